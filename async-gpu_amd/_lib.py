@@ -1,0 +1,149 @@
+"""ctypes binding of include/agpu.h.  Device memory comes from the caller (torch tensors or
+agpu_malloc); every pointer argument accepts an int address, a torch tensor or None."""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libagpu_hip.so")
+
+# error codes of include/agpu.h
+ERR_SHAPE_MISMATCH, ERR_DIM_OUT_OF_RANGE, ERR_KERNEL_NOT_FOUND = -1, -2, -3
+ERR_NULL_POINTER, ERR_UNSUPPORTED, ERR_WORKSPACE = -4, -5, -6
+
+EPI_NONE, EPI_GELU_TANH, EPI_GELU_QUICK, EPI_FORCE_LITERAL = 0, 1, 2, 0x100
+QUANT_RUST, QUANT_SCRIPT = 0, 1
+GELU_TANH, GELU_QUICK = 0, 1
+
+
+class AgpuError(RuntimeError):
+    """Mirrors nn::NnError (nn/error.rs:7-29): .code is the C return value."""
+
+    def __init__(self, code, message):
+        super().__init__(f"agpu error {code}: {message}")
+        self.code = code
+        self.message = message
+
+
+def lib_path():
+    return _SO
+
+
+def library_available():
+    return os.path.exists(_SO)
+
+
+_cdll = None
+
+_i32, _u32, _sz, _vp, _f = C.c_int32, C.c_uint32, C.c_size_t, C.c_void_p, C.c_float
+
+# name -> (restype, argtypes); the complete export list of include/agpu.h
+SIGNATURES = {
+    "agpu_ctx_create": (_i32, [_i32, C.POINTER(_vp)]),
+    "agpu_ctx_create_on_stream": (_i32, [_i32, _vp, C.POINTER(_vp)]),
+    "agpu_ctx_destroy": (_i32, [_vp]),
+    "agpu_last_error_string": (C.c_char_p, [_vp]),
+    "agpu_ctx_stream": (_vp, [_vp]),
+    "agpu_malloc": (_i32, [_vp, _sz, C.POINTER(_vp)]),
+    "agpu_free": (_i32, [_vp, _vp]),
+    "agpu_memcpy_h2d": (_i32, [_vp, _vp, _vp, _sz]),
+    "agpu_memcpy_d2h": (_i32, [_vp, _vp, _vp, _sz]),
+    "agpu_memcpy_d2d": (_i32, [_vp, _vp, _vp, _sz]),
+    "agpu_sync": (_i32, [_vp]),
+    "agpu_kernel_lookup": (_i32, [_vp, C.c_char_p, C.POINTER(C.c_char_p)]),
+    "agpu_int4_linear": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32]),
+    "agpu_ln_int4_linear": (_i32, [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32]),
+    "agpu_int4_dequantize": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32]),
+    "agpu_int4_quantize": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32]),
+    "agpu_int4_quantize_host": (_i32, [_vp, _vp, _vp, _i32, _i32, _i32, _i32]),
+    "agpu_layer_norm": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _f]),
+    "agpu_add_layer_norm_dual": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _f]),
+    "agpu_gelu": (_i32, [_vp, _vp, _vp, _sz, _i32]),
+    "agpu_add_inplace": (_i32, [_vp, _vp, _vp, _sz]),
+    "agpu_bias_add": (_i32, [_vp, _vp, _vp, _i32, _i32]),
+    "agpu_softmax_rows": (_i32, [_vp, _vp, _vp, _i32, _i32]),
+    "agpu_embedding": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32]),
+    "agpu_argmax_rows": (_i32, [_vp, _vp, _vp, _i32, _i32, _i32]),
+    "agpu_split_qkv": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32]),
+    "agpu_concat_heads": (_i32, [_vp, _vp, _vp, _i32, _i32, _i32]),
+    "agpu_attention": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32]),
+    "agpu_kv_append": (_i32, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32]),
+    "agpu_gemm_f32": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32]),
+}
+
+
+def cdll():
+    """Load libagpu_hip.so (once).  No fallback: a missing library is an error."""
+    global _cdll
+    if _cdll is None:
+        if not os.path.exists(_SO):
+            raise AgpuError(ERR_KERNEL_NOT_FOUND,
+                            f"{_SO} is not built; run __graft_entry__.build() (hipcc --offload-arch=gfx950)")
+        lib = C.CDLL(_SO)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _cdll = lib
+    return _cdll
+
+
+def ptr(x):
+    """int address of a torch tensor / numpy array / int / None."""
+    if x is None:
+        return None
+    if isinstance(x, int):
+        return x
+    if hasattr(x, "data_ptr"):
+        return x.data_ptr()
+    if hasattr(x, "ctypes"):
+        return x.ctypes.data
+    raise TypeError(f"cannot take a pointer of {type(x)}")
+
+
+class Context:
+    """KernelRegistry + device handle (nn/registry.rs:26-144).  `stream` is a raw hipStream_t
+    (e.g. torch.cuda.current_stream().cuda_stream); None makes the library create its own."""
+
+    def __init__(self, device=0, stream=None):
+        self._lib = cdll()
+        h = _vp()
+        if stream is None:
+            rc = self._lib.agpu_ctx_create(device, C.byref(h))
+        else:
+            rc = self._lib.agpu_ctx_create_on_stream(device, _vp(stream), C.byref(h))
+        if rc != 0:
+            raise AgpuError(rc, "agpu_ctx_create failed")
+        self.handle = h
+        self.device = device
+
+    def close(self):
+        if getattr(self, "handle", None):
+            self._lib.agpu_ctx_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def call(self, name, *args):
+        fn = getattr(self._lib, name)
+        conv = [ptr(a) if (t is _vp) else a for a, t in zip(args, fn.argtypes[1:])]
+        rc = fn(self.handle, *conv)
+        if rc != 0:
+            raise AgpuError(rc, self._lib.agpu_last_error_string(self.handle).decode())
+        return rc
+
+    def stream(self):
+        return self._lib.agpu_ctx_stream(self.handle)
+
+    def sync(self):
+        self.call("agpu_sync")
+
+    def get(self, name):
+        """registry.get(name): entry point serving a reference kernel name, or KernelNotFound."""
+        out = C.c_char_p()
+        rc = self._lib.agpu_kernel_lookup(self.handle, name.encode(), C.byref(out))
+        if rc != 0:
+            raise AgpuError(rc, self._lib.agpu_last_error_string(self.handle).decode())
+        return out.value.decode()

@@ -1,0 +1,19 @@
+// Launch parameters of the attention kernels, shared by the C ABI wrapper and the model driver.
+#pragma once
+#include "agpu_internal.h"
+
+struct AttnParams {
+    const float *q;  // element (b, h, i, e) at q[b*q_batch_stride + h*q_head_stride + i*q_row_stride + e]
+    const float *k;  // [batch*n_heads, kv_stride, 64]
+    const float *v;
+    float *o;        // element (b, h, i, e) at o[b*o_batch_stride + h*o_head_stride + i*o_row_stride + e]
+    int n_heads, batch, q_len, kv_len, q_offset, kv_stride, causal;
+    long long q_batch_stride, q_head_stride, q_row_stride;
+    long long o_batch_stride, o_head_stride, o_row_stride;
+    // When non-null the kernels read the number of positions already cached from here and use
+    // kv_len = *pos_dev + q_len, q_offset = *pos_dev (lets one captured launch serve every step).
+    const int *pos_dev;
+};
+
+// max_kv_len bounds kv_len for launches that read it from pos_dev (sizes the key split).
+int32_t agpu_attention_launch(agpu_ctx *ctx, const AttnParams &p, int max_kv_len);

@@ -1,0 +1,290 @@
+// Causal attention for gfx950, d_head = 64, fp32.
+//   * attn_mfma_kernel: prefill / chunked prefill.  One wave per 32 query rows; S^T = K Q^T and
+//     O^T = V^T P^T on v_mfma_f32_32x32x2_f32 with online softmax; K/V tiles of 32 keys in LDS.
+//   * attn_splitkv_kernel: decode (few query rows).  The keys are split over workgroups and waves;
+//     16 lanes share one key (float4 each), partial (m, l, o) are merged in a fixed order.
+#include "agpu_internal.h"
+#include "attention.h"
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int DH = 64;
+constexpr int KLD = 68;  // K tile row stride in floats: 8 consecutive lanes' b128 reads hit distinct banks
+
+__device__ __forceinline__ void resolve_positions(const AttnParams &p, int &kv_len, int &q_offset) {
+    kv_len = p.kv_len;
+    q_offset = p.q_offset;
+    if (p.pos_dev) {
+        const int pos = *p.pos_dev;
+        kv_len = pos + p.q_len;
+        q_offset = pos;
+    }
+}
+
+// grid (ceil(q_len/32), n_heads * batch), 64 threads.
+__global__ __launch_bounds__(64) void attn_mfma_kernel(const AttnParams p) {
+    __shared__ __align__(16) float Ks[32 * KLD];
+    __shared__ __align__(16) float Vs[32 * DH];
+    const int lane = threadIdx.x, c = lane & 31, h2 = lane >> 5;
+    const int hb = blockIdx.y, b = hb / p.n_heads, h = hb % p.n_heads;
+    const int i0 = blockIdx.x * 32;
+    int kv_len, q_offset;
+    resolve_positions(p, kv_len, q_offset);
+
+    const float *kh = p.k + (size_t)hb * p.kv_stride * DH;
+    const float *vh = p.v + (size_t)hb * p.kv_stride * DH;
+
+    // Q fragment: lane (c, h2) holds Q[i0+c][32*h2 + s], pre-multiplied by 1/8 (exact).
+    float qreg[32];
+    {
+        const int qi = i0 + c;
+        const float *qrow = p.q + (size_t)b * p.q_batch_stride + (size_t)h * p.q_head_stride + (size_t)qi * p.q_row_stride + 32 * h2;
+#pragma unroll
+        for (int s = 0; s < 32; s += 4) {
+            float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (qi < p.q_len) t = *reinterpret_cast<const float4 *>(qrow + s);
+            qreg[s] = t.x * 0.125f; qreg[s + 1] = t.y * 0.125f; qreg[s + 2] = t.z * 0.125f; qreg[s + 3] = t.w * 0.125f;
+        }
+    }
+    floatx16 o0 = {0}, o1 = {0};
+    float m_run = -INFINITY, l_run = 0.0f;
+    const int last_q = min(p.q_len, i0 + 32) - 1;
+    const int jmax = p.causal ? min(kv_len, q_offset + last_q + 1) : kv_len;  // keys [0, jmax)
+    const int my_limit = p.causal ? q_offset + i0 + c : 0x7fffffff;            // last visible key of my query
+
+    for (int j0 = 0; j0 < jmax; j0 += 32) {
+        // stage K and V rows j0..j0+31 (zero beyond kv_len)
+        __syncthreads();
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int idx = it * 64 + lane;
+            const int r = idx >> 4, c4 = (idx & 15) * 4;
+            float4 kv4 = make_float4(0.f, 0.f, 0.f, 0.f), vv4 = kv4;
+            if (j0 + r < kv_len) {
+                kv4 = *reinterpret_cast<const float4 *>(kh + (size_t)(j0 + r) * DH + c4);
+                vv4 = *reinterpret_cast<const float4 *>(vh + (size_t)(j0 + r) * DH + c4);
+            }
+            *reinterpret_cast<float4 *>(&Ks[r * KLD + c4]) = kv4;
+            *reinterpret_cast<float4 *>(&Vs[r * DH + c4]) = vv4;
+        }
+        __syncthreads();
+
+        // S^T[key][query]: A = K[key = c][32*h2 + s], B = Q[query = c][32*h2 + s]
+        floatx16 sacc = {0};
+        const float *krow = &Ks[c * KLD + 32 * h2];
+#pragma unroll
+        for (int s = 0; s < 32; s += 4) {
+            const float4 k4 = *reinterpret_cast<const float4 *>(krow + s);
+            sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(k4.x, qreg[s], sacc, 0, 0, 0);
+            sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(k4.y, qreg[s + 1], sacc, 0, 0, 0);
+            sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(k4.z, qreg[s + 2], sacc, 0, 0, 0);
+            sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(k4.w, qreg[s + 3], sacc, 0, 0, 0);
+        }
+        // register r holds key j0 + 8*(r/4) + 4*h2 + r%4 for query c
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int j = j0 + 8 * (r >> 2) + 4 * h2 + (r & 3);
+            const bool vis = (j <= my_limit) && (j < kv_len);
+            sacc[r] = vis ? sacc[r] : -INFINITY;
+            tmax = fmaxf(tmax, sacc[r]);
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+        const float m_new = fmaxf(m_run, tmax);
+        // m_new is finite from the first tile on: key 0 is visible to every query.
+        const float alpha = expf(m_run - m_new);
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            sacc[r] = expf(sacc[r] - m_new);
+            psum += sacc[r];
+        }
+        psum += __shfl_xor(psum, 32, kWave);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            o0[r] *= alpha;
+            o1[r] *= alpha;
+        }
+        // O^T[d][query] += V^T[d][key] P^T[key][query]: A = V[key(r,h2)][32*dt + c], B = p[r]
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int kl = 8 * (r >> 2) + 4 * h2 + (r & 3);
+            const float va = Vs[kl * DH + c];
+            const float vb = Vs[kl * DH + 32 + c];
+            o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(va, sacc[r], o0, 0, 0, 0);
+            o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vb, sacc[r], o1, 0, 0, 0);
+        }
+    }
+    const int qi = i0 + c;
+    if (qi < p.q_len) {
+        const float inv_l = 1.0f / l_run;
+        float *orow = p.o + (size_t)b * p.o_batch_stride + (size_t)h * p.o_head_stride + (size_t)qi * p.o_row_stride;
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb) {
+            const int d = 8 * rb + 4 * h2;
+            *reinterpret_cast<float4 *>(orow + d) =
+                make_float4(o0[4 * rb] * inv_l, o0[4 * rb + 1] * inv_l, o0[4 * rb + 2] * inv_l, o0[4 * rb + 3] * inv_l);
+            *reinterpret_cast<float4 *>(orow + 32 + d) =
+                make_float4(o1[4 * rb] * inv_l, o1[4 * rb + 1] * inv_l, o1[4 * rb + 2] * inv_l, o1[4 * rb + 3] * inv_l);
+        }
+    }
+}
+
+// Merge (m, l, o) of `other` into (m, l, o); empty partials have l == 0 and m == -inf.
+__device__ __forceinline__ void merge_partial(float &m, float &l, float4 &o, float m2, float l2, float4 o2) {
+    const float mn = fmaxf(m, m2);
+    if (mn == -INFINITY) return;
+    const float a = expf(m - mn), b = expf(m2 - mn);
+    l = l * a + l2 * b;
+    o.x = o.x * a + o2.x * b; o.y = o.y * a + o2.y * b; o.z = o.z * a + o2.z * b; o.w = o.w * a + o2.w * b;
+    m = mn;
+}
+
+// grid (nsplit, q_len, n_heads * batch), 256 threads.  Workgroup (s, i, hb) takes keys
+// [s*chunk, (s+1)*chunk) that query row i may see.  Lane layout: 16 lanes x float4 per key,
+// 4 keys per wave step, 16 keys per workgroup step.
+__global__ __launch_bounds__(256) void attn_splitkv_kernel(const AttnParams p, int chunk, float *part,
+                                                            unsigned int *counters) {
+    __shared__ float sm[4], sl[4];
+    __shared__ __align__(16) float so[4][DH];
+    __shared__ int s_last;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int gq = lane >> 4, sub = lane & 15;
+    const int split = blockIdx.x, nsplit = gridDim.x, qi = blockIdx.y, hb = blockIdx.z;
+    const int b = hb / p.n_heads, h = hb % p.n_heads;
+    int kv_len, q_offset;
+    resolve_positions(p, kv_len, q_offset);
+    const int vis = p.causal ? min(kv_len, q_offset + qi + 1) : kv_len;  // keys [0, vis)
+    const int ja = split * chunk, jb = min(vis, ja + chunk);
+
+    const float *kh = p.k + (size_t)hb * p.kv_stride * DH;
+    const float *vh = p.v + (size_t)hb * p.kv_stride * DH;
+    const float *qrow = p.q + (size_t)b * p.q_batch_stride + (size_t)h * p.q_head_stride + (size_t)qi * p.q_row_stride;
+    float4 q4 = *reinterpret_cast<const float4 *>(qrow + 4 * sub);
+    q4.x *= 0.125f; q4.y *= 0.125f; q4.z *= 0.125f; q4.w *= 0.125f;
+
+    float m = -INFINITY, l = 0.0f;
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int j = ja + wave * 4 + gq; j < jb; j += 16) {
+        const float4 k4 = *reinterpret_cast<const float4 *>(kh + (size_t)j * DH + 4 * sub);
+        const float4 v4 = *reinterpret_cast<const float4 *>(vh + (size_t)j * DH + 4 * sub);
+        float s = (q4.x * k4.x + q4.y * k4.y) + (q4.z * k4.z + q4.w * k4.w);
+        s += __shfl_xor(s, 8, kWave);
+        s += __shfl_xor(s, 4, kWave);
+        s += __shfl_xor(s, 2, kWave);
+        s += __shfl_xor(s, 1, kWave);
+        const float mn = fmaxf(m, s);
+        const float a = expf(m - mn), pj = expf(s - mn);
+        l = l * a + pj;
+        o.x = o.x * a + pj * v4.x; o.y = o.y * a + pj * v4.y; o.z = o.z * a + pj * v4.z; o.w = o.w * a + pj * v4.w;
+        m = mn;
+    }
+    // merge the 4 lane groups of the wave (xor 16, then xor 32): fixed order
+#pragma unroll
+    for (int off = 16; off <= 32; off <<= 1) {
+        const float m2 = __shfl_xor(m, off, kWave), l2 = __shfl_xor(l, off, kWave);
+        float4 o2;
+        o2.x = __shfl_xor(o.x, off, kWave); o2.y = __shfl_xor(o.y, off, kWave);
+        o2.z = __shfl_xor(o.z, off, kWave); o2.w = __shfl_xor(o.w, off, kWave);
+        // both partners must combine in the same operand order to stay bit-identical
+        if ((lane & off) == 0) merge_partial(m, l, o, m2, l2, o2);
+        else {
+            float mm = m2, ll = l2;
+            float4 oo = o2;
+            merge_partial(mm, ll, oo, m, l, o);
+            m = mm; l = ll; o = oo;
+        }
+    }
+    if (lane < 16) {
+        if (lane == 0) { sm[wave] = m; sl[wave] = l; }
+        *reinterpret_cast<float4 *>(&so[wave][4 * sub]) = o;
+    }
+    __syncthreads();
+    // partial record: [m, l, o[64]] = 66 floats per (hb, qi, split)
+    const size_t rec = ((size_t)hb * p.q_len + qi) * nsplit;
+    if (wave == 0 && lane < 16) {
+        m = sm[0]; l = sl[0];
+        o = *reinterpret_cast<const float4 *>(&so[0][4 * sub]);
+        for (int w = 1; w < 4; ++w) merge_partial(m, l, o, sm[w], sl[w], *reinterpret_cast<const float4 *>(&so[w][4 * sub]));
+        if (nsplit == 1) {
+            const float inv = 1.0f / l;
+            float *orow = p.o + (size_t)b * p.o_batch_stride + (size_t)h * p.o_head_stride + (size_t)qi * p.o_row_stride;
+            *reinterpret_cast<float4 *>(orow + 4 * sub) = make_float4(o.x * inv, o.y * inv, o.z * inv, o.w * inv);
+        } else {
+            float *pr = part + (rec + split) * 66;
+            if (lane == 0) { pr[0] = m; pr[1] = l; }
+            pr[2 + 4 * sub] = o.x; pr[3 + 4 * sub] = o.y; pr[4 + 4 * sub] = o.z; pr[5 + 4 * sub] = o.w;
+        }
+    }
+    if (nsplit == 1) return;
+    __threadfence();
+    __syncthreads();
+    const int cidx = hb * p.q_len + qi;
+    if (tid == 0) {
+        const unsigned int t = atomicAdd(&counters[cidx], 1u);
+        s_last = (t == (unsigned int)(nsplit - 1));
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();
+    if (wave == 0 && lane < 16) {
+        m = -INFINITY; l = 0.0f;
+        o = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int s = 0; s < nsplit; ++s) {
+            const float *pr = part + (rec + s) * 66;
+            const float m2 = __builtin_nontemporal_load(pr), l2 = __builtin_nontemporal_load(pr + 1);
+            float4 o2;
+            o2.x = __builtin_nontemporal_load(pr + 2 + 4 * sub); o2.y = __builtin_nontemporal_load(pr + 3 + 4 * sub);
+            o2.z = __builtin_nontemporal_load(pr + 4 + 4 * sub); o2.w = __builtin_nontemporal_load(pr + 5 + 4 * sub);
+            merge_partial(m, l, o, m2, l2, o2);
+        }
+        const float inv = 1.0f / l;
+        float *orow = p.o + (size_t)b * p.o_batch_stride + (size_t)h * p.o_head_stride + (size_t)qi * p.o_row_stride;
+        *reinterpret_cast<float4 *>(orow + 4 * sub) = make_float4(o.x * inv, o.y * inv, o.z * inv, o.w * inv);
+    }
+    if (tid == 0) counters[cidx] = 0u;
+}
+
+}  // namespace
+
+int32_t agpu_attention_launch(agpu_ctx *ctx, const AttnParams &p, int max_kv_len) {
+    const int hb = p.n_heads * p.batch;
+    if (p.q_len <= 8) {
+        const int chunk = 64;
+        const int nsplit = ceil_div(max_kv_len, chunk);
+        if ((size_t)hb * p.q_len > (size_t)kNumCounters ||
+            (size_t)hb * p.q_len * nsplit * 66 * sizeof(float) > kWorkspaceBytes)
+            return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "attention: heads*q_len*splits too large");
+        hipLaunchKernelGGL(attn_splitkv_kernel, dim3(nsplit, p.q_len, hb), dim3(256), 0, ctx->stream, p, chunk,
+                           reinterpret_cast<float *>(ctx->workspace), ctx->counters);
+        return AGPU_LAUNCH_CHECK(ctx, "attn_splitkv_kernel");
+    }
+    hipLaunchKernelGGL(attn_mfma_kernel, dim3(ceil_div(p.q_len, 32), hb), dim3(64), 0, ctx->stream, p);
+    return AGPU_LAUNCH_CHECK(ctx, "attn_mfma_kernel");
+}
+
+AGPU_EXPORT int32_t agpu_attention(agpu_ctx *ctx, const float *q, const float *k, const float *v, float *o,
+                                   int32_t n_heads, int32_t q_len, int32_t kv_len, int32_t q_offset,
+                                   int32_t kv_stride, int32_t d_head, int32_t causal) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (!q || !k || !v || !o) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "attention: null pointer");
+    if (d_head != DH)
+        return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "attention: expected d_head = 64, got d_head = %d", d_head);
+    if (n_heads <= 0 || q_len < 0 || kv_len < 1 || q_offset < 0 || kv_stride < kv_len)
+        return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH,
+                         "attention: bad dims heads=%d q_len=%d kv_len=%d q_offset=%d kv_stride=%d", n_heads, q_len,
+                         kv_len, q_offset, kv_stride);
+    if (q_len == 0) return AGPU_OK;
+    AttnParams p{};
+    p.q = q; p.k = k; p.v = v; p.o = o;
+    p.n_heads = n_heads; p.batch = 1; p.q_len = q_len; p.kv_len = kv_len; p.q_offset = q_offset;
+    p.kv_stride = kv_stride; p.causal = causal ? 1 : 0;
+    p.q_batch_stride = 0; p.q_head_stride = (long long)q_len * DH; p.q_row_stride = DH;
+    p.o_batch_stride = 0; p.o_head_stride = (long long)q_len * DH; p.o_row_stride = DH;
+    p.pos_dev = nullptr;
+    return agpu_attention_launch(ctx, p, kv_len);
+}

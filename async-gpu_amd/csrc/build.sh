@@ -1,0 +1,19 @@
+#!/bin/bash
+# Compiles libagpu_hip.so for gfx950 in-tree (no GPU needed: hipcc cross-compiles).
+set -euo pipefail
+cd "$(dirname "$0")"
+HIPCC=${HIPCC:-/opt/rocm/bin/hipcc}
+FLAGS=(--offload-arch=gfx950 -O3 -std=c++17 -fPIC -fvisibility=hidden -ffp-contract=off
+       -Xclang -target-feature -Xclang -packed-fp32-ops -Wall -Wno-unused-function)
+mkdir -p build
+pids=()
+for src in *.hip; do
+  obj="build/${src%.hip}.o"
+  "$HIPCC" "${FLAGS[@]}" -c "$src" -o "$obj" &
+  pids+=($!)
+done
+g++ -O2 -std=c++17 -fPIC -fopenmp -fvisibility=hidden -ffp-contract=off -c quantize_host.cpp -o build/quantize_host.o &
+pids+=($!)
+for p in "${pids[@]}"; do wait "$p"; done
+"$HIPCC" --offload-arch=gfx950 -shared -fPIC -o ../libagpu_hip.so build/*.o -fopenmp
+echo "built $(cd .. && pwd)/libagpu_hip.so"

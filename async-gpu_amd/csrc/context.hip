@@ -1,0 +1,175 @@
+// Context, device memory and the kernel-name table of libagpu_hip.so.
+#include <cstring>
+#include <new>
+
+#include "agpu_internal.h"
+
+static int32_t ctx_init(agpu_ctx *c) {
+    hipDeviceProp_t prop;
+    hipError_t e = hipGetDeviceProperties(&prop, c->device);
+    if (e != hipSuccess) return agpu_hip(c, e, "hipGetDeviceProperties");
+    c->num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    e = hipMalloc((void **)&c->workspace, kWorkspaceBytes);
+    if (e != hipSuccess) return agpu_hip(c, e, "hipMalloc(workspace)");
+    e = hipMalloc((void **)&c->counters, kNumCounters * sizeof(unsigned int));
+    if (e != hipSuccess) return agpu_hip(c, e, "hipMalloc(counters)");
+    e = hipMemset(c->counters, 0, kNumCounters * sizeof(unsigned int));
+    if (e != hipSuccess) return agpu_hip(c, e, "hipMemset(counters)");
+    return AGPU_OK;
+}
+
+AGPU_EXPORT int32_t agpu_ctx_create(int32_t device, agpu_ctx **out) {
+    if (!out) return AGPU_ERR_NULL_POINTER;
+    *out = nullptr;
+    hipError_t e = hipSetDevice(device);
+    if (e != hipSuccess) return (int32_t)e;
+    agpu_ctx *c = new (std::nothrow) agpu_ctx();
+    if (!c) return AGPU_ERR_NULL_POINTER;
+    c->device = device;
+    e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) {
+        delete c;
+        return (int32_t)e;
+    }
+    c->owns_stream = true;
+    int32_t rc = ctx_init(c);
+    if (rc != AGPU_OK) {
+        agpu_ctx_destroy(c);
+        return rc;
+    }
+    *out = c;
+    return AGPU_OK;
+}
+
+AGPU_EXPORT int32_t agpu_ctx_create_on_stream(int32_t device, void *hip_stream, agpu_ctx **out) {
+    if (!out) return AGPU_ERR_NULL_POINTER;
+    *out = nullptr;
+    hipError_t e = hipSetDevice(device);
+    if (e != hipSuccess) return (int32_t)e;
+    agpu_ctx *c = new (std::nothrow) agpu_ctx();
+    if (!c) return AGPU_ERR_NULL_POINTER;
+    c->device = device;
+    c->stream = (hipStream_t)hip_stream;
+    c->owns_stream = false;
+    int32_t rc = ctx_init(c);
+    if (rc != AGPU_OK) {
+        agpu_ctx_destroy(c);
+        return rc;
+    }
+    *out = c;
+    return AGPU_OK;
+}
+
+AGPU_EXPORT int32_t agpu_ctx_destroy(agpu_ctx *ctx) {
+    if (!ctx) return AGPU_OK;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream || !ctx->owns_stream) (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->workspace) (void)hipFree(ctx->workspace);
+    if (ctx->counters) (void)hipFree(ctx->counters);
+    if (ctx->owns_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return AGPU_OK;
+}
+
+AGPU_EXPORT const char *agpu_last_error_string(const agpu_ctx *ctx) { return ctx ? ctx->err : "null context"; }
+
+AGPU_EXPORT void *agpu_ctx_stream(const agpu_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
+
+AGPU_EXPORT int32_t agpu_malloc(agpu_ctx *ctx, size_t bytes, void **out) {
+    AGPU_REQUIRE_CTX(ctx);
+    AGPU_REQUIRE_PTR(ctx, out);
+    *out = nullptr;
+    if (bytes == 0) return AGPU_OK;
+    hipError_t e = hipMalloc(out, bytes);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipMalloc");
+    e = hipMemsetAsync(*out, 0, bytes, ctx->stream);
+    return agpu_hip(ctx, e, "hipMemsetAsync");
+}
+
+AGPU_EXPORT int32_t agpu_free(agpu_ctx *ctx, void *ptr) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (!ptr) return AGPU_OK;
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipStreamSynchronize");
+    return agpu_hip(ctx, hipFree(ptr), "hipFree");
+}
+
+AGPU_EXPORT int32_t agpu_memcpy_h2d(agpu_ctx *ctx, void *dst, const void *src_host, size_t bytes) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (bytes == 0) return AGPU_OK;
+    AGPU_REQUIRE_PTR(ctx, dst);
+    AGPU_REQUIRE_PTR(ctx, src_host);
+    hipError_t e = hipMemcpyAsync(dst, src_host, bytes, hipMemcpyHostToDevice, ctx->stream);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipMemcpyAsync(h2d)");
+    return agpu_hip(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+AGPU_EXPORT int32_t agpu_memcpy_d2h(agpu_ctx *ctx, void *dst_host, const void *src, size_t bytes) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (bytes == 0) return AGPU_OK;
+    AGPU_REQUIRE_PTR(ctx, dst_host);
+    AGPU_REQUIRE_PTR(ctx, src);
+    hipError_t e = hipMemcpyAsync(dst_host, src, bytes, hipMemcpyDeviceToHost, ctx->stream);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipMemcpyAsync(d2h)");
+    return agpu_hip(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+AGPU_EXPORT int32_t agpu_memcpy_d2d(agpu_ctx *ctx, void *dst, const void *src, size_t bytes) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (bytes == 0) return AGPU_OK;
+    AGPU_REQUIRE_PTR(ctx, dst);
+    AGPU_REQUIRE_PTR(ctx, src);
+    return agpu_hip(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->stream),
+                    "hipMemcpyAsync(d2d)");
+}
+
+AGPU_EXPORT int32_t agpu_sync(agpu_ctx *ctx) {
+    AGPU_REQUIRE_CTX(ctx);
+    return agpu_hip(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+// The reference's kernel names on this path (nn/registry.rs:34-103) and the entry
+// point that serves each.
+static const struct {
+    const char *name;
+    const char *entry;
+} kKernelTable[] = {
+    {"int4_gemm_w4a16", "agpu_int4_linear"},
+    {"bias_add", "agpu_bias_add"},
+    {"layer_norm", "agpu_layer_norm"},
+    {"layer_norm_v2", "agpu_layer_norm"},
+    {"layer_norm_v3", "agpu_layer_norm"},
+    {"layer_norm_residual", "agpu_add_layer_norm_dual"},
+    {"layer_norm_residual_dual", "agpu_add_layer_norm_dual"},
+    {"gelu_forward", "agpu_gelu"},
+    {"gelu_forward_v2", "agpu_gelu"},
+    {"elementwise_add", "agpu_add_inplace"},
+    {"elementwise_add_v2", "agpu_add_inplace"},
+    {"elementwise_add_v3", "agpu_add_inplace"},
+    {"split_qkv", "agpu_split_qkv"},
+    {"concat_heads", "agpu_concat_heads"},
+    {"flash_attention", "agpu_attention"},
+    {"flash_attention_v2", "agpu_attention"},
+    {"flash_attn_v3", "agpu_attention"},
+    {"flash_attention_kv", "agpu_attention"},
+    {"kv_cache_append", "agpu_kv_append"},
+    {"embedding_lookup", "agpu_embedding"},
+    {"gemm_f32", "agpu_gemm_f32"},
+    {"gemm_f32_v2", "agpu_gemm_f32"},
+    {"gemm_f32_v3", "agpu_gemm_f32"},
+};
+
+AGPU_EXPORT int32_t agpu_kernel_lookup(const agpu_ctx *ctx, const char *name, const char **entry_point_out) {
+    if (entry_point_out) *entry_point_out = nullptr;
+    if (!name) return AGPU_ERR_NULL_POINTER;
+    for (const auto &e : kKernelTable) {
+        if (std::strcmp(e.name, name) == 0) {
+            if (entry_point_out) *entry_point_out = e.entry;
+            return AGPU_OK;
+        }
+    }
+    if (ctx) {
+        agpu_fail(const_cast<agpu_ctx *>(ctx), AGPU_ERR_KERNEL_NOT_FOUND, "kernel not found in registry: %s", name);
+    }
+    return AGPU_ERR_KERNEL_NOT_FOUND;
+}

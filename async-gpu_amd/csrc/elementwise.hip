@@ -1,0 +1,390 @@
+// LayerNorm, add+LayerNorm, GELU, residual add, bias add, row softmax, embedding, argmax and
+// the QKV layout kernels.  All of them move each byte once: they are HBM-bound, one wave per
+// row where a row reduction is needed.
+#include "agpu_internal.h"
+
+namespace {
+
+constexpr int LN_CACHE = 32;  // values per lane kept in registers: rows up to 2048 wide are read once
+
+// One wave per row.  Two-pass statistics (mean, then centred second moment), as
+// nn/cpu_ref.rs:38-47 does; population variance, eps inside the square root.
+// ADD: x = a + b first (nn/ops/norm.rs:105-196), optionally stored to sum_out.
+template <bool ADD>
+__global__ __launch_bounds__(256) void layer_norm_kernel(const float *a, const float *b, const float *__restrict__ gamma,
+                                                          const float *__restrict__ beta, float *sum_out, float *y,
+                                                          int rows, int d, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float *ar = a + (size_t)row * d;
+    const float *br = ADD ? b + (size_t)row * d : nullptr;
+    float *sr = (ADD && sum_out) ? sum_out + (size_t)row * d : nullptr;
+    float *yr = y + (size_t)row * d;
+    const bool cached = d <= 64 * LN_CACHE;
+    float v[LN_CACHE];
+    float s = 0.0f;
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < LN_CACHE; ++i) {
+            const int k = lane + 64 * i;
+            float t = 0.0f;
+            if (k < d) {
+                t = ar[k];
+                if (ADD) {
+                    t += br[k];
+                    if (sr) sr[k] = t;
+                }
+            }
+            v[i] = t;
+            s += t;
+        }
+    } else {
+        for (int k = lane; k < d; k += 64) {
+            float t = ar[k];
+            if (ADD) {
+                t += br[k];
+                if (sr) sr[k] = t;
+            }
+            s += t;
+        }
+    }
+    const float mean = wave_sum(s) / (float)d;
+    float q = 0.0f;
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < LN_CACHE; ++i) {
+            const int k = lane + 64 * i;
+            if (k < d) {
+                const float df = v[i] - mean;
+                q += df * df;
+            }
+        }
+    } else {
+        for (int k = lane; k < d; k += 64) {
+            const float t = ADD ? ar[k] + br[k] : ar[k];
+            const float df = t - mean;
+            q += df * df;
+        }
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)d + eps);
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < LN_CACHE; ++i) {
+            const int k = lane + 64 * i;
+            if (k < d) yr[k] = (v[i] - mean) * rstd * gamma[k] + beta[k];
+        }
+    } else {
+        for (int k = lane; k < d; k += 64) {
+            const float t = ADD ? ar[k] + br[k] : ar[k];
+            yr[k] = (t - mean) * rstd * gamma[k] + beta[k];
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void gelu_kernel(const float *x, float *y, size_t n, int mode) {
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i + 3 < n && (((uintptr_t)x | (uintptr_t)y) & 15) == 0) {
+        float4 v = *reinterpret_cast<const float4 *>(x + i);
+        if (mode == AGPU_GELU_TANH) {
+            v.x = gelu_tanh_dev(v.x); v.y = gelu_tanh_dev(v.y); v.z = gelu_tanh_dev(v.z); v.w = gelu_tanh_dev(v.w);
+        } else {
+            v.x = gelu_quick_dev(v.x); v.y = gelu_quick_dev(v.y); v.z = gelu_quick_dev(v.z); v.w = gelu_quick_dev(v.w);
+        }
+        *reinterpret_cast<float4 *>(y + i) = v;
+    } else {
+        for (size_t j = i; j < n && j < i + 4; ++j)
+            y[j] = mode == AGPU_GELU_TANH ? gelu_tanh_dev(x[j]) : gelu_quick_dev(x[j]);
+    }
+}
+
+__global__ __launch_bounds__(256) void add_inplace_kernel(float *a, const float *__restrict__ b, size_t n) {
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i + 3 < n && (((uintptr_t)a | (uintptr_t)b) & 15) == 0) {
+        float4 u = *reinterpret_cast<float4 *>(a + i);
+        const float4 w = *reinterpret_cast<const float4 *>(b + i);
+        u.x += w.x; u.y += w.y; u.z += w.z; u.w += w.w;
+        *reinterpret_cast<float4 *>(a + i) = u;
+    } else {
+        for (size_t j = i; j < n && j < i + 4; ++j) a[j] += b[j];
+    }
+}
+
+__global__ __launch_bounds__(256) void bias_add_kernel(float *data, const float *__restrict__ bias, size_t total,
+                                                        int n_cols) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < total) data[i] += bias[i % (size_t)n_cols];
+}
+
+// One wave per row; expf (not the fast exponent) and a true division.
+__global__ __launch_bounds__(256) void softmax_rows_kernel(const float *x, float *y, int rows, int cols) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float *xr = x + (size_t)row * cols;
+    float *yr = y + (size_t)row * cols;
+    float mx = -INFINITY;
+    for (int k = lane; k < cols; k += 64) mx = fmaxf(mx, xr[k]);
+    mx = wave_max(mx);
+    float s = 0.0f;
+    for (int k = lane; k < cols; k += 64) s += expf(xr[k] - mx);
+    s = wave_sum(s);
+    for (int k = lane; k < cols; k += 64) yr[k] = expf(xr[k] - mx) / s;
+}
+
+// out[p,:] = wte[tok[p],:] + wpe[p+pos_offset,:]  (compute_transformer.rs:1320-1329)
+__global__ __launch_bounds__(256) void embedding_kernel(const uint32_t *__restrict__ tokens,
+                                                         const float *__restrict__ wte,
+                                                         const float *__restrict__ wpe, float *out, int seq, int d,
+                                                         int pos_offset) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (size_t)seq * d) return;
+    const int p = (int)(i / d), j = (int)(i % d);
+    out[i] = wte[(size_t)tokens[p] * d + j] + wpe[(size_t)(p + pos_offset) * d + j];
+}
+
+// [seq,3d] -> Q,K,V [H,seq,dh]  (compute_transformer.rs:1620-1660)
+__global__ __launch_bounds__(256) void split_qkv_kernel(const float *__restrict__ qkv, float *q, float *k, float *v,
+                                                         int seq, int n_heads, int d_head) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const int d = n_heads * d_head;
+    if (i >= (size_t)seq * d) return;
+    const int e = (int)(i % d_head);
+    const int s = (int)((i / d_head) % seq);
+    const int h = (int)(i / ((size_t)d_head * seq));
+    const size_t src = (size_t)s * 3 * d + (size_t)h * d_head + e;
+    q[i] = qkv[src];
+    k[i] = qkv[src + d];
+    v[i] = qkv[src + 2 * d];
+}
+
+// [H,seq,dh] -> [seq,H*dh]  (compute_transformer.rs:1671-1703)
+__global__ __launch_bounds__(256) void concat_heads_kernel(const float *__restrict__ in, float *out, int seq,
+                                                            int n_heads, int d_head) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const int d = n_heads * d_head;
+    if (i >= (size_t)seq * d) return;
+    const int j = (int)(i % d), s = (int)(i / d);
+    const int h = j / d_head, e = j % d_head;
+    out[i] = in[((size_t)h * seq + s) * d_head + e];
+}
+
+// row 0 of src [H, src_stride, dh] -> cache[h, write_pos, :]  (compute_transformer.rs:1777-1812)
+__global__ __launch_bounds__(256) void kv_append_kernel(const float *__restrict__ src, float *cache, int n_heads,
+                                                         int src_stride, int max_seq, int write_pos, int d_head) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n_heads * d_head) return;
+    const int h = i / d_head, e = i % d_head;
+    cache[((size_t)h * max_seq + write_pos) * d_head + e] = src[(size_t)h * src_stride * d_head + e];
+}
+
+// Arg-max of each row in two levels: every workgroup reduces one chunk to (value, index),
+// the last workgroup of a row to arrive reduces the chunk results in chunk order.
+// Ties: the smaller index wins (last_index == 0) or the larger one.
+__device__ __forceinline__ bool better(float v, unsigned int i, float bv, unsigned int bi, int last_index) {
+    return (v > bv) || (v == bv && (last_index ? i > bi : i < bi));
+}
+
+__global__ __launch_bounds__(256) void argmax_rows_kernel(const float *__restrict__ x, uint32_t *idx_out,
+                                                           float *part_val, unsigned int *part_idx,
+                                                           unsigned int *counters, int cols, int chunk,
+                                                           int last_index) {
+    __shared__ float sv[4];
+    __shared__ unsigned int si[4];
+    __shared__ int s_last;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int row = blockIdx.y, nchunks = gridDim.x;
+    const float *xr = x + (size_t)row * cols;
+    const int c0 = blockIdx.x * chunk, c1 = min(cols, c0 + chunk);
+    float bv = -INFINITY;
+    unsigned int bi = last_index ? 0u : 0xFFFFFFFFu;
+    for (int c = c0 + tid; c < c1; c += 256) {
+        const float v = xr[c];
+        if (better(v, (unsigned int)c, bv, bi, last_index)) { bv = v; bi = (unsigned int)c; }
+    }
+    auto wave_reduce = [&](float &v, unsigned int &i) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ov = __shfl_xor(v, off, kWave);
+            const unsigned int oi = __shfl_xor(i, off, kWave);
+            if (better(ov, oi, v, i, last_index)) { v = ov; i = oi; }
+        }
+    };
+    wave_reduce(bv, bi);
+    if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < 4; ++w)
+            if (better(sv[w], si[w], bv, bi, last_index)) { bv = sv[w]; bi = si[w]; }
+        if (nchunks == 1) {
+            idx_out[row] = (bi == 0xFFFFFFFFu) ? 0u : bi;
+        } else {
+            part_val[(size_t)row * nchunks + blockIdx.x] = bv;
+            part_idx[(size_t)row * nchunks + blockIdx.x] = bi;
+        }
+    }
+    if (nchunks == 1) return;
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned int t = atomicAdd(&counters[row], 1u);
+        s_last = (t == (unsigned int)(nchunks - 1));
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();
+    if (wave == 0) {
+        bv = -INFINITY;
+        bi = last_index ? 0u : 0xFFFFFFFFu;
+        for (int c = lane; c < nchunks; c += 64) {
+            const float v = __builtin_nontemporal_load(&part_val[(size_t)row * nchunks + c]);
+            const unsigned int i = __builtin_nontemporal_load(&part_idx[(size_t)row * nchunks + c]);
+            if (better(v, i, bv, bi, last_index)) { bv = v; bi = i; }
+        }
+        wave_reduce(bv, bi);
+        if (lane == 0) {
+            idx_out[row] = (bi == 0xFFFFFFFFu) ? 0u : bi;
+            counters[row] = 0u;
+        }
+    }
+}
+
+inline unsigned grid_1d(size_t n, int per_block) { return (unsigned)((n + per_block - 1) / per_block); }
+
+}  // namespace
+
+int32_t agpu_layer_norm_impl(agpu_ctx *ctx, const float *x, const float *gamma, const float *beta, float *y,
+                             int rows, int d, float eps) {
+    hipLaunchKernelGGL((layer_norm_kernel<false>), dim3(ceil_div(rows, 4)), dim3(256), 0, ctx->stream, x,
+                       (const float *)nullptr, gamma, beta, (float *)nullptr, y, rows, d, eps);
+    return AGPU_LAUNCH_CHECK(ctx, "layer_norm_kernel");
+}
+
+AGPU_EXPORT int32_t agpu_layer_norm(agpu_ctx *ctx, const float *x, const float *gamma, const float *beta, float *y,
+                                    int32_t rows, int32_t d, float eps) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (!x || !gamma || !beta || !y) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "layer_norm: null pointer");
+    if (rows < 0 || d <= 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "layer_norm: bad dims rows=%d d=%d", rows, d);
+    if (rows == 0) return AGPU_OK;
+    return agpu_layer_norm_impl(ctx, x, gamma, beta, y, rows, d, eps);
+}
+
+AGPU_EXPORT int32_t agpu_add_layer_norm_dual(agpu_ctx *ctx, const float *a, const float *b, const float *gamma,
+                                             const float *beta, float *sum_out, float *norm_out, int32_t rows,
+                                             int32_t d, float eps) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (!a || !b || !gamma || !beta || !norm_out)
+        return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "add_layer_norm_dual: null pointer");
+    if (rows < 0 || d <= 0)
+        return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "add_layer_norm_dual: bad dims rows=%d d=%d", rows, d);
+    if (rows == 0) return AGPU_OK;
+    hipLaunchKernelGGL((layer_norm_kernel<true>), dim3(ceil_div(rows, 4)), dim3(256), 0, ctx->stream, a, b, gamma,
+                       beta, sum_out, norm_out, rows, d, eps);
+    return AGPU_LAUNCH_CHECK(ctx, "add_layer_norm_kernel");
+}
+
+AGPU_EXPORT int32_t agpu_gelu(agpu_ctx *ctx, const float *x, float *y, size_t n, int32_t mode) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (n == 0) return AGPU_OK;
+    if (!x || !y) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "gelu: null pointer");
+    if (mode != AGPU_GELU_TANH && mode != AGPU_GELU_QUICK)
+        return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "gelu: unknown mode %d", mode);
+    hipLaunchKernelGGL(gelu_kernel, dim3(grid_1d(n, 1024)), dim3(256), 0, ctx->stream, x, y, n, mode);
+    return AGPU_LAUNCH_CHECK(ctx, "gelu_kernel");
+}
+
+AGPU_EXPORT int32_t agpu_add_inplace(agpu_ctx *ctx, float *a, const float *b, size_t n) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (n == 0) return AGPU_OK;
+    if (!a || !b) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "add_inplace: null pointer");
+    hipLaunchKernelGGL(add_inplace_kernel, dim3(grid_1d(n, 1024)), dim3(256), 0, ctx->stream, a, b, n);
+    return AGPU_LAUNCH_CHECK(ctx, "add_inplace_kernel");
+}
+
+AGPU_EXPORT int32_t agpu_bias_add(agpu_ctx *ctx, float *data, const float *bias, int32_t rows, int32_t n_cols) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (!data || !bias) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "bias_add: null pointer");
+    if (rows < 0 || n_cols <= 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "bias_add: bad dims rows=%d n_cols=%d", rows, n_cols);
+    const size_t total = (size_t)rows * n_cols;
+    if (total == 0) return AGPU_OK;
+    hipLaunchKernelGGL(bias_add_kernel, dim3(grid_1d(total, 256)), dim3(256), 0, ctx->stream, data, bias, total, n_cols);
+    return AGPU_LAUNCH_CHECK(ctx, "bias_add_kernel");
+}
+
+AGPU_EXPORT int32_t agpu_softmax_rows(agpu_ctx *ctx, const float *x, float *y, int32_t rows, int32_t cols) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (!x || !y) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "softmax_rows: null pointer");
+    if (rows < 0 || cols <= 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "softmax_rows: bad dims rows=%d cols=%d", rows, cols);
+    if (rows == 0) return AGPU_OK;
+    hipLaunchKernelGGL(softmax_rows_kernel, dim3(ceil_div(rows, 4)), dim3(256), 0, ctx->stream, x, y, rows, cols);
+    return AGPU_LAUNCH_CHECK(ctx, "softmax_rows_kernel");
+}
+
+AGPU_EXPORT int32_t agpu_embedding(agpu_ctx *ctx, const uint32_t *tokens, const float *wte, const float *wpe,
+                                   float *out, int32_t seq, int32_t d, int32_t pos_offset) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (!tokens || !wte || !wpe || !out) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "embedding: null pointer");
+    if (seq < 0 || d <= 0 || pos_offset < 0)
+        return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "embedding: bad dims seq=%d d=%d pos_offset=%d", seq, d, pos_offset);
+    if (seq == 0) return AGPU_OK;
+    hipLaunchKernelGGL(embedding_kernel, dim3(grid_1d((size_t)seq * d, 256)), dim3(256), 0, ctx->stream, tokens, wte,
+                       wpe, out, seq, d, pos_offset);
+    return AGPU_LAUNCH_CHECK(ctx, "embedding_kernel");
+}
+
+AGPU_EXPORT int32_t agpu_argmax_rows(agpu_ctx *ctx, const float *x, uint32_t *idx_out, int32_t rows, int32_t cols,
+                                     int32_t last_index) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (!x || !idx_out) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "argmax_rows: null pointer");
+    if (rows < 0 || cols <= 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "argmax_rows: bad dims rows=%d cols=%d", rows, cols);
+    if (rows == 0) return AGPU_OK;
+    if (rows > kNumCounters) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "argmax_rows: rows=%d too large", rows);
+    const int chunk = 2048;
+    const int nchunks = ceil_div(cols, chunk);
+    if ((size_t)rows * nchunks * 8 > kWorkspaceBytes)
+        return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "argmax_rows: rows*cols too large");
+    float *pv = reinterpret_cast<float *>(ctx->workspace);
+    unsigned int *pi = reinterpret_cast<unsigned int *>(ctx->workspace) + (size_t)rows * nchunks;
+    hipLaunchKernelGGL(argmax_rows_kernel, dim3(nchunks, rows), dim3(256), 0, ctx->stream, x, idx_out, pv, pi,
+                       ctx->counters, cols, chunk, last_index ? 1 : 0);
+    return AGPU_LAUNCH_CHECK(ctx, "argmax_rows_kernel");
+}
+
+AGPU_EXPORT int32_t agpu_split_qkv(agpu_ctx *ctx, const float *qkv, float *q, float *k, float *v, int32_t seq,
+                                   int32_t n_heads, int32_t d_head) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (!qkv || !q || !k || !v) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "split_qkv: null pointer");
+    if (seq < 0 || n_heads <= 0 || d_head <= 0)
+        return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "split_qkv: bad dims seq=%d heads=%d d_head=%d", seq, n_heads, d_head);
+    const size_t total = (size_t)seq * n_heads * d_head;
+    if (total == 0) return AGPU_OK;
+    hipLaunchKernelGGL(split_qkv_kernel, dim3(grid_1d(total, 256)), dim3(256), 0, ctx->stream, qkv, q, k, v, seq,
+                       n_heads, d_head);
+    return AGPU_LAUNCH_CHECK(ctx, "split_qkv_kernel");
+}
+
+AGPU_EXPORT int32_t agpu_concat_heads(agpu_ctx *ctx, const float *in, float *out, int32_t seq, int32_t n_heads,
+                                      int32_t d_head) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (!in || !out) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "concat_heads: null pointer");
+    if (seq < 0 || n_heads <= 0 || d_head <= 0)
+        return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "concat_heads: bad dims seq=%d heads=%d d_head=%d", seq, n_heads, d_head);
+    const size_t total = (size_t)seq * n_heads * d_head;
+    if (total == 0) return AGPU_OK;
+    hipLaunchKernelGGL(concat_heads_kernel, dim3(grid_1d(total, 256)), dim3(256), 0, ctx->stream, in, out, seq,
+                       n_heads, d_head);
+    return AGPU_LAUNCH_CHECK(ctx, "concat_heads_kernel");
+}
+
+AGPU_EXPORT int32_t agpu_kv_append(agpu_ctx *ctx, const float *src, float *cache, int32_t n_heads,
+                                   int32_t src_stride, int32_t max_seq, int32_t write_pos, int32_t d_head) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (!src || !cache) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "kv_append: null pointer");
+    if (n_heads <= 0 || d_head <= 0 || src_stride <= 0 || max_seq <= 0)
+        return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "kv_append: bad dims");
+    if (write_pos < 0 || write_pos >= max_seq)
+        return agpu_fail(ctx, AGPU_ERR_DIM_OUT_OF_RANGE, "kv_append: write_pos %d out of range for max_seq %d", write_pos, max_seq);
+    hipLaunchKernelGGL(kv_append_kernel, dim3(grid_1d((size_t)n_heads * d_head, 256)), dim3(256), 0, ctx->stream, src,
+                       cache, n_heads, src_stride, max_seq, write_pos, d_head);
+    return AGPU_LAUNCH_CHECK(ctx, "kv_append_kernel");
+}

@@ -1,0 +1,182 @@
+/*
+ * agpu.h — C ABI of libagpu_hip.so: hand-written gfx950 (MI355X) kernels behind the
+ * operator surface of async_gpu's `nn` module, for the quantized GPT-2 inference path.
+ *
+ * What this boundary replaces in the reference (paths relative to the reference
+ * checkout, crates/core/gpu-host/src/ unless a crate is named):
+ *   - nn/registry.rs:34-144   `KernelRegistry::{new,get}` + `func.launch(cfg, args)`:
+ *     one C function per kernel the path loads; agpu_kernel_lookup() answers
+ *     the `get(name)` question for the reference's kernel names.
+ *   - nn/ops/ wrappers        shape checks move into these functions; outputs are
+ *     caller-allocated (the Rust/C++ wrapper allocates, as nn/ops does today).
+ *   - nn/error.rs:7-29        NnError -> int32 codes below.
+ *
+ * Conventions
+ *   - all tensors dense, row-major, fp32; packed weights and token ids uint32;
+ *   - every pointer is a DEVICE pointer unless the parameter name ends in `_host`;
+ *   - every launcher is asynchronous on the context's stream, in call order; none
+ *     allocates or synchronises, so a sequence of calls may be captured in a HIP graph;
+ *   - return value: 0 ok; <0 argument/shape error found on the host before any
+ *     launch; >0 a hipError_t.  agpu_last_error_string() describes the last failure.
+ *   - a context is used by one thread at a time; different contexts are independent.
+ */
+#ifndef AGPU_H
+#define AGPU_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AGPU_OK 0
+#define AGPU_ERR_SHAPE_MISMATCH (-1)   /* NnError::ShapeMismatch   (nn/error.rs:9-14)  */
+#define AGPU_ERR_DIM_OUT_OF_RANGE (-2) /* NnError::DimOutOfRange   (nn/error.rs:16-21) */
+#define AGPU_ERR_KERNEL_NOT_FOUND (-3) /* NnError::KernelNotFound  (nn/error.rs:23-26) */
+#define AGPU_ERR_NULL_POINTER (-4)
+#define AGPU_ERR_UNSUPPORTED (-5)
+#define AGPU_ERR_WORKSPACE (-6)        /* split-K scratch too small for the request */
+
+typedef struct agpu_ctx agpu_ctx;
+
+/* ---- context, memory (cudarc CudaDevice as used by nn/tensor.rs:47-120) ------------- */
+
+/* KernelRegistry::init_default (nn/registry.rs:131-135): device + its own stream. */
+int32_t agpu_ctx_create(int32_t device, agpu_ctx **out);
+/* Same, but launches go to a stream the caller owns (hipStream_t passed as void*;
+ * NULL = the legacy default stream).  For hosts that already have a stream. */
+int32_t agpu_ctx_create_on_stream(int32_t device, void *hip_stream, agpu_ctx **out);
+int32_t agpu_ctx_destroy(agpu_ctx *ctx);
+const char *agpu_last_error_string(const agpu_ctx *ctx);
+void *agpu_ctx_stream(const agpu_ctx *ctx);
+
+int32_t agpu_malloc(agpu_ctx *ctx, size_t bytes, void **out);              /* alloc_zeros: memory is zeroed */
+int32_t agpu_free(agpu_ctx *ctx, void *ptr);
+int32_t agpu_memcpy_h2d(agpu_ctx *ctx, void *dst, const void *src_host, size_t bytes); /* htod_sync_copy */
+int32_t agpu_memcpy_d2h(agpu_ctx *ctx, void *dst_host, const void *src, size_t bytes); /* dtoh_sync_copy */
+int32_t agpu_memcpy_d2d(agpu_ctx *ctx, void *dst, const void *src, size_t bytes);      /* clone_tensor, tensor.rs:270-282 */
+int32_t agpu_sync(agpu_ctx *ctx);                                                       /* dev.synchronize() */
+
+/* registry.get(name) (nn/registry.rs:140-144): 0 if `name` is one of the reference's
+ * kernel names this library implements, AGPU_ERR_KERNEL_NOT_FOUND otherwise.
+ * *entry_point_out (optional) receives the name of the C function that serves it. */
+int32_t agpu_kernel_lookup(const agpu_ctx *ctx, const char *name, const char **entry_point_out);
+
+/* ---- int4 weight-only Linear ---------------------------------------------------------- */
+
+/* Epilogue flags for agpu_int4_linear. */
+#define AGPU_EPI_NONE 0u
+#define AGPU_EPI_GELU_TANH 1u  /* compute_transformer.rs:396-443 (tanh form) applied after bias   */
+#define AGPU_EPI_GELU_QUICK 2u /* compute_transformer.rs:1468-1531, x*sigmoid(1.702x)             */
+#define AGPU_EPI_FORCE_LITERAL 0x100u /* one thread per output, fma chain in ascending k — the
+                                          reference kernel's own arithmetic order               */
+
+/*
+ * Y[M,N] = X[M,K] * deq(W) (+ bias[N]) (-> GELU) (+ residual[M,N]).
+ * Replaces kernel int4_gemm_w4a16 (crates/kernel/gpu-kernel-compute/src/compute_gemm.rs:2849-2910)
+ * + bias_add (compute_transformer.rs:1354-1387) as driven by Int4Linear::forward
+ * (nn/layers/int4_linear.rs:71-133) and ops::int4_matmul (nn/ops/gemm.rs:1243-1262).
+ *   packed [K/8, N] u32: nibble i (bits 4i..4i+3) of word [kp, n] holds q(8kp+i, n)+8
+ *   scales [ceil(K/group), N] f32;  w = (float)(nibble-8) * scale[k/group, n]
+ * bias and residual may be NULL; residual may alias y.  K % 8 == 0 is required
+ * (nn/ops/quantize.rs:109); otherwise AGPU_ERR_SHAPE_MISMATCH.
+ */
+int32_t agpu_int4_linear(agpu_ctx *ctx, const float *x, const uint32_t *packed, const float *scales,
+                         const float *bias, const float *residual, float *y, int32_t M, int32_t N,
+                         int32_t K, int32_t group, uint32_t flags);
+
+/* Same with LayerNorm(x; gamma, beta, eps) over K applied to each input row first
+ * (ops::layer_norm followed by Int4Linear::forward, gpt2.rs:1307-1316,1329-1331). */
+int32_t agpu_ln_int4_linear(agpu_ctx *ctx, const float *x, const float *gamma, const float *beta,
+                            float eps, const uint32_t *packed, const float *scales, const float *bias,
+                            const float *residual, float *y, int32_t M, int32_t N, int32_t K,
+                            int32_t group, uint32_t flags);
+
+/* W[K,N] = (float)(nibble-8) * scale: the kernel's inline dequantisation
+ * (compute_gemm.rs:2882-2886) / nn/ops/quantize.rs:158-162 as a standalone, bit-exact hook. */
+int32_t agpu_int4_dequantize(agpu_ctx *ctx, const uint32_t *packed, const float *scales, float *w_out,
+                             int32_t K, int32_t N, int32_t group);
+
+#define AGPU_QUANT_RUST 0   /* nn/ops/quantize.rs:102-153: round half away, v * (1/scale) */
+#define AGPU_QUANT_SCRIPT 1 /* scripts/quantize_gpt2_int4.py:21-62: round half even, v / scale */
+/* quantize_weight_int4 on the device: weight_t [K,N] f32 -> packed, scales. */
+int32_t agpu_int4_quantize(agpu_ctx *ctx, const float *weight_t, uint32_t *packed, float *scales,
+                           int32_t K, int32_t N, int32_t group, int32_t mode);
+/* The same function on the host CPU, where the reference runs it (host pointers). */
+int32_t agpu_int4_quantize_host(const float *weight_t_host, uint32_t *packed_host, float *scales_host,
+                                int32_t K, int32_t N, int32_t group, int32_t mode);
+
+/* ---- normalisation, activation, elementwise ------------------------------------------- */
+
+/* ops::layer_norm (nn/ops/norm.rs:14-81) -> layer_norm_v3 (compute_transformer.rs:236-385).
+ * Two-pass mean/variance as the CPU reference does (nn/cpu_ref.rs:38-47). */
+int32_t agpu_layer_norm(agpu_ctx *ctx, const float *x, const float *gamma, const float *beta, float *y,
+                        int32_t rows, int32_t d, float eps);
+/* ops::layer_norm_residual_dual (nn/ops/norm.rs:248-400): sum = a+b, norm = LN(sum).
+ * sum_out may be NULL (layer_norm_residual, norm.rs:88-237) and may alias a. */
+int32_t agpu_add_layer_norm_dual(agpu_ctx *ctx, const float *a, const float *b, const float *gamma,
+                                 const float *beta, float *sum_out, float *norm_out, int32_t rows,
+                                 int32_t d, float eps);
+#define AGPU_GELU_TANH 0
+#define AGPU_GELU_QUICK 1
+/* ops::gelu (nn/ops/activation.rs:14-16,79-108); mode picks gelu_forward / gelu_forward_v2. y may alias x. */
+int32_t agpu_gelu(agpu_ctx *ctx, const float *x, float *y, size_t n, int32_t mode);
+/* ops::elementwise_add (nn/ops/reshape.rs:161-186): a += b. */
+int32_t agpu_add_inplace(agpu_ctx *ctx, float *a, const float *b, size_t n);
+/* ops::bias_add (nn/ops/reshape.rs:112-136): data[r, j] += bias[j]. */
+int32_t agpu_bias_add(agpu_ctx *ctx, float *data, const float *bias, int32_t rows, int32_t n_cols);
+/* Row softmax; CPU twin cpu_softmax_f64 (nn/cpu_ref.rs:111-125). y may alias x. */
+int32_t agpu_softmax_rows(agpu_ctx *ctx, const float *x, float *y, int32_t rows, int32_t cols);
+/* ops::embedding_lookup (nn/ops/reshape.rs:301-335) with the position offset of
+ * Embedding::forward_tokens_with_offset (nn/layers/embedding.rs:59-93):
+ * out[p,:] = wte[tok[p],:] + wpe[p+pos_offset,:].  Token ids >= vocab or positions
+ * >= n_positions are rejected on the host only when the ids are host-known; here the
+ * caller guarantees them, as the reference kernel does (compute_transformer.rs:1324-1328). */
+int32_t agpu_embedding(agpu_ctx *ctx, const uint32_t *tokens, const float *wte, const float *wpe,
+                       float *out, int32_t seq, int32_t d, int32_t pos_offset);
+/* First index of the row maximum (tests_inference.rs:4504-4515 tie rule); last_index != 0
+ * gives the last one instead (Iterator::max_by, gpt2.rs:991-997). */
+int32_t agpu_argmax_rows(agpu_ctx *ctx, const float *x, uint32_t *idx_out, int32_t rows, int32_t cols,
+                         int32_t last_index);
+
+/* ---- attention ------------------------------------------------------------------------- */
+
+/* ops::split_qkv (nn/ops/attention.rs:105-142): [seq,3d] -> Q,K,V [H,seq,dh]. */
+int32_t agpu_split_qkv(agpu_ctx *ctx, const float *qkv, float *q, float *k, float *v, int32_t seq,
+                       int32_t n_heads, int32_t d_head);
+/* ops::concat_heads (nn/ops/attention.rs:515-549): [H,seq,dh] -> [seq,H*dh]. */
+int32_t agpu_concat_heads(agpu_ctx *ctx, const float *in, float *out, int32_t seq, int32_t n_heads,
+                          int32_t d_head);
+/*
+ * Attention of q_len new query rows against kv_len keys, every head in one launch.
+ * Replaces flash_attention / _v2 (compute_transformer.rs:597-816,837-1065),
+ * flash_attn_v3.cu and flash_attention_kv (compute_transformer.rs:1076-1288) behind
+ * ops::multi_head_flash_attention (nn/ops/attention.rs:151-202) and
+ * ops::scaled_dot_product_attention_kv (nn/ops/attention.rs:557-606).
+ *   q,o [H, q_len, 64]; k,v [H, kv_stride, 64] with the first kv_len rows valid;
+ *   key j is visible to query row i iff !causal or j <= q_offset + i;
+ *   scale = 1/sqrt(d_head) applied to the dot product.
+ * Prefill: q_len == kv_len == kv_stride, q_offset 0.  Decode: q_len 1, q_offset kv_len-1.
+ * d_head must be 64 (nn/ops/attention.rs:223-229); kv_len >= 1; every query row must see
+ * at least one key.
+ */
+int32_t agpu_attention(agpu_ctx *ctx, const float *q, const float *k, const float *v, float *o,
+                       int32_t n_heads, int32_t q_len, int32_t kv_len, int32_t q_offset,
+                       int32_t kv_stride, int32_t d_head, int32_t causal);
+/* kv_cache_append (compute_transformer.rs:1777-1812): row 0 of src [H, src_stride, dh]
+ * -> cache [H, max_seq, dh] at write_pos. */
+int32_t agpu_kv_append(agpu_ctx *ctx, const float *src, float *cache, int32_t n_heads, int32_t src_stride,
+                       int32_t max_seq, int32_t write_pos, int32_t d_head);
+
+/* ---- f32 GEMM (the reference model's f32 LM head) --------------------------------------- */
+
+/* ops::matmul (nn/ops/gemm.rs:20-212) -> gemm_f32 / _v2 / _v3 (compute_gemm.rs:1663,1839,2160):
+ * C[M,N] = A[M,K] * B[K,N]. */
+int32_t agpu_gemm_f32(agpu_ctx *ctx, const float *a, const float *b, float *c, int32_t M, int32_t N,
+                      int32_t K);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AGPU_H */
