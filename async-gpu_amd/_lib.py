@@ -68,7 +68,30 @@ SIGNATURES = {
     "agpu_attention": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32]),
     "agpu_kv_append": (_i32, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32]),
     "agpu_gemm_f32": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32]),
+    # include/agpu_gpt2.h (first argument is the model handle, or the config / context)
+    "agpu_gpt2_config_small": (_i32, [_vp]),
+    "agpu_gpt2_config_xl": (_i32, [_vp]),
+    "agpu_gpt2_create": (_i32, [_vp, _vp, C.POINTER(_vp)]),
+    "agpu_gpt2_destroy": (_i32, [_vp]),
+    "agpu_gpt2_set_embeddings": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32]),
+    "agpu_gpt2_set_layer_norms": (_i32, [_vp, _i32, _vp, _vp, _vp, _vp, _i32]),
+    "agpu_gpt2_set_int4_linear": (_i32, [_vp, _i32, _i32, _vp, _vp, _vp, _i32, _i32, _i32]),
+    "agpu_gpt2_quantize_linear": (_i32, [_vp, _i32, _i32, _vp, _vp, _i32, _i32, _i32, _i32]),
+    "agpu_gpt2_quantized_memory_bytes": (C.c_int64, [_vp]),
+    "agpu_gpt2_reset_cache": (_i32, [_vp]),
+    "agpu_gpt2_cache_len": (_i32, [_vp]),
+    "agpu_gpt2_forward_cached": (_i32, [_vp, _vp, _i32, _i32, _vp, _i32]),
+    "agpu_gpt2_generate_cached": (_i32, [_vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp]),
+    "agpu_gpt2_generate": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, _vp]),
+    "agpu_gpt2_decode_steps": (_i32, [_vp, _i32, _i32, _vp]),
 }
+
+
+class Gpt2ConfigStruct(C.Structure):
+    """agpu_gpt2_config of include/agpu_gpt2.h."""
+    _fields_ = [("n_layer", _i32), ("n_embd", _i32), ("n_head", _i32), ("vocab_size", _i32), ("n_positions", _i32),
+                ("layer_norm_epsilon", _f), ("group_size", _i32), ("max_batch", _i32), ("lm_head", _i32),
+                ("gelu", _i32), ("argmax_last", _i32)]
 
 
 def cdll():

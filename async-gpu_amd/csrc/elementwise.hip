@@ -187,14 +187,14 @@ __device__ __forceinline__ bool better(float v, unsigned int i, float bv, unsign
 
 __global__ __launch_bounds__(256) void argmax_rows_kernel(const float *__restrict__ x, uint32_t *idx_out,
                                                            float *part_val, unsigned int *part_idx,
-                                                           unsigned int *counters, int cols, int chunk,
-                                                           int last_index) {
+                                                           unsigned int *counters, int cols, int row_stride,
+                                                           int chunk, int last_index) {
     __shared__ float sv[4];
     __shared__ unsigned int si[4];
     __shared__ int s_last;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row = blockIdx.y, nchunks = gridDim.x;
-    const float *xr = x + (size_t)row * cols;
+    const float *xr = x + (size_t)row * row_stride;
     const int c0 = blockIdx.x * chunk, c1 = min(cols, c0 + chunk);
     float bv = -INFINITY;
     unsigned int bi = last_index ? 0u : 0xFFFFFFFFu;
@@ -332,12 +332,9 @@ AGPU_EXPORT int32_t agpu_embedding(agpu_ctx *ctx, const uint32_t *tokens, const 
     return AGPU_LAUNCH_CHECK(ctx, "embedding_kernel");
 }
 
-AGPU_EXPORT int32_t agpu_argmax_rows(agpu_ctx *ctx, const float *x, uint32_t *idx_out, int32_t rows, int32_t cols,
-                                     int32_t last_index) {
-    AGPU_REQUIRE_CTX(ctx);
-    if (!x || !idx_out) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "argmax_rows: null pointer");
-    if (rows < 0 || cols <= 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "argmax_rows: bad dims rows=%d cols=%d", rows, cols);
-    if (rows == 0) return AGPU_OK;
+// Rows of `cols` values, `row_stride` floats apart.
+int32_t agpu_argmax_rows_strided(agpu_ctx *ctx, const float *x, uint32_t *idx_out, int rows, int cols, int row_stride,
+                                 int last_index) {
     if (rows > kNumCounters) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "argmax_rows: rows=%d too large", rows);
     const int chunk = 2048;
     const int nchunks = ceil_div(cols, chunk);
@@ -346,8 +343,17 @@ AGPU_EXPORT int32_t agpu_argmax_rows(agpu_ctx *ctx, const float *x, uint32_t *id
     float *pv = reinterpret_cast<float *>(ctx->workspace);
     unsigned int *pi = reinterpret_cast<unsigned int *>(ctx->workspace) + (size_t)rows * nchunks;
     hipLaunchKernelGGL(argmax_rows_kernel, dim3(nchunks, rows), dim3(256), 0, ctx->stream, x, idx_out, pv, pi,
-                       ctx->counters, cols, chunk, last_index ? 1 : 0);
+                       ctx->counters, cols, row_stride, chunk, last_index ? 1 : 0);
     return AGPU_LAUNCH_CHECK(ctx, "argmax_rows_kernel");
+}
+
+AGPU_EXPORT int32_t agpu_argmax_rows(agpu_ctx *ctx, const float *x, uint32_t *idx_out, int32_t rows, int32_t cols,
+                                     int32_t last_index) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (!x || !idx_out) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "argmax_rows: null pointer");
+    if (rows < 0 || cols <= 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "argmax_rows: bad dims rows=%d cols=%d", rows, cols);
+    if (rows == 0) return AGPU_OK;
+    return agpu_argmax_rows_strided(ctx, x, idx_out, rows, cols, cols, last_index);
 }
 
 AGPU_EXPORT int32_t agpu_split_qkv(agpu_ctx *ctx, const float *qkv, float *q, float *k, float *v, int32_t seq,

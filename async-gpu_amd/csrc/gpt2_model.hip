@@ -1,0 +1,758 @@
+// int4 GPT-2 model driver: device-resident weights and KV cache, prefill and cached decode,
+// greedy generation with the decode step replayed as a HIP graph (arg-max and token feed stay
+// on the device, so a step needs no host round trip).
+//
+// Control flow follows the reference's Int4Gpt2Model::forward (nn/models/gpt2.rs:1522-1533),
+// Int4TransformerBlock::forward (gpt2.rs:1307-1338) and Gpt2Model::forward_cached /
+// generate_cached (gpt2.rs:712-783); the per-layer launches are the fused forms of the
+// reference's kernel sequence:
+//   LN1 + QKV Linear + bias            (layer_norm_v3, int4_gemm_w4a16, bias_add)
+//   K/V rows -> cache                  (split_qkv, kv_cache_append)
+//   attention, output already [rows,d] (flash_attention_kv, concat_heads)
+//   proj Linear + bias + residual      (int4_gemm_w4a16, bias_add, elementwise_add_v3)
+//   LN2 + fc Linear + bias + GELU      (layer_norm_v3, int4_gemm_w4a16, bias_add, gelu_forward)
+//   fc-proj Linear + bias + residual   (int4_gemm_w4a16, bias_add, elementwise_add_v3)
+#include <cstring>
+#include <map>
+#include <new>
+#include <vector>
+
+#include "../../include/agpu_gpt2.h"
+#include "agpu_internal.h"
+#include "attention.h"
+
+int32_t agpu_argmax_rows_strided(agpu_ctx *ctx, const float *x, uint32_t *idx_out, int rows, int cols, int row_stride,
+                                 int last_index);
+
+namespace {
+
+struct Int4Lin {
+    uint32_t *packed = nullptr;
+    float *scales = nullptr;
+    float *bias = nullptr;
+    int K = 0, N = 0, Npad = 0;  // Npad: row stride of packed/scales (== N except for the LM head)
+};
+
+struct Block {
+    float *ln1_g = nullptr, *ln1_b = nullptr, *ln2_g = nullptr, *ln2_b = nullptr;
+    Int4Lin lin[4];
+};
+
+struct DevBuf {
+    void *p = nullptr;
+    size_t bytes = 0;
+};
+
+}  // namespace
+
+struct agpu_gpt2 {
+    agpu_ctx *ctx = nullptr;
+    agpu_gpt2_config cfg{};
+    int d = 0, H = 0, ff = 0, V = 0, P = 0, Vpad = 0;
+    float *wte = nullptr, *wpe = nullptr, *lnf_g = nullptr, *lnf_b = nullptr;
+    float *wte_t = nullptr;  // [d, V], only for the f32 LM head
+    std::vector<Block> blocks;
+    Int4Lin lm_head;
+    float *kcache = nullptr, *vcache = nullptr;  // [layer][max_batch][H][P][64]
+    int cache_len = 0;
+    // activations (grown on demand, never inside a captured region)
+    DevBuf hid, qkv, att, ffn, lnb, last, logits, tok_in;
+    uint32_t *cur_tok = nullptr, *next_tok = nullptr, *out_tok = nullptr;
+    int out_capacity = 0;  // steps recorded in out_tok
+    int *pos_dev = nullptr, *step_dev = nullptr;
+    std::map<long long, hipGraphExec_t> graphs;  // key: batch << 32 | kv bucket
+    hipEvent_t ev0 = nullptr, ev1 = nullptr, ev2 = nullptr;
+};
+
+namespace {
+
+constexpr int DH = 64;
+
+__global__ __launch_bounds__(256) void embed_rows_kernel(const uint32_t *__restrict__ tokens,
+                                                          const float *__restrict__ wte,
+                                                          const float *__restrict__ wpe, float *out, int rows,
+                                                          int new_len, int d, const int *pos_dev) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (size_t)rows * d) return;
+    const int r = (int)(i / d), j = (int)(i % d);
+    const int pos = *pos_dev + (r % new_len);
+    out[i] = wte[(size_t)tokens[r] * d + j] + wpe[(size_t)pos * d + j];
+}
+
+// K and V columns of qkv [rows, 3d] -> cache[(b*H + h), pos + s, :]
+__global__ __launch_bounds__(256) void kv_scatter_kernel(const float *__restrict__ qkv, float *kc, float *vc, int rows,
+                                                          int new_len, int H, int P, const int *pos_dev) {
+    const int d = H * DH;
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (size_t)rows * d) return;
+    const int r = (int)(i / d), j = (int)(i % d);
+    const int b = r / new_len, s = r % new_len, h = j / DH, e = j % DH;
+    const size_t dst = ((size_t)(b * H + h) * P + (*pos_dev + s)) * DH + e;
+    kc[dst] = qkv[(size_t)r * 3 * d + d + j];
+    vc[dst] = qkv[(size_t)r * 3 * d + 2 * d + j];
+}
+
+__global__ __launch_bounds__(256) void gather_last_rows_kernel(const float *__restrict__ src, float *dst, int batch,
+                                                                int new_len, int d) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (size_t)batch * d) return;
+    const int b = (int)(i / d), j = (int)(i % d);
+    dst[i] = src[((size_t)b * new_len + new_len - 1) * d + j];
+}
+
+// next tokens become the current tokens, are recorded, and the position / step counters advance.
+__global__ __launch_bounds__(1024) void advance_kernel(const uint32_t *next_tok, uint32_t *cur_tok, uint32_t *out_tok,
+                                                        int *pos_dev, int *step_dev, int batch, int delta,
+                                                        int out_capacity) {
+    const int t = threadIdx.x;
+    const int st = *step_dev;
+    if (t < batch) {
+        cur_tok[t] = next_tok[t];
+        if (st < out_capacity) out_tok[(size_t)st * batch + t] = next_tok[t];
+    }
+    __syncthreads();
+    if (t == 0) {
+        *pos_dev += delta;
+        *step_dev = st + 1;
+    }
+}
+
+__global__ void set_counters_kernel(int *pos_dev, int pos, int *step_dev, int step) {
+    *pos_dev = pos;
+    if (step >= 0) *step_dev = step;
+}
+
+__global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t *p, uint32_t v, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// [rows, cols] -> [cols, rows]
+__global__ __launch_bounds__(256) void transpose_kernel(const float *__restrict__ in, float *out, int rows, int cols) {
+    __shared__ float tile[32][33];
+    const int bx = blockIdx.x * 32, by = blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    for (int r = ty; r < 32; r += 8)
+        if (by + r < rows && bx + tx < cols) tile[r][tx] = in[(size_t)(by + r) * cols + bx + tx];
+    __syncthreads();
+    for (int r = ty; r < 32; r += 8)
+        if (bx + r < cols && by + tx < rows) out[(size_t)(bx + r) * rows + by + tx] = tile[tx][r];
+}
+
+int32_t dev_alloc(agpu_ctx *ctx, void **p, size_t bytes) {
+    hipError_t e = hipMalloc(p, bytes);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipMalloc");
+    return AGPU_OK;
+}
+
+int32_t upload(agpu_ctx *ctx, void *dst, const void *src, size_t bytes, int on_device) {
+    hipError_t e = hipMemcpyAsync(dst, src, bytes, on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, ctx->stream);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipMemcpyAsync");
+    // host sources may be freed by the caller right after the call returns
+    if (!on_device) return agpu_hip(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    return AGPU_OK;
+}
+
+int32_t set_vec(agpu_ctx *ctx, float **dst, const float *src, size_t n, int on_device) {
+    if (!src) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "gpt2: null weight pointer");
+    if (!*dst) {
+        int32_t rc = dev_alloc(ctx, (void **)dst, n * sizeof(float));
+        if (rc != AGPU_OK) return rc;
+    }
+    return upload(ctx, *dst, src, n * sizeof(float), on_device);
+}
+
+void free_lin(Int4Lin &l) {
+    if (l.packed) (void)hipFree(l.packed);
+    if (l.scales) (void)hipFree(l.scales);
+    if (l.bias) (void)hipFree(l.bias);
+    l = Int4Lin{};
+}
+
+void drop_graphs(agpu_gpt2 *m) {
+    for (auto &kv : m->graphs) (void)hipGraphExecDestroy(kv.second);
+    m->graphs.clear();
+}
+
+// Grow a buffer; existing graphs hold the old address, so they are dropped.
+int32_t ensure(agpu_gpt2 *m, DevBuf &b, size_t bytes) {
+    if (b.bytes >= bytes) return AGPU_OK;
+    (void)hipStreamSynchronize(m->ctx->stream);
+    drop_graphs(m);
+    if (b.p) (void)hipFree(b.p);
+    b.p = nullptr;
+    b.bytes = 0;
+    int32_t rc = dev_alloc(m->ctx, &b.p, bytes);
+    if (rc != AGPU_OK) return rc;
+    b.bytes = bytes;
+    return AGPU_OK;
+}
+
+int32_t expected_dims(const agpu_gpt2 *m, int layer, int which, int &K, int &N) {
+    if (layer < 0) {
+        K = m->d;
+        N = m->V;
+        return AGPU_OK;
+    }
+    switch (which) {
+        case AGPU_LINEAR_QKV: K = m->d; N = 3 * m->d; break;
+        case AGPU_LINEAR_PROJ: K = m->d; N = m->d; break;
+        case AGPU_LINEAR_FC: K = m->d; N = m->ff; break;
+        case AGPU_LINEAR_FC_PROJ: K = m->ff; N = m->d; break;
+        default: return AGPU_ERR_DIM_OUT_OF_RANGE;
+    }
+    return AGPU_OK;
+}
+
+int32_t alloc_lin(agpu_gpt2 *m, Int4Lin &l, int K, int N, bool pad, bool with_bias) {
+    free_lin(l);
+    const int g = m->cfg.group_size;
+    l.K = K;
+    l.N = N;
+    l.Npad = pad ? ceil_div(N, 256) * 256 : N;
+    const size_t nw = (size_t)(K / 8) * l.Npad, ns = (size_t)ceil_div(K, g) * l.Npad;
+    int32_t rc = dev_alloc(m->ctx, (void **)&l.packed, nw * 4);
+    if (rc == AGPU_OK) rc = dev_alloc(m->ctx, (void **)&l.scales, ns * 4);
+    if (rc == AGPU_OK && with_bias) rc = dev_alloc(m->ctx, (void **)&l.bias, (size_t)N * 4);
+    if (rc != AGPU_OK) return rc;
+    if (pad && l.Npad != N) {
+        // pad columns: nibble 8 (= 0) and scale 0, so they produce exact zeros
+        hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((nw + 255) / 256)), dim3(256), 0, m->ctx->stream, l.packed,
+                           0x88888888u, nw);
+        hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((ns + 255) / 256)), dim3(256), 0, m->ctx->stream,
+                           reinterpret_cast<uint32_t *>(l.scales), 0u, ns);
+        rc = AGPU_LAUNCH_CHECK(m->ctx, "fill_u32_kernel");
+    }
+    return rc;
+}
+
+int32_t copy_rows(agpu_ctx *ctx, void *dst, size_t dst_stride, const void *src, size_t src_stride, size_t width,
+                  size_t rows, int on_device) {
+    hipError_t e = hipMemcpy2DAsync(dst, dst_stride, src, src_stride, width, rows,
+                                    on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, ctx->stream);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipMemcpy2DAsync");
+    if (!on_device) return agpu_hip(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    return AGPU_OK;
+}
+
+Int4Lin *lin_slot(agpu_gpt2 *m, int layer, int which) {
+    return layer < 0 ? &m->lm_head : &m->blocks[layer].lin[which];
+}
+
+int32_t check_layer(agpu_gpt2 *m, int layer, int which, int K, int N) {
+    if (layer >= m->cfg.n_layer || layer < -1)
+        return agpu_fail(m->ctx, AGPU_ERR_DIM_OUT_OF_RANGE, "gpt2: layer %d out of range for %d layers", layer, m->cfg.n_layer);
+    int eK = 0, eN = 0;
+    if (expected_dims(m, layer, which, eK, eN) != AGPU_OK)
+        return agpu_fail(m->ctx, AGPU_ERR_DIM_OUT_OF_RANGE, "gpt2: linear index %d out of range", which);
+    if (K != eK || N != eN)
+        return agpu_fail(m->ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2: expected [K=%d, N=%d], got [K=%d, N=%d]", eK, eN, K, N);
+    return AGPU_OK;
+}
+
+// One forward over `new_len` tokens per sequence.  Every kernel reads the number of cached
+// positions from pos_dev, so the same launch sequence serves eager calls and graph replays.
+// max_kv bounds cache_len + new_len for sizing the attention key split.
+int32_t launch_forward(agpu_gpt2 *m, const uint32_t *tokens, int B, int new_len, int max_kv, bool all_rows_logits) {
+    agpu_ctx *ctx = m->ctx;
+    const int d = m->d, H = m->H, ff = m->ff, P = m->P, g = m->cfg.group_size;
+    const int R = B * new_len;
+    const float eps = m->cfg.layer_norm_epsilon;
+    float *hid = (float *)m->hid.p, *qkv = (float *)m->qkv.p, *att = (float *)m->att.p, *ffn = (float *)m->ffn.p;
+    const uint32_t gelu_flag = m->cfg.gelu == AGPU_GELU_QUICK ? AGPU_EPI_GELU_QUICK : AGPU_EPI_GELU_TANH;
+    int32_t rc;
+
+    hipLaunchKernelGGL(embed_rows_kernel, dim3((unsigned)(((size_t)R * d + 255) / 256)), dim3(256), 0, ctx->stream, tokens,
+                       m->wte, m->wpe, hid, R, new_len, d, m->pos_dev);
+    if ((rc = AGPU_LAUNCH_CHECK(ctx, "embed_rows_kernel")) != AGPU_OK) return rc;
+
+    const size_t layer_stride = (size_t)m->cfg.max_batch * H * P * DH;
+    for (int L = 0; L < m->cfg.n_layer; ++L) {
+        const Block &b = m->blocks[L];
+        const Int4Lin &wq = b.lin[AGPU_LINEAR_QKV], &wp = b.lin[AGPU_LINEAR_PROJ], &wf = b.lin[AGPU_LINEAR_FC],
+                      &wo = b.lin[AGPU_LINEAR_FC_PROJ];
+        rc = agpu_ln_int4_linear(ctx, hid, b.ln1_g, b.ln1_b, eps, wq.packed, wq.scales, wq.bias, nullptr, qkv, R, 3 * d,
+                                 d, g, 0);
+        if (rc != AGPU_OK) return rc;
+        float *kc = m->kcache + L * layer_stride, *vc = m->vcache + L * layer_stride;
+        hipLaunchKernelGGL(kv_scatter_kernel, dim3((unsigned)(((size_t)R * d + 255) / 256)), dim3(256), 0, ctx->stream, qkv,
+                           kc, vc, R, new_len, H, P, m->pos_dev);
+        if ((rc = AGPU_LAUNCH_CHECK(ctx, "kv_scatter_kernel")) != AGPU_OK) return rc;
+        AttnParams ap{};
+        ap.q = qkv; ap.k = kc; ap.v = vc; ap.o = att;
+        ap.n_heads = H; ap.batch = B; ap.q_len = new_len; ap.kv_len = 0; ap.q_offset = 0; ap.kv_stride = P; ap.causal = 1;
+        ap.q_batch_stride = (long long)new_len * 3 * d; ap.q_head_stride = DH; ap.q_row_stride = 3 * d;
+        ap.o_batch_stride = (long long)new_len * d; ap.o_head_stride = DH; ap.o_row_stride = d;
+        ap.pos_dev = m->pos_dev;
+        if ((rc = agpu_attention_launch(ctx, ap, max_kv)) != AGPU_OK) return rc;
+        rc = agpu_int4_linear(ctx, att, wp.packed, wp.scales, wp.bias, hid, hid, R, d, d, g, 0);
+        if (rc != AGPU_OK) return rc;
+        rc = agpu_ln_int4_linear(ctx, hid, b.ln2_g, b.ln2_b, eps, wf.packed, wf.scales, wf.bias, nullptr, ffn, R, ff, d, g,
+                                 gelu_flag);
+        if (rc != AGPU_OK) return rc;
+        rc = agpu_int4_linear(ctx, ffn, wo.packed, wo.scales, wo.bias, hid, hid, R, d, ff, g, 0);
+        if (rc != AGPU_OK) return rc;
+    }
+
+    // final LayerNorm + LM head on the rows whose logits are wanted
+    const float *head_in = hid;
+    int Rl = R;
+    if (!all_rows_logits && new_len > 1) {
+        hipLaunchKernelGGL(gather_last_rows_kernel, dim3((unsigned)(((size_t)B * d + 255) / 256)), dim3(256), 0, ctx->stream,
+                           hid, (float *)m->last.p, B, new_len, d);
+        if ((rc = AGPU_LAUNCH_CHECK(ctx, "gather_last_rows_kernel")) != AGPU_OK) return rc;
+        head_in = (float *)m->last.p;
+        Rl = B;
+    } else if (!all_rows_logits) {
+        Rl = B;
+    }
+    float *logits = (float *)m->logits.p;
+    if (m->cfg.lm_head == AGPU_LM_HEAD_INT4) {
+        rc = agpu_ln_int4_linear(ctx, head_in, m->lnf_g, m->lnf_b, eps, m->lm_head.packed, m->lm_head.scales, nullptr, nullptr,
+                                 logits, Rl, m->Vpad, d, g, 0);
+    } else {
+        rc = agpu_layer_norm(ctx, head_in, m->lnf_g, m->lnf_b, (float *)m->lnb.p, Rl, d, eps);
+        if (rc == AGPU_OK) rc = agpu_gemm_f32(ctx, (float *)m->lnb.p, m->wte_t, logits, Rl, m->V, d);
+    }
+    return rc;
+}
+
+int logits_stride(const agpu_gpt2 *m) { return m->cfg.lm_head == AGPU_LM_HEAD_INT4 ? m->Vpad : m->V; }
+
+int32_t ensure_buffers(agpu_gpt2 *m, int B, int new_len, bool all_rows_logits) {
+    const size_t R = (size_t)B * new_len, d = m->d;
+    const size_t Rl = all_rows_logits ? R : (size_t)B;
+    int32_t rc;
+    if ((rc = ensure(m, m->hid, R * d * 4)) != AGPU_OK) return rc;
+    if ((rc = ensure(m, m->qkv, R * 3 * d * 4)) != AGPU_OK) return rc;
+    if ((rc = ensure(m, m->att, R * d * 4)) != AGPU_OK) return rc;
+    if ((rc = ensure(m, m->ffn, R * m->ff * 4)) != AGPU_OK) return rc;
+    if ((rc = ensure(m, m->lnb, Rl * d * 4)) != AGPU_OK) return rc;
+    if ((rc = ensure(m, m->last, (size_t)B * d * 4)) != AGPU_OK) return rc;
+    if ((rc = ensure(m, m->logits, Rl * logits_stride(m) * 4)) != AGPU_OK) return rc;
+    return AGPU_OK;
+}
+
+int32_t check_ready(agpu_gpt2 *m) {
+    if (!m->wte || !m->wpe || !m->lnf_g || !m->lnf_b) return agpu_fail(m->ctx, AGPU_ERR_NULL_POINTER, "gpt2: embeddings not set");
+    for (int L = 0; L < m->cfg.n_layer; ++L) {
+        const Block &b = m->blocks[L];
+        if (!b.ln1_g || !b.ln2_g) return agpu_fail(m->ctx, AGPU_ERR_NULL_POINTER, "gpt2: layer norms of layer %d not set", L);
+        for (int w = 0; w < 4; ++w)
+            if (!b.lin[w].packed) return agpu_fail(m->ctx, AGPU_ERR_NULL_POINTER, "gpt2: linear %d of layer %d not set", w, L);
+    }
+    if (m->cfg.lm_head == AGPU_LM_HEAD_INT4 && !m->lm_head.packed)
+        return agpu_fail(m->ctx, AGPU_ERR_NULL_POINTER, "gpt2: int4 LM head not set");
+    return AGPU_OK;
+}
+
+int32_t set_counters(agpu_gpt2 *m, int pos, int step) {
+    hipLaunchKernelGGL(set_counters_kernel, dim3(1), dim3(1), 0, m->ctx->stream, m->pos_dev, pos, m->step_dev, step);
+    return AGPU_LAUNCH_CHECK(m->ctx, "set_counters_kernel");
+}
+
+int32_t launch_argmax_advance(agpu_gpt2 *m, int B, int delta) {
+    int32_t rc = agpu_argmax_rows_strided(m->ctx, (float *)m->logits.p, m->next_tok, B, m->V, logits_stride(m),
+                                          m->cfg.argmax_last);
+    if (rc != AGPU_OK) return rc;
+    hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1024), 0, m->ctx->stream, m->next_tok, m->cur_tok, m->out_tok,
+                       m->pos_dev, m->step_dev, B, delta, m->out_capacity);
+    return AGPU_LAUNCH_CHECK(m->ctx, "advance_kernel");
+}
+
+int kv_bucket(const agpu_gpt2 *m, int kv_len) {
+    int b = 128;
+    while (b < kv_len) b *= 2;
+    return b < m->P ? b : m->P;
+}
+
+// The captured decode step for (batch, kv bucket); captured on first use.
+int32_t decode_graph(agpu_gpt2 *m, int B, int bucket, hipGraphExec_t *out) {
+    const long long key = ((long long)B << 32) | (unsigned)bucket;
+    auto it = m->graphs.find(key);
+    if (it != m->graphs.end()) {
+        *out = it->second;
+        return AGPU_OK;
+    }
+    agpu_ctx *ctx = m->ctx;
+    if (ctx->stream == nullptr)
+        return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "gpt2: graph capture needs a context with its own stream (agpu_ctx_create)");
+    hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipStreamBeginCapture");
+    int32_t rc = launch_forward(m, m->cur_tok, B, 1, bucket, false);
+    if (rc == AGPU_OK) rc = launch_argmax_advance(m, B, 1);
+    hipGraph_t graph = nullptr;
+    e = hipStreamEndCapture(ctx->stream, &graph);
+    if (rc != AGPU_OK) {
+        if (graph) (void)hipGraphDestroy(graph);
+        return rc;
+    }
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipStreamEndCapture");
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipGraphInstantiate");
+    m->graphs[key] = exec;
+    *out = exec;
+    return AGPU_OK;
+}
+
+int32_t ensure_out_tokens(agpu_gpt2 *m, int steps, int B) {
+    if (m->out_capacity >= steps && m->out_tok) return AGPU_OK;
+    (void)hipStreamSynchronize(m->ctx->stream);
+    drop_graphs(m);
+    if (m->out_tok) (void)hipFree(m->out_tok);
+    m->out_tok = nullptr;
+    const int cap = steps > m->P ? steps : m->P;
+    int32_t rc = dev_alloc(m->ctx, (void **)&m->out_tok, (size_t)cap * m->cfg.max_batch * sizeof(uint32_t));
+    if (rc != AGPU_OK) return rc;
+    m->out_capacity = cap;
+    (void)B;
+    return AGPU_OK;
+}
+
+// Replays `steps` decode steps; the host only tracks the position to pick the graph.
+int32_t run_decode_steps(agpu_gpt2 *m, int B, int steps) {
+    for (int s = 0; s < steps; ++s) {
+        hipGraphExec_t exec;
+        int32_t rc = decode_graph(m, B, kv_bucket(m, m->cache_len + 1), &exec);
+        if (rc != AGPU_OK) return rc;
+        hipError_t e = hipGraphLaunch(exec, m->ctx->stream);
+        if (e != hipSuccess) return agpu_hip(m->ctx, e, "hipGraphLaunch");
+        m->cache_len += 1;
+    }
+    return AGPU_OK;
+}
+
+void fill_config(agpu_gpt2_config *c, int n_layer, int n_embd, int n_head) {
+    c->n_layer = n_layer;
+    c->n_embd = n_embd;
+    c->n_head = n_head;
+    c->vocab_size = 50257;
+    c->n_positions = 1024;
+    c->layer_norm_epsilon = 1e-5f;
+    c->group_size = 32;
+    c->max_batch = 1;
+    c->lm_head = AGPU_LM_HEAD_INT4;
+    c->gelu = AGPU_GELU_TANH;
+    c->argmax_last = 0;
+}
+
+}  // namespace
+
+AGPU_EXPORT int32_t agpu_gpt2_config_small(agpu_gpt2_config *out) {
+    if (!out) return AGPU_ERR_NULL_POINTER;
+    fill_config(out, 12, 768, 12);
+    return AGPU_OK;
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_config_xl(agpu_gpt2_config *out) {
+    if (!out) return AGPU_ERR_NULL_POINTER;
+    fill_config(out, 48, 1600, 25);
+    return AGPU_OK;
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_create(agpu_ctx *ctx, const agpu_gpt2_config *cfg, agpu_gpt2 **out) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (!cfg || !out) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "gpt2_create: null pointer");
+    *out = nullptr;
+    if (cfg->n_layer <= 0 || cfg->n_embd <= 0 || cfg->n_head <= 0 || cfg->vocab_size <= 0 || cfg->n_positions <= 0 ||
+        cfg->group_size <= 0 || cfg->max_batch <= 0 || cfg->max_batch > 1024)
+        return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_create: bad configuration");
+    if (cfg->n_embd % cfg->n_head != 0 || cfg->n_embd / cfg->n_head != DH)
+        return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_create: expected head_dim = 64, got n_embd/n_head = %d/%d",
+                         cfg->n_embd, cfg->n_head);
+    if (cfg->n_embd % 8 != 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_create: n_embd must be divisible by 8");
+    agpu_gpt2 *m = new (std::nothrow) agpu_gpt2();
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    m->ctx = ctx;
+    m->cfg = *cfg;
+    m->d = cfg->n_embd;
+    m->H = cfg->n_head;
+    m->ff = 4 * cfg->n_embd;  // Gpt2Config::ffn_dim, gpt2.rs:90-92
+    m->V = cfg->vocab_size;
+    m->P = cfg->n_positions;
+    m->Vpad = ceil_div(m->V, 256) * 256;
+    m->blocks.resize(cfg->n_layer);
+    const size_t cache_elems = (size_t)cfg->n_layer * cfg->max_batch * m->H * m->P * DH;
+    int32_t rc = dev_alloc(ctx, (void **)&m->kcache, cache_elems * 4);
+    if (rc == AGPU_OK) rc = dev_alloc(ctx, (void **)&m->vcache, cache_elems * 4);
+    if (rc == AGPU_OK) rc = dev_alloc(ctx, (void **)&m->cur_tok, (size_t)cfg->max_batch * 4);
+    if (rc == AGPU_OK) rc = dev_alloc(ctx, (void **)&m->next_tok, (size_t)cfg->max_batch * 4);
+    if (rc == AGPU_OK) rc = dev_alloc(ctx, (void **)&m->pos_dev, 2 * sizeof(int));
+    if (rc == AGPU_OK) {
+        m->step_dev = m->pos_dev + 1;
+        rc = agpu_hip(ctx, hipMemset(m->pos_dev, 0, 2 * sizeof(int)), "hipMemset");
+    }
+    if (rc == AGPU_OK) rc = agpu_hip(ctx, hipEventCreate(&m->ev0), "hipEventCreate");
+    if (rc == AGPU_OK) rc = agpu_hip(ctx, hipEventCreate(&m->ev1), "hipEventCreate");
+    if (rc == AGPU_OK) rc = agpu_hip(ctx, hipEventCreate(&m->ev2), "hipEventCreate");
+    if (rc != AGPU_OK) {
+        agpu_gpt2_destroy(m);
+        return rc;
+    }
+    *out = m;
+    return AGPU_OK;
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_destroy(agpu_gpt2 *m) {
+    if (!m) return AGPU_OK;
+    if (m->ctx) (void)hipStreamSynchronize(m->ctx->stream);
+    drop_graphs(m);
+    for (auto &b : m->blocks) {
+        for (float *p : {b.ln1_g, b.ln1_b, b.ln2_g, b.ln2_b})
+            if (p) (void)hipFree(p);
+        for (auto &l : b.lin) free_lin(l);
+    }
+    free_lin(m->lm_head);
+    for (void *p : {(void *)m->wte, (void *)m->wpe, (void *)m->lnf_g, (void *)m->lnf_b, (void *)m->wte_t, (void *)m->kcache,
+                    (void *)m->vcache, (void *)m->cur_tok, (void *)m->next_tok, (void *)m->out_tok, (void *)m->pos_dev,
+                    m->hid.p, m->qkv.p, m->att.p, m->ffn.p, m->lnb.p, m->last.p, m->logits.p, m->tok_in.p})
+        if (p) (void)hipFree(p);
+    for (hipEvent_t e : {m->ev0, m->ev1, m->ev2})
+        if (e) (void)hipEventDestroy(e);
+    delete m;
+    return AGPU_OK;
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_set_embeddings(agpu_gpt2 *m, const float *wte, const float *wpe, const float *lnf_g,
+                                             const float *lnf_b, int32_t on_device) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    agpu_ctx *ctx = m->ctx;
+    int32_t rc = set_vec(ctx, &m->wte, wte, (size_t)m->V * m->d, on_device);
+    if (rc == AGPU_OK) rc = set_vec(ctx, &m->wpe, wpe, (size_t)m->P * m->d, on_device);
+    if (rc == AGPU_OK) rc = set_vec(ctx, &m->lnf_g, lnf_g, m->d, on_device);
+    if (rc == AGPU_OK) rc = set_vec(ctx, &m->lnf_b, lnf_b, m->d, on_device);
+    if (rc == AGPU_OK && m->cfg.lm_head == AGPU_LM_HEAD_F32) {
+        // Linear::new stores the weight transposed, [in, out] (nn/layers/linear.rs:67-74)
+        if (!m->wte_t) rc = dev_alloc(ctx, (void **)&m->wte_t, (size_t)m->V * m->d * 4);
+        if (rc == AGPU_OK) {
+            hipLaunchKernelGGL(transpose_kernel, dim3(ceil_div(m->d, 32), ceil_div(m->V, 32)), dim3(256), 0, ctx->stream,
+                               m->wte, m->wte_t, m->V, m->d);
+            rc = AGPU_LAUNCH_CHECK(ctx, "transpose_kernel");
+        }
+    }
+    return rc;
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_set_layer_norms(agpu_gpt2 *m, int32_t layer, const float *ln1_g, const float *ln1_b,
+                                              const float *ln2_g, const float *ln2_b, int32_t on_device) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    if (layer < 0 || layer >= m->cfg.n_layer)
+        return agpu_fail(m->ctx, AGPU_ERR_DIM_OUT_OF_RANGE, "gpt2: layer %d out of range for %d layers", layer, m->cfg.n_layer);
+    Block &b = m->blocks[layer];
+    int32_t rc = set_vec(m->ctx, &b.ln1_g, ln1_g, m->d, on_device);
+    if (rc == AGPU_OK) rc = set_vec(m->ctx, &b.ln1_b, ln1_b, m->d, on_device);
+    if (rc == AGPU_OK) rc = set_vec(m->ctx, &b.ln2_g, ln2_g, m->d, on_device);
+    if (rc == AGPU_OK) rc = set_vec(m->ctx, &b.ln2_b, ln2_b, m->d, on_device);
+    return rc;
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_set_int4_linear(agpu_gpt2 *m, int32_t layer, int32_t which, const uint32_t *packed,
+                                              const float *scales, const float *bias, int32_t K, int32_t N,
+                                              int32_t on_device) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    int32_t rc = check_layer(m, layer, which, K, N);
+    if (rc != AGPU_OK) return rc;
+    if (!packed || !scales) return agpu_fail(m->ctx, AGPU_ERR_NULL_POINTER, "gpt2_set_int4_linear: null pointer");
+    drop_graphs(m);
+    Int4Lin &l = *lin_slot(m, layer, which);
+    rc = alloc_lin(m, l, K, N, layer < 0, bias != nullptr && layer >= 0);
+    if (rc != AGPU_OK) return rc;
+    const int ng = ceil_div(K, m->cfg.group_size);
+    rc = copy_rows(m->ctx, l.packed, (size_t)l.Npad * 4, packed, (size_t)N * 4, (size_t)N * 4, K / 8, on_device);
+    if (rc == AGPU_OK) rc = copy_rows(m->ctx, l.scales, (size_t)l.Npad * 4, scales, (size_t)N * 4, (size_t)N * 4, ng, on_device);
+    if (rc == AGPU_OK && l.bias) rc = upload(m->ctx, l.bias, bias, (size_t)N * 4, on_device);
+    return rc;
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_quantize_linear(agpu_gpt2 *m, int32_t layer, int32_t which, const float *weight_t,
+                                              const float *bias, int32_t K, int32_t N, int32_t mode, int32_t on_device) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    int32_t rc = check_layer(m, layer, which, K, N);
+    if (rc != AGPU_OK) return rc;
+    if (!weight_t) return agpu_fail(m->ctx, AGPU_ERR_NULL_POINTER, "gpt2_quantize_linear: null pointer");
+    agpu_ctx *ctx = m->ctx;
+    const int g = m->cfg.group_size, ng = ceil_div(K, g);
+    float *w_dev = nullptr;
+    uint32_t *p_dev = nullptr;
+    float *s_dev = nullptr;
+    const float *w_src = weight_t;
+    if (!on_device) {
+        rc = dev_alloc(ctx, (void **)&w_dev, (size_t)K * N * 4);
+        if (rc == AGPU_OK) rc = upload(ctx, w_dev, weight_t, (size_t)K * N * 4, 0);
+        w_src = w_dev;
+    }
+    if (rc == AGPU_OK) rc = dev_alloc(ctx, (void **)&p_dev, (size_t)(K / 8) * N * 4);
+    if (rc == AGPU_OK) rc = dev_alloc(ctx, (void **)&s_dev, (size_t)ng * N * 4);
+    if (rc == AGPU_OK) rc = agpu_int4_quantize(ctx, w_src, p_dev, s_dev, K, N, g, mode);
+    if (rc == AGPU_OK) {
+        // bias may be a host pointer while the quantized data is on the device: set in two steps
+        rc = agpu_gpt2_set_int4_linear(m, layer, which, p_dev, s_dev, nullptr, K, N, 1);
+        if (rc == AGPU_OK && bias && layer >= 0) {
+            Int4Lin &l = *lin_slot(m, layer, which);
+            rc = dev_alloc(ctx, (void **)&l.bias, (size_t)N * 4);
+            if (rc == AGPU_OK) rc = upload(ctx, l.bias, bias, (size_t)N * 4, on_device);
+        }
+    }
+    (void)hipStreamSynchronize(ctx->stream);
+    for (void *p : {(void *)w_dev, (void *)p_dev, (void *)s_dev})
+        if (p) (void)hipFree(p);
+    return rc;
+}
+
+AGPU_EXPORT int64_t agpu_gpt2_quantized_memory_bytes(const agpu_gpt2 *m) {
+    if (!m) return 0;
+    int64_t total = 0;
+    const int g = m->cfg.group_size;
+    for (const auto &b : m->blocks)
+        for (const auto &l : b.lin)
+            if (l.packed) total += (int64_t)(l.K / 8) * l.N * 4 + (int64_t)ceil_div(l.K, g) * l.N * 4 + (l.bias ? (int64_t)l.N * 4 : 0);
+    return total;
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_reset_cache(agpu_gpt2 *m) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    m->cache_len = 0;
+    return set_counters(m, 0, 0);
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_cache_len(const agpu_gpt2 *m) { return m ? m->cache_len : 0; }
+
+AGPU_EXPORT int32_t agpu_gpt2_forward_cached(agpu_gpt2 *m, const uint32_t *tokens, int32_t batch, int32_t new_len,
+                                             float *logits, int32_t all_rows) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    agpu_ctx *ctx = m->ctx;
+    if (!tokens) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "gpt2_forward_cached: null tokens");
+    if (batch <= 0 || batch > m->cfg.max_batch)
+        return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_forward_cached: batch %d not in 1..%d", batch, m->cfg.max_batch);
+    if (new_len <= 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_forward_cached: new_len must be positive");
+    if (m->cache_len + new_len > m->P)
+        return agpu_fail(ctx, AGPU_ERR_DIM_OUT_OF_RANGE, "gpt2_forward_cached: %d cached + %d new positions exceed n_positions %d",
+                         m->cache_len, new_len, m->P);
+    int32_t rc = check_ready(m);
+    if (rc != AGPU_OK) return rc;
+    if ((rc = ensure_buffers(m, batch, new_len, all_rows != 0)) != AGPU_OK) return rc;
+    if ((rc = ensure_out_tokens(m, m->P, batch)) != AGPU_OK) return rc;
+    if ((rc = set_counters(m, m->cache_len, -1)) != AGPU_OK) return rc;
+    if ((rc = launch_forward(m, tokens, batch, new_len, m->cache_len + new_len, all_rows != 0)) != AGPU_OK) return rc;
+    // keep the device-side generation state usable: next token = arg-max of the last rows
+    if (!all_rows) {
+        if ((rc = launch_argmax_advance(m, batch, new_len)) != AGPU_OK) return rc;
+    } else {
+        if ((rc = set_counters(m, m->cache_len + new_len, -1)) != AGPU_OK) return rc;
+    }
+    m->cache_len += new_len;
+    if (logits) {
+        const size_t rows = all_rows ? (size_t)batch * new_len : (size_t)batch;
+        hipError_t e = hipMemcpy2DAsync(logits, (size_t)m->V * 4, m->logits.p, (size_t)logits_stride(m) * 4, (size_t)m->V * 4,
+                                        rows, hipMemcpyDeviceToDevice, ctx->stream);
+        if (e != hipSuccess) return agpu_hip(ctx, e, "hipMemcpy2DAsync(logits)");
+    }
+    return AGPU_OK;
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_decode_steps(agpu_gpt2 *m, int32_t batch, int32_t steps, float *ms_total_out_host) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    agpu_ctx *ctx = m->ctx;
+    if (batch <= 0 || batch > m->cfg.max_batch || steps < 0)
+        return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_decode_steps: bad batch/steps");
+    if (m->cache_len == 0) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "gpt2_decode_steps: run a prefill first");
+    if (m->cache_len + steps > m->P)
+        return agpu_fail(ctx, AGPU_ERR_DIM_OUT_OF_RANGE, "gpt2_decode_steps: %d cached + %d steps exceed n_positions %d",
+                         m->cache_len, steps, m->P);
+    int32_t rc = ensure_buffers(m, batch, 1, false);
+    if (rc != AGPU_OK) return rc;
+    // capture outside the timed region
+    hipGraphExec_t exec;
+    for (int s = 0; s < steps; ++s)
+        if ((rc = decode_graph(m, batch, kv_bucket(m, m->cache_len + 1 + s), &exec)) != AGPU_OK) return rc;
+    if ((rc = agpu_hip(ctx, hipEventRecord(m->ev0, ctx->stream), "hipEventRecord")) != AGPU_OK) return rc;
+    if ((rc = run_decode_steps(m, batch, steps)) != AGPU_OK) return rc;
+    if ((rc = agpu_hip(ctx, hipEventRecord(m->ev1, ctx->stream), "hipEventRecord")) != AGPU_OK) return rc;
+    if ((rc = agpu_hip(ctx, hipEventSynchronize(m->ev1), "hipEventSynchronize")) != AGPU_OK) return rc;
+    if (ms_total_out_host) (void)hipEventElapsedTime(ms_total_out_host, m->ev0, m->ev1);
+    return AGPU_OK;
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_generate_cached(agpu_gpt2 *m, const uint32_t *prompt_host, int32_t batch, int32_t prompt_len,
+                                              int32_t max_new_tokens, int32_t eos, uint32_t *tokens_out_host,
+                                              int32_t *lengths_out_host, float *timing_ms_out_host) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    agpu_ctx *ctx = m->ctx;
+    if (!prompt_host || !tokens_out_host || !lengths_out_host)
+        return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "gpt2_generate_cached: null pointer");
+    if (batch <= 0 || batch > m->cfg.max_batch || prompt_len <= 0 || max_new_tokens < 0)
+        return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_generate_cached: bad batch/prompt_len/max_new_tokens");
+    // the last generated token is never fed back, so prompt_len + max_new_tokens - 1 positions are cached
+    if (prompt_len + (max_new_tokens > 0 ? max_new_tokens - 1 : 0) > m->P)
+        return agpu_fail(ctx, AGPU_ERR_DIM_OUT_OF_RANGE, "gpt2_generate_cached: prompt %d + %d new tokens exceed n_positions %d",
+                         prompt_len, max_new_tokens, m->P);
+    const int total = prompt_len + max_new_tokens;
+    for (int b = 0; b < batch; ++b) {
+        std::memcpy(tokens_out_host + (size_t)b * total, prompt_host + (size_t)b * prompt_len, (size_t)prompt_len * 4);
+        lengths_out_host[b] = prompt_len;
+    }
+    if (max_new_tokens == 0) return AGPU_OK;
+    int32_t rc = check_ready(m);
+    if (rc != AGPU_OK) return rc;
+    if ((rc = ensure(m, m->tok_in, (size_t)batch * prompt_len * 4)) != AGPU_OK) return rc;
+    if ((rc = ensure_buffers(m, batch, prompt_len, false)) != AGPU_OK) return rc;
+    if ((rc = ensure_out_tokens(m, max_new_tokens, batch)) != AGPU_OK) return rc;
+    if ((rc = upload(ctx, m->tok_in.p, prompt_host, (size_t)batch * prompt_len * 4, 0)) != AGPU_OK) return rc;
+    if ((rc = agpu_gpt2_reset_cache(m)) != AGPU_OK) return rc;
+
+    (void)hipEventRecord(m->ev0, ctx->stream);
+    if ((rc = agpu_gpt2_forward_cached(m, (const uint32_t *)m->tok_in.p, batch, prompt_len, nullptr, 0)) != AGPU_OK) return rc;
+    (void)hipEventRecord(m->ev1, ctx->stream);
+    if ((rc = run_decode_steps(m, batch, max_new_tokens - 1)) != AGPU_OK) return rc;
+    (void)hipEventRecord(m->ev2, ctx->stream);
+
+    std::vector<uint32_t> gen((size_t)max_new_tokens * batch);
+    rc = agpu_memcpy_d2h(ctx, gen.data(), m->out_tok, gen.size() * 4);
+    if (rc != AGPU_OK) return rc;
+    if (timing_ms_out_host) {
+        (void)hipEventElapsedTime(&timing_ms_out_host[0], m->ev0, m->ev1);
+        (void)hipEventElapsedTime(&timing_ms_out_host[1], m->ev1, m->ev2);
+    }
+    for (int b = 0; b < batch; ++b) {
+        int len = prompt_len;
+        for (int s = 0; s < max_new_tokens; ++s) {
+            const uint32_t t = gen[(size_t)s * batch + b];
+            if (eos >= 0 && t == (uint32_t)eos) break;  // stop before appending (gpt2.rs:762,776)
+            tokens_out_host[(size_t)b * total + len++] = t;
+        }
+        lengths_out_host[b] = len;
+    }
+    return AGPU_OK;
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_generate(agpu_gpt2 *m, const uint32_t *prompt_host, int32_t prompt_len, int32_t max_new_tokens,
+                                       int32_t eos, uint32_t *tokens_out_host, int32_t *length_out_host) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    agpu_ctx *ctx = m->ctx;
+    if (!prompt_host || !tokens_out_host || !length_out_host)
+        return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "gpt2_generate: null pointer");
+    if (prompt_len <= 0 || max_new_tokens < 0)
+        return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_generate: bad prompt_len/max_new_tokens");
+    std::memcpy(tokens_out_host, prompt_host, (size_t)prompt_len * 4);
+    int len = prompt_len;
+    int32_t rc = check_ready(m);
+    if (rc != AGPU_OK) return rc;
+    for (int step = 0; step < max_new_tokens; ++step) {
+        if (len > m->P) {
+            rc = agpu_fail(ctx, AGPU_ERR_DIM_OUT_OF_RANGE, "gpt2_generate: sequence length %d exceeds n_positions %d", len, m->P);
+            break;
+        }
+        if ((rc = ensure(m, m->tok_in, (size_t)len * 4)) != AGPU_OK) break;
+        if ((rc = upload(ctx, m->tok_in.p, tokens_out_host, (size_t)len * 4, 0)) != AGPU_OK) break;
+        if ((rc = agpu_gpt2_reset_cache(m)) != AGPU_OK) break;
+        if ((rc = agpu_gpt2_forward_cached(m, (const uint32_t *)m->tok_in.p, 1, len, nullptr, 0)) != AGPU_OK) break;
+        uint32_t next = 0;
+        if ((rc = agpu_memcpy_d2h(ctx, &next, m->next_tok, 4)) != AGPU_OK) break;
+        if (eos >= 0 && next == (uint32_t)eos) break;
+        tokens_out_host[len++] = next;
+    }
+    *length_out_host = len;
+    return rc;
+}

@@ -1,0 +1,184 @@
+"""Int4Gpt2Model over the model-level C ABI (include/agpu_gpt2.h); mirrors
+nn::models::gpt2::{Gpt2Config, Int4Gpt2Model, KvCache} (nn/models/gpt2.rs:20-93,1341-1580,712-783)."""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from ._lib import AgpuError
+
+LM_HEAD_INT4, LM_HEAD_F32 = 0, 1
+LINEAR_INDEX = {"qkv": 0, "proj": 1, "fc": 2, "fc_proj": 3}
+
+
+class Gpt2Config:
+    """Gpt2Config (gpt2.rs:20-93) plus the build's knobs (group size, batch, head mode, GELU form, tie rule)."""
+
+    def __init__(self, n_layer, n_embd, n_head, vocab_size=50257, n_positions=1024, layer_norm_epsilon=1e-5,
+                 group_size=32, max_batch=1, lm_head=LM_HEAD_INT4, gelu=_lib.GELU_TANH, argmax_last=False):
+        self.n_layer, self.n_embd, self.n_head = n_layer, n_embd, n_head
+        self.vocab_size, self.n_positions, self.layer_norm_epsilon = vocab_size, n_positions, layer_norm_epsilon
+        self.group_size, self.max_batch, self.lm_head, self.gelu, self.argmax_last = group_size, max_batch, lm_head, gelu, argmax_last
+
+    @classmethod
+    def small(cls, **kw):
+        return cls(12, 768, 12, **kw)
+
+    @classmethod
+    def xl(cls, **kw):
+        return cls(48, 1600, 25, **kw)
+
+    def head_dim(self):
+        return self.n_embd // self.n_head
+
+    def ffn_dim(self):
+        return 4 * self.n_embd
+
+    def struct(self):
+        return _lib.Gpt2ConfigStruct(self.n_layer, self.n_embd, self.n_head, self.vocab_size, self.n_positions,
+                                     self.layer_norm_epsilon, self.group_size, self.max_batch, self.lm_head, self.gelu,
+                                     int(self.argmax_last))
+
+
+def _np(a, dtype):
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+class Int4Gpt2Model:
+    """Device-resident int4 GPT-2.  `ctx` must own its stream (Context(device) without a stream
+    argument): the decode loop is captured into HIP graphs on it."""
+
+    def __init__(self, config, ctx=None, device=0):
+        self.config = config
+        self.ctx = ctx if ctx is not None else _lib.Context(device)
+        self._lib = _lib.cdll()
+        h = C.c_void_p()
+        st = config.struct()
+        rc = self._lib.agpu_gpt2_create(self.ctx.handle, C.byref(st), C.byref(h))
+        self._check(rc)
+        self.handle = h
+
+    def _check(self, rc):
+        if rc != 0:
+            raise AgpuError(rc, self._lib.agpu_last_error_string(self.ctx.handle).decode())
+
+    def _call(self, name, *args):
+        fn = getattr(self._lib, name)
+        conv = [_lib.ptr(a) if (t is C.c_void_p) else a for a, t in zip(args, fn.argtypes[1:])]
+        self._check(fn(self.handle, *conv))
+
+    def close(self):
+        if getattr(self, "handle", None):
+            self._lib.agpu_gpt2_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # ---- weights -------------------------------------------------------------------------
+    def set_embeddings(self, wte, wpe, lnf_g, lnf_b):
+        self._call("agpu_gpt2_set_embeddings", _np(wte, np.float32), _np(wpe, np.float32), _np(lnf_g, np.float32),
+                   _np(lnf_b, np.float32), 0)
+
+    def set_layer_norms(self, layer, ln1_g, ln1_b, ln2_g, ln2_b):
+        self._call("agpu_gpt2_set_layer_norms", layer, _np(ln1_g, np.float32), _np(ln1_b, np.float32),
+                   _np(ln2_g, np.float32), _np(ln2_b, np.float32), 0)
+
+    def set_int4_linear(self, layer, which, packed, scales, bias=None):
+        packed, scales = _np(packed, np.uint32), _np(scales, np.float32)
+        b = None if bias is None else _np(bias, np.float32)
+        self._call("agpu_gpt2_set_int4_linear", layer, LINEAR_INDEX.get(which, which), packed, scales, b,
+                   packed.shape[0] * 8, packed.shape[1], 0)
+
+    def quantize_linear(self, layer, which, weight_t, bias=None, mode=_lib.QUANT_RUST):
+        """Int4TransformerBlock::new's path: quantize weight_t [K,N] at load (gpt2.rs:1257-1264)."""
+        w = _np(weight_t, np.float32)
+        b = None if bias is None else _np(bias, np.float32)
+        self._call("agpu_gpt2_quantize_linear", layer, LINEAR_INDEX.get(which, which), w, b, w.shape[0], w.shape[1], mode, 0)
+
+    @classmethod
+    def from_quantized(cls, config, qz, ctx=None, device=0):
+        """qz: the dict produced by workloads.quantize_gpt2."""
+        m = cls(config, ctx, device)
+        m.set_embeddings(qz["wte"], qz["wpe"], qz["lnf_g"], qz["lnf_b"])
+        for li, L in enumerate(qz["layers"]):
+            m.set_layer_norms(li, L["ln1_g"], L["ln1_b"], L["ln2_g"], L["ln2_b"])
+            for name in LINEAR_INDEX:
+                m.set_int4_linear(li, name, *L[name])
+        if config.lm_head == LM_HEAD_INT4:
+            m.set_int4_linear(-1, 0, qz["lm_head"][0], qz["lm_head"][1], None)
+        return m
+
+    @classmethod
+    def from_weights(cls, config, weights, mode=_lib.QUANT_RUST, ctx=None, device=0):
+        """Int4Gpt2Model::from_weights (gpt2.rs:1362-1433): fp32 weights in, quantized at load."""
+        m = cls(config, ctx, device)
+        m.set_embeddings(weights["wte"], weights["wpe"], weights["lnf_g"], weights["lnf_b"])
+        for li, L in enumerate(weights["layers"]):
+            m.set_layer_norms(li, L["ln1_g"], L["ln1_b"], L["ln2_g"], L["ln2_b"])
+            for name in LINEAR_INDEX:
+                m.quantize_linear(li, name, L[name + "_w"], L[name + "_b"], mode)
+        if config.lm_head == LM_HEAD_INT4:
+            m.quantize_linear(-1, 0, np.ascontiguousarray(weights["wte"].T), None, mode)
+        return m
+
+    def quantized_memory_bytes(self):
+        return int(self._lib.agpu_gpt2_quantized_memory_bytes(self.handle))
+
+    # ---- inference -----------------------------------------------------------------------
+    def reset_cache(self):
+        self._call("agpu_gpt2_reset_cache")
+
+    def cache_len(self):
+        return int(self._lib.agpu_gpt2_cache_len(self.handle))
+
+    def forward_cached(self, tokens, all_rows=True):
+        """tokens [batch, new_len] (numpy); returns logits as numpy, [batch, new_len, V] or [batch, V]."""
+        tokens = np.atleast_2d(_np(tokens, np.uint32))
+        B, n = tokens.shape
+        V = self.config.vocab_size
+        p = C.c_void_p()
+        self.ctx.call("agpu_malloc", tokens.nbytes, C.byref(p))
+        rows = B * n if all_rows else B
+        lg = C.c_void_p()
+        self.ctx.call("agpu_malloc", rows * V * 4, C.byref(lg))
+        try:
+            self.ctx.call("agpu_memcpy_h2d", p.value, tokens, tokens.nbytes)
+            self._call("agpu_gpt2_forward_cached", p.value, B, n, lg.value, int(all_rows))
+            out = np.empty((B, n, V) if all_rows else (B, V), np.float32)
+            self.ctx.call("agpu_memcpy_d2h", out, lg.value, out.nbytes)
+        finally:
+            self.ctx.call("agpu_free", p.value)
+            self.ctx.call("agpu_free", lg.value)
+        return out
+
+    def forward(self, tokens):
+        """Int4Gpt2Model::forward (gpt2.rs:1522-1533): uncached, logits [seq, V] of one sequence."""
+        self.reset_cache()
+        return self.forward_cached(np.asarray(tokens).reshape(1, -1), all_rows=True)[0]
+
+    def generate_cached(self, prompt, max_new_tokens, eos=50256):
+        """Returns (list of token arrays per sequence, (prefill_ms, decode_ms))."""
+        prompt = np.atleast_2d(_np(prompt, np.uint32))
+        B, n = prompt.shape
+        out = np.zeros((B, n + max_new_tokens), np.uint32)
+        lens = np.zeros(B, np.int32)
+        ms = np.zeros(2, np.float32)
+        self._call("agpu_gpt2_generate_cached", prompt, B, n, max_new_tokens, eos, out, lens, ms)
+        return [out[b, :lens[b]].copy() for b in range(B)], (float(ms[0]), float(ms[1]))
+
+    def generate(self, prompt, max_new_tokens, eos=50256):
+        prompt = _np(prompt, np.uint32).ravel()
+        out = np.zeros(prompt.size + max_new_tokens, np.uint32)
+        n = C.c_int32(0)
+        self._call("agpu_gpt2_generate", prompt, prompt.size, max_new_tokens, eos, out, C.addressof(n))
+        return out[: n.value].copy()
+
+    def decode_steps(self, batch, steps):
+        """Replays `steps` decode steps from the current state; returns the total milliseconds."""
+        ms = C.c_float(0)
+        self._call("agpu_gpt2_decode_steps", batch, steps, C.addressof(ms))
+        return float(ms.value)

@@ -1,0 +1,113 @@
+/*
+ * agpu_gpt2.h — C ABI of the int4 GPT-2 model driver in libagpu_hip.so.
+ *
+ * Replaces, for the quantized GPT-2 path of async_gpu (paths relative to the reference
+ * checkout, crates/core/gpu-host/src/):
+ *   - nn/models/gpt2.rs:1341-1580  Int4Gpt2Model::{from_weights, forward, generate}
+ *   - nn/models/gpt2.rs:712-783    forward_cached / generate_cached (f32 model only in the
+ *                                  reference; composed here with the int4 Linears)
+ *   - nn/models/gpt2.rs:1064-1117  KvCache — held on the device here, [layer][batch][head][n_positions][64]
+ *   - nn/models/gpt2.rs:991-997    argmax (tie rule selectable, see agpu_gpt2_config.argmax_last)
+ * Weight setters take HOST pointers, like Int4Linear::new(&[u32], &[f32], ...) and
+ * Embedding::new(&[f32], ...) do (nn/layers/int4_linear.rs:40-68, nn/layers/embedding.rs:25-40);
+ * each has an `on_device` switch for data that already lives in device memory.
+ *
+ * Same conventions as agpu.h: int32 return codes, agpu_last_error_string(ctx) for details,
+ * all work on the context's stream.  One model is used by one thread at a time.
+ */
+#ifndef AGPU_GPT2_H
+#define AGPU_GPT2_H
+
+#include "agpu.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct agpu_gpt2 agpu_gpt2;
+
+#define AGPU_LM_HEAD_INT4 0 /* tied head wte^T quantized like every other Linear (K = n_embd, N = vocab) */
+#define AGPU_LM_HEAD_F32 1  /* the reference model's f32 Linear over wte (gpt2.rs:1415-1422) */
+
+typedef struct agpu_gpt2_config {
+    int32_t n_layer, n_embd, n_head, vocab_size, n_positions; /* Gpt2Config, gpt2.rs:20-34 */
+    float layer_norm_epsilon;
+    int32_t group_size;  /* int4 group along K (reference default 128, gpt2.rs:1358) */
+    int32_t max_batch;   /* independent sequences that share the weights (>= 1) */
+    int32_t lm_head;     /* AGPU_LM_HEAD_* */
+    int32_t gelu;        /* AGPU_GELU_TANH (CPU reference, tests_inference.rs:3680) or AGPU_GELU_QUICK (ops::gelu) */
+    int32_t argmax_last; /* 0: first maximal index (tests_inference.rs:4504-4515); 1: last (gpt2.rs:991-997) */
+} agpu_gpt2_config;
+
+/* Gpt2Config::{small, xl} (gpt2.rs:37-82) with group 32, batch 1, int4 head, tanh GELU, first-index argmax. */
+int32_t agpu_gpt2_config_small(agpu_gpt2_config *out);
+int32_t agpu_gpt2_config_xl(agpu_gpt2_config *out);
+
+int32_t agpu_gpt2_create(agpu_ctx *ctx, const agpu_gpt2_config *cfg, agpu_gpt2 **out);
+int32_t agpu_gpt2_destroy(agpu_gpt2 *m);
+
+/* Embedding::new + ln_f (gpt2.rs:1368-1375,1408-1413): wte [vocab, d], wpe [n_positions, d], gains/biases [d]. */
+int32_t agpu_gpt2_set_embeddings(agpu_gpt2 *m, const float *wte, const float *wpe, const float *lnf_g,
+                                 const float *lnf_b, int32_t on_device);
+int32_t agpu_gpt2_set_layer_norms(agpu_gpt2 *m, int32_t layer, const float *ln1_g, const float *ln1_b,
+                                  const float *ln2_g, const float *ln2_b, int32_t on_device);
+#define AGPU_LINEAR_QKV 0     /* c_attn   [d, 3d]  */
+#define AGPU_LINEAR_PROJ 1    /* c_proj   [d, d]   */
+#define AGPU_LINEAR_FC 2      /* mlp fc   [d, 4d]  */
+#define AGPU_LINEAR_FC_PROJ 3 /* mlp proj [4d, d]  */
+/* Int4Linear::new (int4_linear.rs:40-68): packed [K/8, N] u32, scales [ceil(K/group), N] f32, bias [N] or NULL.
+ * layer == -1 sets the tied int4 LM head (K = n_embd, N = vocab_size, no bias). */
+int32_t agpu_gpt2_set_int4_linear(agpu_gpt2 *m, int32_t layer, int32_t which, const uint32_t *packed,
+                                  const float *scales, const float *bias, int32_t K, int32_t N, int32_t on_device);
+/* Int4TransformerBlock::new's path (gpt2.rs:1257-1264): quantize weight_t [K, N] f32 with
+ * quantize_weight_int4 (mode AGPU_QUANT_*) on the device, then keep the packed form. */
+int32_t agpu_gpt2_quantize_linear(agpu_gpt2 *m, int32_t layer, int32_t which, const float *weight_t,
+                                  const float *bias, int32_t K, int32_t N, int32_t mode, int32_t on_device);
+
+/* Int4Gpt2Model::quantized_memory_bytes (gpt2.rs:1565-1577): packed + scales + bias of the block Linears. */
+int64_t agpu_gpt2_quantized_memory_bytes(const agpu_gpt2 *m);
+
+/* KvCache::{new, len} (gpt2.rs:1078-1104): forget every cached position / positions cached. */
+int32_t agpu_gpt2_reset_cache(agpu_gpt2 *m);
+int32_t agpu_gpt2_cache_len(const agpu_gpt2 *m);
+
+/*
+ * forward_cached (gpt2.rs:712-734): run `new_len` new tokens of each of `batch` sequences
+ * (tokens [batch, new_len] u32, DEVICE pointer) at positions cache_len .. cache_len+new_len-1,
+ * append their K/V to the cache and write logits (DEVICE pointer, may be NULL):
+ *   all_rows != 0: [batch, new_len, vocab_size]   (what the reference returns)
+ *   all_rows == 0: [batch, vocab_size], last position only (what generation consumes)
+ * With an empty cache this is Int4Gpt2Model::forward (gpt2.rs:1522-1533).
+ * AGPU_ERR_DIM_OUT_OF_RANGE when cache_len + new_len > n_positions.
+ */
+int32_t agpu_gpt2_forward_cached(agpu_gpt2 *m, const uint32_t *tokens, int32_t batch, int32_t new_len,
+                                 float *logits, int32_t all_rows);
+
+/*
+ * generate_cached (gpt2.rs:740-783), greedy: prefill the prompts [batch, prompt_len] (HOST pointer),
+ * then one token per step; the step loop runs as replayed HIP graphs with arg-max and the token
+ * feed on the device.  A sequence stops before appending `eos` (gpt2.rs:762,776); eos < 0 never stops.
+ *   tokens_out [batch, prompt_len + max_new_tokens] u32 (HOST): prompt followed by generated ids
+ *   lengths_out [batch] (HOST): valid entries per sequence
+ *   timing_ms_out (HOST, optional, 2 floats): prefill time, decode-loop time (first token comes from prefill)
+ */
+int32_t agpu_gpt2_generate_cached(agpu_gpt2 *m, const uint32_t *prompt_host, int32_t batch, int32_t prompt_len,
+                                  int32_t max_new_tokens, int32_t eos, uint32_t *tokens_out_host,
+                                  int32_t *lengths_out_host, float *timing_ms_out_host);
+
+/* Int4Gpt2Model::generate (gpt2.rs:1536-1560): no cache, the whole sequence is re-run per new token. */
+int32_t agpu_gpt2_generate(agpu_gpt2 *m, const uint32_t *prompt_host, int32_t prompt_len, int32_t max_new_tokens,
+                           int32_t eos, uint32_t *tokens_out_host, int32_t *length_out_host);
+
+/*
+ * Benchmark hook: replay `steps` decode steps (one token per sequence per step) starting from the
+ * current cache state and the device-resident current tokens, without any host round trip, and
+ * report the time per step measured with HIP events on the context's stream.  The cache advances by
+ * `steps` positions.  Requires a previous forward/generate call and cache_len + steps <= n_positions.
+ */
+int32_t agpu_gpt2_decode_steps(agpu_gpt2 *m, int32_t batch, int32_t steps, float *ms_total_out_host);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AGPU_GPT2_H */

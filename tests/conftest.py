@@ -47,3 +47,25 @@ def to_dev(a, dev):
 
 def to_np_u32(t):
     return t.cpu().numpy().view(np.uint32)
+
+
+def build_oracle_model(cfg, qz, lm_head_int4=True):
+    """The f64 oracle model (oracle/orc.py Gpt2) loaded from a workloads.quantize_gpt2 dict."""
+    from async_gpu_amd import workloads
+
+    m = orc_mod.Gpt2(**cfg)
+    m.set_embeddings(qz["wte"], qz["wpe"], qz["lnf_g"], qz["lnf_b"])
+    for li, L in enumerate(qz["layers"]):
+        m.set_layer_norms(li, L["ln1_g"], L["ln1_b"], L["ln2_g"], L["ln2_b"])
+        for wi, name in enumerate(workloads.LINEAR_NAMES):
+            m.set_int4_linear(li, wi, L[name][0], L[name][1], L[name][2], qz["group"])
+    if lm_head_int4:
+        m.set_int4_linear(-1, 0, qz["lm_head"][0], qz["lm_head"][1], None, qz["group"])
+    return m
+
+
+def gpu_config(cfg, **kw):
+    from async_gpu_amd import gpt2
+
+    return gpt2.Gpt2Config(cfg["n_layer"], cfg["n_embd"], cfg["n_head"], vocab_size=cfg["vocab"],
+                           n_positions=cfg["n_positions"], **kw)

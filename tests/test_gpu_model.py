@@ -1,0 +1,200 @@
+"""GPU parity of the int4 GPT-2 model driver (include/agpu_gpt2.h) against the f64 CPU oracle:
+logits within 2e-4 after all layers, greedy token ids identical, cached == uncached."""
+import numpy as np
+import pytest
+
+from conftest import build_oracle_model, gpu_config
+
+pytestmark = pytest.mark.gpu
+
+TOL_LOGITS = 2e-4  # logits after all layers vs the f64 CPU path
+
+
+def _quantized(orc, cfg, seed, group=32, std=0.08, **kw):
+    from async_gpu_amd import workloads
+    w = workloads.gpt2_fp32_weights(cfg, seed, std=std, **kw)
+    qz = workloads.quantize_gpt2(w, group, lambda wt, g: orc.quantize_weight_int4(wt, g, orc.SCRIPT))
+    return w, qz
+
+
+def _assert_tokens_match(got, ref, margins, prompt_len, what):
+    """Greedy ids must be identical.  If they are not, name the first divergence and the oracle's
+    top-1/top-2 logit gap there, so a near-tie is distinguishable from a wrong kernel."""
+    n = min(len(got), len(ref))
+    diff = [i for i in range(n) if got[i] != ref[i]]
+    if diff or len(got) != len(ref):
+        i = diff[0] if diff else n
+        gap = margins[i - prompt_len] if prompt_len <= i < prompt_len + len(margins) else float("nan")
+        pytest.fail(f"{what}: tokens diverge at index {i} (gpu {got[i] if i < len(got) else None}, oracle "
+                    f"{ref[i] if i < len(ref) else None}); oracle top-1/top-2 gap there {gap:.3e}")
+
+
+@pytest.fixture(scope="module")
+def tiny(orc, agpu, dev):
+    from async_gpu_amd import gpt2, workloads
+    cfg = workloads.GPT2_TINY
+    w, qz = _quantized(orc, cfg, 11, nonzero_bias=True, random_ln=True)
+    om = build_oracle_model(cfg, qz)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg), qz)
+    return cfg, w, qz, om, gm
+
+
+def test_tiny_forward_logits(tiny, agpu):
+    from async_gpu_amd import workloads
+    cfg, w, qz, om, gm = tiny
+    for n in (1, 9, 17, 40):
+        tokens = workloads.random_prompt(cfg, n, n)
+        om.reset_cache()
+        ref = om.forward(tokens, all_rows=True)
+        got = gm.forward(tokens)
+        assert got.shape == (n, cfg["vocab"])
+        assert np.abs(got - ref).max() <= TOL_LOGITS
+
+
+def test_tiny_chunked_cached_forward(tiny):
+    from async_gpu_amd import workloads
+    cfg, w, qz, om, gm = tiny
+    tokens = workloads.random_prompt(cfg, 5, 30)
+    full = gm.forward(tokens)
+    gm.reset_cache()
+    a = gm.forward_cached(tokens[:7].reshape(1, -1))[0]
+    assert gm.cache_len() == 7
+    b = gm.forward_cached(tokens[7:27].reshape(1, -1))[0]      # GEMM + MFMA attention path with a cache
+    c = gm.forward_cached(tokens[27:28].reshape(1, -1))[0]     # decode path
+    d = gm.forward_cached(tokens[28:].reshape(1, -1), all_rows=False)  # last row only
+    assert gm.cache_len() == 30
+    got = np.concatenate([a, b, c], axis=0)
+    assert np.abs(got - full[:28]).max() <= 1e-5
+    assert np.abs(d[0] - full[29]).max() <= 1e-5
+
+
+def test_tiny_generate_matches_oracle(tiny):
+    from async_gpu_amd import workloads
+    cfg, w, qz, om, gm = tiny
+    prompt = workloads.random_prompt(cfg, 4, 6)
+    ref, margins = om.generate(prompt, 40, cached=True, eos=-1)
+    (got,), _ = gm.generate_cached(prompt, 40, eos=-1)
+    _assert_tokens_match(got, ref, margins, 6, "generate_cached")
+    unc = gm.generate(prompt, 12, eos=-1)
+    _assert_tokens_match(unc, ref[:18], margins, 6, "generate (uncached)")  # tests_inference.rs:6114-6171
+    # replaying is deterministic and graphs survive a second run
+    (again,), _ = gm.generate_cached(prompt, 40, eos=-1)
+    assert np.array_equal(again, got)
+
+
+def test_tiny_eos_and_limits(tiny, agpu):
+    from async_gpu_amd import workloads
+    cfg, w, qz, om, gm = tiny
+    prompt = workloads.random_prompt(cfg, 4, 6)
+    (toks,), _ = gm.generate_cached(prompt, 10, eos=-1)
+    stop = int(toks[8])
+    (cut,), _ = gm.generate_cached(prompt, 10, eos=stop)  # gpt2.rs:762,776: stop before appending
+    first = list(toks[6:]).index(stop)
+    assert np.array_equal(cut, toks[:6 + first])
+    assert np.array_equal(gm.generate(prompt, 10, eos=stop), cut)
+    (zero,), _ = gm.generate_cached(prompt, 0)
+    assert np.array_equal(zero, prompt)
+    # context limit: 64 positions
+    (full,), _ = gm.generate_cached(prompt, 59, eos=-1)
+    assert len(full) == 65 and gm.cache_len() == 64
+    with pytest.raises(agpu.AgpuError) as e:
+        gm.generate_cached(prompt, 60, eos=-1)
+    assert e.value.code == agpu._lib.ERR_DIM_OUT_OF_RANGE
+    with pytest.raises(agpu.AgpuError) as e:
+        gm.forward(np.zeros(65, np.uint32))
+    assert e.value.code == agpu._lib.ERR_DIM_OUT_OF_RANGE
+    with pytest.raises(agpu.AgpuError) as e:
+        gm.generate_cached(np.zeros((2, 4), np.uint32), 3)  # max_batch is 1
+    assert e.value.code == agpu._lib.ERR_SHAPE_MISMATCH
+
+
+def test_from_weights_quantizes_like_the_host_function(tiny, orc, agpu):
+    """Int4Gpt2Model::from_weights (gpt2.rs:1362-1433): fp32 in, quantize_weight_int4 at load."""
+    from async_gpu_amd import gpt2, workloads
+    cfg, w, qz, om, gm = tiny
+    qr = workloads.quantize_gpt2(w, 32, lambda wt, g: orc.quantize_weight_int4(wt, g, orc.RUST))
+    ref_model = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg), qr)
+    dev_model = gpt2.Int4Gpt2Model.from_weights(gpu_config(cfg), w, mode=agpu._lib.QUANT_RUST)
+    tokens = workloads.random_prompt(cfg, 8, 12)
+    assert np.array_equal(ref_model.forward(tokens), dev_model.forward(tokens))
+    assert dev_model.quantized_memory_bytes() == ref_model.quantized_memory_bytes()
+    # Int4Linear::memory_bytes (int4_linear.rs:136-146), summed as gpt2.rs:1565-1577 does
+    d, ff, L = cfg["n_embd"], 4 * cfg["n_embd"], cfg["n_layer"]
+    per = sum(k // 8 * n * 4 + (k + 31) // 32 * n * 4 + n * 4 for k, n in [(d, 3 * d), (d, d), (d, ff), (ff, d)])
+    assert dev_model.quantized_memory_bytes() == L * per
+
+
+def test_f32_lm_head_and_quick_gelu_and_last_index(orc, agpu, dev):
+    """The reference model as it is: f32 head over wte (gpt2.rs:1415-1422); plus the opt-in forms."""
+    from async_gpu_amd import gpt2, workloads
+    cfg = workloads.GPT2_TINY
+    w, qz = _quantized(orc, cfg, 12, nonzero_bias=True)
+    om = build_oracle_model(cfg, qz, lm_head_int4=False)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg, lm_head=gpt2.LM_HEAD_F32), qz)
+    tokens = workloads.random_prompt(cfg, 2, 20)
+    ref = om.forward(tokens, all_rows=True)
+    assert np.abs(gm.forward(tokens) - ref).max() <= TOL_LOGITS
+    refg, margins = om.generate(tokens[:5], 20, cached=True, eos=-1)
+    (got,), _ = gm.generate_cached(tokens[:5], 20, eos=-1)
+    _assert_tokens_match(got, refg, margins, 5, "f32 head")
+    # quick GELU differs from tanh GELU but stays finite and deterministic
+    gq = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg, gelu=agpu._lib.GELU_QUICK), qz)
+    lq = gq.forward(tokens)
+    assert np.isfinite(lq).all() and np.abs(lq - gm.forward(tokens)).max() > 1e-4
+
+
+def test_batch_of_independent_sequences(orc, agpu, dev):
+    """B sequences share the weights; each must equal its own single-sequence run."""
+    from async_gpu_amd import gpt2, workloads
+    cfg = workloads.GPT2_TINY
+    w, qz = _quantized(orc, cfg, 13, nonzero_bias=True, random_ln=True)
+    om = build_oracle_model(cfg, qz)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg, max_batch=16), qz)
+    prompts = workloads.random_prompt(cfg, 6, 9, batch=16)
+    outs, _ = gm.generate_cached(prompts, 20, eos=-1)
+    for b in (0, 3, 15):
+        ref, margins = om.generate(prompts[b], 20, cached=True, eos=-1)
+        _assert_tokens_match(outs[b], ref, margins, 9, f"batch row {b}")
+    lg = gm.forward_cached(prompts[:5, :1], all_rows=False)  # cache holds 28 positions; 5 decode rows
+    assert lg.shape == (5, cfg["vocab"])
+
+
+def test_xl_shaped_layers(orc, agpu, dev):
+    """GPT-2 XL geometry (d=1600, 25 heads, ffn 6400) with 2 layers, batch 1 and 16."""
+    from async_gpu_amd import gpt2, workloads
+    cfg = dict(n_layer=2, n_embd=1600, n_head=25, vocab=2003, n_positions=128)
+    w, qz = _quantized(orc, cfg, 4, std=0.02)
+    om = build_oracle_model(cfg, qz)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg, max_batch=16), qz)
+    prompts = workloads.random_prompt(cfg, 4, 24, batch=16)
+    om.reset_cache()
+    ref = om.forward(prompts[0], all_rows=True)
+    assert np.abs(gm.forward(prompts[0]) - ref).max() <= TOL_LOGITS
+    outs, _ = gm.generate_cached(prompts, 12, eos=-1)
+    for b in (0, 15):
+        refg, margins = om.generate(prompts[b], 12, cached=True, eos=-1)
+        _assert_tokens_match(outs[b], refg, margins, 24, f"xl-shaped batch row {b}")
+
+
+def test_config4_gpt2_small_generation(orc, agpu, dev):
+    """BASELINE config 4: GPT-2 small, random init N(0, 0.02), int4 group 32 (script rounding),
+    prompt of 64 uniform ids, 128 greedy steps, seed 3.  Tokens identical to the f64 CPU path,
+    logits within 2e-4."""
+    from async_gpu_amd import gpt2, workloads
+    cfg = workloads.GPT2_SMALL
+    w = workloads.gpt2_fp32_weights(cfg, 3)
+    qz = workloads.quantize_gpt2(w, 32, lambda wt, g: orc.quantize_weight_int4(wt, g, orc.SCRIPT))
+    om = build_oracle_model(cfg, qz)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg), qz)
+    prompt = workloads.random_prompt(cfg, 3, 64)
+    om.reset_cache()
+    ref_logits = om.forward(prompt, all_rows=False)
+    gm.reset_cache()
+    got_logits = gm.forward_cached(prompt.reshape(1, -1), all_rows=False)
+    err = np.abs(got_logits[0] - ref_logits[0]).max()
+    assert err <= TOL_LOGITS, f"prefill logits differ by {err}"
+    ref, margins = om.generate(prompt, 128, cached=True, eos=-1)
+    (got,), (ms_prefill, ms_decode) = gm.generate_cached(prompt, 128, eos=-1)
+    _assert_tokens_match(got, ref, margins, 64, "config 4")
+    assert len(got) == 192
+    print(f"config4: prefill {ms_prefill:.3f} ms, decode {ms_decode / 127:.4f} ms/token, min oracle margin {margins.min():.3e}")
