@@ -49,9 +49,14 @@ SIGNATURES = {
     "agpu_memcpy_d2h": (_i32, [_vp, _vp, _vp, _sz]),
     "agpu_memcpy_d2d": (_i32, [_vp, _vp, _vp, _sz]),
     "agpu_sync": (_i32, [_vp]),
+    "agpu_timer_start": (_i32, [_vp]),
+    "agpu_timer_stop": (_i32, [_vp, _vp]),
     "agpu_kernel_lookup": (_i32, [_vp, C.c_char_p, C.POINTER(C.c_char_p)]),
     "agpu_int4_linear": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32]),
+    "agpu_int4_gemv_tune": (None, [_i32, _i32]),
     "agpu_ln_int4_linear": (_i32, [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32]),
+    "agpu_bench_int4_linear": (_i32, [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32,
+                                      _i32, C.c_int64, C.c_int64, _i32, _vp]),
     "agpu_int4_dequantize": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32]),
     "agpu_int4_quantize": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32]),
     "agpu_int4_quantize_host": (_i32, [_vp, _vp, _vp, _i32, _i32, _i32, _i32]),
@@ -162,6 +167,30 @@ class Context:
 
     def sync(self):
         self.call("agpu_sync")
+
+    def timer_start(self):
+        self.call("agpu_timer_start")
+
+    def timer_stop(self):
+        ms = C.c_float(0)
+        self.call("agpu_timer_stop", C.addressof(ms))
+        return float(ms.value)
+
+    def malloc(self, nbytes):
+        p = _vp()
+        self.call("agpu_malloc", nbytes, C.byref(p))
+        return p.value
+
+    def free(self, p):
+        self.call("agpu_free", p)
+
+    def upload(self, array):
+        """numpy array -> freshly allocated device buffer (int address)."""
+        import numpy as np
+        a = np.ascontiguousarray(array)
+        p = self.malloc(a.nbytes)
+        self.call("agpu_memcpy_h2d", p, a, a.nbytes)
+        return p
 
     def get(self, name):
         """registry.get(name): entry point serving a reference kernel name, or KernelNotFound."""

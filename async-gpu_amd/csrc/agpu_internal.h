@@ -21,6 +21,7 @@ struct agpu_ctx {
     int num_cus = 256;
     char *workspace = nullptr;      // kWorkspaceBytes of device scratch
     unsigned int *counters = nullptr;  // kNumCounters zeroed uint32; kernels restore zero
+    hipEvent_t t0 = nullptr, t1 = nullptr;  // agpu_timer_*
     char err[512] = {0};
 };
 

@@ -1,8 +1,8 @@
 // Causal attention for gfx950, d_head = 64, fp32.
 //   * attn_mfma_kernel: prefill / chunked prefill.  One wave per 32 query rows; S^T = K Q^T and
 //     O^T = V^T P^T on v_mfma_f32_32x32x2_f32 with online softmax; K/V tiles of 32 keys in LDS.
-//   * attn_splitkv_kernel: decode (few query rows).  The keys are split over workgroups and waves;
-//     16 lanes share one key (float4 each), partial (m, l, o) are merged in a fixed order.
+//   * attn_decode_kernel: decode (few query rows).  One workgroup per (head, query row); its waves
+//     split the keys, 16 lanes share one key (float4 each), partial (m, l, o) merge in a fixed order.
 #include "agpu_internal.h"
 #include "attention.h"
 
@@ -144,53 +144,75 @@ __device__ __forceinline__ void merge_partial(float &m, float &l, float4 &o, flo
     m = mn;
 }
 
-// grid (nsplit, q_len, n_heads * batch), 256 threads.  Workgroup (s, i, hb) takes keys
-// [s*chunk, (s+1)*chunk) that query row i may see.  Lane layout: 16 lanes x float4 per key,
-// 4 keys per wave step, 16 keys per workgroup step.
-__global__ __launch_bounds__(256) void attn_splitkv_kernel(const AttnParams p, int chunk, float *part,
-                                                            unsigned int *counters) {
-    __shared__ float sm[4], sl[4];
-    __shared__ __align__(16) float so[4][DH];
-    __shared__ int s_last;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+// grid (q_len, n_heads * batch), 64*W threads.  One workgroup per (head, query row) takes every
+// visible key, so nothing crosses a workgroup.  Lane layout: 16 lanes x float4 per key, 4 keys
+// per wave step; a lane group handles PASS keys per pass (scores first, then one rescale),
+// the W waves interleave over the keys.  Partials merge in a fixed order: lane groups, then waves.
+constexpr int PASS = 8;
+
+__global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
+    __shared__ float sm[16], sl[16];
+    __shared__ __align__(16) float so[16][DH];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6;
     const int gq = lane >> 4, sub = lane & 15;
-    const int split = blockIdx.x, nsplit = gridDim.x, qi = blockIdx.y, hb = blockIdx.z;
+    const int qi = blockIdx.x, hb = blockIdx.y;
     const int b = hb / p.n_heads, h = hb % p.n_heads;
     int kv_len, q_offset;
     resolve_positions(p, kv_len, q_offset);
     const int vis = p.causal ? min(kv_len, q_offset + qi + 1) : kv_len;  // keys [0, vis)
-    const int ja = split * chunk, jb = min(vis, ja + chunk);
 
-    const float *kh = p.k + (size_t)hb * p.kv_stride * DH;
-    const float *vh = p.v + (size_t)hb * p.kv_stride * DH;
+    const float *kh = p.k + (size_t)hb * p.kv_stride * DH + 4 * sub;
+    const float *vh = p.v + (size_t)hb * p.kv_stride * DH + 4 * sub;
     const float *qrow = p.q + (size_t)b * p.q_batch_stride + (size_t)h * p.q_head_stride + (size_t)qi * p.q_row_stride;
     float4 q4 = *reinterpret_cast<const float4 *>(qrow + 4 * sub);
     q4.x *= 0.125f; q4.y *= 0.125f; q4.z *= 0.125f; q4.w *= 0.125f;
 
     float m = -INFINITY, l = 0.0f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int j = ja + wave * 4 + gq; j < jb; j += 16) {
-        const float4 k4 = *reinterpret_cast<const float4 *>(kh + (size_t)j * DH + 4 * sub);
-        const float4 v4 = *reinterpret_cast<const float4 *>(vh + (size_t)j * DH + 4 * sub);
-        float s = (q4.x * k4.x + q4.y * k4.y) + (q4.z * k4.z + q4.w * k4.w);
-        s += __shfl_xor(s, 8, kWave);
-        s += __shfl_xor(s, 4, kWave);
-        s += __shfl_xor(s, 2, kWave);
-        s += __shfl_xor(s, 1, kWave);
-        const float mn = fmaxf(m, s);
-        const float a = expf(m - mn), pj = expf(s - mn);
-        l = l * a + pj;
-        o.x = o.x * a + pj * v4.x; o.y = o.y * a + pj * v4.y; o.z = o.z * a + pj * v4.z; o.w = o.w * a + pj * v4.w;
+    const int stride = 4 * W;  // keys between two consecutive keys of one lane group
+    for (int base = wave * 4 + gq; base < vis; base += PASS * stride) {
+        float s[PASS];
+        float4 v4[PASS];
+        float bm = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < PASS; ++i) {
+            const int j = base + i * stride;
+            s[i] = -INFINITY;
+            v4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (j < vis) {
+                const float4 k4 = *reinterpret_cast<const float4 *>(kh + (size_t)j * DH);
+                v4[i] = *reinterpret_cast<const float4 *>(vh + (size_t)j * DH);
+                s[i] = (q4.x * k4.x + q4.y * k4.y) + (q4.z * k4.z + q4.w * k4.w);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < PASS; ++i) {
+            // masked lanes carry -inf through the adds unchanged (all 16 lanes of a group agree on j < vis)
+            s[i] += __shfl_xor(s[i], 8, kWave);
+            s[i] += __shfl_xor(s[i], 4, kWave);
+            s[i] += __shfl_xor(s[i], 2, kWave);
+            s[i] += __shfl_xor(s[i], 1, kWave);
+            bm = fmaxf(bm, s[i]);
+        }
+        const float mn = fmaxf(m, bm);  // finite: the first key of the pass is visible
+        const float a = expf(m - mn);
+        l *= a;
+        o.x *= a; o.y *= a; o.z *= a; o.w *= a;
+#pragma unroll
+        for (int i = 0; i < PASS; ++i) {
+            const float pj = expf(s[i] - mn);  // exp(-inf) = 0 for masked keys
+            l += pj;
+            o.x += pj * v4[i].x; o.y += pj * v4[i].y; o.z += pj * v4[i].z; o.w += pj * v4[i].w;
+        }
         m = mn;
     }
-    // merge the 4 lane groups of the wave (xor 16, then xor 32): fixed order
+    // merge the 4 lane groups of the wave (xor 16, then xor 32): both partners use the same operand order
 #pragma unroll
     for (int off = 16; off <= 32; off <<= 1) {
         const float m2 = __shfl_xor(m, off, kWave), l2 = __shfl_xor(l, off, kWave);
         float4 o2;
         o2.x = __shfl_xor(o.x, off, kWave); o2.y = __shfl_xor(o.y, off, kWave);
         o2.z = __shfl_xor(o.z, off, kWave); o2.w = __shfl_xor(o.w, off, kWave);
-        // both partners must combine in the same operand order to stay bit-identical
         if ((lane & off) == 0) merge_partial(m, l, o, m2, l2, o2);
         else {
             float mm = m2, ll = l2;
@@ -204,49 +226,14 @@ __global__ __launch_bounds__(256) void attn_splitkv_kernel(const AttnParams p, i
         *reinterpret_cast<float4 *>(&so[wave][4 * sub]) = o;
     }
     __syncthreads();
-    // partial record: [m, l, o[64]] = 66 floats per (hb, qi, split)
-    const size_t rec = ((size_t)hb * p.q_len + qi) * nsplit;
     if (wave == 0 && lane < 16) {
         m = sm[0]; l = sl[0];
         o = *reinterpret_cast<const float4 *>(&so[0][4 * sub]);
-        for (int w = 1; w < 4; ++w) merge_partial(m, l, o, sm[w], sl[w], *reinterpret_cast<const float4 *>(&so[w][4 * sub]));
-        if (nsplit == 1) {
-            const float inv = 1.0f / l;
-            float *orow = p.o + (size_t)b * p.o_batch_stride + (size_t)h * p.o_head_stride + (size_t)qi * p.o_row_stride;
-            *reinterpret_cast<float4 *>(orow + 4 * sub) = make_float4(o.x * inv, o.y * inv, o.z * inv, o.w * inv);
-        } else {
-            float *pr = part + (rec + split) * 66;
-            if (lane == 0) { pr[0] = m; pr[1] = l; }
-            pr[2 + 4 * sub] = o.x; pr[3 + 4 * sub] = o.y; pr[4 + 4 * sub] = o.z; pr[5 + 4 * sub] = o.w;
-        }
-    }
-    if (nsplit == 1) return;
-    __threadfence();
-    __syncthreads();
-    const int cidx = hb * p.q_len + qi;
-    if (tid == 0) {
-        const unsigned int t = atomicAdd(&counters[cidx], 1u);
-        s_last = (t == (unsigned int)(nsplit - 1));
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-    if (wave == 0 && lane < 16) {
-        m = -INFINITY; l = 0.0f;
-        o = make_float4(0.f, 0.f, 0.f, 0.f);
-        for (int s = 0; s < nsplit; ++s) {
-            const float *pr = part + (rec + s) * 66;
-            const float m2 = __builtin_nontemporal_load(pr), l2 = __builtin_nontemporal_load(pr + 1);
-            float4 o2;
-            o2.x = __builtin_nontemporal_load(pr + 2 + 4 * sub); o2.y = __builtin_nontemporal_load(pr + 3 + 4 * sub);
-            o2.z = __builtin_nontemporal_load(pr + 4 + 4 * sub); o2.w = __builtin_nontemporal_load(pr + 5 + 4 * sub);
-            merge_partial(m, l, o, m2, l2, o2);
-        }
+        for (int w = 1; w < W; ++w) merge_partial(m, l, o, sm[w], sl[w], *reinterpret_cast<const float4 *>(&so[w][4 * sub]));
         const float inv = 1.0f / l;
         float *orow = p.o + (size_t)b * p.o_batch_stride + (size_t)h * p.o_head_stride + (size_t)qi * p.o_row_stride;
         *reinterpret_cast<float4 *>(orow + 4 * sub) = make_float4(o.x * inv, o.y * inv, o.z * inv, o.w * inv);
     }
-    if (tid == 0) counters[cidx] = 0u;
 }
 
 }  // namespace
@@ -254,14 +241,11 @@ __global__ __launch_bounds__(256) void attn_splitkv_kernel(const AttnParams p, i
 int32_t agpu_attention_launch(agpu_ctx *ctx, const AttnParams &p, int max_kv_len) {
     const int hb = p.n_heads * p.batch;
     if (p.q_len <= 8) {
-        const int chunk = 64;
-        const int nsplit = ceil_div(max_kv_len, chunk);
-        if ((size_t)hb * p.q_len > (size_t)kNumCounters ||
-            (size_t)hb * p.q_len * nsplit * 66 * sizeof(float) > kWorkspaceBytes)
-            return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "attention: heads*q_len*splits too large");
-        hipLaunchKernelGGL(attn_splitkv_kernel, dim3(nsplit, p.q_len, hb), dim3(256), 0, ctx->stream, p, chunk,
-                           reinterpret_cast<float *>(ctx->workspace), ctx->counters);
-        return AGPU_LAUNCH_CHECK(ctx, "attn_splitkv_kernel");
+        // waves per workgroup: one per 32 keys of the longest possible context, 1..16
+        int W = ceil_div(max_kv_len, 32);
+        W = W < 1 ? 1 : (W > 16 ? 16 : W);
+        hipLaunchKernelGGL(attn_decode_kernel, dim3(p.q_len, hb), dim3(64 * W), 0, ctx->stream, p);
+        return AGPU_LAUNCH_CHECK(ctx, "attn_decode_kernel");
     }
     hipLaunchKernelGGL(attn_mfma_kernel, dim3(ceil_div(p.q_len, 32), hb), dim3(64), 0, ctx->stream, p);
     return AGPU_LAUNCH_CHECK(ctx, "attn_mfma_kernel");

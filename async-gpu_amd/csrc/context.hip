@@ -64,6 +64,8 @@ AGPU_EXPORT int32_t agpu_ctx_destroy(agpu_ctx *ctx) {
     if (!ctx) return AGPU_OK;
     (void)hipSetDevice(ctx->device);
     if (ctx->stream || !ctx->owns_stream) (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->t0) (void)hipEventDestroy(ctx->t0);
+    if (ctx->t1) (void)hipEventDestroy(ctx->t1);
     if (ctx->workspace) (void)hipFree(ctx->workspace);
     if (ctx->counters) (void)hipFree(ctx->counters);
     if (ctx->owns_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -126,6 +128,26 @@ AGPU_EXPORT int32_t agpu_memcpy_d2d(agpu_ctx *ctx, void *dst, const void *src, s
 AGPU_EXPORT int32_t agpu_sync(agpu_ctx *ctx) {
     AGPU_REQUIRE_CTX(ctx);
     return agpu_hip(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+AGPU_EXPORT int32_t agpu_timer_start(agpu_ctx *ctx) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (!ctx->t0) {
+        hipError_t e = hipEventCreate(&ctx->t0);
+        if (e == hipSuccess) e = hipEventCreate(&ctx->t1);
+        if (e != hipSuccess) return agpu_hip(ctx, e, "hipEventCreate");
+    }
+    return agpu_hip(ctx, hipEventRecord(ctx->t0, ctx->stream), "hipEventRecord");
+}
+
+AGPU_EXPORT int32_t agpu_timer_stop(agpu_ctx *ctx, float *ms_out_host) {
+    AGPU_REQUIRE_CTX(ctx);
+    AGPU_REQUIRE_PTR(ctx, ms_out_host);
+    if (!ctx->t0) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "timer_stop without timer_start");
+    hipError_t e = hipEventRecord(ctx->t1, ctx->stream);
+    if (e == hipSuccess) e = hipEventSynchronize(ctx->t1);
+    if (e == hipSuccess) e = hipEventElapsedTime(ms_out_host, ctx->t0, ctx->t1);
+    return agpu_hip(ctx, e, "timer_stop");
 }
 
 // The reference's kernel names on this path (nn/registry.rs:34-103) and the entry

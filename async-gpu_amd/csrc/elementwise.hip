@@ -2,6 +2,7 @@
 // the QKV layout kernels.  All of them move each byte once: they are HBM-bound, one wave per
 // row where a row reduction is needed.
 #include "agpu_internal.h"
+#include "elementwise.h"
 
 namespace {
 
@@ -178,73 +179,75 @@ __global__ __launch_bounds__(256) void kv_append_kernel(const float *__restrict_
     cache[((size_t)h * max_seq + write_pos) * d_head + e] = src[(size_t)h * src_stride * d_head + e];
 }
 
-// Arg-max of each row in two levels: every workgroup reduces one chunk to (value, index),
-// the last workgroup of a row to arrive reduces the chunk results in chunk order.
+// Arg-max of each row: one workgroup of 1024 threads per row, so no result crosses a workgroup.
 // Ties: the smaller index wins (last_index == 0) or the larger one.
 __device__ __forceinline__ bool better(float v, unsigned int i, float bv, unsigned int bi, int last_index) {
     return (v > bv) || (v == bv && (last_index ? i > bi : i < bi));
 }
 
-__global__ __launch_bounds__(256) void argmax_rows_kernel(const float *__restrict__ x, uint32_t *idx_out,
-                                                           float *part_val, unsigned int *part_idx,
-                                                           unsigned int *counters, int cols, int row_stride,
-                                                           int chunk, int last_index) {
-    __shared__ float sv[4];
-    __shared__ unsigned int si[4];
-    __shared__ int s_last;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int row = blockIdx.y, nchunks = gridDim.x;
+__global__ __launch_bounds__(1024) void argmax_rows_kernel(const float *__restrict__ x, uint32_t *idx_out, int cols,
+                                                            int row_stride, int last_index, const ArgmaxAdvance adv) {
+    __shared__ float sv[16];
+    __shared__ unsigned int si[16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6;
+    const int row = blockIdx.x;
     const float *xr = x + (size_t)row * row_stride;
-    const int c0 = blockIdx.x * chunk, c1 = min(cols, c0 + chunk);
     float bv = -INFINITY;
     unsigned int bi = last_index ? 0u : 0xFFFFFFFFu;
-    for (int c = c0 + tid; c < c1; c += 256) {
-        const float v = xr[c];
-        if (better(v, (unsigned int)c, bv, bi, last_index)) { bv = v; bi = (unsigned int)c; }
-    }
-    auto wave_reduce = [&](float &v, unsigned int &i) {
+    if ((((uintptr_t)xr) & 15) == 0) {
+        // float4 loads, four in flight per thread
+        const int n4 = cols >> 2;
+        const float4 *x4 = reinterpret_cast<const float4 *>(xr);
+        for (int c0 = tid; c0 < n4; c0 += 4 * blockDim.x) {
+            float4 v[4];
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const float ov = __shfl_xor(v, off, kWave);
-            const unsigned int oi = __shfl_xor(i, off, kWave);
-            if (better(ov, oi, v, i, last_index)) { v = ov; i = oi; }
+            for (int u = 0; u < 4; ++u) {
+                const int c = c0 + u * blockDim.x;
+                v[u] = c < n4 ? x4[c] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const unsigned int base = 4u * (unsigned int)(c0 + u * blockDim.x);
+                if (c0 + u * (int)blockDim.x < n4) {
+                    if (better(v[u].x, base, bv, bi, last_index)) { bv = v[u].x; bi = base; }
+                    if (better(v[u].y, base + 1, bv, bi, last_index)) { bv = v[u].y; bi = base + 1; }
+                    if (better(v[u].z, base + 2, bv, bi, last_index)) { bv = v[u].z; bi = base + 2; }
+                    if (better(v[u].w, base + 3, bv, bi, last_index)) { bv = v[u].w; bi = base + 3; }
+                }
+            }
         }
-    };
-    wave_reduce(bv, bi);
+        for (int c = 4 * n4 + tid; c < cols; c += blockDim.x) {
+            const float v = xr[c];
+            if (better(v, (unsigned int)c, bv, bi, last_index)) { bv = v; bi = (unsigned int)c; }
+        }
+    } else {
+        for (int c = tid; c < cols; c += blockDim.x) {
+            const float v = xr[c];
+            if (better(v, (unsigned int)c, bv, bi, last_index)) { bv = v; bi = (unsigned int)c; }
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, kWave);
+        const unsigned int oi = __shfl_xor(bi, off, kWave);
+        if (better(ov, oi, bv, bi, last_index)) { bv = ov; bi = oi; }
+    }
     if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
     __syncthreads();
     if (tid == 0) {
-        for (int w = 1; w < 4; ++w)
+        for (int w = 1; w < W; ++w)
             if (better(sv[w], si[w], bv, bi, last_index)) { bv = sv[w]; bi = si[w]; }
-        if (nchunks == 1) {
-            idx_out[row] = (bi == 0xFFFFFFFFu) ? 0u : bi;
-        } else {
-            part_val[(size_t)row * nchunks + blockIdx.x] = bv;
-            part_idx[(size_t)row * nchunks + blockIdx.x] = bi;
-        }
-    }
-    if (nchunks == 1) return;
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) {
-        const unsigned int t = atomicAdd(&counters[row], 1u);
-        s_last = (t == (unsigned int)(nchunks - 1));
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-    if (wave == 0) {
-        bv = -INFINITY;
-        bi = last_index ? 0u : 0xFFFFFFFFu;
-        for (int c = lane; c < nchunks; c += 64) {
-            const float v = __builtin_nontemporal_load(&part_val[(size_t)row * nchunks + c]);
-            const unsigned int i = __builtin_nontemporal_load(&part_idx[(size_t)row * nchunks + c]);
-            if (better(v, i, bv, bi, last_index)) { bv = v; bi = i; }
-        }
-        wave_reduce(bv, bi);
-        if (lane == 0) {
-            idx_out[row] = (bi == 0xFFFFFFFFu) ? 0u : bi;
-            counters[row] = 0u;
+        const uint32_t best = (bi == 0xFFFFFFFFu) ? 0u : bi;
+        idx_out[row] = best;
+        if (adv.cur_tok) {
+            // token feed: the arg-max becomes the current token of this sequence and is recorded
+            const int st = *adv.step_dev;
+            adv.cur_tok[row] = best;
+            if (st < adv.out_capacity) adv.out_tok[(size_t)st * gridDim.x + row] = best;
+            if (adv.bump_counters) {  // only legal with a single row: nobody else reads the counters
+                *adv.pos_dev += adv.delta;
+                *adv.step_dev = st + 1;
+            }
         }
     }
 }
@@ -332,18 +335,15 @@ AGPU_EXPORT int32_t agpu_embedding(agpu_ctx *ctx, const uint32_t *tokens, const 
     return AGPU_LAUNCH_CHECK(ctx, "embedding_kernel");
 }
 
-// Rows of `cols` values, `row_stride` floats apart.
+// Rows of `cols` values, `row_stride` floats apart; `adv` (optional) fuses the token feed.
 int32_t agpu_argmax_rows_strided(agpu_ctx *ctx, const float *x, uint32_t *idx_out, int rows, int cols, int row_stride,
-                                 int last_index) {
-    if (rows > kNumCounters) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "argmax_rows: rows=%d too large", rows);
-    const int chunk = 2048;
-    const int nchunks = ceil_div(cols, chunk);
-    if ((size_t)rows * nchunks * 8 > kWorkspaceBytes)
-        return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "argmax_rows: rows*cols too large");
-    float *pv = reinterpret_cast<float *>(ctx->workspace);
-    unsigned int *pi = reinterpret_cast<unsigned int *>(ctx->workspace) + (size_t)rows * nchunks;
-    hipLaunchKernelGGL(argmax_rows_kernel, dim3(nchunks, rows), dim3(256), 0, ctx->stream, x, idx_out, pv, pi,
-                       ctx->counters, cols, row_stride, chunk, last_index ? 1 : 0);
+                                 int last_index, const ArgmaxAdvance *adv) {
+    ArgmaxAdvance a{};
+    if (adv) a = *adv;
+    int W = ceil_div(cols, 256);
+    W = W < 1 ? 1 : (W > 16 ? 16 : W);
+    hipLaunchKernelGGL(argmax_rows_kernel, dim3(rows), dim3(64 * W), 0, ctx->stream, x, idx_out, cols, row_stride,
+                       last_index ? 1 : 0, a);
     return AGPU_LAUNCH_CHECK(ctx, "argmax_rows_kernel");
 }
 
@@ -353,7 +353,7 @@ AGPU_EXPORT int32_t agpu_argmax_rows(agpu_ctx *ctx, const float *x, uint32_t *id
     if (!x || !idx_out) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "argmax_rows: null pointer");
     if (rows < 0 || cols <= 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "argmax_rows: bad dims rows=%d cols=%d", rows, cols);
     if (rows == 0) return AGPU_OK;
-    return agpu_argmax_rows_strided(ctx, x, idx_out, rows, cols, cols, last_index);
+    return agpu_argmax_rows_strided(ctx, x, idx_out, rows, cols, cols, last_index, nullptr);
 }
 
 AGPU_EXPORT int32_t agpu_split_qkv(agpu_ctx *ctx, const float *qkv, float *q, float *k, float *v, int32_t seq,

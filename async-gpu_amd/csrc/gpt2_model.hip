@@ -20,9 +20,9 @@
 #include "../../include/agpu_gpt2.h"
 #include "agpu_internal.h"
 #include "attention.h"
+#include "elementwise.h"
+#include "linear_common.h"
 
-int32_t agpu_argmax_rows_strided(agpu_ctx *ctx, const float *x, uint32_t *idx_out, int rows, int cols, int row_stride,
-                                 int last_index);
 
 namespace {
 
@@ -100,21 +100,9 @@ __global__ __launch_bounds__(256) void gather_last_rows_kernel(const float *__re
     dst[i] = src[((size_t)b * new_len + new_len - 1) * d + j];
 }
 
-// next tokens become the current tokens, are recorded, and the position / step counters advance.
-__global__ __launch_bounds__(1024) void advance_kernel(const uint32_t *next_tok, uint32_t *cur_tok, uint32_t *out_tok,
-                                                        int *pos_dev, int *step_dev, int batch, int delta,
-                                                        int out_capacity) {
-    const int t = threadIdx.x;
-    const int st = *step_dev;
-    if (t < batch) {
-        cur_tok[t] = next_tok[t];
-        if (st < out_capacity) out_tok[(size_t)st * batch + t] = next_tok[t];
-    }
-    __syncthreads();
-    if (t == 0) {
-        *pos_dev += delta;
-        *step_dev = st + 1;
-    }
+__global__ void advance_counters_kernel(int *pos_dev, int *step_dev, int delta) {
+    *pos_dev += delta;
+    *step_dev += 1;
 }
 
 __global__ void set_counters_kernel(int *pos_dev, int pos, int *step_dev, int step) {
@@ -271,13 +259,23 @@ int32_t launch_forward(agpu_gpt2 *m, const uint32_t *tokens, int B, int new_len,
         const Block &b = m->blocks[L];
         const Int4Lin &wq = b.lin[AGPU_LINEAR_QKV], &wp = b.lin[AGPU_LINEAR_PROJ], &wf = b.lin[AGPU_LINEAR_FC],
                       &wo = b.lin[AGPU_LINEAR_FC_PROJ];
-        rc = agpu_ln_int4_linear(ctx, hid, b.ln1_g, b.ln1_b, eps, wq.packed, wq.scales, wq.bias, nullptr, qkv, R, 3 * d,
-                                 d, g, 0);
-        if (rc != AGPU_OK) return rc;
         float *kc = m->kcache + L * layer_stride, *vc = m->vcache + L * layer_stride;
-        hipLaunchKernelGGL(kv_scatter_kernel, dim3((unsigned)(((size_t)R * d + 255) / 256)), dim3(256), 0, ctx->stream, qkv,
-                           kc, vc, R, new_len, H, P, m->pos_dev);
-        if ((rc = AGPU_LAUNCH_CHECK(ctx, "kv_scatter_kernel")) != AGPU_OK) return rc;
+        if (new_len == 1 && R <= 16 && g % 8 == 0 && agpu_int4_gemv_can_fuse_ln(R, d)) {
+            // decode: LN1 + QKV + bias with the K/V rows written straight into the cache
+            GemvArgs ga{};
+            ga.x = hid; ga.packed = wq.packed; ga.scales = wq.scales; ga.bias = wq.bias; ga.residual = nullptr; ga.y = qkv;
+            ga.ln_gamma = b.ln1_g; ga.ln_beta = b.ln1_b; ga.ln_eps = eps;
+            ga.M = R; ga.N = 3 * d; ga.K = d; ga.group = g; ga.flags = 0;
+            ga.kcache = kc; ga.vcache = vc; ga.pos_dev = m->pos_dev; ga.n_heads = H; ga.n_positions = P;
+            if ((rc = agpu_int4_gemv_launch(ctx, ga)) != AGPU_OK) return rc;
+        } else {
+            rc = agpu_ln_int4_linear(ctx, hid, b.ln1_g, b.ln1_b, eps, wq.packed, wq.scales, wq.bias, nullptr, qkv, R,
+                                     3 * d, d, g, 0);
+            if (rc != AGPU_OK) return rc;
+            hipLaunchKernelGGL(kv_scatter_kernel, dim3((unsigned)(((size_t)R * d + 255) / 256)), dim3(256), 0, ctx->stream,
+                               qkv, kc, vc, R, new_len, H, P, m->pos_dev);
+            if ((rc = AGPU_LAUNCH_CHECK(ctx, "kv_scatter_kernel")) != AGPU_OK) return rc;
+        }
         AttnParams ap{};
         ap.q = qkv; ap.k = kc; ap.v = vc; ap.o = att;
         ap.n_heads = H; ap.batch = B; ap.q_len = new_len; ap.kv_len = 0; ap.q_offset = 0; ap.kv_stride = P; ap.causal = 1;
@@ -352,12 +350,15 @@ int32_t set_counters(agpu_gpt2 *m, int pos, int step) {
 }
 
 int32_t launch_argmax_advance(agpu_gpt2 *m, int B, int delta) {
+    ArgmaxAdvance adv{};
+    adv.cur_tok = m->cur_tok; adv.out_tok = m->out_tok; adv.pos_dev = m->pos_dev; adv.step_dev = m->step_dev;
+    adv.delta = delta; adv.out_capacity = m->out_capacity; adv.bump_counters = (B == 1);
     int32_t rc = agpu_argmax_rows_strided(m->ctx, (float *)m->logits.p, m->next_tok, B, m->V, logits_stride(m),
-                                          m->cfg.argmax_last);
-    if (rc != AGPU_OK) return rc;
-    hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1024), 0, m->ctx->stream, m->next_tok, m->cur_tok, m->out_tok,
-                       m->pos_dev, m->step_dev, B, delta, m->out_capacity);
-    return AGPU_LAUNCH_CHECK(m->ctx, "advance_kernel");
+                                          m->cfg.argmax_last, &adv);
+    if (rc != AGPU_OK || B == 1) return rc;
+    // several rows: the counters advance once every row has read them
+    hipLaunchKernelGGL(advance_counters_kernel, dim3(1), dim3(1), 0, m->ctx->stream, m->pos_dev, m->step_dev, delta);
+    return AGPU_LAUNCH_CHECK(m->ctx, "advance_counters_kernel");
 }
 
 int kv_bucket(const agpu_gpt2 *m, int kv_len) {

@@ -1,4 +1,4 @@
-// int4 weight-only Linear for gfx950: quantize, dequantize, decode GEMV (M <= 16),
+// int4 weight-only Linear for gfx950: quantize, dequantize, the dispatch to the decode GEMV (M <= 16),
 // prefill GEMM on fp32 MFMA (M > 16), and the literal one-thread-per-output kernel.
 //
 // Weight layout is the reference's (nn/ops/quantize.rs:93-101,133-148):
@@ -6,7 +6,8 @@
 //   scales [ceil(K/group), N] f32
 // so one packed row is N contiguous words: a wave reading one row touches 256 B
 // (one word per lane) or 1 KiB (four words per lane) of contiguous memory.
-#include "agpu_internal.h"
+#include "elementwise.h"
+#include "linear_common.h"
 
 namespace {
 
@@ -70,19 +71,6 @@ __global__ __launch_bounds__(256) void int4_pack_kernel(const float *__restrict_
 }
 
 // ------------------------------------------------------------------------------------
-// shared epilogue
-// ------------------------------------------------------------------------------------
-
-__device__ __forceinline__ float epilogue(float v, int m, int n, int N, const float *bias, const float *residual,
-                                          uint32_t flags) {
-    if (bias) v += bias[n];
-    if (flags & AGPU_EPI_GELU_TANH) v = gelu_tanh_dev(v);
-    else if (flags & AGPU_EPI_GELU_QUICK) v = gelu_quick_dev(v);
-    if (residual) v += residual[(size_t)m * N + n];
-    return v;
-}
-
-// ------------------------------------------------------------------------------------
 // literal kernel: the reference's arithmetic order (compute_gemm.rs:2868-2900)
 // ------------------------------------------------------------------------------------
 
@@ -107,262 +95,6 @@ __global__ __launch_bounds__(256) void int4_gemm_literal_kernel(const float *__r
         }
     }
     y[gid] = epilogue(acc, row, col, N, bias, residual, flags);
-}
-
-// ------------------------------------------------------------------------------------
-// decode GEMV, M <= 16
-// ------------------------------------------------------------------------------------
-//
-// grid (col_blocks, ksplit), 256 threads = 4 waves.  A workgroup owns 64*CPL columns
-// and a contiguous range of "units"; a unit is `rpu` packed rows that share one scale
-// row (rpu = group/8 when that divides K/8, else 1).  Wave w takes units w, w+4, ...
-// Each lane owns CPL adjacent columns: one 4*CPL-byte load per packed row, so a wave
-// reads 256*CPL contiguous bytes per row.
-//
-// Per unit a lane accumulates s = sum_k x[k] * nibble[k] with the nibble as an unsigned
-// float (v_cvt_f32_ubyteN on the masked word) and then adds scale * (s - 8 * sum_k x[k]);
-// sum_k x[k] per unit is computed once per workgroup while x is staged in LDS.
-//
-// Split-K: waves reduce through LDS in wave order; workgroups write partials to the
-// workspace and the last one to arrive (ticket counter) adds them in split order, so the
-// result does not depend on arrival order.
-
-struct GemvParams {
-    const float *x;
-    const uint32_t *packed;
-    const float *scales;
-    const float *bias;
-    const float *residual;
-    float *y;
-    float *partial;           // [ksplit, M, N]
-    unsigned int *counters;   // [col_blocks], zero on entry and on exit
-    const float *ln_gamma;    // non-null: LayerNorm over K applied to x rows first
-    const float *ln_beta;
-    float ln_eps;
-    int M, N, K, group;
-    int rpu;                  // packed rows per unit
-    int n_units;              // ceil((K/8) / rpu)
-    int units_per_split;
-    uint32_t flags;
-};
-
-template <int CPL>
-struct WordVec;
-template <>
-struct WordVec<1> {
-    using U = uint32_t;
-    using F = float;
-};
-template <>
-struct WordVec<2> {
-    using U = uint2;
-    using F = float2;
-};
-template <>
-struct WordVec<4> {
-    using U = uint4;
-    using F = float4;
-};
-
-template <int CPL>
-__device__ __forceinline__ void load_words(const uint32_t *p, uint32_t (&w)[CPL]) {
-    using U = typename WordVec<CPL>::U;
-    const U v = *reinterpret_cast<const U *>(p);
-    if constexpr (CPL == 1) w[0] = v;
-    if constexpr (CPL == 2) { w[0] = v.x; w[1] = v.y; }
-    if constexpr (CPL == 4) { w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w; }
-}
-
-template <int CPL>
-__device__ __forceinline__ void load_floats(const float *p, float (&f)[CPL]) {
-    using F = typename WordVec<CPL>::F;
-    const F v = *reinterpret_cast<const F *>(p);
-    if constexpr (CPL == 1) f[0] = v;
-    if constexpr (CPL == 2) { f[0] = v.x; f[1] = v.y; }
-    if constexpr (CPL == 4) { f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w; }
-}
-
-// The 8 nibbles of a word as unsigned floats, nf[i] = nibble i.
-__device__ __forceinline__ void unpack_u8(uint32_t w, float (&nf)[8]) {
-    const uint32_t lo = w & 0x0F0F0F0Fu;         // nibbles 0,2,4,6 in bytes 0..3
-    const uint32_t hi = (w >> 4) & 0x0F0F0F0Fu;  // nibbles 1,3,5,7
-    nf[0] = (float)(lo & 0xFFu);
-    nf[1] = (float)(hi & 0xFFu);
-    nf[2] = (float)((lo >> 8) & 0xFFu);
-    nf[3] = (float)((hi >> 8) & 0xFFu);
-    nf[4] = (float)((lo >> 16) & 0xFFu);
-    nf[5] = (float)((hi >> 16) & 0xFFu);
-    nf[6] = (float)(lo >> 24);
-    nf[7] = (float)(hi >> 24);
-}
-
-template <int MT, int CPL>
-__global__ __launch_bounds__(256) void int4_gemv_kernel(const GemvParams p) {
-    extern __shared__ __align__(16) float smem[];
-    constexpr int COLS = 64 * CPL;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int bx = blockIdx.x, by = blockIdx.y;
-    const int ksplit = gridDim.y;
-    const int u0 = by * p.units_per_split;
-    const int u1 = min(p.n_units, u0 + p.units_per_split);
-    const int kp_total = p.K / 8;
-    const int k0 = u0 * p.rpu * 8;                         // first k of this split
-    const int kslice = p.units_per_split * p.rpu * 8;      // staged k range (zero padded)
-    const int n_units_local = p.units_per_split;
-
-    // LDS: xs[MT][kslice] | xsum[MT][units_per_split] | stats[MT][2]; later reused for the reduction.
-    float *xs = smem;
-    float *xsum = xs + MT * kslice;
-    float *stats = xsum + MT * n_units_local;
-
-    // ---- optional LayerNorm statistics (two-pass, per row; every workgroup recomputes) ----
-    if (p.ln_gamma) {
-        for (int m = wave; m < MT; m += 4) {
-            float mean = 0.0f, rstd = 0.0f;
-            if (m < p.M) {
-                const float *row = p.x + (size_t)m * p.K;
-                float s = 0.0f;
-                for (int k = lane; k < p.K; k += 64) s += row[k];
-                mean = wave_sum(s) / (float)p.K;
-                float v = 0.0f;
-                for (int k = lane; k < p.K; k += 64) {
-                    const float d = row[k] - mean;
-                    v += d * d;
-                }
-                rstd = 1.0f / sqrtf(wave_sum(v) / (float)p.K + p.ln_eps);
-            }
-            if (lane == 0) {
-                stats[2 * m] = mean;
-                stats[2 * m + 1] = rstd;
-            }
-        }
-        __syncthreads();
-    }
-
-    // ---- stage x[:, k0 .. k0+kslice) ----
-    for (int i = tid; i < MT * kslice; i += 256) {
-        const int m = i / kslice, kk = i - m * kslice, k = k0 + kk;
-        float v = 0.0f;
-        if (m < p.M && k < p.K) {
-            v = p.x[(size_t)m * p.K + k];
-            if (p.ln_gamma) v = (v - stats[2 * m]) * stats[2 * m + 1] * p.ln_gamma[k] + p.ln_beta[k];
-        }
-        xs[i] = v;
-    }
-    __syncthreads();
-    for (int i = tid; i < MT * n_units_local; i += 256) {
-        const int m = i / n_units_local, u = i - m * n_units_local;
-        const float *src = xs + m * kslice + u * p.rpu * 8;
-        float s = 0.0f;
-        for (int j = 0; j < p.rpu * 8; ++j) s += src[j];
-        xsum[i] = s;
-    }
-    __syncthreads();
-
-    // ---- main loop ----
-    const int c0 = bx * COLS + lane * CPL;
-    const bool col_ok = c0 < p.N;  // N % CPL == 0 is guaranteed by the launcher
-    float acc[MT][CPL];
-#pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-        for (int c = 0; c < CPL; ++c) acc[m][c] = 0.0f;
-
-    if (col_ok) {
-        for (int u = u0 + wave; u < u1; u += 4) {
-            const int kp0 = u * p.rpu;
-            const int g = (kp0 * 8) / p.group;
-            float sc[CPL];
-            load_floats<CPL>(p.scales + (size_t)g * p.N + c0, sc);
-            float part[MT][CPL];
-#pragma unroll
-            for (int m = 0; m < MT; ++m)
-#pragma unroll
-                for (int c = 0; c < CPL; ++c) part[m][c] = 0.0f;
-            const int rows = min(p.rpu, kp_total - kp0);
-            const float *xu = xs + (u - u0) * p.rpu * 8;
-#pragma unroll 4
-            for (int r = 0; r < rows; ++r) {
-                uint32_t w[CPL];
-                load_words<CPL>(p.packed + (size_t)(kp0 + r) * p.N + c0, w);
-                float nf[CPL][8];
-#pragma unroll
-                for (int c = 0; c < CPL; ++c) unpack_u8(w[c], nf[c]);
-#pragma unroll
-                for (int m = 0; m < MT; ++m) {
-                    const float4 xa = *reinterpret_cast<const float4 *>(xu + m * kslice + r * 8);
-                    const float4 xb = *reinterpret_cast<const float4 *>(xu + m * kslice + r * 8 + 4);
-#pragma unroll
-                    for (int c = 0; c < CPL; ++c) {
-                        float s = part[m][c];
-                        s = fmaf(xa.x, nf[c][0], s);
-                        s = fmaf(xa.y, nf[c][1], s);
-                        s = fmaf(xa.z, nf[c][2], s);
-                        s = fmaf(xa.w, nf[c][3], s);
-                        s = fmaf(xb.x, nf[c][4], s);
-                        s = fmaf(xb.y, nf[c][5], s);
-                        s = fmaf(xb.z, nf[c][6], s);
-                        s = fmaf(xb.w, nf[c][7], s);
-                        part[m][c] = s;
-                    }
-                }
-            }
-#pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                const float xs8 = 8.0f * xsum[m * n_units_local + (u - u0)];
-#pragma unroll
-                for (int c = 0; c < CPL; ++c) acc[m][c] = fmaf(sc[c], part[m][c] - xs8, acc[m][c]);
-            }
-        }
-    }
-
-    // ---- reduce the 4 waves through LDS (reuses the staging area) ----
-    __syncthreads();
-    float *red = smem;  // [4][MT][COLS]
-#pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-        for (int c = 0; c < CPL; ++c) red[(wave * MT + m) * COLS + lane * CPL + c] = acc[m][c];
-    __syncthreads();
-
-    __shared__ int s_last;
-    const int n_out = MT * COLS;
-    if (ksplit == 1) {
-        for (int i = tid; i < n_out; i += 256) {
-            const int m = i / COLS, cc = i - m * COLS, n = bx * COLS + cc;
-            if (m < p.M && n < p.N) {
-                const float v = (red[i] + red[n_out + i]) + (red[2 * n_out + i] + red[3 * n_out + i]);
-                p.y[(size_t)m * p.N + n] = epilogue(v, m, n, p.N, p.bias, p.residual, p.flags);
-            }
-        }
-        return;
-    }
-    for (int i = tid; i < n_out; i += 256) {
-        const int m = i / COLS, cc = i - m * COLS, n = bx * COLS + cc;
-        if (m < p.M && n < p.N) {
-            const float v = (red[i] + red[n_out + i]) + (red[2 * n_out + i] + red[3 * n_out + i]);
-            p.partial[((size_t)by * p.M + m) * p.N + n] = v;
-        }
-    }
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) {
-        const unsigned int t = atomicAdd(&p.counters[bx], 1u);
-        s_last = (t == (unsigned int)(ksplit - 1));
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-    for (int i = tid; i < n_out; i += 256) {
-        const int m = i / COLS, cc = i - m * COLS, n = bx * COLS + cc;
-        if (m < p.M && n < p.N) {
-            float v = 0.0f;
-            for (int s = 0; s < ksplit; ++s)
-                v += __builtin_nontemporal_load(&p.partial[((size_t)s * p.M + m) * p.N + n]);
-            p.y[(size_t)m * p.N + n] = epilogue(v, m, n, p.N, p.bias, p.residual, p.flags);
-        }
-    }
-    if (tid == 0) p.counters[bx] = 0u;
 }
 
 // ------------------------------------------------------------------------------------
@@ -459,75 +191,6 @@ __global__ __launch_bounds__(256) void int4_gemm_mfma_kernel(const float *__rest
     }
 }
 
-// Dense fp32 GEMV for M <= 16 (the f32 LM head at decode): lane = column, the 4 waves of a
-// workgroup split K, grid.y splits K further with the same ticket reduction as the int4 GEMV.
-template <int MT>
-__global__ __launch_bounds__(256) void gemv_f32_kernel(const float *__restrict__ x, const float *__restrict__ b,
-                                                        float *y, float *partial, unsigned int *counters, int M,
-                                                        int N, int K, int k_per_split) {
-    __shared__ float red[4][MT][64];
-    __shared__ int s_last;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int bx = blockIdx.x, by = blockIdx.y, ksplit = gridDim.y;
-    const int n = bx * 64 + lane;
-    const int ka = by * k_per_split, kb = min(K, ka + k_per_split);
-    float acc[MT];
-#pragma unroll
-    for (int m = 0; m < MT; ++m) acc[m] = 0.0f;
-    if (n < N) {
-        for (int k = ka + wave; k < kb; k += 4) {
-            const float w = b[(size_t)k * N + n];
-#pragma unroll
-            for (int m = 0; m < MT; ++m)
-                if (m < M) acc[m] = fmaf(x[(size_t)m * K + k], w, acc[m]);
-        }
-    }
-#pragma unroll
-    for (int m = 0; m < MT; ++m) red[wave][m][lane] = acc[m];
-    __syncthreads();
-    if (wave != 0) {
-        if (ksplit == 1) return;
-    }
-    float v[MT];
-    if (wave == 0) {
-#pragma unroll
-        for (int m = 0; m < MT; ++m) v[m] = (red[0][m][lane] + red[1][m][lane]) + (red[2][m][lane] + red[3][m][lane]);
-    }
-    if (ksplit == 1) {
-        if (n < N)
-#pragma unroll
-            for (int m = 0; m < MT; ++m)
-                if (m < M) y[(size_t)m * N + n] = v[m];
-        return;
-    }
-    if (wave == 0 && n < N) {
-#pragma unroll
-        for (int m = 0; m < MT; ++m)
-            if (m < M) partial[((size_t)by * M + m) * N + n] = v[m];
-    }
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) {
-        const unsigned int t = atomicAdd(&counters[bx], 1u);
-        s_last = (t == (unsigned int)(ksplit - 1));
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-    if (wave == 0 && n < N) {
-#pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            if (m < M) {
-                float s = 0.0f;
-                for (int sp = 0; sp < ksplit; ++sp)
-                    s += __builtin_nontemporal_load(&partial[((size_t)sp * M + m) * N + n]);
-                y[(size_t)m * N + n] = s;
-            }
-        }
-    }
-    if (tid == 0) counters[bx] = 0u;
-}
-
 // ------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------
@@ -541,77 +204,8 @@ int32_t check_linear_args(agpu_ctx *ctx, const void *x, const void *packed, cons
     return AGPU_OK;
 }
 
-template <int MT, int CPL>
-int32_t launch_gemv_t(agpu_ctx *ctx, GemvParams &p, dim3 grid, size_t lds) {
-    hipLaunchKernelGGL((int4_gemv_kernel<MT, CPL>), grid, dim3(256), lds, ctx->stream, p);
-    return AGPU_LAUNCH_CHECK(ctx, "int4_gemv_kernel");
-}
-
-template <int CPL>
-int32_t launch_gemv_m(agpu_ctx *ctx, GemvParams &p, int MT, dim3 grid, size_t lds) {
-    switch (MT) {
-        case 1: return launch_gemv_t<1, CPL>(ctx, p, grid, lds);
-        case 2: return launch_gemv_t<2, CPL>(ctx, p, grid, lds);
-        case 4: return launch_gemv_t<4, CPL>(ctx, p, grid, lds);
-        case 8: return launch_gemv_t<8, CPL>(ctx, p, grid, lds);
-        default: return launch_gemv_t<16, CPL>(ctx, p, grid, lds);
-    }
-}
-
-int32_t launch_gemv(agpu_ctx *ctx, const float *x, const float *ln_gamma, const float *ln_beta, float ln_eps,
-                    const uint32_t *packed, const float *scales, const float *bias, const float *residual,
-                    float *y, int M, int N, int K, int group, uint32_t flags) {
-    GemvParams p{};
-    p.x = x; p.packed = packed; p.scales = scales; p.bias = bias; p.residual = residual; p.y = y;
-    p.ln_gamma = ln_gamma; p.ln_beta = ln_beta; p.ln_eps = ln_eps;
-    p.M = M; p.N = N; p.K = K; p.group = group; p.flags = flags;
-    const int kp_total = K / 8;
-    const int wpg = group / 8;
-    p.rpu = (kp_total % wpg == 0) ? wpg : 1;
-    // keep units at <= 16 rows so a short K still splits across waves
-    while (p.rpu > 16 && p.rpu % 2 == 0) p.rpu /= 2;
-    p.n_units = kp_total / p.rpu;
-    const int MT = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
-
-    const bool aligned16 = (N % 4 == 0) && (((uintptr_t)packed | (uintptr_t)scales) % 16 == 0);
-    const bool aligned8 = (N % 2 == 0) && (((uintptr_t)packed | (uintptr_t)scales) % 8 == 0);
-    const int max_split = max(1, p.n_units / 4);
-    const int target_wgs = 2 * ctx->num_cus;
-    int cpl = 1;
-    if (aligned16 && MT <= 8 && ceil_div(N, 256) * max_split >= target_wgs) cpl = 4;
-    else if (aligned8 && ceil_div(N, 128) * max_split >= target_wgs) cpl = 2;
-    const int col_blocks = ceil_div(N, 64 * cpl);
-    int ksplit = min(max_split, max(1, ceil_div(target_wgs, col_blocks)));
-    // LDS budget (staging and reduction share the buffer) and workspace budget
-    auto lds_bytes = [&](int ks) {
-        const int ups = ceil_div(p.n_units, ks);
-        const size_t stage = (size_t)MT * ups * p.rpu * 8 + (size_t)MT * ups + 2 * MT;
-        const size_t red = (size_t)4 * MT * 64 * cpl;
-        return sizeof(float) * (stage > red ? stage : red);
-    };
-    while (lds_bytes(ksplit) > 60 * 1024 && ksplit < p.n_units) ++ksplit;
-    if (lds_bytes(ksplit) > 60 * 1024)
-        return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "int4_linear: K=%d too large for the decode kernel", K);
-    while (ksplit > 1 && (size_t)ksplit * M * N * sizeof(float) > kWorkspaceBytes) --ksplit;
-    p.units_per_split = ceil_div(p.n_units, ksplit);
-    ksplit = ceil_div(p.n_units, p.units_per_split);
-    if (col_blocks > kNumCounters) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_linear: N=%d too large", N);
-    p.partial = reinterpret_cast<float *>(ctx->workspace);
-    p.counters = ctx->counters;
-    const dim3 grid(col_blocks, ksplit);
-    const size_t lds = lds_bytes(ksplit);
-    switch (cpl) {
-        case 4: return launch_gemv_m<4>(ctx, p, MT, grid, lds);
-        case 2: return launch_gemv_m<2>(ctx, p, MT, grid, lds);
-        default: return launch_gemv_m<1>(ctx, p, MT, grid, lds);
-    }
-}
-
 }  // namespace
 
-// Defined in elementwise.hip.
-int32_t agpu_layer_norm_impl(agpu_ctx *ctx, const float *x, const float *gamma, const float *beta, float *y,
-                             int rows, int d, float eps);
 
 AGPU_EXPORT int32_t agpu_ln_int4_linear(agpu_ctx *ctx, const float *x, const float *gamma, const float *beta,
                                         float eps, const uint32_t *packed, const float *scales, const float *bias,
@@ -626,7 +220,7 @@ AGPU_EXPORT int32_t agpu_ln_int4_linear(agpu_ctx *ctx, const float *x, const flo
     const bool literal = (flags & AGPU_EPI_FORCE_LITERAL) || (group % 8 != 0 && M <= 16);
     const uint32_t epi = flags & (AGPU_EPI_GELU_TANH | AGPU_EPI_GELU_QUICK);
     const float *xin = x;
-    if (gamma && (literal || M > 16)) {
+    if (gamma && (literal || M > 16 || !agpu_int4_gemv_can_fuse_ln(M, K))) {
         // LayerNorm into the workspace tail, then the plain kernels.
         const size_t need = (size_t)M * K * sizeof(float);
         if (need > kWorkspaceBytes / 2)
@@ -643,7 +237,13 @@ AGPU_EXPORT int32_t agpu_ln_int4_linear(agpu_ctx *ctx, const float *x, const flo
                            xin, packed, scales, bias, residual, y, M, N, K, group, epi);
         return AGPU_LAUNCH_CHECK(ctx, "int4_gemm_literal_kernel");
     }
-    if (M <= 16) return launch_gemv(ctx, xin, gamma, beta, eps, packed, scales, bias, residual, y, M, N, K, group, epi);
+    if (M <= 16) {
+        GemvArgs a{};
+        a.x = xin; a.packed = packed; a.scales = scales; a.bias = bias; a.residual = residual; a.y = y;
+        a.ln_gamma = gamma; a.ln_beta = beta; a.ln_eps = eps;
+        a.M = M; a.N = N; a.K = K; a.group = group; a.flags = epi;
+        return agpu_int4_gemv_launch(ctx, a);
+    }
     const dim3 grid(ceil_div(N, GEMM_BN), ceil_div(M, GEMM_BM));
     hipLaunchKernelGGL((int4_gemm_mfma_kernel<false>), grid, dim3(256), 0, ctx->stream, xin, packed, scales,
                        (const float *)nullptr, bias, residual, y, M, N, K, group, epi);
@@ -655,6 +255,48 @@ AGPU_EXPORT int32_t agpu_int4_linear(agpu_ctx *ctx, const float *x, const uint32
                                      int32_t K, int32_t group, uint32_t flags) {
     return agpu_ln_int4_linear(ctx, x, nullptr, nullptr, 0.0f, packed, scales, bias, residual, y, M, N, K, group,
                                flags);
+}
+
+AGPU_EXPORT int32_t agpu_bench_int4_linear(agpu_ctx *ctx, const float *x, const float *gamma, const float *beta, float eps,
+                                           const uint32_t *packed, const float *scales, const float *bias,
+                                           const float *residual, float *y, int32_t M, int32_t N, int32_t K,
+                                           int32_t group, uint32_t flags, int32_t n_weight_sets,
+                                           int64_t packed_set_stride, int64_t scales_set_stride, int32_t reps,
+                                           float *us_per_launch_out_host) {
+    AGPU_REQUIRE_CTX(ctx);
+    AGPU_REQUIRE_PTR(ctx, us_per_launch_out_host);
+    if (reps <= 0 || n_weight_sets <= 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "bench_int4_linear: reps and n_weight_sets must be positive");
+    if (!ctx->stream) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "bench_int4_linear: needs a context with its own stream");
+    // one untimed pass outside the graph validates the arguments
+    int32_t rc = agpu_ln_int4_linear(ctx, x, gamma, beta, eps, packed, scales, bias, residual, y, M, N, K, group, flags);
+    if (rc != AGPU_OK) return rc;
+    hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipStreamBeginCapture");
+    for (int i = 0; i < reps && rc == AGPU_OK; ++i) {
+        const int set = i % n_weight_sets;
+        rc = agpu_ln_int4_linear(ctx, x, gamma, beta, eps, packed + (size_t)set * packed_set_stride,
+                                 scales + (size_t)set * scales_set_stride, bias, residual, y, M, N, K, group, flags);
+    }
+    hipGraph_t graph = nullptr;
+    e = hipStreamEndCapture(ctx->stream, &graph);
+    if (rc != AGPU_OK || e != hipSuccess) {
+        if (graph) (void)hipGraphDestroy(graph);
+        return rc != AGPU_OK ? rc : agpu_hip(ctx, e, "hipStreamEndCapture");
+    }
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipGraphInstantiate");
+    float ms = 0.0f;
+    e = hipGraphLaunch(exec, ctx->stream);  // warm-up replay
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e == hipSuccess) rc = agpu_timer_start(ctx);
+    if (e == hipSuccess && rc == AGPU_OK) e = hipGraphLaunch(exec, ctx->stream);
+    if (e == hipSuccess && rc == AGPU_OK) rc = agpu_timer_stop(ctx, &ms);
+    (void)hipGraphExecDestroy(exec);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipGraphLaunch");
+    *us_per_launch_out_host = ms * 1000.0f / (float)reps;
+    return rc;
 }
 
 AGPU_EXPORT int32_t agpu_int4_dequantize(agpu_ctx *ctx, const uint32_t *packed, const float *scales, float *w_out,
@@ -692,29 +334,7 @@ AGPU_EXPORT int32_t agpu_gemm_f32(agpu_ctx *ctx, const float *a, const float *b,
     if (!a || !b || !c) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "gemm_f32: null pointer");
     if (M < 0 || N <= 0 || K <= 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gemm_f32: bad dims M=%d N=%d K=%d", M, N, K);
     if (M == 0) return AGPU_OK;
-    if (M <= 16) {
-        const int MT = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
-        const int col_blocks = ceil_div(N, 64);
-        int ksplit = max(1, min(K / 32, ceil_div(2 * ctx->num_cus, col_blocks)));
-        while (ksplit > 1 && (size_t)ksplit * M * N * sizeof(float) > kWorkspaceBytes) --ksplit;
-        const int kps = ceil_div(K, ksplit);
-        ksplit = ceil_div(K, kps);
-        if (col_blocks > kNumCounters) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "gemm_f32: N=%d too large", N);
-        const dim3 grid(col_blocks, ksplit);
-        float *partial = reinterpret_cast<float *>(ctx->workspace);
-#define AGPU_GEMV_F32(MTV)                                                                                       \
-    hipLaunchKernelGGL((gemv_f32_kernel<MTV>), grid, dim3(256), 0, ctx->stream, a, b, c, partial, ctx->counters, \
-                       M, N, K, kps)
-        switch (MT) {
-            case 1: AGPU_GEMV_F32(1); break;
-            case 2: AGPU_GEMV_F32(2); break;
-            case 4: AGPU_GEMV_F32(4); break;
-            case 8: AGPU_GEMV_F32(8); break;
-            default: AGPU_GEMV_F32(16); break;
-        }
-#undef AGPU_GEMV_F32
-        return AGPU_LAUNCH_CHECK(ctx, "gemv_f32_kernel");
-    }
+    if (M <= 16) return agpu_f32_gemv_launch(ctx, a, b, c, M, N, K);
     const dim3 grid(ceil_div(N, GEMM_BN), ceil_div(M, GEMM_BM));
     hipLaunchKernelGGL((int4_gemm_mfma_kernel<true>), grid, dim3(256), 0, ctx->stream, a, (const uint32_t *)nullptr,
                        (const float *)nullptr, b, (const float *)nullptr, (const float *)nullptr, c, M, N, K, 8, 0u);

@@ -1,0 +1,55 @@
+// Pieces shared by the int4 Linear kernels: epilogue, nibble unpack, GEMV launch arguments.
+#pragma once
+#include "agpu_internal.h"
+
+// bias -> GELU -> residual, applied to one output element.
+__device__ __forceinline__ float epilogue(float v, int m, int n, int N, const float *bias, const float *residual,
+                                          uint32_t flags) {
+    if (bias) v += bias[n];
+    if (flags & AGPU_EPI_GELU_TANH) v = gelu_tanh_dev(v);
+    else if (flags & AGPU_EPI_GELU_QUICK) v = gelu_quick_dev(v);
+    if (residual) v += residual[(size_t)m * N + n];
+    return v;
+}
+
+// The 8 nibbles of a word as unsigned floats, nf[i] = nibble i (v_cvt_f32_ubyteN on masked words).
+__device__ __forceinline__ void unpack_u8(uint32_t w, float (&nf)[8]) {
+    const uint32_t lo = w & 0x0F0F0F0Fu;         // nibbles 0,2,4,6 in bytes 0..3
+    const uint32_t hi = (w >> 4) & 0x0F0F0F0Fu;  // nibbles 1,3,5,7
+    nf[0] = (float)(lo & 0xFFu);
+    nf[1] = (float)(hi & 0xFFu);
+    nf[2] = (float)((lo >> 8) & 0xFFu);
+    nf[3] = (float)((hi >> 8) & 0xFFu);
+    nf[4] = (float)((lo >> 16) & 0xFFu);
+    nf[5] = (float)((hi >> 16) & 0xFFu);
+    nf[6] = (float)(lo >> 24);
+    nf[7] = (float)(hi >> 24);
+}
+
+// Arguments of the decode GEMV (M <= 16 rows).
+struct GemvArgs {
+    const float *x;         // [M, K]
+    const uint32_t *packed; // [K/8, N]
+    const float *scales;    // [ceil(K/group), N]
+    const float *bias;      // [N] or null
+    const float *residual;  // [M, N] or null (may alias y)
+    float *y;               // [M, N]
+    const float *ln_gamma;  // non-null: LayerNorm over K applied to the rows of x first
+    const float *ln_beta;
+    float ln_eps;
+    int M, N, K, group;
+    uint32_t flags;         // AGPU_EPI_GELU_*
+    // Optional K/V scatter for a fused QKV projection with N = 3*d_model, one new position per
+    // row: columns [d, 2d) also go to kcache[(m*n_heads + h), *pos_dev, e], columns [2d, 3d) to vcache.
+    float *kcache;
+    float *vcache;
+    const int *pos_dev;
+    int n_heads, n_positions;
+};
+
+int32_t agpu_int4_gemv_launch(agpu_ctx *ctx, const GemvArgs &a);
+// Whether the GEMV can apply LayerNorm itself for this shape (otherwise normalise first).
+bool agpu_int4_gemv_can_fuse_ln(int M, int K);
+
+// Dense fp32 GEMV, C[M,N] = A[M,K] B[K,N], M <= 16.
+int32_t agpu_f32_gemv_launch(agpu_ctx *ctx, const float *a, const float *b, float *c, int M, int N, int K);

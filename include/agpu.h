@@ -58,6 +58,13 @@ int32_t agpu_memcpy_d2h(agpu_ctx *ctx, void *dst_host, const void *src, size_t b
 int32_t agpu_memcpy_d2d(agpu_ctx *ctx, void *dst, const void *src, size_t bytes);      /* clone_tensor, tensor.rs:270-282 */
 int32_t agpu_sync(agpu_ctx *ctx);                                                       /* dev.synchronize() */
 
+/* Stage timing as Gpt2Model::forward_profiled does it (synchronize + clock around a stage,
+ * nn/models/gpt2.rs:529-568), with HIP events on the context's stream instead of a host clock:
+ * agpu_timer_start records an event; agpu_timer_stop records a second one, waits for it and
+ * writes the milliseconds between the two to *ms_out_host. */
+int32_t agpu_timer_start(agpu_ctx *ctx);
+int32_t agpu_timer_stop(agpu_ctx *ctx, float *ms_out_host);
+
 /* registry.get(name) (nn/registry.rs:140-144): 0 if `name` is one of the reference's
  * kernel names this library implements, AGPU_ERR_KERNEL_NOT_FOUND otherwise.
  * *entry_point_out (optional) receives the name of the C function that serves it. */
@@ -86,12 +93,30 @@ int32_t agpu_int4_linear(agpu_ctx *ctx, const float *x, const uint32_t *packed, 
                          const float *bias, const float *residual, float *y, int32_t M, int32_t N,
                          int32_t K, int32_t group, uint32_t flags);
 
+/* Tuning hook of the decode GEMV (M <= 16): how many workgroups a launch aims at (0 = one per
+ * CU, the default) and how many packed rows (8 k each) a wave keeps at least (default 8).
+ * Process-wide; results stay deterministic for any setting. */
+void agpu_int4_gemv_tune(int32_t target_wgs, int32_t min_rows_per_wave);
+
 /* Same with LayerNorm(x; gamma, beta, eps) over K applied to each input row first
  * (ops::layer_norm followed by Int4Linear::forward, gpt2.rs:1307-1316,1329-1331). */
 int32_t agpu_ln_int4_linear(agpu_ctx *ctx, const float *x, const float *gamma, const float *beta,
                             float eps, const uint32_t *packed, const float *scales, const float *bias,
                             const float *residual, float *y, int32_t M, int32_t N, int32_t K,
                             int32_t group, uint32_t flags);
+
+/* Measurement helper (no counterpart in the reference, whose benches time host-side loops,
+ * nn/ops/norm.rs:578-633): records `reps` back-to-back launches of agpu_ln_int4_linear
+ * (gamma/beta may be NULL) into a HIP graph, replays it and writes the mean microseconds per
+ * launch, measured with HIP events on the context's stream.  Launch i uses weight set
+ * i % n_weight_sets at packed + set*packed_set_stride / scales + set*scales_set_stride
+ * (strides in elements), so a rotation larger than the caches measures HBM, not cache, bandwidth.
+ * Needs a context that owns its stream. */
+int32_t agpu_bench_int4_linear(agpu_ctx *ctx, const float *x, const float *gamma, const float *beta, float eps,
+                               const uint32_t *packed, const float *scales, const float *bias,
+                               const float *residual, float *y, int32_t M, int32_t N, int32_t K, int32_t group,
+                               uint32_t flags, int32_t n_weight_sets, int64_t packed_set_stride,
+                               int64_t scales_set_stride, int32_t reps, float *us_per_launch_out_host);
 
 /* W[K,N] = (float)(nibble-8) * scale: the kernel's inline dequantisation
  * (compute_gemm.rs:2882-2886) / nn/ops/quantize.rs:158-162 as a standalone, bit-exact hook. */
