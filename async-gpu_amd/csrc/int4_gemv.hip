@@ -30,6 +30,7 @@ namespace {
 struct GemvParams {
     GemvArgs a;
     int rows_per_split;  // packed rows per workgroup (grid.y slices of K)
+    int col_blocks;      // column tiles of 16*CPL columns; a workgroup strides over them
     float *partial;      // [ksplit, M, N], only with ksplit > 1
     unsigned int *counters;  // [col_blocks] tickets, zero on entry and on exit
 };
@@ -94,8 +95,10 @@ __device__ __forceinline__ float block_sum(float v, float *scratch, int lane, in
     return t;
 }
 
-// LDS layout (floats): xs[MT][xs_len] | xsum[MT][rows_per_split] | red[W][MT][COLS] (after the loop,
-// aliasing xs) | scratch[16].  xs_len = K when LayerNorm is fused (whole rows), else the K slice.
+// LDS layout (floats): xs[MT][xs_len] | xsum[MT][rows_per_split] | red[W][MT][COLS].
+// xs_len = K when LayerNorm is fused (whole rows), else the K slice.
+// A workgroup handles the column tiles blockIdx.x, blockIdx.x + gridDim.x, ...: x is staged once
+// and the loads of the next tile's first two row trips are issued before the current tile is reduced.
 template <int MT, int CPL, bool LN>
 __global__ __launch_bounds__(MT <= 4 ? 1024 : 512) void int4_gemv_kernel(const GemvParams p) {
     extern __shared__ __align__(16) float smem[];
@@ -113,38 +116,33 @@ __global__ __launch_bounds__(MT <= 4 ? 1024 : 512) void int4_gemv_kernel(const G
     const int xs_len = LN ? a.K : p.rows_per_split * 8;
     float *xs = smem;
     float *xsum = smem + MT * xs_len;
+    float *red = xsum + MT * p.rows_per_split;  // [W][MT][COLS]
     const int n_out = MT * COLS;
-
-    // the first two row groups of this lane: their loads go out before anything else
-    const int c0 = blockIdx.x * COLS + cg * CPL;
-    const bool col_ok = c0 < a.N;  // N % CPL == 0 is guaranteed by the launcher
     const int row_a = r0 + 4 * wave + rs, row_b = row_a + 4 * W;
+
+    // the first two row trips of a tile, for this lane
     uint32_t wa[CPL], wb[CPL];
     float sa[CPL], sb[CPL];
+    auto preload = [&](int tile) {
+        const int c0 = tile * COLS + cg * CPL;
+        const bool ok = tile < p.col_blocks && c0 < a.N;  // N % CPL == 0 is guaranteed by the launcher
 #pragma unroll
-    for (int c = 0; c < CPL; ++c) {
-        wa[c] = wb[c] = 0x88888888u;
-        sa[c] = sb[c] = 0.0f;
-    }
-    if (col_ok && row_a < r1) {
-        load_words<CPL>(a.packed + (size_t)row_a * a.N + c0, wa);
-        load_floats<CPL>(a.scales + (size_t)((row_a * 8) / a.group) * a.N + c0, sa);
-    }
-    if (col_ok && row_b < r1) {
-        load_words<CPL>(a.packed + (size_t)row_b * a.N + c0, wb);
-        load_floats<CPL>(a.scales + (size_t)((row_b * 8) / a.group) * a.N + c0, sb);
-    }
-    // epilogue operands of this thread's output element, fetched early
-    float e_bias = 0.0f, e_res = 0.0f;
-    {
-        const int m = tid / COLS, n = blockIdx.x * COLS + (tid - m * COLS);
-        if (tid < n_out && m < a.M && n < a.N) {
-            if (a.bias) e_bias = a.bias[n];
-            if (a.residual) e_res = a.residual[(size_t)m * a.N + n];
+        for (int c = 0; c < CPL; ++c) {
+            wa[c] = wb[c] = 0x88888888u;
+            sa[c] = sb[c] = 0.0f;
         }
-    }
+        if (ok && row_a < r1) {
+            load_words<CPL>(a.packed + (size_t)row_a * a.N + c0, wa);
+            load_floats<CPL>(a.scales + (size_t)((row_a * 8) / a.group) * a.N + c0, sa);
+        }
+        if (ok && row_b < r1) {
+            load_words<CPL>(a.packed + (size_t)row_b * a.N + c0, wb);
+            load_floats<CPL>(a.scales + (size_t)((row_b * 8) / a.group) * a.N + c0, sb);
+        }
+    };
+    preload(blockIdx.x);  // these loads go out before anything else
 
-    // ---- stage x ----
+    // ---- stage x once ----
     if constexpr (LN) {
         // whole rows into LDS, two-pass statistics over the workgroup, normalise the slice in place
         for (int i = tid; i < MT * a.K; i += T) {
@@ -184,12 +182,8 @@ __global__ __launch_bounds__(MT <= 4 ? 1024 : 512) void int4_gemv_kernel(const G
         xsum[m * p.rows_per_split + r] = 8.0f * (((xa.x + xa.y) + (xa.z + xa.w)) + ((xb.x + xb.y) + (xb.z + xb.w)));
     }
     __syncthreads();
-    // ---- main loop: row = r0 + 4*wave + rs + 4*W*i; trips 0 and 1 were loaded at the top ----
+
     float acc[MT][CPL];
-#pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-        for (int c = 0; c < CPL; ++c) acc[m][c] = 0.0f;
     auto consume = [&](const uint32_t (&w)[CPL], const float (&sc)[CPL], int row) {
         const int r = row - r0;
 #pragma unroll
@@ -214,17 +208,38 @@ __global__ __launch_bounds__(MT <= 4 ? 1024 : 512) void int4_gemv_kernel(const G
             }
         }
     };
-    if (col_ok) {
+
+    for (int tile = blockIdx.x; tile < p.col_blocks; tile += gridDim.x) {
+        const int c0 = tile * COLS + cg * CPL;
+        const bool col_ok = c0 < a.N;
+        // epilogue operands of this thread's output element, fetched early
+        float e_bias = 0.0f, e_res = 0.0f;
+        {
+            const int m = tid / COLS, n = tile * COLS + (tid - m * COLS);
+            if (tid < n_out && m < a.M && n < a.N) {
+                if (a.bias) e_bias = a.bias[n];
+                if (a.residual) e_res = a.residual[(size_t)m * a.N + n];
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) acc[m][c] = 0.0f;
+        // rows r0 + 4*wave + rs + 4*W*i; trips 0 and 1 are already in registers
         for (int row = row_a; row < r1; row += 8 * W) {
-            // issue the next pair, then consume the pair in registers
             uint32_t wn0[CPL], wn1[CPL];
             float sn0[CPL], sn1[CPL];
             const int rn0 = row + 8 * W, rn1 = row + 12 * W;
-            if (rn0 < r1) {
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) {
+                wn0[c] = wn1[c] = 0x88888888u;
+                sn0[c] = sn1[c] = 0.0f;
+            }
+            if (col_ok && rn0 < r1) {
                 load_words<CPL>(a.packed + (size_t)rn0 * a.N + c0, wn0);
                 load_floats<CPL>(a.scales + (size_t)((rn0 * 8) / a.group) * a.N + c0, sn0);
             }
-            if (rn1 < r1) {
+            if (col_ok && rn1 < r1) {
                 load_words<CPL>(a.packed + (size_t)rn1 * a.N + c0, wn1);
                 load_floats<CPL>(a.scales + (size_t)((rn1 * 8) / a.group) * a.N + c0, sn1);
             }
@@ -236,72 +251,72 @@ __global__ __launch_bounds__(MT <= 4 ? 1024 : 512) void int4_gemv_kernel(const G
                 wb[c] = wn1[c]; sb[c] = sn1[c];
             }
         }
-    }
-    // row slots -> lanes 0..15 (fixed order), then waves through LDS
-#pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-        for (int c = 0; c < CPL; ++c) {
-            float v = acc[m][c];
-            v += __shfl_xor(v, 16, kWave);
-            v += __shfl_xor(v, 32, kWave);
-            acc[m][c] = v;
-        }
-    __syncthreads();  // xs is dead from here on
-    float *red = smem;  // [W][MT][COLS]
-    if (rs == 0) {
+        preload(tile + gridDim.x);  // next tile's loads fly during the reduction below
+        // row slots -> lanes 0..15 (fixed order), then waves through LDS
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
-            for (int c = 0; c < CPL; ++c) red[(wave * MT + m) * COLS + cg * CPL + c] = acc[m][c];
-    }
-    __syncthreads();
-    if (ksplit == 1) {
+            for (int c = 0; c < CPL; ++c) {
+                float v = acc[m][c];
+                v += __shfl_xor(v, 16, kWave);
+                v += __shfl_xor(v, 32, kWave);
+                acc[m][c] = v;
+            }
+        __syncthreads();  // the previous tile's readers of red are done
+        if (rs == 0) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m)
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) red[(wave * MT + m) * COLS + cg * CPL + c] = acc[m][c];
+        }
+        __syncthreads();
+        if (ksplit == 1) {
+            for (int i = tid; i < n_out; i += T) {
+                const int m = i / COLS, n = tile * COLS + (i - m * COLS);
+                if (m < a.M && n < a.N) {
+                    float v = 0.0f;
+                    for (int w = 0; w < W; ++w) v += red[w * n_out + i];
+                    if (i != tid) {
+                        e_bias = a.bias ? a.bias[n] : 0.0f;
+                        e_res = a.residual ? a.residual[(size_t)m * a.N + n] : 0.0f;
+                    }
+                    finish_output(a, v, e_bias, e_res, m, n);
+                }
+            }
+            continue;
+        }
+        // publish this workgroup's partial sums past the L2, then take a ticket
         for (int i = tid; i < n_out; i += T) {
-            const int m = i / COLS, n = blockIdx.x * COLS + (i - m * COLS);
+            const int m = i / COLS, n = tile * COLS + (i - m * COLS);
             if (m < a.M && n < a.N) {
                 float v = 0.0f;
                 for (int w = 0; w < W; ++w) v += red[w * n_out + i];
+                __hip_atomic_store(&p.partial[((size_t)split * a.M + m) * a.N + n], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned int t = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_last = (t == (unsigned int)(ksplit - 1));
+        }
+        __syncthreads();
+        if (!s_last) continue;  // uniform over the workgroup
+        for (int i = tid; i < n_out; i += T) {
+            const int m = i / COLS, n = tile * COLS + (i - m * COLS);
+            if (m < a.M && n < a.N) {
+                float t = 0.0f;
+                for (int sp = 0; sp < ksplit; ++sp)
+                    t += __hip_atomic_load(&p.partial[((size_t)sp * a.M + m) * a.N + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 if (i != tid) {
                     e_bias = a.bias ? a.bias[n] : 0.0f;
                     e_res = a.residual ? a.residual[(size_t)m * a.N + n] : 0.0f;
                 }
-                finish_output(a, v, e_bias, e_res, m, n);
+                finish_output(a, t, e_bias, e_res, m, n);
             }
         }
-        return;
+        if (tid == 0) __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    // publish this workgroup's partial sums past the L2, then take a ticket
-    for (int i = tid; i < n_out; i += T) {
-        const int m = i / COLS, n = blockIdx.x * COLS + (i - m * COLS);
-        if (m < a.M && n < a.N) {
-            float v = 0.0f;
-            for (int w = 0; w < W; ++w) v += red[w * n_out + i];
-            __hip_atomic_store(&p.partial[((size_t)split * a.M + m) * a.N + n], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (tid == 0) {
-        const unsigned int t = __hip_atomic_fetch_add(&p.counters[blockIdx.x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (t == (unsigned int)(ksplit - 1));
-    }
-    __syncthreads();
-    if (!s_last) return;
-    for (int i = tid; i < n_out; i += T) {
-        const int m = i / COLS, n = blockIdx.x * COLS + (i - m * COLS);
-        if (m < a.M && n < a.N) {
-            float t = 0.0f;
-            for (int sp = 0; sp < ksplit; ++sp)
-                t += __hip_atomic_load(&p.partial[((size_t)sp * a.M + m) * a.N + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (i != tid) {
-                e_bias = a.bias ? a.bias[n] : 0.0f;
-                e_res = a.residual ? a.residual[(size_t)m * a.N + n] : 0.0f;
-            }
-            finish_output(a, t, e_bias, e_res, m, n);
-        }
-    }
-    if (tid == 0) __hip_atomic_store(&p.counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Dense fp32 GEMV: lane = column, the W waves of a workgroup split K, reduced in wave order.
@@ -362,15 +377,16 @@ int32_t launch_m(agpu_ctx *ctx, const GemvParams &p, int MT, dim3 grid, int W, s
 }
 
 int g_tune_target_wgs = 0;    // 0: default
-int g_tune_min_rows = 8;      // packed rows per wave that split-K aims to keep
+int g_tune_rows_per_split = 256;  // packed rows a workgroup takes at most
 
 }  // namespace
 
 bool agpu_int4_gemv_can_fuse_ln(int M, int K) { return M <= 2 && (size_t)M * K * sizeof(float) <= 32 * 1024; }
 
-AGPU_EXPORT void agpu_int4_gemv_tune(int32_t target_wgs, int32_t min_rows_per_wave) {
+AGPU_EXPORT void agpu_int4_gemv_tune(int32_t max_wgs, int32_t min_rows_per_wave) {
+    const int32_t target_wgs = max_wgs;
     g_tune_target_wgs = target_wgs;
-    g_tune_min_rows = min_rows_per_wave > 0 ? min_rows_per_wave : 8;
+    g_tune_rows_per_split = min_rows_per_wave > 0 ? min_rows_per_wave : 256;
 }
 
 int32_t agpu_int4_gemv_launch(agpu_ctx *ctx, const GemvArgs &a) {
@@ -380,7 +396,6 @@ int32_t agpu_int4_gemv_launch(agpu_ctx *ctx, const GemvArgs &a) {
         return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "int4_gemv: fused LayerNorm needs M <= 2 and M*K <= 8192");
     const int kp_total = a.K / 8;
     const int MT = a.M <= 1 ? 1 : a.M <= 2 ? 2 : a.M <= 4 ? 4 : a.M <= 8 ? 8 : 16;
-    const int target = g_tune_target_wgs > 0 ? g_tune_target_wgs : ctx->num_cus;
     const bool aligned16 = (a.N % 4 == 0) && (((uintptr_t)a.packed | (uintptr_t)a.scales) % 16 == 0);
     const int cpl = aligned16 ? 4 : 1;
     const int col_blocks = ceil_div(a.N, 16 * cpl);
@@ -388,18 +403,14 @@ int32_t agpu_int4_gemv_launch(agpu_ctx *ctx, const GemvArgs &a) {
 
     // K split over workgroups: a workgroup of 16 waves covers 64 packed rows per trip and keeps two
     // trips in flight, so up to 4 trips (256 rows) per workgroup cost two memory round trips.
-    // More splits only pay when they are needed to occupy the chip (g_tune_target_wgs).
-    int ksplit = ceil_div(kp_total, 256);
-    if (g_tune_target_wgs > 0 && ksplit * col_blocks < target) ksplit = ceil_div(target, col_blocks);
-    const int max_split = kp_total / (4 * g_tune_min_rows) > 0 ? kp_total / (4 * g_tune_min_rows) : 1;
-    if (ksplit > max_split) ksplit = max_split;
+    int ksplit = ceil_div(kp_total, g_tune_rows_per_split);
     while (ksplit > 1 && (size_t)ksplit * a.M * a.N * sizeof(float) > kWorkspaceBytes / 2) --ksplit;
     auto stage_floats = [&](int ks) {
         const int rps = ceil_div(kp_total, ks);
         const size_t xs_len = a.ln_gamma ? (size_t)a.K : (size_t)rps * 8;
         return (size_t)MT * xs_len + (size_t)MT * rps;
     };
-    constexpr size_t kLdsBudget = 60 * 1024;
+    constexpr size_t kLdsBudget = 40 * 1024;
     while (stage_floats(ksplit) * sizeof(float) > kLdsBudget && ksplit < kp_total) ++ksplit;
     p.rows_per_split = ceil_div(kp_total, ksplit);
     ksplit = ceil_div(kp_total, p.rows_per_split);
@@ -412,12 +423,17 @@ int32_t agpu_int4_gemv_launch(agpu_ctx *ctx, const GemvArgs &a) {
     const int max_w = MT <= 4 ? 16 : 8;
     int W = ceil_div(p.rows_per_split, 8);  // two trips of 4 rows per wave
     W = W < 1 ? 1 : (W > max_w ? max_w : W);
-    while (W > 1 && (size_t)W * MT * 16 * cpl * sizeof(float) > kLdsBudget) --W;
+    while (W > 1 && ((size_t)W * MT * 16 * cpl + stage_floats(ksplit)) * sizeof(float) > 64 * 1024) --W;
     const size_t red_floats = (size_t)W * MT * 16 * cpl;
-    const size_t lds = sizeof(float) * (stage_floats(ksplit) > red_floats ? stage_floats(ksplit) : red_floats);
+    const size_t lds = sizeof(float) * (stage_floats(ksplit) + red_floats);
     p.partial = reinterpret_cast<float *>(ctx->workspace);
     p.counters = ctx->counters;
-    const dim3 grid(col_blocks, ksplit);
+    p.col_blocks = col_blocks;
+    // at most one workgroup per CU (measured best for the LM head); each strides over the column tiles
+    int gx = col_blocks;
+    const int cap = g_tune_target_wgs > 0 ? g_tune_target_wgs : ctx->num_cus;
+    if (gx * ksplit > cap) gx = cap / ksplit > 0 ? cap / ksplit : 1;
+    const dim3 grid(gx, ksplit);
     return cpl == 4 ? launch_m<4>(ctx, p, MT, grid, W, lds) : launch_m<1>(ctx, p, MT, grid, W, lds);
 }
 

@@ -93,10 +93,11 @@ int32_t agpu_int4_linear(agpu_ctx *ctx, const float *x, const uint32_t *packed, 
                          const float *bias, const float *residual, float *y, int32_t M, int32_t N,
                          int32_t K, int32_t group, uint32_t flags);
 
-/* Tuning hook of the decode GEMV (M <= 16): how many workgroups a launch aims at (0 = one per
- * CU, the default) and how many packed rows (8 k each) a wave keeps at least (default 8).
+/* Tuning hook of the decode GEMV (M <= 16): the most workgroups a launch uses (0 = one per CU,
+ * the default; each workgroup strides over the column tiles) and the most packed rows (8 k each)
+ * one workgroup takes before K is split over workgroups (0 = 256, the default).
  * Process-wide; results stay deterministic for any setting. */
-void agpu_int4_gemv_tune(int32_t target_wgs, int32_t min_rows_per_wave);
+void agpu_int4_gemv_tune(int32_t max_wgs, int32_t max_rows_per_wg);
 
 /* Same with LayerNorm(x; gamma, beta, eps) over K applied to each input row first
  * (ops::layer_norm followed by Int4Linear::forward, gpt2.rs:1307-1316,1329-1331). */
