@@ -17,3 +17,7 @@ pids+=($!)
 for p in "${pids[@]}"; do wait "$p"; done
 "$HIPCC" --offload-arch=gfx950 -shared -fPIC -o ../libagpu_hip.so build/*.o -fopenmp
 echo "built $(cd .. && pwd)/libagpu_hip.so"
+# C++ host-layer test (include/agpu_nn.hpp); runs on the GPU box from tests/test_gpu_cpp.py
+g++ -O1 -std=c++17 -I../../include ../../tests/cpp/test_nn.cpp -o ../../tests/cpp/test_nn \
+    -L.. -lagpu_hip -Wl,-rpath,'$ORIGIN/../../async-gpu_amd' -Wl,-rpath,/opt/rocm/lib -L/opt/rocm/lib -lamdhip64
+echo "built tests/cpp/test_nn"
