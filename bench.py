@@ -24,6 +24,9 @@ sys.path.insert(0, ROOT)
 import __graft_entry__ as entry  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, GB/s
+# HBM bytes per launch of the roofline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
+# a device copy of known size (profiles/gemv_lm_head_pmc_traffic.md); None until measured.
+TRAFFIC_BYTES_PER_LAUNCH = 24548000
 
 
 def step_bytes(cfg, group, context_len):
@@ -44,6 +47,42 @@ def gemv_bytes(K, N, group, M=1):
     return K * N / 2 + ((K + group - 1) // group) * N * 4 + M * K * 4 + M * N * 4
 
 
+def roofline_kernel(ctx, cfg, group, workloads):
+    """The dominant kernel: the int4 dequant-GEMV (about 85% of the step's GPU time), timed on the
+    LM-head shape, its largest launch (31% of the step's bytes).  240 back-to-back launches are
+    recorded into a HIP graph and replayed; HIP events on the context's stream bracket the replay.
+    Two figures: a rotation over 12 weight copies (290 MB, larger than the caches) is the HBM
+    figure reported as `achieved`; the same weights every launch (cache resident, as in decode,
+    where the 78 MB model stays in the 256 MB Infinity Cache) is reported beside it."""
+    import ctypes as C
+    K, N = cfg["n_embd"], ((cfg["vocab"] + 255) // 256) * 256
+    rng = np.random.default_rng(0)
+    n_sets = 12
+    packed, scales, _ = workloads.random_int4_linear(rng, K, N, group)
+    dp = ctx.upload(np.tile(packed, (n_sets, 1)))
+    ds = ctx.upload(np.tile(scales, (n_sets, 1)))
+    dx = ctx.upload(rng.standard_normal((1, K)).astype(np.float32))
+    dy = ctx.malloc(N * 4)
+
+    def time_gemv(sets, reps=240):
+        us = C.c_float(0)
+        ctx.call("agpu_bench_int4_linear", dx, None, None, 0.0, dp, ds, None, None, dy, 1, N, K, group, 0, sets,
+                 packed.size, scales.size, reps, C.addressof(us))
+        return float(us.value)
+
+    us_hot = time_gemv(1)
+    us = time_gemv(n_sets)
+    gb = gemv_bytes(K, N, group)
+    for p in (dp, ds, dx, dy):
+        ctx.free(p)
+    achieved = gb / (us * 1e-6) / 1e9
+    return {"bound": "hbm", "kernel": "int4_gemv_kernel<1,4,false> (LM head shape M=1 K=768 N=50432 g=32)",
+            "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5),
+            "traffic": TRAFFIC_BYTES_PER_LAUNCH, "bytes_per_launch": int(gb), "us_per_launch": round(us, 3),
+            "weight_sets_rotated": n_sets, "cache_resident_GBps": round(gb / (us_hot * 1e-6) / 1e9, 2),
+            "cache_resident_us_per_launch": round(us_hot, 3)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -51,6 +90,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-steps", type=int, default=24)
+    ap.add_argument("--roofline-only", action="store_true",
+                    help="only the dominant-kernel loop plus a 64 MiB device copy (calibration for rocprofv3 --pmc runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (every GPU box here has one MI355X); run with --gpus 1")
@@ -66,6 +107,18 @@ def main():
     group, prompt_len = 32, 64
     if prompt_len + args.warmup + args.steps > cfg["n_positions"]:
         sys.exit(f"bench.py: prompt {prompt_len} + warmup + steps must stay within {cfg['n_positions']} positions")
+
+    if args.roofline_only:
+        ctx = _lib.Context(0)
+        r = roofline_kernel(ctx, cfg, group, workloads)
+        n = 64 << 20
+        a, b = ctx.malloc(n), ctx.malloc(n)
+        for _ in range(10):
+            ctx.call("agpu_memcpy_d2d", b, a, n)
+        ctx.sync()
+        r["calibration_copy_bytes"] = n
+        print(json.dumps({"roofline": r}))
+        return
 
     t0 = time.time()
     weights = workloads.gpt2_fp32_weights(cfg, seed=3)
@@ -89,36 +142,7 @@ def main():
     ctx_mid = ctx0 + args.steps // 2
     sb = step_bytes(cfg, group, ctx_mid)
 
-    # dominant kernel: the int4 dequant-GEMV (about 85% of the step's GPU time).  Timed on the
-    # LM-head shape, its largest launch (31% of the step's bytes): `reps` back-to-back launches
-    # recorded into a HIP graph and replayed, HIP events on the context's stream around the replay.
-    # Two figures: the same weights every launch (cache resident, as in decode where the 78 MB
-    # model stays in the 256 MB Infinity Cache) and a rotation over 12 weight copies (290 MB,
-    # larger than the caches), which is the HBM figure reported as roofline.achieved.
-    import ctypes as C
-    ctx = model.ctx
-    K, N = cfg["n_embd"], ((cfg["vocab"] + 255) // 256) * 256
-    rng = np.random.default_rng(0)
-    n_sets = 12
-    packed, scales, _ = workloads.random_int4_linear(rng, K, N, group)
-    dp = ctx.upload(np.tile(packed, (n_sets, 1)))
-    ds = ctx.upload(np.tile(scales, (n_sets, 1)))
-    dx = ctx.upload(rng.standard_normal((1, K)).astype(np.float32))
-    dy = ctx.malloc(N * 4)
-
-    def time_gemv(sets, reps=240):
-        us = C.c_float(0)
-        ctx.call("agpu_bench_int4_linear", dx, None, None, 0.0, dp, ds, None, None, dy, 1, N, K, group, 0, sets,
-                 packed.size, scales.size, reps, C.addressof(us))
-        return float(us.value)
-
-    gemv_us_hot = time_gemv(1)
-    gemv_us = time_gemv(n_sets)
-    gb = gemv_bytes(K, N, group)
-    achieved = gb / (gemv_us * 1e-6) / 1e9
-    achieved_hot = gb / (gemv_us_hot * 1e-6) / 1e9
-    for p in (dp, ds, dx, dy):
-        ctx.free(p)
+    roof = roofline_kernel(model.ctx, cfg, group, workloads)
 
     out = {
         "metric": "GPT-2 int4 decode tok/s (B=1); dequant-GEMV HBM GB/s vs peak",
@@ -137,12 +161,7 @@ def main():
                    "context_at_start": ctx0, "steps_event_ms": round(ms_events, 4), "model_build_s": round(build_s, 2)},
         "step_hbm": {"algorithmic_bytes_per_step": int(sb), "achieved_GBps": round(sb / (ms_per_step * 1e-3) / 1e9, 2),
                      "frac_of_8TBps": round(sb / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 5)},
-        "roofline": {"bound": "hbm", "kernel": "int4_gemv_kernel<1,4,false> (LM head shape M=1 K=768 N=50432 g=32)",
-                     "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 5), "traffic": None,
-                     "bytes_per_launch": int(gb), "us_per_launch": round(gemv_us, 3),
-                     "weight_sets_rotated": n_sets, "cache_resident_GBps": round(achieved_hot, 2),
-                     "cache_resident_us_per_launch": round(gemv_us_hot, 3)},
+        "roofline": roof,
     }
 
     if not args.no_cpu_baseline:
