@@ -53,7 +53,7 @@ SIGNATURES = {
     "agpu_timer_stop": (_i32, [_vp, _vp]),
     "agpu_kernel_lookup": (_i32, [_vp, C.c_char_p, C.POINTER(C.c_char_p)]),
     "agpu_int4_linear": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32]),
-    "agpu_int4_gemv_tune": (None, [_i32, _i32]),
+    "agpu_int4_gemv_tune": (None, [_i32, _i32, _i32]),
     "agpu_ln_int4_linear": (_i32, [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32]),
     "agpu_bench_int4_linear": (_i32, [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32,
                                       _i32, C.c_int64, C.c_int64, _i32, _vp]),
@@ -71,6 +71,7 @@ SIGNATURES = {
     "agpu_split_qkv": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32]),
     "agpu_concat_heads": (_i32, [_vp, _vp, _vp, _i32, _i32, _i32]),
     "agpu_attention": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32]),
+    "agpu_bench_attention": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
     "agpu_kv_append": (_i32, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32]),
     "agpu_gemm_f32": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32]),
     # include/agpu_gpt2.h (first argument is the model handle, or the config / context)

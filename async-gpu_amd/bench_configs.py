@@ -1,0 +1,126 @@
+#!/usr/bin/env python3
+"""Per-configuration measurements of the quantized GPT-2 path on one MI355X (the benchmark
+configurations other than the headline one, which bench.py covers): isolated int4 GEMV / GEMM,
+attention prefill / decode, and GPT-2 XL-shaped decode at batch 1 and 16.  Prints one JSON line per
+case.  Kernel cases are timed as graph replays with HIP events on the context's stream.
+
+    python3 async-gpu_amd/bench_configs.py [--xl-layers 48] [--skip-xl] [--skip-kernels]
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as entry  # noqa: E402
+
+HBM_GBS, MFMA_F32_TFLOPS = 8000.0, 157.3
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--xl-layers", type=int, default=48)
+    ap.add_argument("--skip-xl", action="store_true")
+    ap.add_argument("--skip-kernels", action="store_true")
+    args = ap.parse_args()
+    entry.load_package()
+    from async_gpu_amd import _lib, gpt2, workloads
+
+    ctx = _lib.Context(0)
+
+    def emit(**kw):
+        print(json.dumps(kw), flush=True)
+
+    def bench_linear(M, K, N, group=32, reps=100):
+        w = workloads.config1_gemv(seed=0 if M == 1 else 1, M=M, K=K, N=N, group=group)
+        dp, ds, dx = ctx.upload(w["packed"]), ctx.upload(w["scales"]), ctx.upload(w["x"])
+        dy = ctx.malloc(M * N * 4)
+        us = C.c_float(0)
+        ctx.call("agpu_bench_int4_linear", dx, None, None, 0.0, dp, ds, None, None, dy, M, N, K, group, 0, 1, 0, 0, reps,
+                 C.addressof(us))
+        for p in (dp, ds, dx, dy):
+            ctx.free(p)
+        return us.value
+
+    if not args.skip_kernels:
+        kernel_cases(ctx, emit, bench_linear, workloads)
+    if args.skip_xl:
+        return
+    xl_cases(ctx, emit, args, _lib, gpt2, workloads)
+
+
+def kernel_cases(ctx, emit, bench_linear, workloads):
+    # config 1: single dequant-GEMV, the MLP fc shape
+    us = bench_linear(1, 768, 3072)
+    b = 768 * 3072 // 2 + 24 * 3072 * 4 + 768 * 4 + 3072 * 4
+    emit(case="config1 int4 GEMV M=1 K=768 N=3072 g=32", us=round(us, 3), algorithmic_bytes=b,
+         GBps=round(b / us / 1e3, 1), frac_hbm=round(b / us / 1e3 / HBM_GBS, 4))
+    # config 2: prefill QKV dequant-GEMM
+    for M in (128, 512, 1024):
+        us = bench_linear(M, 768, 2304, reps=50)
+        fl = 2.0 * M * 768 * 2304
+        emit(case=f"config2 int4 GEMM M={M} K=768 N=2304 g=32", us=round(us, 3), flops=fl,
+             TFLOPs=round(fl / us / 1e6, 2), frac_mfma_f32=round(fl / us / 1e6 / MFMA_F32_TFLOPS, 4))
+    # config 3: attention prefill and decode
+    w = workloads.config3_attention()
+    dq, dk, dv = ctx.upload(w["q"]), ctx.upload(w["k"]), ctx.upload(w["v"])
+    do = ctx.malloc(w["q"].nbytes)
+    us = C.c_float(0)
+    ctx.call("agpu_bench_attention", dq, dk, dv, do, 12, 1024, 1024, 0, 1024, 64, 1, 20, C.addressof(us))
+    fl = 4.0 * 12 * 64 * 1024 * 1025 / 2
+    emit(case="config3 attention prefill H=12 seq=1024", us=round(us.value, 3), flops=fl,
+         TFLOPs=round(fl / us.value / 1e6, 2), frac_mfma_f32=round(fl / us.value / 1e6 / MFMA_F32_TFLOPS, 4))
+    dq1 = ctx.upload(np.ascontiguousarray(w["q"][:, 1023:1024]))
+    ctx.call("agpu_bench_attention", dq1, dk, dv, do, 12, 1, 1024, 1023, 1024, 64, 1, 200, C.addressof(us))
+    b = 2 * 12 * 1024 * 64 * 4
+    emit(case="config3 attention decode H=12 kv=1024", us=round(us.value, 3), algorithmic_bytes=b,
+         GBps=round(b / us.value / 1e3, 1), frac_hbm=round(b / us.value / 1e3 / HBM_GBS, 4))
+    for p in (dq, dk, dv, do, dq1):
+        ctx.free(p)
+
+
+
+def xl_cases(ctx, emit, args, _lib, gpt2, workloads):
+    # config 5: GPT-2 XL-shaped decode, prompt 256, batch 1 and 16 (weights quantized on the device at load)
+    cfg = dict(workloads.GPT2_XL, n_layer=args.xl_layers)
+    t0 = time.time()
+    gcfg = gpt2.Gpt2Config(cfg["n_layer"], cfg["n_embd"], cfg["n_head"], group_size=32, max_batch=16)
+    model = gpt2.Int4Gpt2Model(gcfg, ctx)
+    rng = np.random.default_rng(4)
+    d, ff, V, P = cfg["n_embd"], 4 * cfg["n_embd"], cfg["vocab"], cfg["n_positions"]
+    nrm = lambda *s: rng.standard_normal(s, dtype=np.float32) * np.float32(0.02)
+    wte = nrm(V, d)
+    model.set_embeddings(wte, nrm(P, d), np.ones(d, np.float32), np.zeros(d, np.float32))
+    for L in range(cfg["n_layer"]):
+        model.set_layer_norms(L, np.ones(d, np.float32), np.zeros(d, np.float32), np.ones(d, np.float32), np.zeros(d, np.float32))
+        for name, (k, n) in (("qkv", (d, 3 * d)), ("proj", (d, d)), ("fc", (d, ff)), ("fc_proj", (ff, d))):
+            model.quantize_linear(L, name, nrm(k, n), np.zeros(n, np.float32), _lib.QUANT_SCRIPT)
+    model.quantize_linear(-1, 0, np.ascontiguousarray(wte.T), None, _lib.QUANT_SCRIPT)
+    build_s = time.time() - t0
+    per_w = 0.5 + 4.0 / 32
+    wbytes = cfg["n_layer"] * (12 * d * d * per_w + (3 * d + d + ff + d) * 4 + 4 * d * 4) + d * V * per_w
+    for B in (1, 16):
+        prompts = workloads.random_prompt(cfg, 4, 256, batch=B)
+        model.reset_cache()
+        t0 = time.time()
+        model.forward_cached(prompts, all_rows=False)
+        prefill_s = time.time() - t0
+        model.decode_steps(B, 8)
+        steps = 64
+        ms = model.decode_steps(B, steps)
+        ctx_mid = 256 + 8 + steps // 2
+        kv = cfg["n_layer"] * 2 * d * 4 * (ctx_mid + 2) * B
+        bytes_step = wbytes + kv
+        emit(case=f"config5 GPT-2 XL-shaped ({cfg['n_layer']} layers) int4 decode B={B}, prompt 256", ms_per_step=round(ms / steps, 4),
+             tok_s=round(B * steps / (ms / 1e3), 1), algorithmic_bytes_per_step=int(bytes_step),
+             GBps=round(bytes_step / (ms / steps) / 1e6, 1), frac_hbm=round(bytes_step / (ms / steps) / 1e6 / HBM_GBS, 4),
+             prefill_wall_s=round(prefill_s, 3), model_build_s=round(build_s, 1))
+
+
+if __name__ == "__main__":
+    main()

@@ -272,3 +272,39 @@ AGPU_EXPORT int32_t agpu_attention(agpu_ctx *ctx, const float *q, const float *k
     p.pos_dev = nullptr;
     return agpu_attention_launch(ctx, p, kv_len);
 }
+
+AGPU_EXPORT int32_t agpu_bench_attention(agpu_ctx *ctx, const float *q, const float *k, const float *v, float *o,
+                                         int32_t n_heads, int32_t q_len, int32_t kv_len, int32_t q_offset,
+                                         int32_t kv_stride, int32_t d_head, int32_t causal, int32_t reps,
+                                         float *us_per_launch_out_host) {
+    AGPU_REQUIRE_CTX(ctx);
+    AGPU_REQUIRE_PTR(ctx, us_per_launch_out_host);
+    if (reps <= 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "bench_attention: reps must be positive");
+    if (!ctx->stream) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "bench_attention: needs a context with its own stream");
+    int32_t rc = agpu_attention(ctx, q, k, v, o, n_heads, q_len, kv_len, q_offset, kv_stride, d_head, causal);
+    if (rc != AGPU_OK) return rc;
+    hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipStreamBeginCapture");
+    for (int i = 0; i < reps && rc == AGPU_OK; ++i)
+        rc = agpu_attention(ctx, q, k, v, o, n_heads, q_len, kv_len, q_offset, kv_stride, d_head, causal);
+    hipGraph_t graph = nullptr;
+    e = hipStreamEndCapture(ctx->stream, &graph);
+    if (rc != AGPU_OK || e != hipSuccess) {
+        if (graph) (void)hipGraphDestroy(graph);
+        return rc != AGPU_OK ? rc : agpu_hip(ctx, e, "hipStreamEndCapture");
+    }
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipGraphInstantiate");
+    float ms = 0.0f;
+    e = hipGraphLaunch(exec, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e == hipSuccess) rc = agpu_timer_start(ctx);
+    if (e == hipSuccess && rc == AGPU_OK) e = hipGraphLaunch(exec, ctx->stream);
+    if (e == hipSuccess && rc == AGPU_OK) rc = agpu_timer_stop(ctx, &ms);
+    (void)hipGraphExecDestroy(exec);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipGraphLaunch");
+    *us_per_launch_out_host = ms * 1000.0f / (float)reps;
+    return rc;
+}

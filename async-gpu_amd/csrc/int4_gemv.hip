@@ -64,26 +64,6 @@ __device__ __forceinline__ void load_floats(const float *p, float (&f)[CPL]) {
     if constexpr (CPL == 4) { f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w; }
 }
 
-// Epilogue for one output element, plus the optional K/V scatter of a fused QKV projection.
-__device__ __forceinline__ void finish_output(const GemvArgs &a, float v, float bias, float resid, int m, int n) {
-    v += bias;
-    if (a.flags & AGPU_EPI_GELU_TANH) v = gelu_tanh_dev(v);
-    else if (a.flags & AGPU_EPI_GELU_QUICK) v = gelu_quick_dev(v);
-    v += resid;
-    a.y[(size_t)m * a.N + n] = v;
-    if (a.kcache) {
-        const int d_model = a.N / 3;
-        if (n >= d_model) {
-            const int j = n - d_model;
-            const bool is_v = j >= d_model;
-            const int jj = is_v ? j - d_model : j;
-            const int h = jj >> 6, e = jj & 63;
-            float *dst = is_v ? a.vcache : a.kcache;
-            dst[((size_t)(m * a.n_heads + h) * a.n_positions + *a.pos_dev) * 64 + e] = v;
-        }
-    }
-}
-
 // Sum over the workgroup, result in every thread.  scratch: 16 floats of LDS.
 __device__ __forceinline__ float block_sum(float v, float *scratch, int lane, int wave, int W) {
     v = wave_sum(v);
@@ -100,7 +80,7 @@ __device__ __forceinline__ float block_sum(float v, float *scratch, int lane, in
 // A workgroup handles the column tiles blockIdx.x, blockIdx.x + gridDim.x, ...: x is staged once
 // and the loads of the next tile's first two row trips are issued before the current tile is reduced.
 template <int MT, int CPL, bool LN>
-__global__ __launch_bounds__(MT <= 4 ? 1024 : 512) void int4_gemv_kernel(const GemvParams p) {
+__global__ __launch_bounds__(MT == 1 ? 1024 : 512) void int4_gemv_kernel(const GemvParams p) {
     extern __shared__ __align__(16) float smem[];
     __shared__ float s_scratch[16];
     __shared__ int s_last;
@@ -377,13 +357,15 @@ int32_t launch_m(agpu_ctx *ctx, const GemvParams &p, int MT, dim3 grid, int W, s
 }
 
 int g_tune_target_wgs = 0;    // 0: default
+int g_tune_max_waves = 0;         // 0: the launch bound of the instantiation
 int g_tune_rows_per_split = 256;  // packed rows a workgroup takes at most
 
 }  // namespace
 
 bool agpu_int4_gemv_can_fuse_ln(int M, int K) { return M <= 2 && (size_t)M * K * sizeof(float) <= 32 * 1024; }
 
-AGPU_EXPORT void agpu_int4_gemv_tune(int32_t max_wgs, int32_t min_rows_per_wave) {
+AGPU_EXPORT void agpu_int4_gemv_tune(int32_t max_wgs, int32_t min_rows_per_wave, int32_t max_waves) {
+    g_tune_max_waves = max_waves;
     const int32_t target_wgs = max_wgs;
     g_tune_target_wgs = target_wgs;
     g_tune_rows_per_split = min_rows_per_wave > 0 ? min_rows_per_wave : 256;
@@ -420,7 +402,8 @@ int32_t agpu_int4_gemv_launch(agpu_ctx *ctx, const GemvArgs &a) {
         return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_gemv: split-K partials exceed the workspace (M=%d N=%d K=%d)", a.M, a.N, a.K);
     // waves: one per 4*g_tune_min_rows rows of the slice, bounded by the launch bound of the
     // instantiation and by the LDS the cross-wave reduction needs
-    const int max_w = MT <= 4 ? 16 : 8;
+    int max_w = MT == 1 ? 16 : 8;
+    if (g_tune_max_waves > 0 && g_tune_max_waves < max_w) max_w = g_tune_max_waves;
     int W = ceil_div(p.rows_per_split, 8);  // two trips of 4 rows per wave
     W = W < 1 ? 1 : (W > max_w ? max_w : W);
     while (W > 1 && ((size_t)W * MT * 16 * cpl + stage_floats(ksplit)) * sizeof(float) > 64 * 1024) --W;

@@ -47,7 +47,30 @@ struct GemvArgs {
     int n_heads, n_positions;
 };
 
+// Epilogue for one output element, plus the optional K/V scatter of a fused QKV projection.
+__device__ __forceinline__ void finish_output(const GemvArgs &a, float v, float bias, float resid, int m, int n) {
+    v += bias;
+    if (a.flags & AGPU_EPI_GELU_TANH) v = gelu_tanh_dev(v);
+    else if (a.flags & AGPU_EPI_GELU_QUICK) v = gelu_quick_dev(v);
+    v += resid;
+    a.y[(size_t)m * a.N + n] = v;
+    if (a.kcache) {
+        const int d_model = a.N / 3;
+        if (n >= d_model) {
+            const int j = n - d_model;
+            const bool is_v = j >= d_model;
+            const int jj = is_v ? j - d_model : j;
+            const int h = jj >> 6, e = jj & 63;
+            float *dst = is_v ? a.vcache : a.kcache;
+            dst[((size_t)(m * a.n_heads + h) * a.n_positions + *a.pos_dev) * 64 + e] = v;
+        }
+    }
+}
+
 int32_t agpu_int4_gemv_launch(agpu_ctx *ctx, const GemvArgs &a);
+// MFMA variant for 4 < M <= 16 (needs group % 32 == 0, K % 32 == 0, N % 4 == 0, 16-byte aligned weights).
+bool agpu_int4_skinny_supported(const GemvArgs &a);
+int32_t agpu_int4_skinny_launch(agpu_ctx *ctx, const GemvArgs &a);
 // Whether the GEMV can apply LayerNorm itself for this shape (otherwise normalise first).
 bool agpu_int4_gemv_can_fuse_ln(int M, int K);
 

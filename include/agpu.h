@@ -95,9 +95,10 @@ int32_t agpu_int4_linear(agpu_ctx *ctx, const float *x, const uint32_t *packed, 
 
 /* Tuning hook of the decode GEMV (M <= 16): the most workgroups a launch uses (0 = one per CU,
  * the default; each workgroup strides over the column tiles) and the most packed rows (8 k each)
- * one workgroup takes before K is split over workgroups (0 = 256, the default).
+ * one workgroup takes before K is split over workgroups (0 = 256, the default), and the most waves per
+ * workgroup (0 = 16 for M = 1, 8 otherwise).
  * Process-wide; results stay deterministic for any setting. */
-void agpu_int4_gemv_tune(int32_t max_wgs, int32_t max_rows_per_wg);
+void agpu_int4_gemv_tune(int32_t max_wgs, int32_t max_rows_per_wg, int32_t max_waves_per_wg);
 
 /* Same with LayerNorm(x; gamma, beta, eps) over K applied to each input row first
  * (ops::layer_norm followed by Int4Linear::forward, gpt2.rs:1307-1316,1329-1331). */
@@ -190,6 +191,12 @@ int32_t agpu_concat_heads(agpu_ctx *ctx, const float *in, float *out, int32_t se
 int32_t agpu_attention(agpu_ctx *ctx, const float *q, const float *k, const float *v, float *o,
                        int32_t n_heads, int32_t q_len, int32_t kv_len, int32_t q_offset,
                        int32_t kv_stride, int32_t d_head, int32_t causal);
+/* Measurement helper for agpu_attention, built like agpu_bench_int4_linear: `reps` launches in a
+ * HIP graph, mean microseconds per launch from HIP events on the context's stream. */
+int32_t agpu_bench_attention(agpu_ctx *ctx, const float *q, const float *k, const float *v, float *o,
+                             int32_t n_heads, int32_t q_len, int32_t kv_len, int32_t q_offset,
+                             int32_t kv_stride, int32_t d_head, int32_t causal, int32_t reps,
+                             float *us_per_launch_out_host);
 /* kv_cache_append (compute_transformer.rs:1777-1812): row 0 of src [H, src_stride, dh]
  * -> cache [H, max_seq, dh] at write_pos. */
 int32_t agpu_kv_append(agpu_ctx *ctx, const float *src, float *cache, int32_t n_heads, int32_t src_stride,
