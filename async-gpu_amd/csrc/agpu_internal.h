@@ -1,6 +1,7 @@
 // Internal declarations shared by the HIP translation units of libagpu_hip.so.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <atomic>
 
 #include <cstdarg>
 #include <cstdint>
@@ -23,7 +24,11 @@ struct agpu_ctx {
     unsigned int *counters = nullptr;  // kNumCounters zeroed uint32; kernels restore zero
     hipEvent_t t0 = nullptr, t1 = nullptr;  // agpu_timer_*
     char err[512] = {0};
+    std::atomic<int> refs{1};  // the handle itself + one per model created on the context
 };
+
+// Drops one reference; the context's resources go with the last one.
+void agpu_ctx_release(agpu_ctx *ctx);
 
 inline int32_t agpu_fail(agpu_ctx *ctx, int32_t code, const char *fmt, ...) {
     if (ctx) {

@@ -62,6 +62,12 @@ AGPU_EXPORT int32_t agpu_ctx_create_on_stream(int32_t device, void *hip_stream, 
 
 AGPU_EXPORT int32_t agpu_ctx_destroy(agpu_ctx *ctx) {
     if (!ctx) return AGPU_OK;
+    agpu_ctx_release(ctx);
+    return AGPU_OK;
+}
+
+void agpu_ctx_release(agpu_ctx *ctx) {
+    if (ctx->refs.fetch_sub(1) > 1) return;  // a model still runs on this context
     (void)hipSetDevice(ctx->device);
     if (ctx->stream || !ctx->owns_stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->t0) (void)hipEventDestroy(ctx->t0);
@@ -70,7 +76,6 @@ AGPU_EXPORT int32_t agpu_ctx_destroy(agpu_ctx *ctx) {
     if (ctx->counters) (void)hipFree(ctx->counters);
     if (ctx->owns_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
-    return AGPU_OK;
 }
 
 AGPU_EXPORT const char *agpu_last_error_string(const agpu_ctx *ctx) { return ctx ? ctx->err : "null context"; }

@@ -83,6 +83,72 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const float *a, const f
     }
 }
 
+// One 256-thread workgroup per row, for launches with few rows (decode): every load of the row is in
+// flight at once and the code stays short.  d <= 256 * LNW_CACHE.
+constexpr int LNW_CACHE = 8;
+template <bool ADD>
+__global__ __launch_bounds__(256) void layer_norm_row_kernel(const float *a, const float *b, const float *__restrict__ gamma,
+                                                              const float *__restrict__ beta, float *sum_out, float *y,
+                                                              int d, float eps) {
+    __shared__ float s_part[2][4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const size_t base = (size_t)blockIdx.x * d;
+    float v[LNW_CACHE], g[LNW_CACHE], be[LNW_CACHE];
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < LNW_CACHE; ++i) {
+        const int k = tid + 256 * i;
+        float t = 0.0f;
+        g[i] = 0.0f;
+        be[i] = 0.0f;
+        if (k < d) {
+            t = a[base + k];
+            if (ADD) t += b[base + k];
+            g[i] = gamma[k];
+            be[i] = beta[k];
+        }
+        v[i] = t;
+        s += t;
+    }
+    if (ADD && sum_out) {
+#pragma unroll
+        for (int i = 0; i < LNW_CACHE; ++i) {
+            const int k = tid + 256 * i;
+            if (k < d) sum_out[base + k] = v[i];
+        }
+    }
+    s = wave_sum(s);
+    if (lane == 0) s_part[0][wave] = s;
+    __syncthreads();
+    const float mean = ((s_part[0][0] + s_part[0][1]) + (s_part[0][2] + s_part[0][3])) / (float)d;
+    float q = 0.0f;
+#pragma unroll
+    for (int i = 0; i < LNW_CACHE; ++i) {
+        const int k = tid + 256 * i;
+        const float df = v[i] - mean;
+        if (k < d) q += df * df;
+    }
+    q = wave_sum(q);
+    if (lane == 0) s_part[1][wave] = q;
+    __syncthreads();
+    const float rstd = 1.0f / sqrtf(((s_part[1][0] + s_part[1][1]) + (s_part[1][2] + s_part[1][3])) / (float)d + eps);
+#pragma unroll
+    for (int i = 0; i < LNW_CACHE; ++i) {
+        const int k = tid + 256 * i;
+        if (k < d) y[base + k] = (v[i] - mean) * rstd * g[i] + be[i];
+    }
+}
+
+template <bool ADD>
+void launch_layer_norm(agpu_ctx *ctx, const float *a, const float *b, const float *gamma, const float *beta, float *sum_out,
+                       float *y, int rows, int d, float eps) {
+    if (rows <= 512 && d <= 256 * LNW_CACHE)
+        hipLaunchKernelGGL((layer_norm_row_kernel<ADD>), dim3(rows), dim3(256), 0, ctx->stream, a, b, gamma, beta, sum_out, y, d, eps);
+    else
+        hipLaunchKernelGGL((layer_norm_kernel<ADD>), dim3(ceil_div(rows, 4)), dim3(256), 0, ctx->stream, a, b, gamma, beta,
+                           sum_out, y, rows, d, eps);
+}
+
 __global__ __launch_bounds__(256) void gelu_kernel(const float *x, float *y, size_t n, int mode) {
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i + 3 < n && (((uintptr_t)x | (uintptr_t)y) & 15) == 0) {
@@ -258,8 +324,7 @@ inline unsigned grid_1d(size_t n, int per_block) { return (unsigned)((n + per_bl
 
 int32_t agpu_layer_norm_impl(agpu_ctx *ctx, const float *x, const float *gamma, const float *beta, float *y,
                              int rows, int d, float eps) {
-    hipLaunchKernelGGL((layer_norm_kernel<false>), dim3(ceil_div(rows, 4)), dim3(256), 0, ctx->stream, x,
-                       (const float *)nullptr, gamma, beta, (float *)nullptr, y, rows, d, eps);
+    launch_layer_norm<false>(ctx, x, nullptr, gamma, beta, nullptr, y, rows, d, eps);
     return AGPU_LAUNCH_CHECK(ctx, "layer_norm_kernel");
 }
 
@@ -281,8 +346,7 @@ AGPU_EXPORT int32_t agpu_add_layer_norm_dual(agpu_ctx *ctx, const float *a, cons
     if (rows < 0 || d <= 0)
         return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "add_layer_norm_dual: bad dims rows=%d d=%d", rows, d);
     if (rows == 0) return AGPU_OK;
-    hipLaunchKernelGGL((layer_norm_kernel<true>), dim3(ceil_div(rows, 4)), dim3(256), 0, ctx->stream, a, b, gamma,
-                       beta, sum_out, norm_out, rows, d, eps);
+    launch_layer_norm<true>(ctx, a, b, gamma, beta, sum_out, norm_out, rows, d, eps);
     return AGPU_LAUNCH_CHECK(ctx, "add_layer_norm_kernel");
 }
 

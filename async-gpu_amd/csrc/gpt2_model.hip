@@ -467,6 +467,7 @@ AGPU_EXPORT int32_t agpu_gpt2_create(agpu_ctx *ctx, const agpu_gpt2_config *cfg,
     agpu_gpt2 *m = new (std::nothrow) agpu_gpt2();
     if (!m) return AGPU_ERR_NULL_POINTER;
     m->ctx = ctx;
+    ctx->refs.fetch_add(1);
     m->cfg = *cfg;
     m->d = cfg->n_embd;
     m->H = cfg->n_head;
@@ -512,6 +513,7 @@ AGPU_EXPORT int32_t agpu_gpt2_destroy(agpu_gpt2 *m) {
         if (p) (void)hipFree(p);
     for (hipEvent_t e : {m->ev0, m->ev1, m->ev2})
         if (e) (void)hipEventDestroy(e);
+    agpu_ctx_release(m->ctx);
     delete m;
     return AGPU_OK;
 }

@@ -285,9 +285,20 @@ __global__ __launch_bounds__(MT == 1 ? 1024 : 512) void int4_gemv_kernel(const G
         for (int i = tid; i < n_out; i += T) {
             const int m = i / COLS, n = tile * COLS + (i - m * COLS);
             if (m < a.M && n < a.N) {
+                const float *src = p.partial + (size_t)m * a.N + n;
+                const size_t stride = (size_t)a.M * a.N;
                 float t = 0.0f;
-                for (int sp = 0; sp < ksplit; ++sp)
-                    t += __hip_atomic_load(&p.partial[((size_t)sp * a.M + m) * a.N + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (int sp0 = 0; sp0 < ksplit; sp0 += 8) {  // 8 loads in flight, summed in split order
+                    float part[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+                        part[u] = sp0 + u < ksplit
+                                      ? __hip_atomic_load(src + (size_t)(sp0 + u) * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                      : 0.0f;
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+                        if (sp0 + u < ksplit) t += part[u];
+                }
                 if (i != tid) {
                     e_bias = a.bias ? a.bias[n] : 0.0f;
                     e_res = a.residual ? a.residual[(size_t)m * a.N + n] : 0.0f;

@@ -47,6 +47,8 @@ int32_t agpu_ctx_create(int32_t device, agpu_ctx **out);
 /* Same, but launches go to a stream the caller owns (hipStream_t passed as void*;
  * NULL = the legacy default stream).  For hosts that already have a stream. */
 int32_t agpu_ctx_create_on_stream(int32_t device, void *hip_stream, agpu_ctx **out);
+/* Models created on the context keep it alive: its memory and stream are released once the
+ * context and every such model have been destroyed, in either order. */
 int32_t agpu_ctx_destroy(agpu_ctx *ctx);
 const char *agpu_last_error_string(const agpu_ctx *ctx);
 void *agpu_ctx_stream(const agpu_ctx *ctx);

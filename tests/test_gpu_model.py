@@ -198,3 +198,19 @@ def test_config4_gpt2_small_generation(orc, agpu, dev):
     _assert_tokens_match(got, ref, margins, 64, "config 4")
     assert len(got) == 192
     print(f"config4: prefill {ms_prefill:.3f} ms, decode {ms_decode / 127:.4f} ms/token, min oracle margin {margins.min():.3e}")
+
+
+def test_context_may_be_destroyed_before_its_model(orc, agpu, dev):
+    """Garbage collectors finalize a context and a model that refers to it in any order; the library
+    keeps the context's memory until both are gone."""
+    from async_gpu_amd import _lib, gpt2, workloads
+    cfg = workloads.GPT2_TINY
+    _, qz = _quantized(orc, cfg, 5)
+    ctx = _lib.Context(0)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg), qz, ctx=ctx)
+    prompt = workloads.random_prompt(cfg, 1, 6)
+    toks = gm.generate_cached(prompt.reshape(1, -1), 4, eos=-1)[0]
+    assert len(toks[0]) == 10
+    ctx.close()
+    gm.close()  # must not touch freed memory
+    gm.close()
