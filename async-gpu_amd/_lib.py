@@ -10,7 +10,7 @@ _SO = os.path.join(_HERE, "libagpu_hip.so")
 ERR_SHAPE_MISMATCH, ERR_DIM_OUT_OF_RANGE, ERR_KERNEL_NOT_FOUND = -1, -2, -3
 ERR_NULL_POINTER, ERR_UNSUPPORTED, ERR_WORKSPACE = -4, -5, -6
 
-EPI_NONE, EPI_GELU_TANH, EPI_GELU_QUICK, EPI_FORCE_LITERAL = 0, 1, 2, 0x100
+EPI_NONE, EPI_GELU_TANH, EPI_GELU_QUICK, EPI_FORCE_LITERAL, EPI_FORCE_FP32_GEMV = 0, 1, 2, 0x100, 0x200
 QUANT_RUST, QUANT_SCRIPT = 0, 1
 GELU_TANH, GELU_QUICK = 0, 1
 

@@ -387,6 +387,8 @@ int32_t agpu_int4_gemv_launch(agpu_ctx *ctx, const GemvArgs &a) {
     p.a = a;
     if (a.ln_gamma && !agpu_int4_gemv_can_fuse_ln(a.M, a.K))
         return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "int4_gemv: fused LayerNorm needs M <= 2 and M*K <= 8192");
+    if (!(a.flags & AGPU_EPI_FORCE_FP32_GEMV) && agpu_int4_gemv_i8_supported(a))
+        return agpu_int4_gemv_i8_launch(ctx, a, g_tune_rows_per_split / 8, g_tune_target_wgs);
     const int kp_total = a.K / 8;
     const int MT = a.M <= 1 ? 1 : a.M <= 2 ? 2 : a.M <= 4 ? 4 : a.M <= 8 ? 8 : 16;
     const bool aligned16 = (a.N % 4 == 0) && (((uintptr_t)a.packed | (uintptr_t)a.scales) % 16 == 0);

@@ -1,0 +1,383 @@
+// Decode GEMV of the int4 weight-only Linear for M <= 2 rows on the int8 matrix cores of gfx950.
+//
+// The fp32 VALU GEMV spends about 2.4 instructions per nibble (convert, multiply-add).  Here the
+// multiply-adds run on v_mfma_i32_16x16x64_i8 and the VALU only masks nibbles into bytes
+// (3 instructions per 8 nibbles), with results that are at least as accurate:
+//
+//   * x is turned into fixed point once per launch: with amax = max|x| of the row and s chosen so that
+//     |x * 2^s| < 2^30, X = rint(x * 2^s) is an int32 (exact for the large elements, off by at most
+//     amax * 2^-31 for the small ones; s is capped at 96, so elements below 2^-97 count as zero), split
+//     into four signed base-256 digits X = sum_d D_d * 256^d.
+//   * B operand = the nibbles as bytes 0..15 straight from the packed words; A operand = the digits.
+//     The 16 rows of A are 4 slots x 4 digits; a slot is (row of x, 32-k chunk of the 64-k trip), and a
+//     slot's row is zero outside its chunk, so one MFMA yields, per slot, the four exact integer sums
+//     sum_k D_d[k] * nibble[k] of one scale group chunk for 16 columns.
+//   * Per chunk and column: u = 2^-s * sum_d 256^d * S_d - 8 * sum_k x[k]  (the zero point), acc += scale * u,
+//     in fp32 as in the VALU kernel.
+//
+// Register / lane layout (q = lane / 16, cg = lane % 16), one trip = 8 packed rows = 64 k:
+//   B: lane (cg, q) holds rows 2q and 2q+1 of the trip for its 4 columns (two global_load_dwordx4);
+//      for column c the four B registers are {w0 & 0x0f0f0f0f, (w0 >> 4) & 0x0f0f0f0f, same for w1}.
+//   A: lane (i, q), i = lane % 16: slot = i / 4 = 2 * m + chunk, digit = i % 4; non-zero only when
+//      chunk == q / 2; 16 bytes from LDS, stored at staging time in the byte order the B registers have.
+//   D: lane (cg, q) receives rows 4q..4q+3 = the four digit sums of slot q for column 4 * cg + c.
+// Whatever k index the hardware assigns to (lane group, register, byte), A and B use the same one.
+//
+// Work decomposition, cross-wave reduction and split-K are those of the VALU kernel: a workgroup owns
+// 64 columns x one K slice per tile, each wave at most two trips per tile whose loads are issued before
+// anything else (and for the next tile before the current one is reduced); waves reduce through LDS in
+// wave order; with ksplit > 1 partial sums are published write-through and the last workgroup to take a
+// ticket adds them in split order.  Rows with a NaN or infinity produce NaN outputs.
+#include "linear_common.h"
+
+namespace {
+
+typedef int intx4 __attribute__((ext_vector_type(4)));
+
+struct I8Params {
+    GemvArgs a;
+    int trips_per_split;  // 64-k trips per workgroup, at most 2 per wave
+    int col_blocks;       // tiles of 64 columns
+    float *partial;       // [ksplit, M, N]
+    unsigned int *counters;
+};
+
+// Reduces N values over the workgroup at once; every thread gets the results.  scratch is [N][16] floats
+// whose columns >= W hold 0 (the neutral element for sums and for maxima of non-negative values) and are
+// never written.  One barrier; lanes read the per-wave values in parallel and finish with a 16-lane butterfly,
+// so the order of the additions is fixed.
+template <int N, bool MAX>
+__device__ __forceinline__ void block_reduce(float (&v)[N], float *scratch, int lane, int wave) {
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+        v[n] = MAX ? wave_max(v[n]) : wave_sum(v[n]);
+        if (lane == 0) scratch[n * 16 + wave] = v[n];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+        float t = scratch[n * 16 + (lane & 15)];
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) {
+            const float o = __shfl_xor(t, off, kWave);
+            t = MAX ? fmaxf(t, o) : t + o;
+        }
+        v[n] = t;
+    }
+}
+
+// LDS: xd bytes [MT][tps][4 digits][4 q][16] | xsum float [MT][2 * tps rounded up to 4] | red float [16][MT][64]
+// (rows >= W of red stay zero).  x never goes through LDS as floats: thread r owns packed row r (8 values) of
+// every x row in registers through LayerNorm, the fixed-point conversion and the chunk sums.
+template <int MT, bool LN>
+__global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
+    extern __shared__ __align__(16) float smem[];
+    __shared__ float s_scratch[3][MT * 16];
+    __shared__ int s_last;
+    const GemvArgs &a = p.a;
+    constexpr int COLS = 64;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6, T = blockDim.x;
+    const int q = lane >> 4, cg = lane & 15;
+    const int ksplit = gridDim.y, split = blockIdx.y;
+    const int tps = p.trips_per_split;
+    const int trips_total = a.K / 64;
+    const int t0 = split * tps, t1 = min(trips_total, t0 + tps);
+    unsigned char *xd = reinterpret_cast<unsigned char *>(smem);
+    float *xsum = smem + MT * tps * 64;  // the digit planes take tps * 256 bytes per row
+    const int xsum_len = (2 * tps + 3) & ~3;
+    float *red = xsum + MT * xsum_len;
+    constexpr int n_out = MT * COLS;
+    const int trip_a = t0 + wave, trip_b = trip_a + W;
+
+    uint4 wa0, wa1, wb0, wb1;  // rows 2q, 2q+1 of trips a and b
+    float4 sa, sb;             // scales of chunk q % 2 of trips a and b
+    auto load_trip = [&](int trip, bool ok, uint4 &w0, uint4 &w1, float4 &sc, int c0) {
+        w0 = w1 = make_uint4(0u, 0u, 0u, 0u);
+        sc = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (ok && trip < t1) {
+            const uint32_t *src = a.packed + (size_t)(8 * trip + 2 * q) * a.N + c0;
+            w0 = *reinterpret_cast<const uint4 *>(src);
+            w1 = *reinterpret_cast<const uint4 *>(src + a.N);
+            sc = *reinterpret_cast<const float4 *>(a.scales + (size_t)((64 * trip + 32 * (q & 1)) / a.group) * a.N + c0);
+        }
+    };
+    auto preload = [&](int tile) {
+        const int c0 = tile * COLS + cg * 4;
+        const bool ok = tile < p.col_blocks && c0 < a.N;
+        load_trip(trip_a, ok, wa0, wa1, sa, c0);
+        load_trip(trip_b, ok, wb0, wb1, sb, c0);
+    };
+    preload(blockIdx.x);
+
+    // ---- x: packed row `row` of every x row into registers ----
+    // With LayerNorm the statistics need the whole row of x, so thread r owns row r of all K / 8; otherwise
+    // only the slice's rows are loaded.  The launcher provides at least that many threads.
+    const int row = LN ? tid : 8 * t0 + tid;       // packed row of x this thread owns
+    const int row_end = LN ? a.K / 8 : 8 * t1;
+    const bool own = row < row_end;
+    const bool in_slice = own && row >= 8 * t0 && row < 8 * t1;
+    float xv[MT][8];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        float4 lo = make_float4(0.f, 0.f, 0.f, 0.f), hi = lo;
+        if (own && m < a.M) {
+            const float *src = a.x + (size_t)m * a.K + 8 * row;
+            lo = *reinterpret_cast<const float4 *>(src);
+            hi = *reinterpret_cast<const float4 *>(src + 4);
+        }
+        xv[m][0] = lo.x; xv[m][1] = lo.y; xv[m][2] = lo.z; xv[m][3] = lo.w;
+        xv[m][4] = hi.x; xv[m][5] = hi.y; xv[m][6] = hi.z; xv[m][7] = hi.w;
+    }
+    if (tid < 16) {  // neutral columns of the reduction scratch and the unused rows of red
+        if (tid >= W)
+            for (int j = 0; j < 3 * MT; ++j) (&s_scratch[0][0])[j * 16 + tid] = 0.0f;
+    }
+    for (int i = W * n_out + tid; i < 16 * n_out; i += T) red[i] = 0.0f;
+    if constexpr (LN) {
+        float g8[8], b8[8];
+        {
+            float4 glo = make_float4(0.f, 0.f, 0.f, 0.f), ghi = glo, blo = glo, bhi = glo;
+            if (own) {
+                glo = *reinterpret_cast<const float4 *>(a.ln_gamma + 8 * row);
+                ghi = *reinterpret_cast<const float4 *>(a.ln_gamma + 8 * row + 4);
+                blo = *reinterpret_cast<const float4 *>(a.ln_beta + 8 * row);
+                bhi = *reinterpret_cast<const float4 *>(a.ln_beta + 8 * row + 4);
+            }
+            g8[0] = glo.x; g8[1] = glo.y; g8[2] = glo.z; g8[3] = glo.w; g8[4] = ghi.x; g8[5] = ghi.y; g8[6] = ghi.z; g8[7] = ghi.w;
+            b8[0] = blo.x; b8[1] = blo.y; b8[2] = blo.z; b8[3] = blo.w; b8[4] = bhi.x; b8[5] = bhi.y; b8[6] = bhi.z; b8[7] = bhi.w;
+        }
+        float st[MT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+            st[m] = ((xv[m][0] + xv[m][1]) + (xv[m][2] + xv[m][3])) + ((xv[m][4] + xv[m][5]) + (xv[m][6] + xv[m][7]));
+        block_reduce<MT, false>(st, s_scratch[0], lane, wave);
+        float mean[MT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            mean[m] = st[m] / (float)a.K;
+            float v = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float d = own ? xv[m][j] - mean[m] : 0.0f;
+                v += d * d;
+            }
+            st[m] = v;
+        }
+        block_reduce<MT, false>(st, s_scratch[1], lane, wave);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const float rstd = 1.0f / sqrtf(st[m] / (float)a.K + a.ln_eps);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) xv[m][j] = in_slice && m < a.M ? (xv[m][j] - mean[m]) * rstd * g8[j] + b8[j] : 0.0f;
+        }
+    }
+    // ---- fixed point: amax of the slice, digits, chunk sums ----
+    float amax[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        float t = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float v = fabsf(xv[m][j]);
+            t = fmaxf(t, v == v ? v : __builtin_inff());  // a NaN counts as infinity
+        }
+        amax[m] = in_slice ? t : 0.0f;
+    }
+    block_reduce<MT, true>(amax, s_scratch[2], lane, wave);
+    float c0m[MT], c1m[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        int e = 0;
+        (void)frexpf(amax[m], &e);  // amax < 2^e
+        int s = 30 - e;
+        s = s > 96 ? 96 : s;
+        const bool finite = amax[m] <= 3.0e38f;
+        const float up = finite ? ldexpf(1.0f, s) : 0.0f;
+        c0m[m] = finite ? ldexpf(1.0f, -s) : __builtin_nanf("");
+        c1m[m] = finite ? ldexpf(1.0f, 16 - s) : __builtin_nanf("");
+        // this thread's row: two 32-bit words (even / odd nibbles) per digit plane, and its part of the chunk sum
+        uint32_t dg[4][2] = {{0u, 0u}, {0u, 0u}, {0u, 0u}, {0u, 0u}};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            int v = __float2int_rn(xv[m][j] * up);
+#pragma unroll
+            for (int d = 0; d < 3; ++d) {
+                const int lo = (int)(signed char)(v & 0xff);
+                dg[d][j & 1] |= (uint32_t)(lo & 0xff) << (8 * (j >> 1));
+                v = (v - lo) >> 8;
+            }
+            dg[3][j & 1] |= (uint32_t)(v & 0xff) << (8 * (j >> 1));
+        }
+        float s8 = ((xv[m][0] + xv[m][1]) + (xv[m][2] + xv[m][3])) + ((xv[m][4] + xv[m][5]) + (xv[m][6] + xv[m][7]));
+        s8 += __shfl_xor(s8, 1, kWave);
+        s8 += __shfl_xor(s8, 2, kWave);  // 4 consecutive rows = one 32-k chunk
+        if (in_slice) {
+            const int rl = row - 8 * t0, tl = rl >> 3, rr = rl & 7;
+            unsigned char *dst = xd + ((size_t)(m * tps + tl) * 4) * 64 + 16 * (rr >> 1) + 8 * (rr & 1);
+#pragma unroll
+            for (int d = 0; d < 4; ++d) *reinterpret_cast<uint2 *>(dst + d * 64) = make_uint2(dg[d][0], dg[d][1]);
+            if ((rl & 3) == 0) xsum[m * xsum_len + (rl >> 2)] = 8.0f * s8;
+        }
+    }
+    __syncthreads();
+
+    // A operand addressing of this lane, D-side constants of this lane
+    const int ai = lane & 15, a_slot = ai >> 2, a_m = a_slot >> 1;
+    const bool a_active = a_m < MT && (a_slot & 1) == (q >> 1);
+    const unsigned char *a_src = xd + ((size_t)(a_m < MT ? a_m : 0) * tps * 4 + (ai & 3)) * 64 + 16 * q;
+    const int d_m = q >> 1;
+    const bool d_ok = d_m < MT;
+    float c0f = 0.0f, c1f = 0.0f;
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+        if (d_m == m) { c0f = c0m[m]; c1f = c1m[m]; }
+    const float *d_xsum = xsum + (d_ok ? d_m : 0) * xsum_len + (q & 1);
+
+    float acc[4];
+    auto consume = [&](const uint4 &w0v, const uint4 &w1v, const float4 &scv, int trip) {
+        const int tl = trip - t0;
+        intx4 av = {0, 0, 0, 0};
+        if (a_active) av = *reinterpret_cast<const intx4 *>(a_src + (size_t)tl * 256);
+        const float xs8 = d_ok ? d_xsum[2 * tl] : 0.0f;
+        const uint32_t w0[4] = {w0v.x, w0v.y, w0v.z, w0v.w};
+        const uint32_t w1[4] = {w1v.x, w1v.y, w1v.z, w1v.w};
+        const float sc[4] = {scv.x, scv.y, scv.z, scv.w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const intx4 bv = {(int)(w0[c] & 0x0f0f0f0fu), (int)((w0[c] >> 4) & 0x0f0f0f0fu), (int)(w1[c] & 0x0f0f0f0fu),
+                              (int)((w1[c] >> 4) & 0x0f0f0f0fu)};
+            const intx4 zero = {0, 0, 0, 0};
+            const intx4 d = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bv, zero, 0, 0, 0);
+            const int vlo = d[0] + (d[1] << 8), vhi = d[2] + (d[3] << 8);
+            const float u = fmaf((float)vhi, c1f, fmaf((float)vlo, c0f, -xs8));
+            acc[c] = fmaf(sc[c], u, acc[c]);
+        }
+    };
+
+    for (int tile = blockIdx.x; tile < p.col_blocks; tile += gridDim.x) {
+        float e_bias = 0.0f, e_res = 0.0f;  // epilogue operands of this thread's output element, fetched early
+        {
+            const int m = tid / COLS, n = tile * COLS + (tid - m * COLS);
+            if (tid < n_out && m < a.M && n < a.N) {
+                if (a.bias) e_bias = a.bias[n];
+                if (a.residual) e_res = a.residual[(size_t)m * a.N + n];
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[c] = 0.0f;
+        if (trip_a < t1) consume(wa0, wa1, sa, trip_a);
+        if (trip_b < t1) consume(wb0, wb1, sb, trip_b);
+        preload(tile + gridDim.x);  // the next tile's loads fly during the reduction below
+        // the two chunks of a trip sit in lane groups q and q ^ 1
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[c] += __shfl_xor(acc[c], 16, kWave);
+        __syncthreads();  // the previous tile's readers of red are done
+        if ((q & 1) == 0 && d_ok)
+            *reinterpret_cast<float4 *>(red + (wave * MT + d_m) * COLS + cg * 4) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+        __syncthreads();
+        if (ksplit == 1) {
+            for (int i = tid; i < n_out; i += T) {
+                const int m = i / COLS, n = tile * COLS + (i - m * COLS);
+                if (m < a.M && n < a.N) {
+                    float v = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < 16; ++w) v += red[w * n_out + i];
+                    if (i != tid) {
+                        e_bias = a.bias ? a.bias[n] : 0.0f;
+                        e_res = a.residual ? a.residual[(size_t)m * a.N + n] : 0.0f;
+                    }
+                    finish_output(a, v, e_bias, e_res, m, n);
+                }
+            }
+            continue;
+        }
+        for (int i = tid; i < n_out; i += T) {
+            const int m = i / COLS, n = tile * COLS + (i - m * COLS);
+            if (m < a.M && n < a.N) {
+                float v = 0.0f;
+#pragma unroll
+                for (int w = 0; w < 16; ++w) v += red[w * n_out + i];
+                __hip_atomic_store(&p.partial[((size_t)split * a.M + m) * a.N + n], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned int t = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_last = (t == (unsigned int)(ksplit - 1));
+        }
+        __syncthreads();
+        if (!s_last) continue;  // uniform over the workgroup
+        for (int i = tid; i < n_out; i += T) {
+            const int m = i / COLS, n = tile * COLS + (i - m * COLS);
+            if (m < a.M && n < a.N) {
+                const float *src = p.partial + (size_t)m * a.N + n;
+                const size_t stride = (size_t)a.M * a.N;
+                float t = 0.0f;
+                for (int sp0 = 0; sp0 < ksplit; sp0 += 8) {  // 8 loads in flight, summed in split order
+                    float part[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+                        part[u] = sp0 + u < ksplit
+                                      ? __hip_atomic_load(src + (size_t)(sp0 + u) * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                      : 0.0f;
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+                        if (sp0 + u < ksplit) t += part[u];
+                }
+                if (i != tid) {
+                    e_bias = a.bias ? a.bias[n] : 0.0f;
+                    e_res = a.residual ? a.residual[(size_t)m * a.N + n] : 0.0f;
+                }
+                finish_output(a, t, e_bias, e_res, m, n);
+            }
+        }
+        if (tid == 0) __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+}  // namespace
+
+bool agpu_int4_gemv_i8_supported(const GemvArgs &a) {
+    return a.M >= 1 && a.M <= 2 && a.group % 32 == 0 && a.K % 64 == 0 && a.N % 4 == 0 &&
+           (((uintptr_t)a.packed | (uintptr_t)a.scales | (uintptr_t)a.x | (uintptr_t)a.ln_gamma | (uintptr_t)a.ln_beta) % 16 == 0) &&
+           (!a.ln_gamma || (agpu_int4_gemv_can_fuse_ln(a.M, a.K) && a.K <= 8192));
+}
+
+int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips_per_split, int max_wgs) {
+    I8Params p{};
+    p.a = a;
+    const int MT = a.M <= 1 ? 1 : 2;
+    const int trips_total = a.K / 64;
+    const int col_blocks = ceil_div(a.N, 64);
+    if (col_blocks > kNumCounters) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_gemv: N=%d too large", a.N);
+    int tps_max = max_trips_per_split < 1 ? 1 : (max_trips_per_split > 32 ? 32 : max_trips_per_split);  // 2 trips x 16 waves
+    auto stage_bytes = [&](int tps) {
+        return (size_t)MT * tps * 256 + sizeof(float) * (size_t)MT * ((2 * tps + 3) & ~3);
+    };
+    int ksplit = ceil_div(trips_total, tps_max);
+    const int tps = ceil_div(trips_total, ksplit);
+    ksplit = ceil_div(trips_total, tps);
+    if ((size_t)ksplit * a.M * a.N * sizeof(float) > kWorkspaceBytes / 2)
+        return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_gemv: split-K partials exceed the workspace (M=%d N=%d K=%d)", a.M, a.N, a.K);
+    int W = tps <= 16 ? tps : ceil_div(tps, 2);
+    if (a.ln_gamma && W < ceil_div(a.K, 512)) W = ceil_div(a.K, 512);  // one thread per packed row of the whole x row
+    if (W > 16) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "int4_gemv: K=%d too large for the fused LayerNorm", a.K);
+    p.trips_per_split = tps;
+    p.col_blocks = col_blocks;
+    p.partial = reinterpret_cast<float *>(ctx->workspace);
+    p.counters = ctx->counters;
+    const size_t lds = stage_bytes(tps) + sizeof(float) * (size_t)16 * MT * 64;
+    int gx = col_blocks;
+    const int cap = max_wgs > 0 ? max_wgs : ctx->num_cus;
+    if (gx * ksplit > cap) gx = cap / ksplit > 0 ? cap / ksplit : 1;
+    const dim3 grid(gx, ksplit), block(64 * W);
+    if (a.ln_gamma) {
+        if (MT == 1) hipLaunchKernelGGL((int4_gemv_i8_kernel<1, true>), grid, block, lds, ctx->stream, p);
+        else hipLaunchKernelGGL((int4_gemv_i8_kernel<2, true>), grid, block, lds, ctx->stream, p);
+    } else {
+        if (MT == 1) hipLaunchKernelGGL((int4_gemv_i8_kernel<1, false>), grid, block, lds, ctx->stream, p);
+        else hipLaunchKernelGGL((int4_gemv_i8_kernel<2, false>), grid, block, lds, ctx->stream, p);
+    }
+    return AGPU_LAUNCH_CHECK(ctx, "int4_gemv_i8_kernel");
+}

@@ -241,8 +241,8 @@ AGPU_EXPORT int32_t agpu_ln_int4_linear(agpu_ctx *ctx, const float *x, const flo
         GemvArgs a{};
         a.x = xin; a.packed = packed; a.scales = scales; a.bias = bias; a.residual = residual; a.y = y;
         a.ln_gamma = gamma; a.ln_beta = beta; a.ln_eps = eps;
-        a.M = M; a.N = N; a.K = K; a.group = group; a.flags = epi;
-        if (agpu_int4_skinny_supported(a)) return agpu_int4_skinny_launch(ctx, a);
+        a.M = M; a.N = N; a.K = K; a.group = group; a.flags = epi | (flags & AGPU_EPI_FORCE_FP32_GEMV);
+        if (!(flags & AGPU_EPI_FORCE_FP32_GEMV) && agpu_int4_skinny_supported(a)) return agpu_int4_skinny_launch(ctx, a);
         return agpu_int4_gemv_launch(ctx, a);
     }
     const dim3 grid(ceil_div(N, GEMM_BN), ceil_div(M, GEMM_BM));

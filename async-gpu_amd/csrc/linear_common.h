@@ -68,6 +68,9 @@ __device__ __forceinline__ void finish_output(const GemvArgs &a, float v, float 
 }
 
 int32_t agpu_int4_gemv_launch(agpu_ctx *ctx, const GemvArgs &a);
+// int8-MFMA variant for M <= 2 (needs group % 32 == 0, K % 64 == 0, N % 4 == 0, 16-byte aligned weights).
+bool agpu_int4_gemv_i8_supported(const GemvArgs &a);
+int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips_per_split, int max_wgs);
 // MFMA variant for 4 < M <= 16 (needs group % 32 == 0, K % 32 == 0, N % 4 == 0, 16-byte aligned weights).
 bool agpu_int4_skinny_supported(const GemvArgs &a);
 int32_t agpu_int4_skinny_launch(agpu_ctx *ctx, const GemvArgs &a);

@@ -81,6 +81,70 @@ def test_gemv_shapes(agpu, orc, dev, M, K, N, g):
     assert np.abs(y.cpu().numpy() - ref).max() <= TOL_LINEAR
 
 
+@pytest.mark.parametrize("M", [1, 2, 8, 16])
+@pytest.mark.parametrize("K,N,g", [(768, 2304, 32), (3072, 768, 32), (768, 768, 128), (1600, 6400, 32), (64, 70, 16)])
+def test_gemv_fp32_valu_kernel(agpu, orc, dev, M, K, N, g):
+    """The fp32 VALU GEMV stays reachable (it serves the shapes the matrix-core kernels do not take)."""
+    from async_gpu_amd import ops, workloads
+    rng = np.random.default_rng(M * 77 + K + N)
+    packed, scales, bias = workloads.random_int4_linear(rng, K, N, g, bias=True)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    y = ops.int4_linear(to_dev(x, dev), to_dev(packed, dev), to_dev(scales, dev), bias=to_dev(bias, dev), group=g,
+                        flags=agpu._lib.EPI_FORCE_FP32_GEMV)
+    assert np.abs(y.cpu().numpy() - orc.int4_gemm_f64(x, packed, scales, g, bias=bias)).max() <= TOL_LINEAR
+
+
+@pytest.mark.parametrize("M", [1, 2])
+@pytest.mark.parametrize("K,N,g", [(64, 4, 32), (64, 68, 64), (128, 132, 32), (768, 2304, 64), (6400, 1600, 32),
+                                   (3072, 768, 128), (4096, 260, 32), (1600, 4800, 32)])
+def test_gemv_int8_matrix_core_shapes(agpu, orc, dev, M, K, N, g):
+    """M <= 2, group % 32 == 0, K % 64 == 0, N % 4 == 0: fixed-point x on the int8 matrix cores.  One trip,
+    ragged last column tile, two trips per wave, split K, groups spanning several 32-k chunks."""
+    from async_gpu_amd import ops, workloads
+    rng = np.random.default_rng(M * 31 + K + N + g)
+    packed, scales, bias = workloads.random_int4_linear(rng, K, N, g, bias=True)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    y = ops.int4_linear(to_dev(x, dev), to_dev(packed, dev), to_dev(scales, dev), bias=to_dev(bias, dev),
+                        residual=to_dev(res, dev), group=g)
+    ref = orc.int4_gemm_f64(x, packed, scales, g, bias=bias) + res
+    assert np.abs(y.cpu().numpy() - ref).max() <= TOL_LINEAR
+
+
+def test_gemv_int8_fixed_point_ranges(agpu, orc, dev):
+    """The fixed-point scale follows max|x| of the row: wide dynamic range, tiny and huge rows, an all-zero
+    row, and the extreme nibbles 0 and 15 everywhere keep the relative error at fp32 level; NaN poisons its row."""
+    from async_gpu_amd import ops, workloads
+    rng = np.random.default_rng(12)
+    K, N, g = 768, 256, 32
+    packed, scales, _ = workloads.random_int4_linear(rng, K, N, g)
+    packed[::2] = 0xFFFFFFFF  # nibble 15 -> +7
+    packed[1::2] = 0x00000000  # nibble 0 -> -8
+    dp, ds = to_dev(packed, dev), to_dev(scales, dev)
+    base = rng.standard_normal((2, K)).astype(np.float32)
+    cases = {
+        "wide range": base * np.exp(rng.uniform(-12, 4, (2, K))).astype(np.float32),
+        "tiny": base * np.float32(1e-20),
+        "below the fixed-point floor (2^-97 per element)": base * np.float32(1e-33),
+        "huge": base * np.float32(1e30),
+        "one spike": np.where(np.arange(K) == 5, np.float32(3e4), base).astype(np.float32),
+        "zero row": np.stack([np.zeros(K, np.float32), base[1]]),
+    }
+    for name, x in cases.items():
+        y = ops.int4_linear(to_dev(x, dev), dp, ds, group=g).cpu().numpy()
+        ref = orc.int4_gemm_f64(x, packed, scales, g)
+        bound = np.abs(x).astype(np.float64) @ np.abs(orc.int4_dequantize(packed, scales, g)).astype(np.float64)
+        err = np.abs(y - ref)
+        assert np.all(err <= 4e-7 * bound + 1e-27), (name, float((err / (bound + 1e-300)).max()))
+    x = base.copy()
+    x[0, 100] = np.nan
+    y = ops.int4_linear(to_dev(x, dev), dp, ds, group=g).cpu().numpy()
+    assert np.isnan(y[0]).all() and np.abs(y[1] - orc.int4_gemm_f64(x[1:], packed, scales, g)[0]).max() <= TOL_LINEAR
+    x[0, 100] = np.inf
+    y = ops.int4_linear(to_dev(x, dev), dp, ds, group=g).cpu().numpy()
+    assert not np.isfinite(y[0]).any() and np.isfinite(y[1]).all()
+
+
 @pytest.mark.parametrize("M", [128, 512, 1024, 17, 100])
 def test_config2_gemm(agpu, orc, dev, M):
     """BASELINE config 2: K=768, N=2304, group 32, seed 1, M in {128, 512, 1024} (+ ragged M)."""
