@@ -59,23 +59,53 @@ inline int32_t agpu_hip(agpu_ctx *ctx, hipError_t e, const char *what) {
 
 // ---- device helpers ---------------------------------------------------------------
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+// Cross-lane moves as DPP modifiers of ordinary VALU instructions (a few cycles each; a ds_bpermute
+// round trip through the LDS crossbar costs on the order of a hundred).
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float old, float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, v), CTRL,
+                                                                 ROW_MASK, 0xf, false));
+}
+
+// Sum / maximum over each row of 16 lanes, result in every lane of the row.
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_move<0xb1, 0xf>(0.0f, v);   // quad_perm [1,0,3,2]
+    v += dpp_move<0x4e, 0xf>(0.0f, v);   // quad_perm [2,3,0,1]
+    v += dpp_move<0x124, 0xf>(0.0f, v);  // row_ror:4
+    v += dpp_move<0x128, 0xf>(0.0f, v);  // row_ror:8
     return v;
+}
+
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_move<0xb1, 0xf>(v, v));
+    v = fmaxf(v, dpp_move<0x4e, 0xf>(v, v));
+    v = fmaxf(v, dpp_move<0x124, 0xf>(v, v));
+    v = fmaxf(v, dpp_move<0x128, 0xf>(v, v));
+    return v;
+}
+
+// Sum / maximum over the 64 lanes, result in every lane: rows of 16 first, then row_bcast:15 into rows 1
+// and 3 and row_bcast:31 into rows 2 and 3 leave the total in lane 63.  The order of additions is fixed.
+__device__ __forceinline__ float wave_sum(float v) {
+    v = row16_sum(v);
+    v += dpp_move<0x142, 0xa>(0.0f, v);
+    v += dpp_move<0x143, 0xc>(0.0f, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-    return v;
+    v = row16_max(v);
+    v = fmaxf(v, dpp_move<0x142, 0xa>(v, v));
+    v = fmaxf(v, dpp_move<0x143, 0xc>(v, v));
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
-// tanh GELU, 0.5x(1+tanh(c(x+0.044715x^3))); accurate tanhf, no fast-math.
+// tanh GELU, 0.5x(1+tanh(c(x+0.044715x^3))), accurate expf, no fast-math.
 __device__ __forceinline__ float gelu_tanh_dev(float x) {
+    // 0.5 * (1 + tanh(u)) == 1 / (1 + exp(-2u)): one exp and one division instead of a tanh expansion
     const float c = 0.7978845608028654f, k = 0.044715f;
     const float inner = c * (x + k * x * x * x);
-    return 0.5f * x * (1.0f + tanhf(inner));
+    return x / (1.0f + expf(-2.0f * inner));
 }
 
 __device__ __forceinline__ float gelu_quick_dev(float x) { return x / (1.0f + expf(-1.702f * x)); }

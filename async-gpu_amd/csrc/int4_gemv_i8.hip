@@ -38,6 +38,7 @@ struct I8Params {
     GemvArgs a;
     int trips_per_split;  // 64-k trips per workgroup, at most 2 per wave
     int col_blocks;       // tiles of 64 columns
+    int chunk_shift;      // log2(group / 32): 32-k chunk index >> chunk_shift = scale row
     float *partial;       // [ksplit, M, N]
     unsigned int *counters;
 };
@@ -56,18 +57,14 @@ __device__ __forceinline__ void block_reduce(float (&v)[N], float *scratch, int 
     __syncthreads();
 #pragma unroll
     for (int n = 0; n < N; ++n) {
-        float t = scratch[n * 16 + (lane & 15)];
-#pragma unroll
-        for (int off = 8; off > 0; off >>= 1) {
-            const float o = __shfl_xor(t, off, kWave);
-            t = MAX ? fmaxf(t, o) : t + o;
-        }
+        const float t0 = scratch[n * 16 + (lane & 15)];
+        const float t = MAX ? row16_max(t0) : row16_sum(t0);
         v[n] = t;
     }
 }
 
-// LDS: xd bytes [MT][tps][4 digits][4 q][16] | xsum float [MT][2 * tps rounded up to 4] | red float [16][MT][64]
-// (rows >= W of red stay zero).  x never goes through LDS as floats: thread r owns packed row r (8 values) of
+// LDS: xd bytes [MT][tps][4 digits][4 q][16] | xsum float [MT][2 * tps rounded up to 4] | red float [32][MT][64]
+// (rows >= 2 W of red stay zero).  x never goes through LDS as floats: thread r owns packed row r (8 values) of
 // every x row in registers through LayerNorm, the fixed-point conversion and the chunk sums.
 template <int MT, bool LN>
 __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
@@ -91,19 +88,21 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
 
     uint4 wa0, wa1, wb0, wb1;  // rows 2q, 2q+1 of trips a and b
     float4 sa, sb;             // scales of chunk q % 2 of trips a and b
+    // Loads are unconditional (an out-of-range trip or column reads a valid address and is zeroed afterwards),
+    // which keeps the code short: the instruction cache is cold at every launch.
     auto load_trip = [&](int trip, bool ok, uint4 &w0, uint4 &w1, float4 &sc, int c0) {
-        w0 = w1 = make_uint4(0u, 0u, 0u, 0u);
-        sc = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (ok && trip < t1) {
-            const uint32_t *src = a.packed + (size_t)(8 * trip + 2 * q) * a.N + c0;
-            w0 = *reinterpret_cast<const uint4 *>(src);
-            w1 = *reinterpret_cast<const uint4 *>(src + a.N);
-            sc = *reinterpret_cast<const float4 *>(a.scales + (size_t)((64 * trip + 32 * (q & 1)) / a.group) * a.N + c0);
-        }
+        ok = ok && trip < t1;
+        const int tr = trip < t1 ? trip : t0;
+        const uint32_t *src = a.packed + (size_t)(8 * tr + 2 * q) * a.N + c0;
+        w0 = *reinterpret_cast<const uint4 *>(src);
+        w1 = *reinterpret_cast<const uint4 *>(src + a.N);
+        sc = *reinterpret_cast<const float4 *>(a.scales + (size_t)((2 * tr + (q & 1)) >> p.chunk_shift) * a.N + c0);
+        if (!ok) sc = make_float4(0.f, 0.f, 0.f, 0.f);  // the weights then do not matter
     };
     auto preload = [&](int tile) {
-        const int c0 = tile * COLS + cg * 4;
-        const bool ok = tile < p.col_blocks && c0 < a.N;
+        const int c_raw = tile * COLS + cg * 4;
+        const bool ok = tile < p.col_blocks && c_raw < a.N;
+        const int c0 = ok ? c_raw : 0;
         load_trip(trip_a, ok, wa0, wa1, sa, c0);
         load_trip(trip_b, ok, wb0, wb1, sb, c0);
     };
@@ -132,7 +131,7 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
         if (tid >= W)
             for (int j = 0; j < 3 * MT; ++j) (&s_scratch[0][0])[j * 16 + tid] = 0.0f;
     }
-    for (int i = W * n_out + tid; i < 16 * n_out; i += T) red[i] = 0.0f;
+    for (int i = 2 * W * n_out + tid; i < 32 * n_out; i += T) red[i] = 0.0f;
     if constexpr (LN) {
         float g8[8], b8[8];
         {
@@ -187,30 +186,36 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
     float c0m[MT], c1m[MT];
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
-        int e = 0;
-        (void)frexpf(amax[m], &e);  // amax < 2^e
+        // amax < 2^e with e from the exponent field (a denormal amax gives e = -126; s is capped anyway)
+        const int e = (int)((__float_as_uint(amax[m]) >> 23) & 0xffu) - 126;
         int s = 30 - e;
         s = s > 96 ? 96 : s;
         const bool finite = amax[m] <= 3.0e38f;
-        const float up = finite ? ldexpf(1.0f, s) : 0.0f;
-        c0m[m] = finite ? ldexpf(1.0f, -s) : __builtin_nanf("");
-        c1m[m] = finite ? ldexpf(1.0f, 16 - s) : __builtin_nanf("");
-        // this thread's row: two 32-bit words (even / odd nibbles) per digit plane, and its part of the chunk sum
-        uint32_t dg[4][2] = {{0u, 0u}, {0u, 0u}, {0u, 0u}, {0u, 0u}};
+        const float up = finite ? __uint_as_float((uint32_t)(127 + s) << 23) : 0.0f;
+        c0m[m] = finite ? __uint_as_float((uint32_t)(127 - s) << 23) : __builtin_nanf("");
+        c1m[m] = finite ? __uint_as_float((uint32_t)(143 - s) << 23) : __builtin_nanf("");
+        // Digits: with u = X + 0x00808080 the low three bytes of u ^ 0x00808080 are the signed digits
+        // D_0..D_2 (each byte of u is D_i + 128) and the top byte is D_3.  A 4x4 byte transpose then gives,
+        // per digit plane, the word of the even and of the odd nibbles of this thread's row.
+        uint32_t dw[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            int v = __float2int_rn(xv[m][j] * up);
+        for (int j = 0; j < 8; ++j) dw[j] = ((uint32_t)__float2int_rn(xv[m][j] * up) + 0x00808080u) ^ 0x00808080u;
+        uint32_t dg[4][2];
 #pragma unroll
-            for (int d = 0; d < 3; ++d) {
-                const int lo = (int)(signed char)(v & 0xff);
-                dg[d][j & 1] |= (uint32_t)(lo & 0xff) << (8 * (j >> 1));
-                v = (v - lo) >> 8;
-            }
-            dg[3][j & 1] |= (uint32_t)(v & 0xff) << (8 * (j >> 1));
+        for (int par = 0; par < 2; ++par) {
+            const uint32_t A = dw[par], B = dw[par + 2], Cw = dw[par + 4], Dw = dw[par + 6];
+            const uint32_t ab_lo = __builtin_amdgcn_perm(B, A, 0x05010400u);   // A0 B0 A1 B1
+            const uint32_t ab_hi = __builtin_amdgcn_perm(B, A, 0x07030602u);   // A2 B2 A3 B3
+            const uint32_t cd_lo = __builtin_amdgcn_perm(Dw, Cw, 0x05010400u);  // C0 D0 C1 D1
+            const uint32_t cd_hi = __builtin_amdgcn_perm(Dw, Cw, 0x07030602u);  // C2 D2 C3 D3
+            dg[0][par] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100u);  // A0 B0 C0 D0
+            dg[1][par] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302u);  // A1 B1 C1 D1
+            dg[2][par] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x05040100u);
+            dg[3][par] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302u);
         }
         float s8 = ((xv[m][0] + xv[m][1]) + (xv[m][2] + xv[m][3])) + ((xv[m][4] + xv[m][5]) + (xv[m][6] + xv[m][7]));
-        s8 += __shfl_xor(s8, 1, kWave);
-        s8 += __shfl_xor(s8, 2, kWave);  // 4 consecutive rows = one 32-k chunk
+        s8 += dpp_move<0xb1, 0xf>(0.0f, s8);
+        s8 += dpp_move<0x4e, 0xf>(0.0f, s8);  // 4 consecutive rows = one 32-k chunk
         if (in_slice) {
             const int rl = row - 8 * t0, tl = rl >> 3, rr = rl & 7;
             unsigned char *dst = xd + ((size_t)(m * tps + tl) * 4) * 64 + 16 * (rr >> 1) + 8 * (rr & 1);
@@ -268,62 +273,51 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
         if (trip_a < t1) consume(wa0, wa1, sa, trip_a);
         if (trip_b < t1) consume(wb0, wb1, sb, trip_b);
         preload(tile + gridDim.x);  // the next tile's loads fly during the reduction below
-        // the two chunks of a trip sit in lane groups q and q ^ 1
-#pragma unroll
-        for (int c = 0; c < 4; ++c) acc[c] += __shfl_xor(acc[c], 16, kWave);
+        // lane groups q = 0, 1 (2, 3 for the second x row) hold the two chunks of a trip: 32 rows of red
         __syncthreads();  // the previous tile's readers of red are done
-        if ((q & 1) == 0 && d_ok)
-            *reinterpret_cast<float4 *>(red + (wave * MT + d_m) * COLS + cg * 4) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+        if (d_ok)
+            *reinterpret_cast<float4 *>(red + ((wave * 2 + (q & 1)) * MT + d_m) * COLS + cg * 4) =
+                make_float4(acc[0], acc[1], acc[2], acc[3]);
         __syncthreads();
-        if (ksplit == 1) {
+        if (ksplit > 1) {
+            // publish this workgroup's partial sums past the L2, then take a ticket
             for (int i = tid; i < n_out; i += T) {
                 const int m = i / COLS, n = tile * COLS + (i - m * COLS);
                 if (m < a.M && n < a.N) {
                     float v = 0.0f;
 #pragma unroll
-                    for (int w = 0; w < 16; ++w) v += red[w * n_out + i];
-                    if (i != tid) {
-                        e_bias = a.bias ? a.bias[n] : 0.0f;
-                        e_res = a.residual ? a.residual[(size_t)m * a.N + n] : 0.0f;
-                    }
-                    finish_output(a, v, e_bias, e_res, m, n);
+                    for (int w = 0; w < 32; ++w) v += red[w * n_out + i];
+                    __hip_atomic_store(&p.partial[((size_t)split * a.M + m) * a.N + n], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
-            continue;
-        }
-        for (int i = tid; i < n_out; i += T) {
-            const int m = i / COLS, n = tile * COLS + (i - m * COLS);
-            if (m < a.M && n < a.N) {
-                float v = 0.0f;
-#pragma unroll
-                for (int w = 0; w < 16; ++w) v += red[w * n_out + i];
-                __hip_atomic_store(&p.partial[((size_t)split * a.M + m) * a.N + n], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (tid == 0) {
+                const unsigned int t = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                s_last = (t == (unsigned int)(ksplit - 1));
             }
+            __syncthreads();
+            if (!s_last) continue;  // uniform over the workgroup
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (tid == 0) {
-            const unsigned int t = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            s_last = (t == (unsigned int)(ksplit - 1));
-        }
-        __syncthreads();
-        if (!s_last) continue;  // uniform over the workgroup
         for (int i = tid; i < n_out; i += T) {
             const int m = i / COLS, n = tile * COLS + (i - m * COLS);
             if (m < a.M && n < a.N) {
-                const float *src = p.partial + (size_t)m * a.N + n;
-                const size_t stride = (size_t)a.M * a.N;
                 float t = 0.0f;
-                for (int sp0 = 0; sp0 < ksplit; sp0 += 8) {  // 8 loads in flight, summed in split order
-                    float part[8];
+                if (ksplit == 1) {
 #pragma unroll
-                    for (int u = 0; u < 8; ++u)
-                        part[u] = sp0 + u < ksplit
-                                      ? __hip_atomic_load(src + (size_t)(sp0 + u) * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                                      : 0.0f;
+                    for (int w = 0; w < 32; ++w) t += red[w * n_out + i];
+                } else {
+                    const float *src = p.partial + (size_t)m * a.N + n;
+                    const size_t stride = (size_t)a.M * a.N;
+                    for (int sp0 = 0; sp0 < ksplit; sp0 += 4) {  // 4 loads in flight, summed in split order
+                        float part[4];
 #pragma unroll
-                    for (int u = 0; u < 8; ++u)
-                        if (sp0 + u < ksplit) t += part[u];
+                        for (int u = 0; u < 4; ++u)
+                            part[u] = __hip_atomic_load(src + (size_t)(sp0 + u < ksplit ? sp0 + u : 0) * stride, __ATOMIC_RELAXED,
+                                                        __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) t += sp0 + u < ksplit ? part[u] : 0.0f;
+                    }
                 }
                 if (i != tid) {
                     e_bias = a.bias ? a.bias[n] : 0.0f;
@@ -332,6 +326,7 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
                 finish_output(a, t, e_bias, e_res, m, n);
             }
         }
+        if (ksplit == 1) continue;
         if (tid == 0) __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
@@ -339,7 +334,7 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
 }  // namespace
 
 bool agpu_int4_gemv_i8_supported(const GemvArgs &a) {
-    return a.M >= 1 && a.M <= 2 && a.group % 32 == 0 && a.K % 64 == 0 && a.N % 4 == 0 &&
+    return a.M >= 1 && a.M <= 2 && a.group % 32 == 0 && ((a.group / 32) & (a.group / 32 - 1)) == 0 && a.K % 64 == 0 && a.N % 4 == 0 &&
            (((uintptr_t)a.packed | (uintptr_t)a.scales | (uintptr_t)a.x | (uintptr_t)a.ln_gamma | (uintptr_t)a.ln_beta) % 16 == 0) &&
            (!a.ln_gamma || (agpu_int4_gemv_can_fuse_ln(a.M, a.K) && a.K <= 8192));
 }
@@ -364,10 +359,11 @@ int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips
     if (a.ln_gamma && W < ceil_div(a.K, 512)) W = ceil_div(a.K, 512);  // one thread per packed row of the whole x row
     if (W > 16) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "int4_gemv: K=%d too large for the fused LayerNorm", a.K);
     p.trips_per_split = tps;
+    p.chunk_shift = __builtin_ctz((unsigned)(a.group / 32));
     p.col_blocks = col_blocks;
     p.partial = reinterpret_cast<float *>(ctx->workspace);
     p.counters = ctx->counters;
-    const size_t lds = stage_bytes(tps) + sizeof(float) * (size_t)16 * MT * 64;
+    const size_t lds = stage_bytes(tps) + sizeof(float) * (size_t)32 * MT * 64;
     int gx = col_blocks;
     const int cap = max_wgs > 0 ? max_wgs : ctx->num_cus;
     if (gx * ksplit > cap) gx = cap / ksplit > 0 ? cap / ksplit : 1;
