@@ -33,11 +33,13 @@
 namespace {
 
 typedef int intx4 __attribute__((ext_vector_type(4)));
+constexpr int kMaxTilesPerPass = 4;
 
 struct I8Params {
     GemvArgs a;
     int trips_per_split;  // 64-k trips per workgroup, at most 2 per wave
     int col_blocks;       // tiles of 64 columns
+    int tiles_per_pass;   // tiles a workgroup reduces together, <= kMaxTilesPerPass
     int chunk_shift;      // log2(group / 32): 32-k chunk index >> chunk_shift = scale row
     float *partial;       // [ksplit, M, N]
     unsigned int *counters;
@@ -63,14 +65,14 @@ __device__ __forceinline__ void block_reduce(float (&v)[N], float *scratch, int 
     }
 }
 
-// LDS: xd bytes [MT][tps][4 digits][4 q][16] | xsum float [MT][2 * tps rounded up to 4] | red float [32][MT][64]
-// (rows >= 2 W of red stay zero).  x never goes through LDS as floats: thread r owns packed row r (8 values) of
+// LDS: xd bytes [MT][tps][4 digits][4 q][16] | xsum float [MT][2 * tps rounded up to 4] | red float [tiles_per_pass][32][MT][64]
+// (rows >= 2 W of every region of red stay zero).  x never goes through LDS as floats: thread r owns packed row r (8 values) of
 // every x row in registers through LayerNorm, the fixed-point conversion and the chunk sums.
 template <int MT, bool LN>
 __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
     extern __shared__ __align__(16) float smem[];
     __shared__ float s_scratch[3][MT * 16];
-    __shared__ int s_last;
+    __shared__ int s_last[kMaxTilesPerPass];
     const GemvArgs &a = p.a;
     constexpr int COLS = 64;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6, T = blockDim.x;
@@ -131,7 +133,8 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
         if (tid >= W)
             for (int j = 0; j < 3 * MT; ++j) (&s_scratch[0][0])[j * 16 + tid] = 0.0f;
     }
-    for (int i = 2 * W * n_out + tid; i < 32 * n_out; i += T) red[i] = 0.0f;
+    for (int i = tid; i < p.tiles_per_pass * 32 * n_out; i += T)
+        if ((i % (32 * n_out)) >= 2 * W * n_out) red[i] = 0.0f;
     if constexpr (LN) {
         float g8[8], b8[8];
         {
@@ -259,53 +262,65 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
         }
     };
 
-    for (int tile = blockIdx.x; tile < p.col_blocks; tile += gridDim.x) {
-        float e_bias = 0.0f, e_res = 0.0f;  // epilogue operands of this thread's output element, fetched early
-        {
-            const int m = tid / COLS, n = tile * COLS + (tid - m * COLS);
-            if (tid < n_out && m < a.M && n < a.N) {
+    // Tiles blockIdx.x, blockIdx.x + gridDim.x, ... in passes of up to p.tiles_per_pass: the waves leave their
+    // sums for tile j of the pass in region j of red, and one pair of barriers serves the whole pass.
+    constexpr int region = 32 * n_out;
+    const int my_tiles = blockIdx.x < p.col_blocks ? (p.col_blocks - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
+    for (int first = 0; first < my_tiles; first += p.tiles_per_pass) {
+        const int nt = min(p.tiles_per_pass, my_tiles - first);
+        // epilogue operands of this thread's first output element of the pass, fetched early
+        float e_bias = 0.0f, e_res = 0.0f;
+        if (tid < nt * n_out) {
+            const int j = tid / n_out, i = tid - j * n_out;
+            const int m = i / COLS, n = (blockIdx.x + (first + j) * gridDim.x) * COLS + (i - m * COLS);
+            if (m < a.M && n < a.N) {
                 if (a.bias) e_bias = a.bias[n];
                 if (a.residual) e_res = a.residual[(size_t)m * a.N + n];
             }
         }
+        for (int j = 0; j < nt; ++j) {
+            const int tile = blockIdx.x + (first + j) * gridDim.x;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) acc[c] = 0.0f;
-        if (trip_a < t1) consume(wa0, wa1, sa, trip_a);
-        if (trip_b < t1) consume(wb0, wb1, sb, trip_b);
-        preload(tile + gridDim.x);  // the next tile's loads fly during the reduction below
-        // lane groups q = 0, 1 (2, 3 for the second x row) hold the two chunks of a trip: 32 rows of red
-        __syncthreads();  // the previous tile's readers of red are done
-        if (d_ok)
-            *reinterpret_cast<float4 *>(red + ((wave * 2 + (q & 1)) * MT + d_m) * COLS + cg * 4) =
-                make_float4(acc[0], acc[1], acc[2], acc[3]);
+            for (int c = 0; c < 4; ++c) acc[c] = 0.0f;
+            if (trip_a < t1) consume(wa0, wa1, sa, trip_a);
+            if (trip_b < t1) consume(wb0, wb1, sb, trip_b);
+            if (first + j + 1 < my_tiles) preload(tile + gridDim.x);  // the next tile's loads fly meanwhile
+            // lane groups q = 0, 1 (2, 3 for the second x row) hold the two chunks of a trip: 32 rows per region
+            if (d_ok)
+                *reinterpret_cast<float4 *>(red + j * region + ((wave * 2 + (q & 1)) * MT + d_m) * COLS + cg * 4) =
+                    make_float4(acc[0], acc[1], acc[2], acc[3]);
+        }
         __syncthreads();
         if (ksplit > 1) {
-            // publish this workgroup's partial sums past the L2, then take a ticket
-            for (int i = tid; i < n_out; i += T) {
-                const int m = i / COLS, n = tile * COLS + (i - m * COLS);
+            // publish this workgroup's partial sums past the L2, then take one ticket per tile
+            for (int idx = tid; idx < nt * n_out; idx += T) {
+                const int j = idx / n_out, i = idx - j * n_out;
+                const int m = i / COLS, n = (blockIdx.x + (first + j) * gridDim.x) * COLS + (i - m * COLS);
                 if (m < a.M && n < a.N) {
                     float v = 0.0f;
 #pragma unroll
-                    for (int w = 0; w < 32; ++w) v += red[w * n_out + i];
+                    for (int w = 0; w < 32; ++w) v += red[j * region + w * n_out + i];
                     __hip_atomic_store(&p.partial[((size_t)split * a.M + m) * a.N + n], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
-            if (tid == 0) {
+            if (tid < nt) {
+                const int tile = blockIdx.x + (first + tid) * gridDim.x;
                 const unsigned int t = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                s_last = (t == (unsigned int)(ksplit - 1));
+                s_last[tid] = (t == (unsigned int)(ksplit - 1));
+                if (s_last[tid]) __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
             __syncthreads();
-            if (!s_last) continue;  // uniform over the workgroup
         }
-        for (int i = tid; i < n_out; i += T) {
-            const int m = i / COLS, n = tile * COLS + (i - m * COLS);
-            if (m < a.M && n < a.N) {
+        for (int idx = tid; idx < nt * n_out; idx += T) {
+            const int j = idx / n_out, i = idx - j * n_out;
+            const int m = i / COLS, n = (blockIdx.x + (first + j) * gridDim.x) * COLS + (i - m * COLS);
+            if (m < a.M && n < a.N && (ksplit == 1 || s_last[j])) {
                 float t = 0.0f;
                 if (ksplit == 1) {
 #pragma unroll
-                    for (int w = 0; w < 32; ++w) t += red[w * n_out + i];
+                    for (int w = 0; w < 32; ++w) t += red[j * region + w * n_out + i];
                 } else {
                     const float *src = p.partial + (size_t)m * a.N + n;
                     const size_t stride = (size_t)a.M * a.N;
@@ -319,15 +334,14 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
                         for (int u = 0; u < 4; ++u) t += sp0 + u < ksplit ? part[u] : 0.0f;
                     }
                 }
-                if (i != tid) {
+                if (idx != tid) {
                     e_bias = a.bias ? a.bias[n] : 0.0f;
                     e_res = a.residual ? a.residual[(size_t)m * a.N + n] : 0.0f;
                 }
                 finish_output(a, t, e_bias, e_res, m, n);
             }
         }
-        if (ksplit == 1) continue;
-        if (tid == 0) __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (first + nt < my_tiles) __syncthreads();  // the next pass reuses red and s_last
     }
 }
 
@@ -363,10 +377,14 @@ int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips
     p.col_blocks = col_blocks;
     p.partial = reinterpret_cast<float *>(ctx->workspace);
     p.counters = ctx->counters;
-    const size_t lds = stage_bytes(tps) + sizeof(float) * (size_t)32 * MT * 64;
     int gx = col_blocks;
     const int cap = max_wgs > 0 ? max_wgs : ctx->num_cus;
     if (gx * ksplit > cap) gx = cap / ksplit > 0 ? cap / ksplit : 1;
+    const int tiles_per_wg = ceil_div(col_blocks, gx);
+    p.tiles_per_pass = tiles_per_wg < kMaxTilesPerPass ? tiles_per_wg : kMaxTilesPerPass;
+    while (p.tiles_per_pass > 1 && stage_bytes(tps) + sizeof(float) * (size_t)p.tiles_per_pass * 32 * MT * 64 > 60 * 1024)
+        --p.tiles_per_pass;
+    const size_t lds = stage_bytes(tps) + sizeof(float) * (size_t)p.tiles_per_pass * 32 * MT * 64;
     const dim3 grid(gx, ksplit), block(64 * W);
     if (a.ln_gamma) {
         if (MT == 1) hipLaunchKernelGGL((int4_gemv_i8_kernel<1, true>), grid, block, lds, ctx->stream, p);
