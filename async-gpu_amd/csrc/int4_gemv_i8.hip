@@ -37,7 +37,8 @@ constexpr int kMaxTilesPerPass = 4;
 
 struct I8Params {
     GemvArgs a;
-    int trips_per_split;  // 64-k trips per workgroup, at most 2 per wave
+    int trips_per_split;  // 64-k trips per workgroup
+    int trips_per_wave;   // ceil(trips_per_split / waves), 1 or even
     int col_blocks;       // tiles of 64 columns
     int tiles_per_pass;   // tiles a workgroup reduces together, <= kMaxTilesPerPass
     int chunk_shift;      // log2(group / 32): 32-k chunk index >> chunk_shift = scale row
@@ -86,29 +87,30 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
     const int xsum_len = (2 * tps + 3) & ~3;
     float *red = xsum + MT * xsum_len;
     constexpr int n_out = MT * COLS;
-    const int trip_a = t0 + wave, trip_b = trip_a + W;
-
-    uint4 wa0, wa1, wb0, wb1;  // rows 2q, 2q+1 of trips a and b
-    float4 sa, sb;             // scales of chunk q % 2 of trips a and b
-    // Loads are unconditional (an out-of-range trip or column reads a valid address and is zeroed afterwards),
-    // which keeps the code short: the instruction cache is cold at every launch.
-    auto load_trip = [&](int trip, bool ok, uint4 &w0, uint4 &w1, float4 &sc, int c0) {
-        ok = ok && trip < t1;
-        const int tr = trip < t1 ? trip : t0;
-        const uint32_t *src = a.packed + (size_t)(8 * tr + 2 * q) * a.N + c0;
+    // A wave takes trips t0 + wave + k * W, k < p.trips_per_wave, of every tile.  Two register sets hold loads in
+    // flight: set a the even k, set b the odd k (trips_per_wave is 1 or even), each refilled right after use
+    // with the wave's next trip of that parity, which may belong to the next tile.
+    const int trip_a = t0 + wave;
+    const int ntw = p.trips_per_wave;
+    uint4 wa0, wa1, wb0, wb1;  // rows 2q, 2q+1 of a trip
+    float4 sa, sb;             // scales of chunk q % 2 of a trip
+    // Out-of-range columns read column 0 and get a zero scale (then the weights do not matter).
+    auto load_trip = [&](int tile, int k, uint4 &w0, uint4 &w1, float4 &sc) {
+        const int trip = trip_a + k * W;
+        if (tile >= p.col_blocks || trip >= t1) return;  // wave-uniform
+        const int c_raw = tile * COLS + cg * 4;
+        const bool ok = c_raw < a.N;
+        const int c0 = ok ? c_raw : 0;
+        const uint32_t *src = a.packed + (size_t)(8 * trip + 2 * q) * a.N + c0;
         w0 = *reinterpret_cast<const uint4 *>(src);
         w1 = *reinterpret_cast<const uint4 *>(src + a.N);
-        sc = *reinterpret_cast<const float4 *>(a.scales + (size_t)((2 * tr + (q & 1)) >> p.chunk_shift) * a.N + c0);
-        if (!ok) sc = make_float4(0.f, 0.f, 0.f, 0.f);  // the weights then do not matter
+        sc = *reinterpret_cast<const float4 *>(a.scales + (size_t)((2 * trip + (q & 1)) >> p.chunk_shift) * a.N + c0);
+        if (!ok) sc = make_float4(0.f, 0.f, 0.f, 0.f);
     };
-    auto preload = [&](int tile) {
-        const int c_raw = tile * COLS + cg * 4;
-        const bool ok = tile < p.col_blocks && c_raw < a.N;
-        const int c0 = ok ? c_raw : 0;
-        load_trip(trip_a, ok, wa0, wa1, sa, c0);
-        load_trip(trip_b, ok, wb0, wb1, sb, c0);
-    };
-    preload(blockIdx.x);
+    wa0 = wa1 = wb0 = wb1 = make_uint4(0u, 0u, 0u, 0u);
+    sa = sb = make_float4(0.f, 0.f, 0.f, 0.f);
+    load_trip(blockIdx.x, 0, wa0, wa1, sa);
+    if (ntw > 1) load_trip(blockIdx.x, 1, wb0, wb1, sb);
 
     // ---- x: packed row `row` of every x row into registers ----
     // With LayerNorm the statistics need the whole row of x, so thread r owns row r of all K / 8; otherwise
@@ -282,9 +284,16 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
             const int tile = blockIdx.x + (first + j) * gridDim.x;
 #pragma unroll
             for (int c = 0; c < 4; ++c) acc[c] = 0.0f;
-            if (trip_a < t1) consume(wa0, wa1, sa, trip_a);
-            if (trip_b < t1) consume(wb0, wb1, sb, trip_b);
-            if (first + j + 1 < my_tiles) preload(tile + gridDim.x);  // the next tile's loads fly meanwhile
+            for (int k = 0; k < ntw; k += 2) {
+                if (trip_a + k * W < t1) consume(wa0, wa1, sa, trip_a + k * W);
+                if (k + 2 < ntw) load_trip(tile, k + 2, wa0, wa1, sa);
+                else if (first + j + 1 < my_tiles) load_trip(tile + gridDim.x, 0, wa0, wa1, sa);
+                if (ntw > 1) {
+                    if (trip_a + (k + 1) * W < t1) consume(wb0, wb1, sb, trip_a + (k + 1) * W);
+                    if (k + 3 < ntw) load_trip(tile, k + 3, wb0, wb1, sb);
+                    else if (first + j + 1 < my_tiles) load_trip(tile + gridDim.x, 1, wb0, wb1, sb);
+                }
+            }
             // lane groups q = 0, 1 (2, 3 for the second x row) hold the two chunks of a trip: 32 rows per region
             if (d_ok)
                 *reinterpret_cast<float4 *>(red + j * region + ((wave * 2 + (q & 1)) * MT + d_m) * COLS + cg * 4) =
@@ -360,18 +369,22 @@ int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips
     const int trips_total = a.K / 64;
     const int col_blocks = ceil_div(a.N, 64);
     if (col_blocks > kNumCounters) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_gemv: N=%d too large", a.N);
-    int tps_max = max_trips_per_split < 1 ? 1 : (max_trips_per_split > 32 ? 32 : max_trips_per_split);  // 2 trips x 16 waves
+    int tps_max = max_trips_per_split < 1 ? 1 : (max_trips_per_split > 128 ? 128 : max_trips_per_split);
     auto stage_bytes = [&](int tps) {
         return (size_t)MT * tps * 256 + sizeof(float) * (size_t)MT * ((2 * tps + 3) & ~3);
     };
+    while (tps_max > 1 && stage_bytes(tps_max) > 24 * 1024) --tps_max;
     int ksplit = ceil_div(trips_total, tps_max);
     const int tps = ceil_div(trips_total, ksplit);
     ksplit = ceil_div(trips_total, tps);
     if ((size_t)ksplit * a.M * a.N * sizeof(float) > kWorkspaceBytes / 2)
         return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_gemv: split-K partials exceed the workspace (M=%d N=%d K=%d)", a.M, a.N, a.K);
-    int W = tps <= 16 ? tps : ceil_div(tps, 2);
-    if (a.ln_gamma && W < ceil_div(a.K, 512)) W = ceil_div(a.K, 512);  // one thread per packed row of the whole x row
-    if (W > 16) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "int4_gemv: K=%d too large for the fused LayerNorm", a.K);
+    int W = tps <= 16 ? tps : 16;
+    if (W < ceil_div(8 * tps, 64)) W = ceil_div(8 * tps, 64);          // one thread per packed row of the slice
+    if (a.ln_gamma && W < ceil_div(a.K, 512)) W = ceil_div(a.K, 512);  // ... of the whole x row with LayerNorm
+    if (W > 16) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "int4_gemv: K=%d too large for one workgroup's staging", a.K);
+    p.trips_per_wave = ceil_div(tps, W);
+    if (p.trips_per_wave > 1 && (p.trips_per_wave & 1)) ++p.trips_per_wave;
     p.trips_per_split = tps;
     p.chunk_shift = __builtin_ctz((unsigned)(a.group / 32));
     p.col_blocks = col_blocks;
