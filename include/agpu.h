@@ -80,8 +80,9 @@ int32_t agpu_kernel_lookup(const agpu_ctx *ctx, const char *name, const char **e
 #define AGPU_EPI_GELU_QUICK 2u /* compute_transformer.rs:1468-1531, x*sigmoid(1.702x)             */
 #define AGPU_EPI_FORCE_LITERAL 0x100u /* one thread per output, fma chain in ascending k — the
                                           reference kernel's own arithmetic order               */
-#define AGPU_EPI_FORCE_FP32_GEMV 0x200u /* M <= 16: the fp32 VALU GEMV even where the int8/fp32 matrix-core
-                                            kernels apply (they need group % 32 == 0 and aligned shapes)  */
+#define AGPU_EPI_FORCE_FP32_GEMV 0x200u /* the fp32 kernels (VALU GEMV for M <= 16, fp32 matrix-core GEMM above)
+                                            even where the int8 matrix-core kernels apply (those need
+                                            group = 32 * 2^n and aligned shapes)                         */
 
 /*
  * Y[M,N] = X[M,K] * deq(W) (+ bias[N]) (-> GELU) (+ residual[M,N]).

@@ -156,6 +156,39 @@ def test_config2_gemm(agpu, orc, dev, M):
     assert np.abs(y - ref).max() <= TOL_LINEAR
 
 
+@pytest.mark.parametrize("K,N,g,M", [(768, 2304, 32, 128), (3072, 768, 128, 64), (1600, 4800, 32, 256), (776, 130, 32, 70)])
+def test_gemm_fp32_matrix_core_kernel(agpu, orc, dev, K, N, g, M):
+    """The fp32 MFMA GEMM stays reachable (it serves the shapes the int8 kernel does not take)."""
+    from async_gpu_amd import ops, workloads
+    rng = np.random.default_rng(K + N + M + 1)
+    packed, scales, bias = workloads.random_int4_linear(rng, K, N, g, bias=True)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    y = ops.int4_linear(to_dev(x, dev), to_dev(packed, dev), to_dev(scales, dev), bias=to_dev(bias, dev), group=g,
+                        flags=agpu._lib.EPI_FORCE_FP32_GEMV)
+    assert np.abs(y.cpu().numpy() - orc.int4_gemm_f64(x, packed, scales, g, bias=bias)).max() <= TOL_LINEAR
+
+
+@pytest.mark.parametrize("K,N,g,M", [(32, 40, 32, 17), (96, 33, 32, 40), (160, 257, 32, 33), (768, 2304, 64, 100),
+                                     (1024, 300, 256, 65), (6400, 1600, 32, 48)])
+def test_gemm_int8_matrix_core_shapes(agpu, orc, dev, K, N, g, M):
+    """M > 16, group = 32 * 2^n, K % 32 == 0: one chunk, a K tail inside a 128-k block, ragged rows and columns,
+    groups spanning several chunks, a long K; with a NaN in one row and a wide dynamic range in another."""
+    from async_gpu_amd import ops, workloads
+    rng = np.random.default_rng(K + N + M + g)
+    packed, scales, bias = workloads.random_int4_linear(rng, K, N, g, bias=True)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    x[1] *= np.exp(rng.uniform(-10, 3, K)).astype(np.float32)
+    x[2] = 0.0
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    y = ops.int4_linear(to_dev(x, dev), to_dev(packed, dev), to_dev(scales, dev), bias=to_dev(bias, dev),
+                        residual=to_dev(res, dev), group=g).cpu().numpy()
+    ref = orc.int4_gemm_f64(x, packed, scales, g, bias=bias) + res
+    assert np.abs(y - ref).max() <= TOL_LINEAR
+    x[3, K // 2] = np.nan
+    y = ops.int4_linear(to_dev(x, dev), to_dev(packed, dev), to_dev(scales, dev), group=g).cpu().numpy()
+    assert np.isnan(y[3]).all() and np.isfinite(np.delete(y, 3, axis=0)).all()
+
+
 @pytest.mark.parametrize("K,N,g,M", [(3072, 768, 128, 64), (776, 130, 32, 70), (64, 70, 12, 33), (1600, 4800, 32, 256)])
 def test_gemm_ragged_and_bias(agpu, orc, dev, K, N, g, M):
     from async_gpu_amd import ops, workloads
