@@ -26,7 +26,7 @@ import __graft_entry__ as entry  # noqa: E402
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, GB/s
 # HBM bytes per launch of the roofline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
 # a device copy of known size (profiles/gemv_lm_head_pmc_traffic.md); None until measured.
-TRAFFIC_BYTES_PER_LAUNCH = 24548000
+TRAFFIC_BYTES_PER_LAUNCH = 24561000
 
 
 def step_bytes(cfg, group, context_len):
@@ -76,7 +76,7 @@ def roofline_kernel(ctx, cfg, group, workloads):
     for p in (dp, ds, dx, dy):
         ctx.free(p)
     achieved = gb / (us * 1e-6) / 1e9
-    return {"bound": "hbm", "kernel": "int4_gemv_kernel<1,4,false> (LM head shape M=1 K=768 N=50432 g=32)",
+    return {"bound": "hbm", "kernel": "int4_gemv_i8_kernel<1,false> (LM head shape M=1 K=768 N=50432 g=32)",
             "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5),
             "traffic": TRAFFIC_BYTES_PER_LAUNCH, "bytes_per_launch": int(gb), "us_per_launch": round(us, 3),
             "weight_sets_rotated": n_sets, "cache_resident_GBps": round(gb / (us_hot * 1e-6) / 1e9, 2),
@@ -155,7 +155,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32 (int4 weights, fp32 scales/activations/accumulate)",
+        "dtype": "int4 weights x 32-bit fixed-point activations on int8 MFMA (exact int32 group sums), fp32 scales and accumulation",
         "data": "synthetic",
         "config": {"workload": "BASELINE config 4: GPT-2 small 124M int4 g32 tied-int4-head, B=1, prompt 64, greedy decode",
                    "context_at_start": ctx0, "steps_event_ms": round(ms_events, 4), "model_build_s": round(build_s, 2)},
