@@ -23,13 +23,22 @@ __device__ __forceinline__ void resolve_positions(const AttnParams &p, int &kv_l
     }
 }
 
-// grid (ceil(q_len/32), n_heads * batch), 64 threads.
-__global__ __launch_bounds__(64) void attn_mfma_kernel(const AttnParams p) {
-    __shared__ __align__(16) float Ks[32 * KLD];
-    __shared__ __align__(16) float Vs[32 * DH];
-    const int lane = threadIdx.x, c = lane & 31, h2 = lane >> 5;
+// grid (ceil(q_len/32), n_heads * batch), 64 * S threads.  A workgroup owns 32 query rows; its S waves
+// split the key tiles of 32 (wave w takes tiles w, w + S, ...), each with its own running (m, l, O) and its
+// own K/V tile in LDS, so no barrier is needed inside the key loop; the next tile travels from global
+// memory into registers while the matrix cores work on the current one.  The S partials are merged
+// through LDS in wave order.  Query blocks are issued last-first: the causal mask makes the last blocks
+// the long ones.
+constexpr int ATT_TILE_FLOATS = 32 * KLD + 32 * DH;  // per wave: K tile (padded rows) + V tile
+
+__global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnParams p) {
+    extern __shared__ __align__(16) float att_smem[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, S = blockDim.x >> 6;
+    const int c = lane & 31, h2 = lane >> 5;
+    float *Ks = att_smem + wave * ATT_TILE_FLOATS;
+    float *Vs = Ks + 32 * KLD;
     const int hb = blockIdx.y, b = hb / p.n_heads, h = hb % p.n_heads;
-    const int i0 = blockIdx.x * 32;
+    const int i0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * 32;
     int kv_len, q_offset;
     resolve_positions(p, kv_len, q_offset);
 
@@ -54,22 +63,30 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(const AttnParams p) {
     const int jmax = p.causal ? min(kv_len, q_offset + last_q + 1) : kv_len;  // keys [0, jmax)
     const int my_limit = p.causal ? q_offset + i0 + c : 0x7fffffff;            // last visible key of my query
 
-    for (int j0 = 0; j0 < jmax; j0 += 32) {
-        // stage K and V rows j0..j0+31 (zero beyond kv_len)
-        __syncthreads();
+    // rows it*4 + lane/16 of a tile, 4 floats at column 4*(lane%16): 8 x (K, V) float4 per lane
+    float4 kpre[8], vpre[8];
+    auto fetch = [&](int j0) {
 #pragma unroll
         for (int it = 0; it < 8; ++it) {
-            const int idx = it * 64 + lane;
-            const int r = idx >> 4, c4 = (idx & 15) * 4;
-            float4 kv4 = make_float4(0.f, 0.f, 0.f, 0.f), vv4 = kv4;
+            const int r = it * 4 + (lane >> 4), c4 = (lane & 15) * 4;
+            kpre[it] = vpre[it] = make_float4(0.f, 0.f, 0.f, 0.f);
             if (j0 + r < kv_len) {
-                kv4 = *reinterpret_cast<const float4 *>(kh + (size_t)(j0 + r) * DH + c4);
-                vv4 = *reinterpret_cast<const float4 *>(vh + (size_t)(j0 + r) * DH + c4);
+                kpre[it] = *reinterpret_cast<const float4 *>(kh + (size_t)(j0 + r) * DH + c4);
+                vpre[it] = *reinterpret_cast<const float4 *>(vh + (size_t)(j0 + r) * DH + c4);
             }
-            *reinterpret_cast<float4 *>(&Ks[r * KLD + c4]) = kv4;
-            *reinterpret_cast<float4 *>(&Vs[r * DH + c4]) = vv4;
         }
-        __syncthreads();
+    };
+    if (wave * 32 < jmax) fetch(wave * 32);
+
+    for (int j0 = wave * 32; j0 < jmax; j0 += 32 * S) {
+        // the tile is private to the wave: LDS operations of one wave complete in order, no barrier
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int r = it * 4 + (lane >> 4), c4 = (lane & 15) * 4;
+            *reinterpret_cast<float4 *>(&Ks[r * KLD + c4]) = kpre[it];
+            *reinterpret_cast<float4 *>(&Vs[r * DH + c4]) = vpre[it];
+        }
+        if (j0 + 32 * S < jmax) fetch(j0 + 32 * S);
 
         // S^T[key][query]: A = K[key = c][32*h2 + s], B = Q[query = c][32*h2 + s]
         floatx16 sacc = {0};
@@ -93,12 +110,13 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(const AttnParams p) {
         }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
         const float m_new = fmaxf(m_run, tmax);
-        // m_new is finite from the first tile on: key 0 is visible to every query.
-        const float alpha = expf(m_run - m_new);
+        // A wave's first tile can be fully masked for some queries (m_new = -inf): keep them empty.
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = expf(m_run - m_use);
         float psum = 0.0f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            sacc[r] = expf(sacc[r] - m_new);
+            sacc[r] = expf(sacc[r] - m_use);
             psum += sacc[r];
         }
         psum += __shfl_xor(psum, 32, kWave);
@@ -118,6 +136,45 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(const AttnParams p) {
             o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(va, sacc[r], o0, 0, 0, 0);
             o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vb, sacc[r], o1, 0, 0, 0);
         }
+    }
+
+    // ---- merge the S partials: each wave leaves m, l and its O^T (64 x 32) in its own tile memory ----
+    // O^T element (d, query c) of lane (c, h2): o0[r] at d = 8*(r/4) + 4*h2 + r%4, o1[r] at d + 32.
+    if (S > 1) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int d = 8 * (r >> 2) + 4 * h2 + (r & 3);
+            Ks[d * 32 + c] = o0[r];
+            Ks[(d + 32) * 32 + c] = o1[r];
+        }
+        if (h2 == 0) {
+            Vs[c] = m_run;
+            Vs[32 + c] = l_run;
+        }
+        __syncthreads();
+        // thread t of the workgroup: query c, dims d = t/32, t/32 + 2S, ... (S waves x 2 halves)
+        const int qi = i0 + c;
+        float m_all = -INFINITY;
+        for (int w = 0; w < S; ++w) m_all = fmaxf(m_all, att_smem[w * ATT_TILE_FLOATS + 32 * KLD + c]);
+        float l_all = 0.0f, fac[4];
+        for (int w = 0; w < 4; ++w) {
+            fac[w] = 0.0f;
+            if (w < S) {
+                const float mw = att_smem[w * ATT_TILE_FLOATS + 32 * KLD + c];
+                fac[w] = mw == -INFINITY ? 0.0f : expf(mw - m_all);
+                l_all += att_smem[w * ATT_TILE_FLOATS + 32 * KLD + 32 + c] * fac[w];
+            }
+        }
+        if (qi < p.q_len) {
+            const float inv_l = 1.0f / l_all;
+            float *orow = p.o + (size_t)b * p.o_batch_stride + (size_t)h * p.o_head_stride + (size_t)qi * p.o_row_stride;
+            for (int d = wave * 2 + h2; d < DH; d += 2 * S) {
+                float acc = 0.0f;
+                for (int w = 0; w < S; ++w) acc += att_smem[w * ATT_TILE_FLOATS + d * 32 + c] * fac[w];
+                orow[d] = acc * inv_l;
+            }
+        }
+        return;
     }
     const int qi = i0 + c;
     if (qi < p.q_len) {
@@ -247,7 +304,12 @@ int32_t agpu_attention_launch(agpu_ctx *ctx, const AttnParams &p, int max_kv_len
         hipLaunchKernelGGL(attn_decode_kernel, dim3(p.q_len, hb), dim3(64 * W), 0, ctx->stream, p);
         return AGPU_LAUNCH_CHECK(ctx, "attn_decode_kernel");
     }
-    hipLaunchKernelGGL(attn_mfma_kernel, dim3(ceil_div(p.q_len, 32), hb), dim3(64), 0, ctx->stream, p);
+    // key split: one wave per 4 key tiles of the longest query block, at most 3 (their tiles fill 64 KiB of LDS)
+    const int tiles = ceil_div(max_kv_len, 32);
+    int S = ceil_div(tiles, 4);
+    S = S < 1 ? 1 : (S > 3 ? 3 : S);
+    hipLaunchKernelGGL(attn_mfma_kernel, dim3(ceil_div(p.q_len, 32), hb), dim3(64 * S), sizeof(float) * ATT_TILE_FLOATS * S,
+                       ctx->stream, p);
     return AGPU_LAUNCH_CHECK(ctx, "attn_mfma_kernel");
 }
 
