@@ -202,53 +202,55 @@ __device__ __forceinline__ void merge_partial(float &m, float &l, float4 &o, flo
 }
 
 // grid (q_len, n_heads * batch), 64*W threads.  One workgroup per (head, query row) takes every
-// visible key, so nothing crosses a workgroup.  Lane layout: 16 lanes x float4 per key, 4 keys
-// per wave step; a lane group handles PASS keys per pass (scores first, then one rescale),
-// the W waves interleave over the keys.  Partials merge in a fixed order: lane groups, then waves.
+// visible key, so nothing crosses a workgroup.  Lane layout: 16 lanes x float4 per key (one DPP row),
+// 4 keys per wave step; a lane group handles PASS keys per pass (scores first, then one rescale), the W
+// waves interleave over the keys.  The launch is a chain of dependent latencies, so: K and V rows are
+// loaded for every slot below kv_stride before the context length (possibly a device-side counter) is
+// known, and masked afterwards; dot products reduce with DPP; the 4W lane-group partials are brought to
+// the common maximum first (one exp each) and then just added, in a fixed order.
 constexpr int PASS = 8;
 
 __global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
-    __shared__ float sm[16], sl[16];
-    __shared__ __align__(16) float so[16][DH];
+    __shared__ float sm[64], sl[64];
+    __shared__ __align__(16) float so[64][DH];  // one row per lane group
+    __shared__ float so2[16][DH];               // one row per wave
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6;
     const int gq = lane >> 4, sub = lane & 15;
     const int qi = blockIdx.x, hb = blockIdx.y;
     const int b = hb / p.n_heads, h = hb % p.n_heads;
-    int kv_len, q_offset;
-    resolve_positions(p, kv_len, q_offset);
-    const int vis = p.causal ? min(kv_len, q_offset + qi + 1) : kv_len;  // keys [0, vis)
 
     const float *kh = p.k + (size_t)hb * p.kv_stride * DH + 4 * sub;
     const float *vh = p.v + (size_t)hb * p.kv_stride * DH + 4 * sub;
     const float *qrow = p.q + (size_t)b * p.q_batch_stride + (size_t)h * p.q_head_stride + (size_t)qi * p.q_row_stride;
     float4 q4 = *reinterpret_cast<const float4 *>(qrow + 4 * sub);
+    const int stride = 4 * W;  // keys between two consecutive keys of one lane group
+    const int first = wave * 4 + gq;
+    float4 k4[PASS], v4[PASS];
+    auto fetch = [&](int base) {  // rows below kv_stride exist whatever the context length is
+#pragma unroll
+        for (int i = 0; i < PASS; ++i) {
+            const int j = base + i * stride;
+            const int jr = j < p.kv_stride ? j : 0;
+            k4[i] = *reinterpret_cast<const float4 *>(kh + (size_t)jr * DH);
+            v4[i] = *reinterpret_cast<const float4 *>(vh + (size_t)jr * DH);
+        }
+    };
+    fetch(first);
+    int kv_len, q_offset;
+    resolve_positions(p, kv_len, q_offset);
+    const int vis = p.causal ? min(kv_len, q_offset + qi + 1) : kv_len;  // keys [0, vis)
     q4.x *= 0.125f; q4.y *= 0.125f; q4.z *= 0.125f; q4.w *= 0.125f;
 
     float m = -INFINITY, l = 0.0f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    const int stride = 4 * W;  // keys between two consecutive keys of one lane group
-    for (int base = wave * 4 + gq; base < vis; base += PASS * stride) {
+    for (int base = first; base < vis; base += PASS * stride) {
+        if (base != first) fetch(base);  // the first pass was fetched before the context length was known
         float s[PASS];
-        float4 v4[PASS];
         float bm = -INFINITY;
 #pragma unroll
         for (int i = 0; i < PASS; ++i) {
-            const int j = base + i * stride;
-            s[i] = -INFINITY;
-            v4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (j < vis) {
-                const float4 k4 = *reinterpret_cast<const float4 *>(kh + (size_t)j * DH);
-                v4[i] = *reinterpret_cast<const float4 *>(vh + (size_t)j * DH);
-                s[i] = (q4.x * k4.x + q4.y * k4.y) + (q4.z * k4.z + q4.w * k4.w);
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < PASS; ++i) {
-            // masked lanes carry -inf through the adds unchanged (all 16 lanes of a group agree on j < vis)
-            s[i] += __shfl_xor(s[i], 8, kWave);
-            s[i] += __shfl_xor(s[i], 4, kWave);
-            s[i] += __shfl_xor(s[i], 2, kWave);
-            s[i] += __shfl_xor(s[i], 1, kWave);
+            const float d = (q4.x * k4[i].x + q4.y * k4[i].y) + (q4.z * k4[i].z + q4.w * k4[i].w);
+            s[i] = base + i * stride < vis ? row16_sum(d) : -INFINITY;
             bm = fmaxf(bm, s[i]);
         }
         const float mn = fmaxf(m, bm);  // finite: the first key of the pass is visible
@@ -259,37 +261,33 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
         for (int i = 0; i < PASS; ++i) {
             const float pj = expf(s[i] - mn);  // exp(-inf) = 0 for masked keys
             l += pj;
-            o.x += pj * v4[i].x; o.y += pj * v4[i].y; o.z += pj * v4[i].z; o.w += pj * v4[i].w;
+            // a masked slot holds whatever the row contains (possibly NaN): select, do not multiply by 0
+            const bool ok = base + i * stride < vis;
+            o.x += ok ? pj * v4[i].x : 0.0f; o.y += ok ? pj * v4[i].y : 0.0f;
+            o.z += ok ? pj * v4[i].z : 0.0f; o.w += ok ? pj * v4[i].w : 0.0f;
         }
         m = mn;
     }
-    // merge the 4 lane groups of the wave (xor 16, then xor 32): both partners use the same operand order
-#pragma unroll
-    for (int off = 16; off <= 32; off <<= 1) {
-        const float m2 = __shfl_xor(m, off, kWave), l2 = __shfl_xor(l, off, kWave);
-        float4 o2;
-        o2.x = __shfl_xor(o.x, off, kWave); o2.y = __shfl_xor(o.y, off, kWave);
-        o2.z = __shfl_xor(o.z, off, kWave); o2.w = __shfl_xor(o.w, off, kWave);
-        if ((lane & off) == 0) merge_partial(m, l, o, m2, l2, o2);
-        else {
-            float mm = m2, ll = l2;
-            float4 oo = o2;
-            merge_partial(mm, ll, oo, m, l, o);
-            m = mm; l = ll; o = oo;
-        }
-    }
-    if (lane < 16) {
-        if (lane == 0) { sm[wave] = m; sl[wave] = l; }
-        *reinterpret_cast<float4 *>(&so[wave][4 * sub]) = o;
-    }
+    // ---- merge the 4W lane-group partials (m, l, o) ----
+    const int g = wave * 4 + gq;
+    if (sub == 0) sm[g] = m;
+    if (tid >= 4 * W && tid < 64) sm[tid] = -INFINITY;
     __syncthreads();
-    if (wave == 0 && lane < 16) {
-        m = sm[0]; l = sl[0];
-        o = *reinterpret_cast<const float4 *>(&so[0][4 * sub]);
-        for (int w = 1; w < W; ++w) merge_partial(m, l, o, sm[w], sl[w], *reinterpret_cast<const float4 *>(&so[w][4 * sub]));
-        const float inv = 1.0f / l;
+    const float m_all = wave_max(sm[lane]);  // finite: key 0 is visible
+    const float fac = expf(m - m_all);       // 0 for an empty partial
+    if (sub == 0) sl[g] = l * fac;
+    if (tid >= 4 * W && tid < 64) sl[tid] = 0.0f;
+    *reinterpret_cast<float4 *>(&so[g][4 * sub]) = make_float4(o.x * fac, o.y * fac, o.z * fac, o.w * fac);
+    // the wave's four rows, column-wise (LDS operations of one wave complete in order)
+    const float ow = (so[wave * 4][lane] + so[wave * 4 + 1][lane]) + (so[wave * 4 + 2][lane] + so[wave * 4 + 3][lane]);
+    so2[wave][lane] = ow;
+    __syncthreads();
+    if (wave == 0) {
+        const float l_all = wave_sum(sl[lane]);
+        float acc = 0.0f;
+        for (int w = 0; w < W; ++w) acc += so2[w][lane];
         float *orow = p.o + (size_t)b * p.o_batch_stride + (size_t)h * p.o_head_stride + (size_t)qi * p.o_row_stride;
-        *reinterpret_cast<float4 *>(orow + 4 * sub) = make_float4(o.x * inv, o.y * inv, o.z * inv, o.w * inv);
+        orow[lane] = acc / l_all;
     }
 }
 
