@@ -109,8 +109,6 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
     };
     wa0 = wa1 = wb0 = wb1 = make_uint4(0u, 0u, 0u, 0u);
     sa = sb = make_float4(0.f, 0.f, 0.f, 0.f);
-    load_trip(blockIdx.x, 0, wa0, wa1, sa);
-    if (ntw > 1) load_trip(blockIdx.x, 1, wb0, wb1, sb);
 
     // ---- x: packed row `row` of every x row into registers ----
     // With LayerNorm the statistics need the whole row of x, so thread r owns row r of all K / 8; otherwise
@@ -131,6 +129,22 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
         xv[m][0] = lo.x; xv[m][1] = lo.y; xv[m][2] = lo.z; xv[m][3] = lo.w;
         xv[m][4] = hi.x; xv[m][5] = hi.y; xv[m][6] = hi.z; xv[m][7] = hi.w;
     }
+    float g8[8], b8[8];
+    if constexpr (LN) {
+        float4 glo = make_float4(0.f, 0.f, 0.f, 0.f), ghi = glo, blo = glo, bhi = glo;
+        if (own) {
+            glo = *reinterpret_cast<const float4 *>(a.ln_gamma + 8 * row);
+            ghi = *reinterpret_cast<const float4 *>(a.ln_gamma + 8 * row + 4);
+            blo = *reinterpret_cast<const float4 *>(a.ln_beta + 8 * row);
+            bhi = *reinterpret_cast<const float4 *>(a.ln_beta + 8 * row + 4);
+        }
+        g8[0] = glo.x; g8[1] = glo.y; g8[2] = glo.z; g8[3] = glo.w; g8[4] = ghi.x; g8[5] = ghi.y; g8[6] = ghi.z; g8[7] = ghi.w;
+        b8[0] = blo.x; b8[1] = blo.y; b8[2] = blo.z; b8[3] = blo.w; b8[4] = bhi.x; b8[5] = bhi.y; b8[6] = bhi.z; b8[7] = bhi.w;
+    }
+    // The weights go out after x: a wave's loads return in order, so x would otherwise wait for them.
+    __builtin_amdgcn_sched_barrier(0);
+    load_trip(blockIdx.x, 0, wa0, wa1, sa);
+    if (ntw > 1) load_trip(blockIdx.x, 1, wb0, wb1, sb);
     if (tid < 16) {  // neutral columns of the reduction scratch and the unused rows of red
         if (tid >= W)
             for (int j = 0; j < 3 * MT; ++j) (&s_scratch[0][0])[j * 16 + tid] = 0.0f;
@@ -138,18 +152,6 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
     for (int i = tid; i < p.tiles_per_pass * 32 * n_out; i += T)
         if ((i % (32 * n_out)) >= 2 * W * n_out) red[i] = 0.0f;
     if constexpr (LN) {
-        float g8[8], b8[8];
-        {
-            float4 glo = make_float4(0.f, 0.f, 0.f, 0.f), ghi = glo, blo = glo, bhi = glo;
-            if (own) {
-                glo = *reinterpret_cast<const float4 *>(a.ln_gamma + 8 * row);
-                ghi = *reinterpret_cast<const float4 *>(a.ln_gamma + 8 * row + 4);
-                blo = *reinterpret_cast<const float4 *>(a.ln_beta + 8 * row);
-                bhi = *reinterpret_cast<const float4 *>(a.ln_beta + 8 * row + 4);
-            }
-            g8[0] = glo.x; g8[1] = glo.y; g8[2] = glo.z; g8[3] = glo.w; g8[4] = ghi.x; g8[5] = ghi.y; g8[6] = ghi.z; g8[7] = ghi.w;
-            b8[0] = blo.x; b8[1] = blo.y; b8[2] = blo.z; b8[3] = blo.w; b8[4] = bhi.x; b8[5] = bhi.y; b8[6] = bhi.z; b8[7] = bhi.w;
-        }
         float st[MT];
 #pragma unroll
         for (int m = 0; m < MT; ++m)
@@ -375,6 +377,8 @@ int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips
     };
     while (tps_max > 1 && stage_bytes(tps_max) > 24 * 1024) --tps_max;
     int ksplit = ceil_div(trips_total, tps_max);
+    // a narrow layer occupies few CUs: split K further, down to one trip per wave (measured on K = 3072, N = 768)
+    if (col_blocks * ksplit < ctx->num_cus / 4 && ceil_div(trips_total, ksplit) > 16) ksplit = ceil_div(trips_total, 16);
     const int tps = ceil_div(trips_total, ksplit);
     ksplit = ceil_div(trips_total, tps);
     if ((size_t)ksplit * a.M * a.N * sizeof(float) > kWorkspaceBytes / 2)
