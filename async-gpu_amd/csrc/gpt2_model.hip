@@ -730,6 +730,68 @@ AGPU_EXPORT int32_t agpu_gpt2_generate_cached(agpu_gpt2 *m, const uint32_t *prom
     return AGPU_OK;
 }
 
+// sampling.hip
+int32_t agpu_top_k_launch(agpu_ctx *ctx, const float *logits, int rows, int n, int stride, int k, float temperature,
+                          uint32_t *idx_out, float *val_out);
+extern "C" uint32_t agpu_top_k_draw_host(const float *ranked_vals, const uint32_t *ranked_idx, int32_t k, float r);
+extern "C" float agpu_simple_rng_next_f32(uint64_t *state);
+
+AGPU_EXPORT int32_t agpu_gpt2_generate_cached_sampling(agpu_gpt2 *m, const uint32_t *prompt_host, int32_t prompt_len,
+                                                       int32_t max_new_tokens, int32_t top_k, float temperature,
+                                                       uint64_t *rng_state, int32_t eos, uint32_t *tokens_out_host,
+                                                       int32_t *length_out_host) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    agpu_ctx *ctx = m->ctx;
+    if (!prompt_host || !tokens_out_host || !length_out_host || !rng_state)
+        return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "gpt2_generate_cached_sampling: null pointer");
+    if (prompt_len <= 0 || max_new_tokens < 0 || top_k <= 0)
+        return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_generate_cached_sampling: bad prompt_len/max_new_tokens/top_k");
+    if (prompt_len + (max_new_tokens > 0 ? max_new_tokens - 1 : 0) > m->P)
+        return agpu_fail(ctx, AGPU_ERR_DIM_OUT_OF_RANGE,
+                         "gpt2_generate_cached_sampling: prompt %d + %d new tokens exceed n_positions %d", prompt_len,
+                         max_new_tokens, m->P);
+    std::memcpy(tokens_out_host, prompt_host, (size_t)prompt_len * 4);
+    int len = prompt_len;
+    *length_out_host = len;
+    if (max_new_tokens == 0) return AGPU_OK;
+    int32_t rc = check_ready(m);
+    if (rc != AGPU_OK) return rc;
+    const int k = top_k < m->V ? top_k : m->V;
+    if (k > 1024) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "gpt2_generate_cached_sampling: top_k = %d exceeds 1024", top_k);
+    uint32_t *idx_dev = nullptr;
+    float *val_dev = nullptr;
+    if ((rc = dev_alloc(ctx, (void **)&idx_dev, (size_t)k * 4)) != AGPU_OK) return rc;
+    if ((rc = dev_alloc(ctx, (void **)&val_dev, (size_t)k * 4)) != AGPU_OK) {
+        (void)hipFree(idx_dev);
+        return rc;
+    }
+    std::vector<uint32_t> idx((size_t)k);
+    std::vector<float> val((size_t)k);
+    if ((rc = ensure(m, m->tok_in, (size_t)prompt_len * 4)) == AGPU_OK) rc = ensure_buffers(m, 1, prompt_len, false);
+    if (rc == AGPU_OK) rc = ensure_out_tokens(m, max_new_tokens, 1);
+    if (rc == AGPU_OK) rc = upload(ctx, m->tok_in.p, prompt_host, (size_t)prompt_len * 4, 0);
+    if (rc == AGPU_OK) rc = agpu_gpt2_reset_cache(m);
+    for (int step = 0; rc == AGPU_OK && step < max_new_tokens; ++step) {
+        // logits of the last position: the prefill first, then one replayed decode step per token.  The
+        // replayed graph also runs the arg-max feed; its token is overwritten by the sampled one below.
+        if (step == 0) rc = agpu_gpt2_forward_cached(m, (const uint32_t *)m->tok_in.p, 1, prompt_len, nullptr, 0);
+        else rc = run_decode_steps(m, 1, 1);
+        if (rc != AGPU_OK) break;
+        rc = agpu_top_k_launch(ctx, (const float *)m->logits.p, 1, m->V, logits_stride(m), k, temperature, idx_dev, val_dev);
+        if (rc == AGPU_OK) rc = agpu_memcpy_d2h(ctx, idx.data(), idx_dev, (size_t)k * 4);
+        if (rc == AGPU_OK) rc = agpu_memcpy_d2h(ctx, val.data(), val_dev, (size_t)k * 4);
+        if (rc != AGPU_OK) break;
+        const uint32_t next = agpu_top_k_draw_host(val.data(), idx.data(), k, agpu_simple_rng_next_f32(rng_state));
+        if (eos >= 0 && next == (uint32_t)eos) break;  // gpt2.rs:956-958, 970-972
+        tokens_out_host[len++] = next;
+        if (step + 1 < max_new_tokens) rc = upload(ctx, m->cur_tok, &next, 4, 0);
+    }
+    (void)hipFree(idx_dev);
+    (void)hipFree(val_dev);
+    *length_out_host = len;
+    return rc;
+}
+
 AGPU_EXPORT int32_t agpu_gpt2_generate(agpu_gpt2 *m, const uint32_t *prompt_host, int32_t prompt_len, int32_t max_new_tokens,
                                        int32_t eos, uint32_t *tokens_out_host, int32_t *length_out_host) {
     if (!m) return AGPU_ERR_NULL_POINTER;

@@ -125,6 +125,27 @@ class Int4Gpt2Model:
             m.quantize_linear(-1, 0, np.ascontiguousarray(weights["wte"].T), None, mode)
         return m
 
+    @classmethod
+    def from_file(cls, path, group_size=32, mode=_lib.QUANT_SCRIPT, ctx=None, device=0, **config_kw):
+        """A GPT-2 safetensors file, fp32 (load_gpt2_weights, model.rs:308-378; quantized here at load like
+        Int4Gpt2Model::from_weights) or int4 (weights.save_gpt2_int4_safetensors).  The geometry comes from the
+        tensor shapes; config_kw passes max_batch, lm_head, gelu, argmax_last on."""
+        from . import weights
+        from safetensors import safe_open
+        with safe_open(path, framework="numpy") as f:
+            is_int4 = any(k.endswith(".int4_packed") for k in f.keys())
+        if is_int4:
+            cfg, qz = weights.load_gpt2_int4_safetensors(path)
+            if qz["lm_head"] is None:
+                config_kw.setdefault("lm_head", LM_HEAD_F32)
+            config = Gpt2Config(cfg["n_layer"], cfg["n_embd"], cfg["n_head"], vocab_size=cfg["vocab"],
+                                n_positions=cfg["n_positions"], group_size=qz["group"], **config_kw)
+            return cls.from_quantized(config, qz, ctx, device)
+        cfg, w = weights.load_gpt2_safetensors(path)
+        config = Gpt2Config(cfg["n_layer"], cfg["n_embd"], cfg["n_head"], vocab_size=cfg["vocab"],
+                            n_positions=cfg["n_positions"], group_size=group_size, **config_kw)
+        return cls.from_weights(config, w, mode, ctx, device)
+
     def quantized_memory_bytes(self):
         return int(self._lib.agpu_gpt2_quantized_memory_bytes(self.handle))
 
@@ -169,6 +190,15 @@ class Int4Gpt2Model:
         ms = np.zeros(2, np.float32)
         self._call("agpu_gpt2_generate_cached", prompt, B, n, max_new_tokens, eos, out, lens, ms)
         return [out[b, :lens[b]].copy() for b in range(B)], (float(ms[0]), float(ms[1]))
+
+    def generate_cached_sampling(self, prompt, max_new_tokens, top_k, temperature, rng, eos=50256):
+        """Int4Gpt2Model::generate_cached_sampling (gpt2.rs:931-977); rng is an ops.SimpleRng and is advanced."""
+        prompt = _np(prompt, np.uint32).ravel()
+        out = np.zeros(prompt.size + max_new_tokens, np.uint32)
+        n = C.c_int32(0)
+        self._call("agpu_gpt2_generate_cached_sampling", prompt, prompt.size, max_new_tokens, top_k, float(temperature),
+                   C.addressof(rng._s), eos, out, C.addressof(n))
+        return out[: n.value].copy()
 
     def generate(self, prompt, max_new_tokens, eos=50256):
         prompt = _np(prompt, np.uint32).ravel()

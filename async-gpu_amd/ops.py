@@ -185,3 +185,43 @@ def gemm_f32(a, b):
     c = torch.empty((M, b.shape[1]), dtype=torch.float32, device=a.device)
     context(a.device.index or 0).call("agpu_gemm_f32", _f32(a), _f32(b), c, M, b.shape[1], K)
     return c
+
+
+class SimpleRng:
+    """SimpleRng (nn/models/gpt2.rs:1000-1023): xorshift64; next_f32 in [0, 1)."""
+
+    def __init__(self, seed):
+        import ctypes as C
+        self._s = C.c_uint64(_lib.cdll().agpu_simple_rng_new(int(seed) & 0xFFFFFFFFFFFFFFFF))
+
+    @property
+    def state(self):
+        return int(self._s.value)
+
+    def next_f32(self):
+        import ctypes as C
+        return float(_lib.cdll().agpu_simple_rng_next_f32(C.addressof(self._s)))
+
+
+def top_k(logits, k, temperature=1.0):
+    """Ranked candidates of top_k_sample (gpt2.rs:1029-1039) per row: (indices [rows, k] int32 view of uint32, values)."""
+    import torch
+
+    lg = logits.contiguous().view(-1, logits.shape[-1])
+    rows, n = lg.shape
+    kk = min(int(k), n)
+    idx = torch.empty((rows, kk), dtype=torch.int32, device=lg.device)
+    val = torch.empty((rows, kk), dtype=torch.float32, device=lg.device)
+    context(lg.device.index or 0).call("agpu_top_k", lg, rows, n, int(k), float(temperature), idx, val)
+    return idx, val
+
+
+def top_k_sample(logits, k, temperature, rng):
+    """top_k_sample (gpt2.rs:1029-1058) on a device logit vector; advances rng; returns the token id."""
+    import ctypes as C
+
+    lg = logits.contiguous().view(-1)
+    tok = C.c_uint32(0)
+    context(lg.device.index or 0).call("agpu_top_k_sample", lg, lg.numel(), int(k), float(temperature), C.addressof(rng._s),
+                                       C.addressof(tok))
+    return int(tok.value)

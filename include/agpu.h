@@ -172,6 +172,25 @@ int32_t agpu_embedding(agpu_ctx *ctx, const uint32_t *tokens, const float *wte, 
 int32_t agpu_argmax_rows(agpu_ctx *ctx, const float *x, uint32_t *idx_out, int32_t rows, int32_t cols,
                          int32_t last_index);
 
+/* ---- sampling --------------------------------------------------------------------------- */
+
+/* The k largest of logits[row, :] / max(temperature, 1e-8) per row, ranked by value (descending) and, among
+ * equal values, by index (ascending): the candidate list of top_k_sample (nn/models/gpt2.rs:1029-1039, a
+ * stable sort).  idx_out, val_out: device [rows, min(k, n)].  n <= 65536, k <= 1024.  NaN ranks lowest. */
+int32_t agpu_top_k(agpu_ctx *ctx, const float *logits, int32_t rows, int32_t n, int32_t k, float temperature,
+                   uint32_t *idx_out, float *val_out);
+/* SimpleRng (gpt2.rs:1000-1023): xorshift64 (13, 7, 17); seed 0 becomes 0xDEADBEEFCAFE1234; next_f32 is
+ * (next_u64 >> 40) / 2^24 in [0, 1).  The state is the caller's 64-bit word. */
+uint64_t agpu_simple_rng_new(uint64_t seed);
+float agpu_simple_rng_next_f32(uint64_t *state);
+/* Host part of top_k_sample (gpt2.rs:1041-1057): softmax over the k ranked values in f32 and the first rank
+ * whose running sum exceeds r (the last rank if none).  Host pointers. */
+uint32_t agpu_top_k_draw_host(const float *ranked_vals, const uint32_t *ranked_idx, int32_t k, float r);
+/* top_k_sample(logits, k, temperature, rng) (gpt2.rs:1029-1058) on device logits [n]: candidates on the device,
+ * k (index, value) pairs to the host, draw with the next value of the generator.  *token_out_host on the host. */
+int32_t agpu_top_k_sample(agpu_ctx *ctx, const float *logits, int32_t n, int32_t k, float temperature,
+                          uint64_t *rng_state, uint32_t *token_out_host);
+
 /* ---- attention ------------------------------------------------------------------------- */
 
 /* ops::split_qkv (nn/ops/attention.rs:105-142): [seq,3d] -> Q,K,V [H,seq,dh]. */

@@ -100,6 +100,17 @@ int32_t agpu_gpt2_generate(agpu_gpt2 *m, const uint32_t *prompt_host, int32_t pr
                            int32_t eos, uint32_t *tokens_out_host, int32_t *length_out_host);
 
 /*
+ * Int4Gpt2Model::generate_cached_sampling (gpt2.rs:931-977): prefill, then one token per step drawn by
+ * top_k_sample from the step's logits with the caller's SimpleRng state (advanced once per token).  A drawn
+ * `eos` ends the sequence before it is appended (eos < 0: never).  One sequence.  tokens_out_host
+ * [prompt_len + max_new_tokens]; *length_out_host = tokens written.  Each step costs one small device-to-host
+ * copy (k candidates) and one token upload: the control flow depends on host random numbers, as in the reference.
+ */
+int32_t agpu_gpt2_generate_cached_sampling(agpu_gpt2 *m, const uint32_t *prompt_host, int32_t prompt_len,
+                                           int32_t max_new_tokens, int32_t top_k, float temperature, uint64_t *rng_state,
+                                           int32_t eos, uint32_t *tokens_out_host, int32_t *length_out_host);
+
+/*
  * Benchmark hook: replay `steps` decode steps (one token per sequence per step) starting from the
  * current cache state and the device-resident current tokens, without any host round trip, and
  * report the time per step measured with HIP events on the context's stream.  The cache advances by

@@ -756,3 +756,96 @@ ORC_API int orc_gpt2_generate(orc_gpt2 *m, const uint32_t *prompt, int prompt_le
     free(logits);
     return len;
 }
+
+/* ------------------------------------------------------------------------ */
+/* sampling: SimpleRng, top_k_sample, generate_cached_sampling               */
+/* ------------------------------------------------------------------------ */
+
+/* SimpleRng::new / next_u64 / next_f32 (nn/models/gpt2.rs:1000-1023): xorshift64 with shifts 13, 7, 17,
+ * seed 0 replaced by 0xDEADBEEFCAFE1234; next_f32 = (next_u64 >> 40) / 2^24 in [0, 1). */
+ORC_API uint64_t orc_simple_rng_new(uint64_t seed) { return seed == 0 ? 0xDEADBEEFCAFE1234ull : seed; }
+
+ORC_API float orc_simple_rng_next_f32(uint64_t *state) {
+    uint64_t x = *state;
+    x ^= x << 13;
+    x ^= x >> 7;
+    x ^= x << 17;
+    *state = x;
+    return (float)(x >> 40) / (float)(1ull << 24);
+}
+
+typedef struct { float v; int i; } orc_pair;
+
+/* descending by value, ties in index order: what a stable sort of (index, value) pairs by
+ * b.partial_cmp(a) gives (gpt2.rs:1036-1038) */
+static int orc_pair_cmp(const void *a, const void *b) {
+    const orc_pair *x = (const orc_pair *)a, *y = (const orc_pair *)b;
+    if (x->v > y->v) return -1;
+    if (x->v < y->v) return 1;
+    return x->i < y->i ? -1 : (x->i > y->i ? 1 : 0);
+}
+
+/*
+ * top_k_sample (gpt2.rs:1029-1058): logits / max(temperature, 1e-8) in f32, the k largest in stable
+ * descending order, softmax over them in f32 (exp of the difference to the first, sequential sum, one
+ * division each), then the first rank whose running sum exceeds r = rng.next_f32(); the last rank if none.
+ * top_idx_out / top_val_out (optional, [k]) receive the ranked candidates.
+ */
+ORC_API uint32_t orc_top_k_sample(const float *logits, int n, int k, float temperature, uint64_t *rng_state,
+                                  uint32_t *top_idx_out, float *top_val_out) {
+    const float temp = temperature < 1e-8f ? 1e-8f : temperature;
+    orc_pair *p = (orc_pair *)malloc(sizeof(orc_pair) * (size_t)n);
+    for (int i = 0; i < n; ++i) {
+        p[i].v = logits[i] / temp;
+        p[i].i = i;
+    }
+    qsort(p, (size_t)n, sizeof(orc_pair), orc_pair_cmp);
+    if (k > n) k = n;
+    float *e = (float *)malloc(sizeof(float) * (size_t)k);
+    float sum = 0.0f;
+    for (int j = 0; j < k; ++j) {
+        e[j] = expf(p[j].v - p[0].v);
+        sum += e[j];
+        if (top_idx_out) top_idx_out[j] = (uint32_t)p[j].i;
+        if (top_val_out) top_val_out[j] = p[j].v;
+    }
+    const float r = orc_simple_rng_next_f32(rng_state);
+    uint32_t pick = (uint32_t)p[k - 1].i;
+    float cum = 0.0f;
+    for (int j = 0; j < k; ++j) {
+        cum += e[j] / sum;
+        if (r < cum) {
+            pick = (uint32_t)p[j].i;
+            break;
+        }
+    }
+    free(e);
+    free(p);
+    return pick;
+}
+
+/*
+ * generate_cached_sampling (gpt2.rs:931-977): prefill, sample from the last row, then one token per step;
+ * a sampled `eos` ends the sequence before it is appended (eos < 0 never stops).  The logits are rounded
+ * to f32 before sampling, as the reference samples from f32 logits.  Returns the total length.
+ */
+ORC_API int orc_gpt2_generate_sampling(orc_gpt2 *m, const uint32_t *prompt, int prompt_len, int max_new_tokens, int top_k,
+                                       float temperature, uint64_t *rng_state, int eos, uint32_t *tokens_out) {
+    double *logits = (double *)malloc(sizeof(double) * (size_t)m->vocab);
+    float *lf = (float *)malloc(sizeof(float) * (size_t)m->vocab);
+    int len = prompt_len;
+    memcpy(tokens_out, prompt, sizeof(uint32_t) * (size_t)prompt_len);
+    orc_gpt2_reset_cache(m);
+    for (int step = 0; step < max_new_tokens; ++step) {
+        const int rc = step == 0 ? orc_gpt2_forward(m, tokens_out, len, 0, logits, NULL)
+                                 : orc_gpt2_forward(m, tokens_out + len - 1, 1, 0, logits, NULL);
+        if (rc != 0) break;
+        for (int i = 0; i < m->vocab; ++i) lf[i] = (float)logits[i];
+        const uint32_t next = orc_top_k_sample(lf, m->vocab, top_k, temperature, rng_state, NULL, NULL);
+        if (eos >= 0 && next == (uint32_t)eos) break;
+        tokens_out[len++] = next;
+    }
+    free(lf);
+    free(logits);
+    return len;
+}

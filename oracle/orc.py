@@ -75,6 +75,10 @@ _g_reset = _sig("orc_gpt2_reset_cache", None, C.c_void_p)
 _g_len = _sig("orc_gpt2_cache_len", _i, C.c_void_p)
 _g_fwd = _sig("orc_gpt2_forward", _i, C.c_void_p, _u32p, _i, _i, C.c_void_p, C.c_void_p)
 _g_gen = _sig("orc_gpt2_generate", _i, C.c_void_p, _u32p, _i, _i, _i, _i, _u32p, C.c_void_p)
+_rng_new = _sig("orc_simple_rng_new", C.c_uint64, C.c_uint64)
+_rng_f32 = _sig("orc_simple_rng_next_f32", C.c_float, C.POINTER(C.c_uint64))
+_topk = _sig("orc_top_k_sample", C.c_uint32, _f32p, _i, _i, C.c_float, C.POINTER(C.c_uint64), C.c_void_p, C.c_void_p)
+_g_samp = _sig("orc_gpt2_generate_sampling", _i, C.c_void_p, _u32p, _i, _i, _i, C.c_float, C.POINTER(C.c_uint64), _i, _u32p)
 
 
 def _f32(a):
@@ -295,6 +299,13 @@ class Gpt2:
             raise ValueError("sequence exceeds n_positions")
         return (logits, hidden) if want_hidden else logits
 
+    def generate_sampling(self, prompt, max_new_tokens, top_k, temperature, rng, eos=50256):
+        """generate_cached_sampling (gpt2.rs:931-977); rng is a SimpleRng and is advanced."""
+        prompt = _u32(prompt)
+        out = np.zeros(prompt.size + max_new_tokens, np.uint32)
+        n = _g_samp(self._h, prompt, prompt.size, max_new_tokens, top_k, temperature, C.byref(rng._s), eos, out)
+        return out[:n].copy()
+
     def generate(self, prompt, max_new_tokens, cached=True, eos=50256):
         prompt = _u32(prompt)
         out = np.zeros(prompt.size + max_new_tokens, np.uint32)
@@ -302,3 +313,28 @@ class Gpt2:
         n = _g_gen(self._h, prompt, prompt.size, max_new_tokens, int(cached), eos, out,
                    margins.ctypes.data_as(C.c_void_p))
         return out[:n].copy(), margins[: max(n - prompt.size, 0)].copy()
+
+
+class SimpleRng:
+    """SimpleRng (nn/models/gpt2.rs:1000-1023): xorshift64, next_f32 in [0, 1) with 24 bits."""
+
+    def __init__(self, seed):
+        self._s = C.c_uint64(_rng_new(int(seed) & 0xFFFFFFFFFFFFFFFF))
+
+    @property
+    def state(self):
+        return int(self._s.value)
+
+    def next_f32(self):
+        return float(_rng_f32(C.byref(self._s)))
+
+
+def top_k_sample(logits, k, temperature, rng, want_candidates=False):
+    """top_k_sample (gpt2.rs:1029-1058) -> token id (and the ranked (indices, scaled values) if asked)."""
+    lg = _f32(logits).ravel()
+    kk = min(int(k), lg.size)
+    idx = np.zeros(kk, np.uint32)
+    val = np.zeros(kk, np.float32)
+    tok = int(_topk(lg, lg.size, int(k), float(temperature), C.byref(rng._s), idx.ctypes.data_as(C.c_void_p),
+                    val.ctypes.data_as(C.c_void_p)))
+    return (tok, idx, val) if want_candidates else tok

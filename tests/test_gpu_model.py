@@ -214,3 +214,22 @@ def test_context_may_be_destroyed_before_its_model(orc, agpu, dev):
     ctx.close()
     gm.close()  # must not touch freed memory
     gm.close()
+
+
+def test_model_from_weight_files(tiny, orc, agpu, dev, tmp_path):
+    """An fp32 safetensors file (quantized at load) and the int4 file written from it give the model built
+    from arrays: identical logits and greedy tokens."""
+    from async_gpu_amd import gpt2, weights, workloads
+    cfg, w, qz, om, gm = tiny
+    src, dst = str(tmp_path / "model.safetensors"), str(tmp_path / "model_int4.safetensors")
+    weights.save_gpt2_safetensors(src, w)
+    weights.quantize_gpt2_file(src, dst, group=32)
+    prompt = workloads.random_prompt(cfg, 9, 7)
+    ref_logits = gm.forward(prompt)
+    ref_tokens = gm.generate_cached(prompt.reshape(1, -1), 12, eos=-1)[0][0]
+    for path in (src, dst):
+        m = gpt2.Int4Gpt2Model.from_file(path, group_size=32, mode=agpu._lib.QUANT_SCRIPT)
+        assert (m.config.n_layer, m.config.n_embd, m.config.vocab_size) == (cfg["n_layer"], cfg["n_embd"], cfg["vocab"])
+        assert np.array_equal(m.forward(prompt), ref_logits)
+        assert np.array_equal(m.generate_cached(prompt.reshape(1, -1), 12, eos=-1)[0][0], ref_tokens)
+        m.close()
