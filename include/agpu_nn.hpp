@@ -296,6 +296,24 @@ inline std::vector<uint32_t> argmax_rows(const GpuTensor &x, const Registry &reg
 }
 }  // namespace ops
 
+// SimpleRng (nn/models/gpt2.rs:1000-1023)
+class SimpleRng {
+public:
+    explicit SimpleRng(uint64_t seed) : s_(agpu_simple_rng_new(seed)) {}
+    float next_f32() { return agpu_simple_rng_next_f32(&s_); }
+    uint64_t *state() { return &s_; }
+
+private:
+    uint64_t s_;
+};
+
+// top_k_sample (gpt2.rs:1029-1058) on a device logit vector
+inline uint32_t top_k_sample(const GpuTensor &logits, size_t k, float temperature, SimpleRng &rng, const Registry &reg) {
+    uint32_t tok = 0;
+    reg->check(agpu_top_k_sample(reg->device(), logits.data(), (int32_t)logits.numel(), (int32_t)k, temperature, rng.state(), &tok));
+    return tok;
+}
+
 // ---- layers (nn/layers/*.rs) --------------------------------------------------------------------
 struct Module {  // trait Module (layers/mod.rs:36-39)
     virtual ~Module() = default;
@@ -488,6 +506,16 @@ public:
         std::vector<uint32_t> out(prompt.size() + max_new_tokens);
         int32_t len = 0;
         reg_->check(agpu_gpt2_generate_cached(h_, prompt.data(), 1, (int32_t)prompt.size(), (int32_t)max_new_tokens, eos, out.data(), &len, nullptr));
+        out.resize((size_t)len);
+        return out;
+    }
+    // generate_cached_sampling (gpt2.rs:931-977)
+    std::vector<uint32_t> generate_cached_sampling(const std::vector<uint32_t> &prompt, size_t max_new_tokens, size_t top_k,
+                                                   float temperature, SimpleRng &rng, int eos = 50256) const {
+        std::vector<uint32_t> out(prompt.size() + max_new_tokens);
+        int32_t len = 0;
+        reg_->check(agpu_gpt2_generate_cached_sampling(h_, prompt.data(), (int32_t)prompt.size(), (int32_t)max_new_tokens, (int32_t)top_k,
+                                                       temperature, rng.state(), eos, out.data(), &len));
         out.resize((size_t)len);
         return out;
     }

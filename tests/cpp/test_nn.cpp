@@ -245,6 +245,16 @@ int main() {
             CHECK(unc.size() == prompt.size() + 10 && unc == cac);
             CHECK(model.cache_len() == prompt.size() + 9);
             CHECK(throws_kind(NnError::Kind::DimOutOfRange, [&] { model.generate_cached(prompt, 61, -1); }));
+            // sampling: same seed, same continuation; k = 1 is the greedy one; the generator is xorshift64
+            SimpleRng r1(7), r2(7), r3(9);
+            auto s1 = model.generate_cached_sampling(prompt, 12, 8, 0.9f, r1, -1);
+            auto s2 = model.generate_cached_sampling(prompt, 12, 8, 0.9f, r2, -1);
+            CHECK(s1.size() == prompt.size() + 12 && s1 == s2);
+            auto g1 = model.generate_cached_sampling(prompt, 10, 1, 1.0f, r3, -1);
+            CHECK(g1 == cac);
+            SimpleRng r4(1);
+            CHECK(r4.next_f32() == 0.0f && *r4.state() == 0x40822041ull);  // one xorshift64 step from 1 (13, 7, 17)
+            CHECK(r4.next_f32() == (float)(1048641ull) / 16777216.0f);
         }
     });
 
