@@ -27,6 +27,7 @@ def main():
     ap.add_argument("--xl-layers", type=int, default=48)
     ap.add_argument("--skip-xl", action="store_true")
     ap.add_argument("--skip-kernels", action="store_true")
+    ap.add_argument("--cpu", action="store_true", help="also time the CPU oracle on configs 1-3 (single thread, as the reference CPU path)")
     args = ap.parse_args()
     entry.load_package()
     from async_gpu_amd import _lib, gpt2, workloads
@@ -36,30 +37,43 @@ def main():
     def emit(**kw):
         print(json.dumps(kw), flush=True)
 
-    def bench_linear(M, K, N, group=32, reps=100):
+    def bench_linear(M, K, N, group=32, reps=100, sets=1):
+        """us per launch; sets > 1 rotates over that many copies of the weights (more than the caches hold)."""
         w = workloads.config1_gemv(seed=0 if M == 1 else 1, M=M, K=K, N=N, group=group)
-        dp, ds, dx = ctx.upload(w["packed"]), ctx.upload(w["scales"]), ctx.upload(w["x"])
+        dp, ds = ctx.upload(np.tile(w["packed"], (sets, 1))), ctx.upload(np.tile(w["scales"], (sets, 1)))
+        dx = ctx.upload(w["x"])
         dy = ctx.malloc(M * N * 4)
         us = C.c_float(0)
-        ctx.call("agpu_bench_int4_linear", dx, None, None, 0.0, dp, ds, None, None, dy, M, N, K, group, 0, 1, 0, 0, reps,
-                 C.addressof(us))
+        ctx.call("agpu_bench_int4_linear", dx, None, None, 0.0, dp, ds, None, None, dy, M, N, K, group, 0, sets,
+                 w["packed"].size, w["scales"].size, reps, C.addressof(us))
         for p in (dp, ds, dx, dy):
             ctx.free(p)
         return us.value
 
     if not args.skip_kernels:
-        kernel_cases(ctx, emit, bench_linear, workloads)
+        kernel_cases(ctx, emit, bench_linear, workloads, args)
     if args.skip_xl:
         return
     xl_cases(ctx, emit, args, _lib, gpt2, workloads)
 
 
-def kernel_cases(ctx, emit, bench_linear, workloads):
-    # config 1: single dequant-GEMV, the MLP fc shape
-    us = bench_linear(1, 768, 3072)
+def kernel_cases(ctx, emit, bench_linear, workloads, args=None):
+    # config 1: single dequant-GEMV, the MLP fc shape: the same weights every launch (single-launch latency, caches
+    # warm) and a rotation over 256 copies (377 MB, more than the Infinity Cache), as the HBM figure
     b = 768 * 3072 // 2 + 24 * 3072 * 4 + 768 * 4 + 3072 * 4
-    emit(case="config1 int4 GEMV M=1 K=768 N=3072 g=32", us=round(us, 3), algorithmic_bytes=b,
+    us = bench_linear(1, 768, 3072)
+    emit(case="config1 int4 GEMV M=1 K=768 N=3072 g=32, same weights", us=round(us, 3), algorithmic_bytes=b,
          GBps=round(b / us / 1e3, 1), frac_hbm=round(b / us / 1e3 / HBM_GBS, 4))
+    us = bench_linear(1, 768, 3072, reps=256, sets=256)
+    emit(case="config1 int4 GEMV M=1 K=768 N=3072 g=32, 256 rotating weight copies", us=round(us, 3), algorithmic_bytes=b,
+         GBps=round(b / us / 1e3, 1), frac_hbm=round(b / us / 1e3 / HBM_GBS, 4))
+    # the two LM-head shapes (GPT-2 small and XL-sized), rotating copies
+    for K, sets in ((768, 12), (1600, 6)):
+        N = 50432
+        b = K * N // 2 + (K // 32) * N * 4 + K * 4 + N * 4
+        us = bench_linear(1, K, N, reps=120, sets=sets)
+        emit(case=f"int4 GEMV M=1 K={K} N={N} g=32 (LM head), {sets} rotating weight copies", us=round(us, 3),
+             algorithmic_bytes=b, GBps=round(b / us / 1e3, 1), frac_hbm=round(b / us / 1e3 / HBM_GBS, 4))
     # config 2: prefill QKV dequant-GEMM
     for M in (128, 512, 1024):
         us = bench_linear(M, 768, 2304, reps=50)
@@ -82,7 +96,36 @@ def kernel_cases(ctx, emit, bench_linear, workloads):
          GBps=round(b / us.value / 1e3, 1), frac_hbm=round(b / us.value / 1e3 / HBM_GBS, 4))
     for p in (dq, dk, dv, do, dq1):
         ctx.free(p)
+    if args is not None and args.cpu:
+        cpu_cases(emit, workloads, w)
 
+
+
+def cpu_cases(emit, workloads, att):
+    """The f64 CPU restatement on one thread (the reference CPU path has no threading), per call."""
+    orc = entry.load_oracle()
+    orc.set_threads(1)
+
+    def per_call(fn, min_s=1.0):
+        n, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            n += 1
+            dt = time.perf_counter() - t0
+            if dt > min_s:
+                return dt / n * 1e6
+
+    w = workloads.config1_gemv()
+    emit(case="cpu oracle config1 GEMV (1 thread)", us=round(per_call(lambda: orc.int4_gemm_f64(w["x"], w["packed"], w["scales"], 32)), 1))
+    w2 = workloads.config2_gemm(M=128)
+    emit(case="cpu oracle config2 GEMM M=128 (1 thread)", us=round(per_call(lambda: orc.int4_gemm_f64(w2["x"], w2["packed"], w2["scales"], 32)), 1))
+    q1 = np.ascontiguousarray(att["q"][:, 1023:1024])
+    emit(case="cpu oracle config3 attention decode kv=1024 (1 thread)",
+         us=round(per_call(lambda: orc.attention_kv(q1, att["k"], att["v"], q_offset=1023)), 1))
+    sub = {k: np.ascontiguousarray(att[k][:, :256]) for k in ("q", "k", "v")}
+    emit(case="cpu oracle config3 attention prefill seq=256 of 1024 (1 thread; flops scale by 16.0 to seq 1024)",
+         us=round(per_call(lambda: orc.attention_kv(sub["q"], sub["k"], sub["v"], q_offset=0)), 1))
+    orc.set_threads(0)
 
 
 def xl_cases(ctx, emit, args, _lib, gpt2, workloads):
