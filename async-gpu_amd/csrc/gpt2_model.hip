@@ -268,6 +268,15 @@ int32_t launch_forward(agpu_gpt2 *m, const uint32_t *tokens, int B, int new_len,
             ga.M = R; ga.N = 3 * d; ga.K = d; ga.group = g; ga.flags = 0;
             ga.kcache = kc; ga.vcache = vc; ga.pos_dev = m->pos_dev; ga.n_heads = H; ga.n_positions = P;
             if ((rc = agpu_int4_gemv_launch(ctx, ga)) != AGPU_OK) return rc;
+        } else if (new_len == 1 && R <= 16 && g % 8 == 0) {
+            // batched decode: LayerNorm on its own, then the QKV projection writes the K/V rows itself
+            if ((rc = agpu_layer_norm_impl(ctx, hid, b.ln1_g, b.ln1_b, (float *)m->lnb.p, R, d, eps)) != AGPU_OK) return rc;
+            GemvArgs ga{};
+            ga.x = (const float *)m->lnb.p; ga.packed = wq.packed; ga.scales = wq.scales; ga.bias = wq.bias; ga.y = qkv;
+            ga.M = R; ga.N = 3 * d; ga.K = d; ga.group = g; ga.flags = 0;
+            ga.kcache = kc; ga.vcache = vc; ga.pos_dev = m->pos_dev; ga.n_heads = H; ga.n_positions = P;
+            rc = agpu_int4_skinny_supported(ga) ? agpu_int4_skinny_launch(ctx, ga) : agpu_int4_gemv_launch(ctx, ga);
+            if (rc != AGPU_OK) return rc;
         } else {
             rc = agpu_ln_int4_linear(ctx, hid, b.ln1_g, b.ln1_b, eps, wq.packed, wq.scales, wq.bias, nullptr, qkv, R,
                                      3 * d, d, g, 0);
