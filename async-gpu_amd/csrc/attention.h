@@ -13,6 +13,9 @@ struct AttnParams {
     // When non-null the kernels read the number of positions already cached from here and use
     // kv_len = *pos_dev + q_len, q_offset = *pos_dev (lets one captured launch serve every step).
     const int *pos_dev;
+    // Decode kernel: fetch the first pass of K/V rows before the context length is known (hides one memory
+    // round trip; reads up to 32 * waves rows whatever the length).  Set by the launcher for small launches.
+    int speculate;
 };
 
 // max_kv_len bounds kv_len for launches that read it from pos_dev (sizes the key split).

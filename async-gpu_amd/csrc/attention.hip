@@ -226,25 +226,26 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
     const int stride = 4 * W;  // keys between two consecutive keys of one lane group
     const int first = wave * 4 + gq;
     float4 k4[PASS], v4[PASS];
-    auto fetch = [&](int base) {  // rows below kv_stride exist whatever the context length is
+    auto fetch = [&](int base, int limit) {  // rows below kv_stride exist whatever the context length is; others read row 0
 #pragma unroll
         for (int i = 0; i < PASS; ++i) {
             const int j = base + i * stride;
-            const int jr = j < p.kv_stride ? j : 0;
+            const int jr = j < limit ? j : 0;
             k4[i] = *reinterpret_cast<const float4 *>(kh + (size_t)jr * DH);
             v4[i] = *reinterpret_cast<const float4 *>(vh + (size_t)jr * DH);
         }
     };
-    fetch(first);
+    if (p.speculate) fetch(first, p.kv_stride);
     int kv_len, q_offset;
     resolve_positions(p, kv_len, q_offset);
     const int vis = p.causal ? min(kv_len, q_offset + qi + 1) : kv_len;  // keys [0, vis)
+    if (!p.speculate && first < vis) fetch(first, vis);
     q4.x *= 0.125f; q4.y *= 0.125f; q4.z *= 0.125f; q4.w *= 0.125f;
 
     float m = -INFINITY, l = 0.0f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int base = first; base < vis; base += PASS * stride) {
-        if (base != first) fetch(base);  // the first pass was fetched before the context length was known
+        if (base != first) fetch(base, vis);  // the first pass is already in registers
         float s[PASS];
         float bm = -INFINITY;
 #pragma unroll
@@ -299,7 +300,9 @@ int32_t agpu_attention_launch(agpu_ctx *ctx, const AttnParams &p, int max_kv_len
         // waves per workgroup: one per 32 keys of the longest possible context, 1..16
         int W = ceil_div(max_kv_len, 32);
         W = W < 1 ? 1 : (W > 16 ? 16 : W);
-        hipLaunchKernelGGL(attn_decode_kernel, dim3(p.q_len, hb), dim3(64 * W), 0, ctx->stream, p);
+        AttnParams pd = p;
+        pd.speculate = p.q_len * hb <= 64 ? 1 : 0;  // latency matters for a few workgroups, bandwidth for many
+        hipLaunchKernelGGL(attn_decode_kernel, dim3(p.q_len, hb), dim3(64 * W), 0, ctx->stream, pd);
         return AGPU_LAUNCH_CHECK(ctx, "attn_decode_kernel");
     }
     // key split: one wave per 4 key tiles of the longest query block, at most 3 (their tiles fill 64 KiB of LDS)
