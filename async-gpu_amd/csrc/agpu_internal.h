@@ -100,6 +100,31 @@ __device__ __forceinline__ float wave_max(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
+// The same for unsigned integers (arg-max index selection).
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ unsigned dpp_move_u32(unsigned old, unsigned v) {
+    return (unsigned)__builtin_amdgcn_update_dpp((int)old, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+
+template <bool MAX>
+__device__ __forceinline__ unsigned row16_minmax_u32(unsigned v) {
+    unsigned o;
+    o = dpp_move_u32<0xb1, 0xf>(v, v); v = MAX ? (o > v ? o : v) : (o < v ? o : v);
+    o = dpp_move_u32<0x4e, 0xf>(v, v); v = MAX ? (o > v ? o : v) : (o < v ? o : v);
+    o = dpp_move_u32<0x124, 0xf>(v, v); v = MAX ? (o > v ? o : v) : (o < v ? o : v);
+    o = dpp_move_u32<0x128, 0xf>(v, v); v = MAX ? (o > v ? o : v) : (o < v ? o : v);
+    return v;
+}
+
+template <bool MAX>
+__device__ __forceinline__ unsigned wave_minmax_u32(unsigned v) {
+    v = row16_minmax_u32<MAX>(v);
+    unsigned o;
+    o = dpp_move_u32<0x142, 0xa>(v, v); v = MAX ? (o > v ? o : v) : (o < v ? o : v);
+    o = dpp_move_u32<0x143, 0xc>(v, v); v = MAX ? (o > v ? o : v) : (o < v ? o : v);
+    return (unsigned)__builtin_amdgcn_readlane((int)v, 63);
+}
+
 // tanh GELU, 0.5x(1+tanh(c(x+0.044715x^3))), accurate expf, no fast-math.
 __device__ __forceinline__ float gelu_tanh_dev(float x) {
     // 0.5 * (1 + tanh(u)) == 1 / (1 + exp(-2u)): one exp and one division instead of a tanh expansion

@@ -251,58 +251,66 @@ __device__ __forceinline__ bool better(float v, unsigned int i, float bv, unsign
     return (v > bv) || (v == bv && (last_index ? i > bi : i < bi));
 }
 
+// Every load of the row is in flight at once (up to 16 float4 per thread, 65536 columns; longer rows loop),
+// and the reductions are DPP: the maximum first, then the smallest (or largest) index among the lanes that hold it.
+constexpr int ARGMAX_UNROLL = 16;
+
 __global__ __launch_bounds__(1024) void argmax_rows_kernel(const float *__restrict__ x, uint32_t *idx_out, int cols,
                                                             int row_stride, int last_index, const ArgmaxAdvance adv) {
     __shared__ float sv[16];
     __shared__ unsigned int si[16];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6, T = blockDim.x;
     const int row = blockIdx.x;
     const float *xr = x + (size_t)row * row_stride;
     float bv = -INFINITY;
     unsigned int bi = last_index ? 0u : 0xFFFFFFFFu;
     if ((((uintptr_t)xr) & 15) == 0) {
-        // float4 loads, four in flight per thread
         const int n4 = cols >> 2;
         const float4 *x4 = reinterpret_cast<const float4 *>(xr);
-        for (int c0 = tid; c0 < n4; c0 += 4 * blockDim.x) {
-            float4 v[4];
+        for (int c0 = tid; c0 < n4; c0 += ARGMAX_UNROLL * T) {
+            float4 v[ARGMAX_UNROLL];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int c = c0 + u * blockDim.x;
-                v[u] = c < n4 ? x4[c] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+            for (int u = 0; u < ARGMAX_UNROLL; ++u) {
+                const int c = c0 + u * T;
+                v[u] = x4[c < n4 ? c : c0];  // a repeated element changes nothing
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const unsigned int base = 4u * (unsigned int)(c0 + u * blockDim.x);
-                if (c0 + u * (int)blockDim.x < n4) {
-                    if (better(v[u].x, base, bv, bi, last_index)) { bv = v[u].x; bi = base; }
-                    if (better(v[u].y, base + 1, bv, bi, last_index)) { bv = v[u].y; bi = base + 1; }
-                    if (better(v[u].z, base + 2, bv, bi, last_index)) { bv = v[u].z; bi = base + 2; }
-                    if (better(v[u].w, base + 3, bv, bi, last_index)) { bv = v[u].w; bi = base + 3; }
-                }
+            for (int u = 0; u < ARGMAX_UNROLL; ++u) {
+                const int c = c0 + u * T;
+                const unsigned int base = 4u * (unsigned int)(c < n4 ? c : c0);
+                if (better(v[u].x, base, bv, bi, last_index)) { bv = v[u].x; bi = base; }
+                if (better(v[u].y, base + 1, bv, bi, last_index)) { bv = v[u].y; bi = base + 1; }
+                if (better(v[u].z, base + 2, bv, bi, last_index)) { bv = v[u].z; bi = base + 2; }
+                if (better(v[u].w, base + 3, bv, bi, last_index)) { bv = v[u].w; bi = base + 3; }
             }
         }
-        for (int c = 4 * n4 + tid; c < cols; c += blockDim.x) {
+        for (int c = 4 * n4 + tid; c < cols; c += T) {
             const float v = xr[c];
             if (better(v, (unsigned int)c, bv, bi, last_index)) { bv = v; bi = (unsigned int)c; }
         }
     } else {
-        for (int c = tid; c < cols; c += blockDim.x) {
+        for (int c = tid; c < cols; c += T) {
             const float v = xr[c];
             if (better(v, (unsigned int)c, bv, bi, last_index)) { bv = v; bi = (unsigned int)c; }
         }
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const float ov = __shfl_xor(bv, off, kWave);
-        const unsigned int oi = __shfl_xor(bi, off, kWave);
-        if (better(ov, oi, bv, bi, last_index)) { bv = ov; bi = oi; }
+    const unsigned int none = last_index ? 0u : 0xFFFFFFFFu;
+    {
+        const float m = wave_max(bv);
+        const unsigned int cand = bv == m ? bi : none;
+        bi = last_index ? wave_minmax_u32<true>(cand) : wave_minmax_u32<false>(cand);
+        bv = m;
     }
     if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
     __syncthreads();
+    if (wave == 0) {
+        const int w = lane & 15;
+        const float v = w < W ? sv[w] : -INFINITY;
+        const float m = row16_max(v);
+        const unsigned int cand = (w < W && v == m) ? si[w] : none;
+        bi = last_index ? row16_minmax_u32<true>(cand) : row16_minmax_u32<false>(cand);
+    }
     if (tid == 0) {
-        for (int w = 1; w < W; ++w)
-            if (better(sv[w], si[w], bv, bi, last_index)) { bv = sv[w]; bi = si[w]; }
         const uint32_t best = (bi == 0xFFFFFFFFu) ? 0u : bi;
         idx_out[row] = best;
         if (adv.cur_tok) {
