@@ -247,12 +247,10 @@ __global__ __launch_bounds__(256) void kv_append_kernel(const float *__restrict_
 
 // Arg-max of each row: one workgroup of 1024 threads per row, so no result crosses a workgroup.
 // Ties: the smaller index wins (last_index == 0) or the larger one.
-__device__ __forceinline__ bool better(float v, unsigned int i, float bv, unsigned int bi, int last_index) {
-    return (v > bv) || (v == bv && (last_index ? i > bi : i < bi));
-}
-
-// Every load of the row is in flight at once (up to 16 float4 per thread, 65536 columns; longer rows loop),
-// and the reductions are DPP: the maximum first, then the smallest (or largest) index among the lanes that hold it.
+// Two short phases instead of one long compare chain (the instruction cache is cold at every launch): the row
+// maximum first (every load of the row in flight at once: up to 16 float4 per thread, 65536 columns per round),
+// then the smallest (or largest) index among the elements equal to it.  NaN never wins; a row without any
+// comparable element gives index 0.
 constexpr int ARGMAX_UNROLL = 16;
 
 __global__ __launch_bounds__(1024) void argmax_rows_kernel(const float *__restrict__ x, uint32_t *idx_out, int cols,
@@ -262,56 +260,60 @@ __global__ __launch_bounds__(1024) void argmax_rows_kernel(const float *__restri
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6, T = blockDim.x;
     const int row = blockIdx.x;
     const float *xr = x + (size_t)row * row_stride;
-    float bv = -INFINITY;
-    unsigned int bi = last_index ? 0u : 0xFFFFFFFFu;
-    if ((((uintptr_t)xr) & 15) == 0) {
-        const int n4 = cols >> 2;
-        const float4 *x4 = reinterpret_cast<const float4 *>(xr);
-        for (int c0 = tid; c0 < n4; c0 += ARGMAX_UNROLL * T) {
-            float4 v[ARGMAX_UNROLL];
+    const bool vec = (((uintptr_t)xr) & 15) == 0 && cols <= 4 * ARGMAX_UNROLL * T;
+    const int n4 = vec ? cols >> 2 : 0;
+    const float4 *x4 = reinterpret_cast<const float4 *>(xr);
+    float4 v[ARGMAX_UNROLL];
+    float m = -INFINITY;
+    if (vec) {
 #pragma unroll
-            for (int u = 0; u < ARGMAX_UNROLL; ++u) {
-                const int c = c0 + u * T;
-                v[u] = x4[c < n4 ? c : c0];  // a repeated element changes nothing
-            }
+        for (int u = 0; u < ARGMAX_UNROLL; ++u) {
+            const int c = tid + u * T;
+            v[u] = c < n4 ? x4[c] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+        }
 #pragma unroll
-            for (int u = 0; u < ARGMAX_UNROLL; ++u) {
-                const int c = c0 + u * T;
-                const unsigned int base = 4u * (unsigned int)(c < n4 ? c : c0);
-                if (better(v[u].x, base, bv, bi, last_index)) { bv = v[u].x; bi = base; }
-                if (better(v[u].y, base + 1, bv, bi, last_index)) { bv = v[u].y; bi = base + 1; }
-                if (better(v[u].z, base + 2, bv, bi, last_index)) { bv = v[u].z; bi = base + 2; }
-                if (better(v[u].w, base + 3, bv, bi, last_index)) { bv = v[u].w; bi = base + 3; }
-            }
-        }
-        for (int c = 4 * n4 + tid; c < cols; c += T) {
-            const float v = xr[c];
-            if (better(v, (unsigned int)c, bv, bi, last_index)) { bv = v; bi = (unsigned int)c; }
-        }
-    } else {
-        for (int c = tid; c < cols; c += T) {
-            const float v = xr[c];
-            if (better(v, (unsigned int)c, bv, bi, last_index)) { bv = v; bi = (unsigned int)c; }
-        }
+        for (int u = 0; u < ARGMAX_UNROLL; ++u) m = fmaxf(fmaxf(m, fmaxf(v[u].x, v[u].y)), fmaxf(v[u].z, v[u].w));
     }
+    for (int c = 4 * n4 + tid; c < cols; c += T) m = fmaxf(m, xr[c]);
+    // phase 1: the row maximum
+    m = wave_max(m);
+    if (lane == 0) sv[wave] = m;
+    __syncthreads();
+    const float M = row16_max((lane & 15) < W ? sv[lane & 15] : -INFINITY);
+    // phase 2: the winning index among the elements equal to it
     const unsigned int none = last_index ? 0u : 0xFFFFFFFFu;
-    {
-        const float m = wave_max(bv);
-        const unsigned int cand = bv == m ? bi : none;
-        bi = last_index ? wave_minmax_u32<true>(cand) : wave_minmax_u32<false>(cand);
-        bv = m;
+    unsigned int lo = 0xFFFFFFFFu, hi = 0u;  // smallest / largest matching index of this thread
+    bool any = false;
+    if (vec) {
+#pragma unroll
+        for (int u = 0; u < ARGMAX_UNROLL; ++u) {
+            const unsigned int base = 4u * (unsigned int)(tid + u * T);
+            const float e[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (e[k] == M && (int)(tid + u * T) < n4) {
+                    lo = min(lo, base + k);
+                    hi = max(hi, base + k);
+                    any = true;
+                }
+        }
     }
-    if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
+    for (int c = 4 * n4 + tid; c < cols; c += T)
+        if (xr[c] == M) {
+            lo = min(lo, (unsigned int)c);
+            hi = max(hi, (unsigned int)c);
+            any = true;
+        }
+    unsigned int cand = any ? (last_index ? hi : lo) : none;
+    cand = last_index ? wave_minmax_u32<true>(cand) : wave_minmax_u32<false>(cand);
+    if (lane == 0) si[wave] = cand;
     __syncthreads();
     if (wave == 0) {
-        const int w = lane & 15;
-        const float v = w < W ? sv[w] : -INFINITY;
-        const float m = row16_max(v);
-        const unsigned int cand = (w < W && v == m) ? si[w] : none;
-        bi = last_index ? row16_minmax_u32<true>(cand) : row16_minmax_u32<false>(cand);
+        const unsigned int c = (lane & 15) < W ? si[lane & 15] : none;
+        cand = last_index ? row16_minmax_u32<true>(c) : row16_minmax_u32<false>(c);
     }
     if (tid == 0) {
-        const uint32_t best = (bi == 0xFFFFFFFFu) ? 0u : bi;
+        const uint32_t best = (cand == 0xFFFFFFFFu) ? 0u : cand;
         idx_out[row] = best;
         if (adv.cur_tok) {
             // token feed: the arg-max becomes the current token of this sequence and is recorded
