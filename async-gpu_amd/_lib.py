@@ -73,6 +73,7 @@ SIGNATURES = {
     "agpu_simple_rng_next_f32": (_f, [_vp]),
     "agpu_top_k_draw_host": (C.c_uint32, [_vp, _vp, _i32, _f]),
     "agpu_top_k_sample": (_i32, [_vp, _vp, _i32, _i32, _f, _vp, _vp]),
+    "agpu_softmax_max_prob": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp]),
     "agpu_split_qkv": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32]),
     "agpu_concat_heads": (_i32, [_vp, _vp, _vp, _i32, _i32, _i32]),
     "agpu_attention": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32]),
@@ -95,6 +96,8 @@ SIGNATURES = {
     "agpu_gpt2_generate_cached": (_i32, [_vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp]),
     "agpu_gpt2_generate": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, _vp]),
     "agpu_gpt2_generate_cached_sampling": (_i32, [_vp, _vp, _i32, _i32, _i32, _f, _vp, _i32, _vp, _vp]),
+    "agpu_gpt2_forward_early_exit": (_i32, [_vp, _vp, _i32, _f, _vp, _vp]),
+    "agpu_gpt2_generate_cached_early_exit": (_i32, [_vp, _vp, _i32, _i32, _f, _i32, _vp, _vp, _vp, _vp]),
     "agpu_gpt2_decode_steps": (_i32, [_vp, _i32, _i32, _vp]),
 }
 

@@ -16,6 +16,6 @@ struct ArgmaxAdvance {
 };
 
 int32_t agpu_argmax_rows_strided(agpu_ctx *ctx, const float *x, uint32_t *idx_out, int rows, int cols, int row_stride,
-                                 int last_index, const ArgmaxAdvance *adv);
+                                 int last_index, const ArgmaxAdvance *adv, float *conf_out = nullptr);
 int32_t agpu_layer_norm_impl(agpu_ctx *ctx, const float *x, const float *gamma, const float *beta, float *y,
                              int rows, int d, float eps);

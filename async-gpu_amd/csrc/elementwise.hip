@@ -251,11 +251,17 @@ __global__ __launch_bounds__(256) void kv_append_kernel(const float *__restrict_
 // maximum first (every load of the row in flight at once: up to 16 float4 per thread, 65536 columns per round),
 // then the smallest (or largest) index among the elements equal to it.  NaN never wins; a row without any
 // comparable element gives index 0.
+// CONF adds a third phase, softmax_max_prob (nn/models/gpt2.rs:983-988): conf_out[row] = 1 / sum(exp(x - M)), the
+// probability of the arg-max under the row's softmax.  The sum is a tree over the workgroup, so it carries less
+// rounding than the reference's sequential f32 sum (which drifts by ~5e-5 relative at 50257 terms).
 constexpr int ARGMAX_UNROLL = 16;
 
+template <bool CONF>
 __global__ __launch_bounds__(1024) void argmax_rows_kernel(const float *__restrict__ x, uint32_t *idx_out, int cols,
-                                                            int row_stride, int last_index, const ArgmaxAdvance adv) {
+                                                            int row_stride, int last_index, const ArgmaxAdvance adv,
+                                                            float *conf_out) {
     __shared__ float sv[16];
+    __shared__ float ss[16];
     __shared__ unsigned int si[16];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6, T = blockDim.x;
     const int row = blockIdx.x;
@@ -312,9 +318,26 @@ __global__ __launch_bounds__(1024) void argmax_rows_kernel(const float *__restri
         const unsigned int c = (lane & 15) < W ? si[lane & 15] : none;
         cand = last_index ? row16_minmax_u32<true>(c) : row16_minmax_u32<false>(c);
     }
+    if (CONF) {
+        float e = 0.0f;
+        if (vec) {
+#pragma unroll
+            for (int u = 0; u < ARGMAX_UNROLL; ++u)
+                if (tid + u * T < n4) e += (expf(v[u].x - M) + expf(v[u].y - M)) + (expf(v[u].z - M) + expf(v[u].w - M));
+        }
+        for (int c = 4 * n4 + tid; c < cols; c += T) e += expf(xr[c] - M);
+        e = wave_sum(e);
+        if (lane == 0) ss[wave] = e;
+        __syncthreads();
+        if (tid == 0) {
+            float t = 0.0f;
+            for (int w = 0; w < W; ++w) t += ss[w];
+            conf_out[row] = 1.0f / t;
+        }
+    }
     if (tid == 0) {
         const uint32_t best = (cand == 0xFFFFFFFFu) ? 0u : cand;
-        idx_out[row] = best;
+        if (idx_out) idx_out[row] = best;
         if (adv.cur_tok) {
             // token feed: the arg-max becomes the current token of this sequence and is recorded
             const int st = *adv.step_dev;
@@ -410,15 +433,29 @@ AGPU_EXPORT int32_t agpu_embedding(agpu_ctx *ctx, const uint32_t *tokens, const 
 }
 
 // Rows of `cols` values, `row_stride` floats apart; `adv` (optional) fuses the token feed.
+// conf_out (optional, [rows]) also receives the softmax probability of each row's arg-max.
 int32_t agpu_argmax_rows_strided(agpu_ctx *ctx, const float *x, uint32_t *idx_out, int rows, int cols, int row_stride,
-                                 int last_index, const ArgmaxAdvance *adv) {
+                                 int last_index, const ArgmaxAdvance *adv, float *conf_out) {
     ArgmaxAdvance a{};
     if (adv) a = *adv;
     int W = ceil_div(cols, 256);
     W = W < 1 ? 1 : (W > 16 ? 16 : W);
-    hipLaunchKernelGGL(argmax_rows_kernel, dim3(rows), dim3(64 * W), 0, ctx->stream, x, idx_out, cols, row_stride,
-                       last_index ? 1 : 0, a);
+    if (conf_out)
+        hipLaunchKernelGGL(argmax_rows_kernel<true>, dim3(rows), dim3(64 * W), 0, ctx->stream, x, idx_out, cols, row_stride,
+                           last_index ? 1 : 0, a, conf_out);
+    else
+        hipLaunchKernelGGL(argmax_rows_kernel<false>, dim3(rows), dim3(64 * W), 0, ctx->stream, x, idx_out, cols, row_stride,
+                           last_index ? 1 : 0, a, conf_out);
     return AGPU_LAUNCH_CHECK(ctx, "argmax_rows_kernel");
+}
+
+AGPU_EXPORT int32_t agpu_softmax_max_prob(agpu_ctx *ctx, const float *logits, int32_t rows, int32_t n, float *conf_out,
+                                          uint32_t *idx_out) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (!logits || !conf_out) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "softmax_max_prob: null pointer");
+    if (rows < 0 || n <= 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "softmax_max_prob: bad dims rows=%d n=%d", rows, n);
+    if (rows == 0) return AGPU_OK;
+    return agpu_argmax_rows_strided(ctx, logits, idx_out, rows, n, n, 0, nullptr, conf_out);
 }
 
 AGPU_EXPORT int32_t agpu_argmax_rows(agpu_ctx *ctx, const float *x, uint32_t *idx_out, int32_t rows, int32_t cols,
@@ -427,7 +464,7 @@ AGPU_EXPORT int32_t agpu_argmax_rows(agpu_ctx *ctx, const float *x, uint32_t *id
     if (!x || !idx_out) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "argmax_rows: null pointer");
     if (rows < 0 || cols <= 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "argmax_rows: bad dims rows=%d cols=%d", rows, cols);
     if (rows == 0) return AGPU_OK;
-    return agpu_argmax_rows_strided(ctx, x, idx_out, rows, cols, cols, last_index, nullptr);
+    return agpu_argmax_rows_strided(ctx, x, idx_out, rows, cols, cols, last_index, nullptr, nullptr);
 }
 
 AGPU_EXPORT int32_t agpu_split_qkv(agpu_ctx *ctx, const float *qkv, float *q, float *k, float *v, int32_t seq,

@@ -62,6 +62,10 @@ struct agpu_gpt2 {
     int *pos_dev = nullptr, *step_dev = nullptr;
     std::map<long long, hipGraphExec_t> graphs;  // key: batch << 32 | kv bucket
     hipEvent_t ev0 = nullptr, ev1 = nullptr, ev2 = nullptr;
+    // early exit: per block one (confidence, arg-max) pair in host-visible memory and one event
+    float *probe_conf_host = nullptr, *probe_conf_dev = nullptr;
+    uint32_t *probe_tok_host = nullptr, *probe_tok_dev = nullptr;
+    std::vector<hipEvent_t> probe_ev;
 };
 
 namespace {
@@ -103,6 +107,24 @@ __global__ __launch_bounds__(256) void gather_last_rows_kernel(const float *__re
 __global__ void advance_counters_kernel(int *pos_dev, int *step_dev, int delta) {
     *pos_dev += delta;
     *step_dev += 1;
+}
+
+// The token chosen on the host becomes the current token; the position advances by one.
+__global__ void feed_token_kernel(uint32_t *cur_tok, uint32_t token, int *pos_dev) {
+    cur_tok[0] = token;
+    *pos_dev += 1;
+}
+
+// Zero K and V rows of one sequence at the current position in blocks layer_from .. layer_from + gridDim.y - 1
+// (the blocks an early exit skipped, gpt2.rs:893-899).  One thread per element of a [H, 64] row pair.
+__global__ __launch_bounds__(256) void kv_zero_rows_kernel(float *kcache, float *vcache, size_t layer_stride, int layer_from,
+                                                            int H, int P, const int *pos_dev) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= H * DH) return;
+    const int h = i / DH, e = i % DH;
+    const size_t at = (size_t)(layer_from + blockIdx.y) * layer_stride + ((size_t)h * P + *pos_dev) * DH + e;
+    kcache[at] = 0.0f;
+    vcache[at] = 0.0f;
 }
 
 __global__ void set_counters_kernel(int *pos_dev, int pos, int *step_dev, int step) {
@@ -238,10 +260,15 @@ int32_t check_layer(agpu_gpt2 *m, int layer, int which, int K, int N) {
     return AGPU_OK;
 }
 
-// One forward over `new_len` tokens per sequence.  Every kernel reads the number of cached
-// positions from pos_dev, so the same launch sequence serves eager calls and graph replays.
-// max_kv bounds cache_len + new_len for sizing the attention key split.
-int32_t launch_forward(agpu_gpt2 *m, const uint32_t *tokens, int B, int new_len, int max_kv, bool all_rows_logits) {
+int32_t launch_embed(agpu_gpt2 *m, const uint32_t *tokens, int B, int new_len) {
+    const int R = B * new_len, d = m->d;
+    hipLaunchKernelGGL(embed_rows_kernel, dim3((unsigned)(((size_t)R * d + 255) / 256)), dim3(256), 0, m->ctx->stream, tokens,
+                       m->wte, m->wpe, (float *)m->hid.p, R, new_len, d, m->pos_dev);
+    return AGPU_LAUNCH_CHECK(m->ctx, "embed_rows_kernel");
+}
+
+// Block L on the hidden rows in place: x += Attn(LN1 x), x += FFN(LN2 x); its K and V rows go into the cache.
+int32_t launch_block(agpu_gpt2 *m, int L, int B, int new_len, int max_kv) {
     agpu_ctx *ctx = m->ctx;
     const int d = m->d, H = m->H, ff = m->ff, P = m->P, g = m->cfg.group_size;
     const int R = B * new_len;
@@ -249,79 +276,82 @@ int32_t launch_forward(agpu_gpt2 *m, const uint32_t *tokens, int B, int new_len,
     float *hid = (float *)m->hid.p, *qkv = (float *)m->qkv.p, *att = (float *)m->att.p, *ffn = (float *)m->ffn.p;
     const uint32_t gelu_flag = m->cfg.gelu == AGPU_GELU_QUICK ? AGPU_EPI_GELU_QUICK : AGPU_EPI_GELU_TANH;
     int32_t rc;
-
-    hipLaunchKernelGGL(embed_rows_kernel, dim3((unsigned)(((size_t)R * d + 255) / 256)), dim3(256), 0, ctx->stream, tokens,
-                       m->wte, m->wpe, hid, R, new_len, d, m->pos_dev);
-    if ((rc = AGPU_LAUNCH_CHECK(ctx, "embed_rows_kernel")) != AGPU_OK) return rc;
-
     const size_t layer_stride = (size_t)m->cfg.max_batch * H * P * DH;
-    for (int L = 0; L < m->cfg.n_layer; ++L) {
-        const Block &b = m->blocks[L];
-        const Int4Lin &wq = b.lin[AGPU_LINEAR_QKV], &wp = b.lin[AGPU_LINEAR_PROJ], &wf = b.lin[AGPU_LINEAR_FC],
-                      &wo = b.lin[AGPU_LINEAR_FC_PROJ];
-        float *kc = m->kcache + L * layer_stride, *vc = m->vcache + L * layer_stride;
-        if (new_len == 1 && R <= 16 && g % 8 == 0 && agpu_int4_gemv_can_fuse_ln(R, d)) {
-            // decode: LN1 + QKV + bias with the K/V rows written straight into the cache
-            GemvArgs ga{};
-            ga.x = hid; ga.packed = wq.packed; ga.scales = wq.scales; ga.bias = wq.bias; ga.residual = nullptr; ga.y = qkv;
-            ga.ln_gamma = b.ln1_g; ga.ln_beta = b.ln1_b; ga.ln_eps = eps;
-            ga.M = R; ga.N = 3 * d; ga.K = d; ga.group = g; ga.flags = 0;
-            ga.kcache = kc; ga.vcache = vc; ga.pos_dev = m->pos_dev; ga.n_heads = H; ga.n_positions = P;
-            if ((rc = agpu_int4_gemv_launch(ctx, ga)) != AGPU_OK) return rc;
-        } else if (new_len == 1 && R <= 16 && g % 8 == 0) {
-            // batched decode: LayerNorm on its own, then the QKV projection writes the K/V rows itself
-            if ((rc = agpu_layer_norm_impl(ctx, hid, b.ln1_g, b.ln1_b, (float *)m->lnb.p, R, d, eps)) != AGPU_OK) return rc;
-            GemvArgs ga{};
-            ga.x = (const float *)m->lnb.p; ga.packed = wq.packed; ga.scales = wq.scales; ga.bias = wq.bias; ga.y = qkv;
-            ga.M = R; ga.N = 3 * d; ga.K = d; ga.group = g; ga.flags = 0;
-            ga.kcache = kc; ga.vcache = vc; ga.pos_dev = m->pos_dev; ga.n_heads = H; ga.n_positions = P;
-            rc = agpu_int4_skinny_supported(ga) ? agpu_int4_skinny_launch(ctx, ga) : agpu_int4_gemv_launch(ctx, ga);
-            if (rc != AGPU_OK) return rc;
-        } else {
-            rc = agpu_ln_int4_linear(ctx, hid, b.ln1_g, b.ln1_b, eps, wq.packed, wq.scales, wq.bias, nullptr, qkv, R,
-                                     3 * d, d, g, 0);
-            if (rc != AGPU_OK) return rc;
-            hipLaunchKernelGGL(kv_scatter_kernel, dim3((unsigned)(((size_t)R * d + 255) / 256)), dim3(256), 0, ctx->stream,
-                               qkv, kc, vc, R, new_len, H, P, m->pos_dev);
-            if ((rc = AGPU_LAUNCH_CHECK(ctx, "kv_scatter_kernel")) != AGPU_OK) return rc;
-        }
-        AttnParams ap{};
-        ap.q = qkv; ap.k = kc; ap.v = vc; ap.o = att;
-        ap.n_heads = H; ap.batch = B; ap.q_len = new_len; ap.kv_len = 0; ap.q_offset = 0; ap.kv_stride = P; ap.causal = 1;
-        ap.q_batch_stride = (long long)new_len * 3 * d; ap.q_head_stride = DH; ap.q_row_stride = 3 * d;
-        ap.o_batch_stride = (long long)new_len * d; ap.o_head_stride = DH; ap.o_row_stride = d;
-        ap.pos_dev = m->pos_dev;
-        if ((rc = agpu_attention_launch(ctx, ap, max_kv)) != AGPU_OK) return rc;
-        rc = agpu_int4_linear(ctx, att, wp.packed, wp.scales, wp.bias, hid, hid, R, d, d, g, 0);
+    const Block &b = m->blocks[L];
+    const Int4Lin &wq = b.lin[AGPU_LINEAR_QKV], &wp = b.lin[AGPU_LINEAR_PROJ], &wf = b.lin[AGPU_LINEAR_FC],
+                  &wo = b.lin[AGPU_LINEAR_FC_PROJ];
+    float *kc = m->kcache + L * layer_stride, *vc = m->vcache + L * layer_stride;
+    if (new_len == 1 && R <= 16 && g % 8 == 0 && agpu_int4_gemv_can_fuse_ln(R, d)) {
+        // decode: LN1 + QKV + bias with the K/V rows written straight into the cache
+        GemvArgs ga{};
+        ga.x = hid; ga.packed = wq.packed; ga.scales = wq.scales; ga.bias = wq.bias; ga.residual = nullptr; ga.y = qkv;
+        ga.ln_gamma = b.ln1_g; ga.ln_beta = b.ln1_b; ga.ln_eps = eps;
+        ga.M = R; ga.N = 3 * d; ga.K = d; ga.group = g; ga.flags = 0;
+        ga.kcache = kc; ga.vcache = vc; ga.pos_dev = m->pos_dev; ga.n_heads = H; ga.n_positions = P;
+        if ((rc = agpu_int4_gemv_launch(ctx, ga)) != AGPU_OK) return rc;
+    } else if (new_len == 1 && R <= 16 && g % 8 == 0) {
+        // batched decode: LayerNorm on its own, then the QKV projection writes the K/V rows itself
+        if ((rc = agpu_layer_norm_impl(ctx, hid, b.ln1_g, b.ln1_b, (float *)m->lnb.p, R, d, eps)) != AGPU_OK) return rc;
+        GemvArgs ga{};
+        ga.x = (const float *)m->lnb.p; ga.packed = wq.packed; ga.scales = wq.scales; ga.bias = wq.bias; ga.y = qkv;
+        ga.M = R; ga.N = 3 * d; ga.K = d; ga.group = g; ga.flags = 0;
+        ga.kcache = kc; ga.vcache = vc; ga.pos_dev = m->pos_dev; ga.n_heads = H; ga.n_positions = P;
+        rc = agpu_int4_skinny_supported(ga) ? agpu_int4_skinny_launch(ctx, ga) : agpu_int4_gemv_launch(ctx, ga);
         if (rc != AGPU_OK) return rc;
-        rc = agpu_ln_int4_linear(ctx, hid, b.ln2_g, b.ln2_b, eps, wf.packed, wf.scales, wf.bias, nullptr, ffn, R, ff, d, g,
-                                 gelu_flag);
-        if (rc != AGPU_OK) return rc;
-        rc = agpu_int4_linear(ctx, ffn, wo.packed, wo.scales, wo.bias, hid, hid, R, d, ff, g, 0);
-        if (rc != AGPU_OK) return rc;
-    }
-
-    // final LayerNorm + LM head on the rows whose logits are wanted
-    const float *head_in = hid;
-    int Rl = R;
-    if (!all_rows_logits && new_len > 1) {
-        hipLaunchKernelGGL(gather_last_rows_kernel, dim3((unsigned)(((size_t)B * d + 255) / 256)), dim3(256), 0, ctx->stream,
-                           hid, (float *)m->last.p, B, new_len, d);
-        if ((rc = AGPU_LAUNCH_CHECK(ctx, "gather_last_rows_kernel")) != AGPU_OK) return rc;
-        head_in = (float *)m->last.p;
-        Rl = B;
-    } else if (!all_rows_logits) {
-        Rl = B;
-    }
-    float *logits = (float *)m->logits.p;
-    if (m->cfg.lm_head == AGPU_LM_HEAD_INT4) {
-        rc = agpu_ln_int4_linear(ctx, head_in, m->lnf_g, m->lnf_b, eps, m->lm_head.packed, m->lm_head.scales, nullptr, nullptr,
-                                 logits, Rl, m->Vpad, d, g, 0);
     } else {
-        rc = agpu_layer_norm(ctx, head_in, m->lnf_g, m->lnf_b, (float *)m->lnb.p, Rl, d, eps);
-        if (rc == AGPU_OK) rc = agpu_gemm_f32(ctx, (float *)m->lnb.p, m->wte_t, logits, Rl, m->V, d);
+        rc = agpu_ln_int4_linear(ctx, hid, b.ln1_g, b.ln1_b, eps, wq.packed, wq.scales, wq.bias, nullptr, qkv, R, 3 * d, d, g,
+                                 0);
+        if (rc != AGPU_OK) return rc;
+        hipLaunchKernelGGL(kv_scatter_kernel, dim3((unsigned)(((size_t)R * d + 255) / 256)), dim3(256), 0, ctx->stream, qkv, kc,
+                           vc, R, new_len, H, P, m->pos_dev);
+        if ((rc = AGPU_LAUNCH_CHECK(ctx, "kv_scatter_kernel")) != AGPU_OK) return rc;
     }
+    AttnParams ap{};
+    ap.q = qkv; ap.k = kc; ap.v = vc; ap.o = att;
+    ap.n_heads = H; ap.batch = B; ap.q_len = new_len; ap.kv_len = 0; ap.q_offset = 0; ap.kv_stride = P; ap.causal = 1;
+    ap.q_batch_stride = (long long)new_len * 3 * d; ap.q_head_stride = DH; ap.q_row_stride = 3 * d;
+    ap.o_batch_stride = (long long)new_len * d; ap.o_head_stride = DH; ap.o_row_stride = d;
+    ap.pos_dev = m->pos_dev;
+    if ((rc = agpu_attention_launch(ctx, ap, max_kv)) != AGPU_OK) return rc;
+    rc = agpu_int4_linear(ctx, att, wp.packed, wp.scales, wp.bias, hid, hid, R, d, d, g, 0);
+    if (rc != AGPU_OK) return rc;
+    rc = agpu_ln_int4_linear(ctx, hid, b.ln2_g, b.ln2_b, eps, wf.packed, wf.scales, wf.bias, nullptr, ffn, R, ff, d, g, gelu_flag);
+    if (rc != AGPU_OK) return rc;
+    return agpu_int4_linear(ctx, ffn, wo.packed, wo.scales, wo.bias, hid, hid, R, d, ff, g, 0);
+}
+
+// Final LayerNorm + LM head on `rows` rows of head_in -> m->logits.
+int32_t launch_head(agpu_gpt2 *m, const float *head_in, int rows) {
+    agpu_ctx *ctx = m->ctx;
+    const int d = m->d, g = m->cfg.group_size;
+    const float eps = m->cfg.layer_norm_epsilon;
+    float *logits = (float *)m->logits.p;
+    if (m->cfg.lm_head == AGPU_LM_HEAD_INT4)
+        return agpu_ln_int4_linear(ctx, head_in, m->lnf_g, m->lnf_b, eps, m->lm_head.packed, m->lm_head.scales, nullptr, nullptr,
+                                   logits, rows, m->Vpad, d, g, 0);
+    int32_t rc = agpu_layer_norm(ctx, head_in, m->lnf_g, m->lnf_b, (float *)m->lnb.p, rows, d, eps);
+    if (rc == AGPU_OK) rc = agpu_gemm_f32(ctx, (float *)m->lnb.p, m->wte_t, logits, rows, m->V, d);
     return rc;
+}
+
+int32_t launch_gather_last(agpu_gpt2 *m, int B, int new_len) {
+    hipLaunchKernelGGL(gather_last_rows_kernel, dim3((unsigned)(((size_t)B * m->d + 255) / 256)), dim3(256), 0, m->ctx->stream,
+                       (float *)m->hid.p, (float *)m->last.p, B, new_len, m->d);
+    return AGPU_LAUNCH_CHECK(m->ctx, "gather_last_rows_kernel");
+}
+
+// One forward over `new_len` tokens per sequence.  Every kernel reads the number of cached
+// positions from pos_dev, so the same launch sequence serves eager calls and graph replays.
+// max_kv bounds cache_len + new_len for sizing the attention key split.
+int32_t launch_forward(agpu_gpt2 *m, const uint32_t *tokens, int B, int new_len, int max_kv, bool all_rows_logits) {
+    int32_t rc = launch_embed(m, tokens, B, new_len);
+    for (int L = 0; rc == AGPU_OK && L < m->cfg.n_layer; ++L) rc = launch_block(m, L, B, new_len, max_kv);
+    if (rc != AGPU_OK) return rc;
+    // final LayerNorm + LM head on the rows whose logits are wanted
+    if (all_rows_logits) return launch_head(m, (float *)m->hid.p, B * new_len);
+    if (new_len == 1) return launch_head(m, (float *)m->hid.p, B);
+    if ((rc = launch_gather_last(m, B, new_len)) != AGPU_OK) return rc;
+    return launch_head(m, (float *)m->last.p, B);
 }
 
 int logits_stride(const agpu_gpt2 *m) { return m->cfg.lm_head == AGPU_LM_HEAD_INT4 ? m->Vpad : m->V; }
@@ -434,6 +464,69 @@ int32_t run_decode_steps(agpu_gpt2 *m, int B, int steps) {
     return AGPU_OK;
 }
 
+int32_t ensure_probes(agpu_gpt2 *m) {
+    if (m->probe_conf_host) return AGPU_OK;
+    agpu_ctx *ctx = m->ctx;
+    const size_t n = (size_t)m->cfg.n_layer;
+    hipError_t e = hipHostMalloc((void **)&m->probe_conf_host, n * sizeof(float), hipHostMallocMapped);
+    if (e == hipSuccess) e = hipHostMalloc((void **)&m->probe_tok_host, n * sizeof(uint32_t), hipHostMallocMapped);
+    if (e == hipSuccess) e = hipHostGetDevicePointer((void **)&m->probe_conf_dev, m->probe_conf_host, 0);
+    if (e == hipSuccess) e = hipHostGetDevicePointer((void **)&m->probe_tok_dev, m->probe_tok_host, 0);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipHostMalloc(probes)");
+    m->probe_ev.assign(n, nullptr);
+    for (size_t i = 0; i < n; ++i)
+        if ((e = hipEventCreateWithFlags(&m->probe_ev[i], hipEventDisableTiming)) != hipSuccess)
+            return agpu_hip(ctx, e, "hipEventCreateWithFlags");
+    return AGPU_OK;
+}
+
+// Confidence and arg-max of logits row 0 into probe slot L, then the slot's event.
+int32_t launch_probe(agpu_gpt2 *m, int L) {
+    int32_t rc = agpu_argmax_rows_strided(m->ctx, (float *)m->logits.p, m->probe_tok_dev + L, 1, m->V, logits_stride(m),
+                                          m->cfg.argmax_last, nullptr, m->probe_conf_dev + L);
+    if (rc != AGPU_OK) return rc;
+    return agpu_hip(m->ctx, hipEventRecord(m->probe_ev[L], m->ctx->stream), "hipEventRecord");
+}
+
+int32_t wait_probe(agpu_gpt2 *m, int L) { return agpu_hip(m->ctx, hipEventSynchronize(m->probe_ev[L]), "hipEventSynchronize"); }
+
+// One decode step of generate_cached_early_exit.  Block L+1 is launched before the host looks at probe L, so the
+// device never idles for a round trip; when probe L ends the step, what block L+1 wrote is discarded: its K/V rows
+// are zeroed with those of the other skipped blocks and the hidden state is rebuilt from the next token.
+int32_t early_exit_step(agpu_gpt2 *m, float threshold, int *used_out, uint32_t *token_out) {
+    agpu_ctx *ctx = m->ctx;
+    const int nl = m->cfg.n_layer, bucket = kv_bucket(m, m->cache_len + 1);
+    int32_t rc = launch_embed(m, m->cur_tok, 1, 1);
+    int used = nl;
+    for (int L = 0; rc == AGPU_OK && L < nl; ++L) {
+        if ((rc = launch_block(m, L, 1, 1, bucket)) != AGPU_OK) break;
+        if ((rc = launch_head(m, (float *)m->hid.p, 1)) != AGPU_OK) break;
+        if ((rc = launch_probe(m, L)) != AGPU_OK) break;
+        if (L >= 1) {
+            if ((rc = wait_probe(m, L - 1)) != AGPU_OK) break;
+            if (m->probe_conf_host[L - 1] >= threshold) {
+                used = L;
+                break;
+            }
+        }
+    }
+    if (rc != AGPU_OK) return rc;
+    if ((rc = wait_probe(m, used - 1)) != AGPU_OK) return rc;
+    const uint32_t token = m->probe_tok_host[used - 1];
+    if (used < nl) {
+        const size_t layer_stride = (size_t)m->cfg.max_batch * m->H * m->P * DH;
+        hipLaunchKernelGGL(kv_zero_rows_kernel, dim3((unsigned)ceil_div(m->H * DH, 256), (unsigned)(nl - used)), dim3(256), 0,
+                           ctx->stream, m->kcache, m->vcache, layer_stride, used, m->H, m->P, m->pos_dev);
+        if ((rc = AGPU_LAUNCH_CHECK(ctx, "kv_zero_rows_kernel")) != AGPU_OK) return rc;
+    }
+    hipLaunchKernelGGL(feed_token_kernel, dim3(1), dim3(1), 0, ctx->stream, m->cur_tok, token, m->pos_dev);
+    if ((rc = AGPU_LAUNCH_CHECK(ctx, "feed_token_kernel")) != AGPU_OK) return rc;
+    m->cache_len += 1;
+    *used_out = used;
+    *token_out = token;
+    return AGPU_OK;
+}
+
 void fill_config(agpu_gpt2_config *c, int n_layer, int n_embd, int n_head) {
     c->n_layer = n_layer;
     c->n_embd = n_embd;
@@ -522,6 +615,10 @@ AGPU_EXPORT int32_t agpu_gpt2_destroy(agpu_gpt2 *m) {
         if (p) (void)hipFree(p);
     for (hipEvent_t e : {m->ev0, m->ev1, m->ev2})
         if (e) (void)hipEventDestroy(e);
+    for (hipEvent_t e : m->probe_ev)
+        if (e) (void)hipEventDestroy(e);
+    if (m->probe_conf_host) (void)hipHostFree(m->probe_conf_host);
+    if (m->probe_tok_host) (void)hipHostFree(m->probe_tok_host);
     agpu_ctx_release(m->ctx);
     delete m;
     return AGPU_OK;
@@ -798,6 +895,94 @@ AGPU_EXPORT int32_t agpu_gpt2_generate_cached_sampling(agpu_gpt2 *m, const uint3
     (void)hipFree(idx_dev);
     (void)hipFree(val_dev);
     *length_out_host = len;
+    return rc;
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_forward_early_exit(agpu_gpt2 *m, const uint32_t *tokens, int32_t seq_len, float threshold,
+                                                 float *logits_out, int32_t *layers_used_out_host) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    agpu_ctx *ctx = m->ctx;
+    if (!tokens || !layers_used_out_host) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "gpt2_forward_early_exit: null pointer");
+    if (seq_len <= 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_forward_early_exit: seq_len must be positive");
+    if (seq_len > m->P)
+        return agpu_fail(ctx, AGPU_ERR_DIM_OUT_OF_RANGE, "gpt2_forward_early_exit: %d tokens exceed n_positions %d", seq_len, m->P);
+    int32_t rc = check_ready(m);
+    if (rc == AGPU_OK) rc = ensure_probes(m);
+    if (rc == AGPU_OK) rc = ensure_buffers(m, 1, seq_len, true);
+    if (rc == AGPU_OK) rc = agpu_gpt2_reset_cache(m);
+    if (rc == AGPU_OK) rc = launch_embed(m, tokens, 1, seq_len);
+    const int nl = m->cfg.n_layer;
+    int used = nl;
+    for (int L = 0; rc == AGPU_OK && L < nl; ++L) {
+        if ((rc = launch_block(m, L, 1, seq_len, seq_len)) != AGPU_OK || L + 1 == nl) break;
+        // confidence of the last position (gpt2.rs:814-819); the other rows' logits are only needed at the end
+        const float *head_in = (float *)m->hid.p;
+        if (seq_len > 1) {
+            if ((rc = launch_gather_last(m, 1, seq_len)) != AGPU_OK) break;
+            head_in = (float *)m->last.p;
+        }
+        if ((rc = launch_head(m, head_in, 1)) != AGPU_OK) break;
+        if ((rc = launch_probe(m, L)) != AGPU_OK) break;
+        if ((rc = wait_probe(m, L)) != AGPU_OK) break;
+        if (m->probe_conf_host[L] >= threshold) {
+            used = L + 1;
+            break;
+        }
+    }
+    if (rc != AGPU_OK) return rc;
+    *layers_used_out_host = used;
+    if (logits_out) {
+        if ((rc = launch_head(m, (float *)m->hid.p, seq_len)) != AGPU_OK) return rc;
+        hipError_t e = hipMemcpy2DAsync(logits_out, (size_t)m->V * 4, m->logits.p, (size_t)logits_stride(m) * 4, (size_t)m->V * 4,
+                                        (size_t)seq_len, hipMemcpyDeviceToDevice, ctx->stream);
+        if (e != hipSuccess) return agpu_hip(ctx, e, "hipMemcpy2DAsync(logits)");
+    }
+    return AGPU_OK;  // the cache counters were never advanced: the cache is empty
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_generate_cached_early_exit(agpu_gpt2 *m, const uint32_t *prompt_host, int32_t prompt_len,
+                                                         int32_t max_new_tokens, float threshold, int32_t eos,
+                                                         uint32_t *tokens_out_host, int32_t *length_out_host,
+                                                         int32_t *layers_out_host, int32_t *steps_out_host) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    agpu_ctx *ctx = m->ctx;
+    if (!prompt_host || !tokens_out_host || !length_out_host || !layers_out_host || !steps_out_host)
+        return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "gpt2_generate_cached_early_exit: null pointer");
+    if (prompt_len <= 0 || max_new_tokens < 0)
+        return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_generate_cached_early_exit: bad prompt_len/max_new_tokens");
+    if (prompt_len + (max_new_tokens > 0 ? max_new_tokens - 1 : 0) > m->P)
+        return agpu_fail(ctx, AGPU_ERR_DIM_OUT_OF_RANGE,
+                         "gpt2_generate_cached_early_exit: prompt %d + %d new tokens exceed n_positions %d", prompt_len,
+                         max_new_tokens, m->P);
+    std::memcpy(tokens_out_host, prompt_host, (size_t)prompt_len * 4);
+    int len = prompt_len, steps = 0;
+    *length_out_host = len;
+    *steps_out_host = 0;
+    int32_t rc = check_ready(m);
+    if (rc == AGPU_OK) rc = ensure_probes(m);
+    if (rc == AGPU_OK) rc = ensure(m, m->tok_in, (size_t)prompt_len * 4);
+    if (rc == AGPU_OK) rc = ensure_buffers(m, 1, prompt_len, false);
+    if (rc == AGPU_OK) rc = ensure_out_tokens(m, m->P, 1);
+    if (rc == AGPU_OK) rc = upload(ctx, m->tok_in.p, prompt_host, (size_t)prompt_len * 4, 0);
+    if (rc == AGPU_OK) rc = agpu_gpt2_reset_cache(m);
+    // prefill: every layer (gpt2.rs:849-857); its arg-max is already the current token on the device
+    if (rc == AGPU_OK) rc = agpu_gpt2_forward_cached(m, (const uint32_t *)m->tok_in.p, 1, prompt_len, nullptr, 0);
+    uint32_t next = 0;
+    if (rc == AGPU_OK) rc = agpu_memcpy_d2h(ctx, &next, m->next_tok, 4);
+    if (rc != AGPU_OK) return rc;
+    layers_out_host[steps++] = m->cfg.n_layer;
+    if (!(eos >= 0 && next == (uint32_t)eos)) {
+        tokens_out_host[len++] = next;
+        for (int t = 1; t < max_new_tokens; ++t) {
+            int used = 0;
+            if ((rc = early_exit_step(m, threshold, &used, &next)) != AGPU_OK) break;
+            layers_out_host[steps++] = used;
+            if (eos >= 0 && next == (uint32_t)eos) break;  // gpt2.rs:915-917
+            tokens_out_host[len++] = next;
+        }
+    }
+    *length_out_host = len;
+    *steps_out_host = steps;
     return rc;
 }
 

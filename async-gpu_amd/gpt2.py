@@ -200,6 +200,35 @@ class Int4Gpt2Model:
                    C.addressof(rng._s), eos, out, C.addressof(n))
         return out[: n.value].copy()
 
+    def forward_early_exit(self, tokens, threshold):
+        """Gpt2Model::forward_early_exit (gpt2.rs:797-830) -> (logits [seq, V] numpy, layers used)."""
+        tokens = _np(tokens, np.uint32).ravel()
+        V = self.config.vocab_size
+        p, lg = C.c_void_p(), C.c_void_p()
+        self.ctx.call("agpu_malloc", tokens.nbytes, C.byref(p))
+        self.ctx.call("agpu_malloc", tokens.size * V * 4, C.byref(lg))
+        used = C.c_int32(0)
+        try:
+            self.ctx.call("agpu_memcpy_h2d", p.value, tokens, tokens.nbytes)
+            self._call("agpu_gpt2_forward_early_exit", p.value, tokens.size, float(threshold), lg.value, C.addressof(used))
+            out = np.empty((tokens.size, V), np.float32)
+            self.ctx.call("agpu_memcpy_d2h", out, lg.value, out.nbytes)
+        finally:
+            self.ctx.call("agpu_free", p.value)
+            self.ctx.call("agpu_free", lg.value)
+        return out, int(used.value)
+
+    def generate_cached_early_exit(self, prompt, max_new_tokens, threshold, eos=50256):
+        """Gpt2Model::generate_cached_early_exit (gpt2.rs:837-922) -> (tokens, blocks used per step)."""
+        prompt = _np(prompt, np.uint32).ravel()
+        rows = max(int(max_new_tokens), 1)
+        out = np.zeros(prompt.size + rows, np.uint32)
+        layers = np.zeros(rows, np.int32)
+        n, steps = C.c_int32(0), C.c_int32(0)
+        self._call("agpu_gpt2_generate_cached_early_exit", prompt, prompt.size, int(max_new_tokens), float(threshold), eos, out,
+                   C.addressof(n), layers, C.addressof(steps))
+        return out[: n.value].copy(), layers[: steps.value].copy()
+
     def generate(self, prompt, max_new_tokens, eos=50256):
         prompt = _np(prompt, np.uint32).ravel()
         out = np.zeros(prompt.size + max_new_tokens, np.uint32)

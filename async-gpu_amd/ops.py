@@ -216,6 +216,18 @@ def top_k(logits, k, temperature=1.0):
     return idx, val
 
 
+def softmax_max_prob(logits):
+    """softmax_max_prob (gpt2.rs:983-988) per row of device logits: (confidence [rows] f32, arg-max [rows] int32 view)."""
+    import torch
+
+    lg = logits.contiguous().view(-1, logits.shape[-1])
+    rows, n = lg.shape
+    conf = torch.empty(rows, dtype=torch.float32, device=lg.device)
+    idx = torch.empty(rows, dtype=torch.int32, device=lg.device)
+    context(lg.device.index or 0).call("agpu_softmax_max_prob", lg, rows, n, conf, idx)
+    return conf, idx
+
+
 def top_k_sample(logits, k, temperature, rng):
     """top_k_sample (gpt2.rs:1029-1058) on a device logit vector; advances rng; returns the token id."""
     import ctypes as C

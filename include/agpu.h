@@ -190,6 +190,13 @@ uint32_t agpu_top_k_draw_host(const float *ranked_vals, const uint32_t *ranked_i
  * k (index, value) pairs to the host, draw with the next value of the generator.  *token_out_host on the host. */
 int32_t agpu_top_k_sample(agpu_ctx *ctx, const float *logits, int32_t n, int32_t k, float temperature,
                           uint64_t *rng_state, uint32_t *token_out_host);
+/* softmax_max_prob (gpt2.rs:983-988), the confidence probed by the early-exit callers: conf_out[row] =
+ * 1 / sum_j exp(logits[row, j] - max_j logits[row, j]), the softmax probability of the row's arg-max; idx_out
+ * (optional) receives that arg-max (first index among equals).  Device pointers; conf_out [rows], idx_out [rows].
+ * The reference downloads the row and sums sequentially in f32; the sum here is a tree, so the two agree to
+ * the rounding of the reference's sum (about 5e-5 relative at 50257 columns). */
+int32_t agpu_softmax_max_prob(agpu_ctx *ctx, const float *logits, int32_t rows, int32_t n, float *conf_out,
+                              uint32_t *idx_out);
 
 /* ---- attention ------------------------------------------------------------------------- */
 

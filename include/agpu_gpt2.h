@@ -111,6 +111,34 @@ int32_t agpu_gpt2_generate_cached_sampling(agpu_gpt2 *m, const uint32_t *prompt_
                                            int32_t eos, uint32_t *tokens_out_host, int32_t *length_out_host);
 
 /*
+ * Gpt2Model::forward_early_exit (gpt2.rs:797-830): uncached forward over seq_len tokens (device ids) that stops
+ * after the first block whose confidence (agpu_softmax_max_prob of the last row's logits behind the final
+ * LayerNorm and the LM head) reaches `threshold`; the last block is never probed.  logits_out (device,
+ * [seq_len, vocab], optional) receives the logits of every row at the layer that ended the forward;
+ * *layers_used_out_host = 1..n_layer.  The confidence crosses to the host as one float per probed layer instead
+ * of the reference's [seq_len, vocab] download.  The KV cache is left empty.
+ */
+int32_t agpu_gpt2_forward_early_exit(agpu_gpt2 *m, const uint32_t *tokens, int32_t seq_len, float threshold,
+                                     float *logits_out, int32_t *layers_used_out_host);
+
+/*
+ * Gpt2Model::generate_cached_early_exit (gpt2.rs:837-922): prefill with every layer, then per token the blocks
+ * run until an intermediate confidence reaches `threshold`; the blocks skipped get zero K and V rows at that
+ * position, and the token is the arg-max of the logits at the layer that ended the step.  One sequence.
+ * As in the reference the first token comes from the prefill whatever max_new_tokens is, and a token equal to
+ * `eos` ends the sequence before it is appended (eos < 0: never) while its step is still counted.
+ *   tokens_out_host [prompt_len + max(max_new_tokens, 1)], *length_out_host = tokens written;
+ *   layers_out_host [max(max_new_tokens, 1)] = blocks used per step (the prefill first), *steps_out_host = entries.
+ * The number of launches per step depends on the data, so the steps are not graph replays; each probe sends 8 bytes
+ * (confidence, arg-max) to host-visible memory, and the host checks probe i while block i+1 already runs (its
+ * results are discarded when probe i ends the step), so no step waits for a round trip per layer.
+ */
+int32_t agpu_gpt2_generate_cached_early_exit(agpu_gpt2 *m, const uint32_t *prompt_host, int32_t prompt_len,
+                                             int32_t max_new_tokens, float threshold, int32_t eos,
+                                             uint32_t *tokens_out_host, int32_t *length_out_host,
+                                             int32_t *layers_out_host, int32_t *steps_out_host);
+
+/*
  * Benchmark hook: replay `steps` decode steps (one token per sequence per step) starting from the
  * current cache state and the device-resident current tokens, without any host round trip, and
  * report the time per step measured with HIP events on the context's stream.  The cache advances by

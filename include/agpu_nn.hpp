@@ -18,6 +18,7 @@
 #include <optional>
 #include <stdexcept>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "agpu.h"
@@ -518,6 +519,32 @@ public:
                                                        temperature, rng.state(), eos, out.data(), &len));
         out.resize((size_t)len);
         return out;
+    }
+    // generate_cached_early_exit (gpt2.rs:837-922) -> (tokens, blocks used per step)
+    std::pair<std::vector<uint32_t>, std::vector<size_t>> generate_cached_early_exit(const std::vector<uint32_t> &prompt,
+                                                                                     size_t max_new_tokens, float threshold,
+                                                                                     int eos = 50256) const {
+        const size_t rows = max_new_tokens > 0 ? max_new_tokens : 1;
+        std::vector<uint32_t> out(prompt.size() + rows);
+        std::vector<int32_t> layers(rows);
+        int32_t len = 0, steps = 0;
+        reg_->check(agpu_gpt2_generate_cached_early_exit(h_, prompt.data(), (int32_t)prompt.size(), (int32_t)max_new_tokens, threshold,
+                                                         eos, out.data(), &len, layers.data(), &steps));
+        out.resize((size_t)len);
+        return {out, std::vector<size_t>(layers.begin(), layers.begin() + steps)};
+    }
+    // forward_early_exit (gpt2.rs:797-830) -> (logits [seq, vocab], layers used); tokens on the host
+    std::pair<GpuTensor, size_t> forward_early_exit(const std::vector<uint32_t> &tokens, float threshold) const {
+        void *ids = nullptr;
+        reg_->check(agpu_malloc(reg_->device(), tokens.size() * 4, &ids));
+        GpuTensor logits = GpuTensor::zeros({tokens.size(), config_.vocab_size}, reg_);
+        int32_t used = 0;
+        int32_t rc = agpu_memcpy_h2d(reg_->device(), ids, tokens.data(), tokens.size() * 4);
+        if (rc == AGPU_OK)
+            rc = agpu_gpt2_forward_early_exit(h_, (const uint32_t *)ids, (int32_t)tokens.size(), threshold, logits.data(), &used);
+        (void)agpu_free(reg_->device(), ids);
+        reg_->check(rc);
+        return {logits, (size_t)used};
     }
     // quantized_memory_bytes (gpt2.rs:1565-1577)
     size_t quantized_memory_bytes() const { return (size_t)agpu_gpt2_quantized_memory_bytes(h_); }

@@ -604,6 +604,112 @@ static void layer_norm_d(const double *x, const float *g, const float *b, double
 ORC_API void orc_gpt2_reset_cache(orc_gpt2 *m) { m->kv_len = 0; }
 ORC_API int orc_gpt2_cache_len(const orc_gpt2 *m) { return m->kv_len; }
 
+typedef struct {
+    double *hid, *ln, *qkv, *att, *tmp, *ffn;
+} orc_work;
+
+static void work_alloc(const orc_gpt2 *m, orc_work *w, int new_len) {
+    const size_t d = (size_t)m->n_embd, n = (size_t)new_len;
+    w->hid = (double *)malloc(sizeof(double) * n * d);
+    w->ln = (double *)malloc(sizeof(double) * n * d);
+    w->qkv = (double *)malloc(sizeof(double) * n * 3 * d);
+    w->att = (double *)malloc(sizeof(double) * n * d);
+    w->tmp = (double *)malloc(sizeof(double) * n * d);
+    w->ffn = (double *)malloc(sizeof(double) * n * (size_t)m->d_ffn);
+}
+
+static void work_free(orc_work *w) {
+    free(w->hid); free(w->ln); free(w->qkv); free(w->att); free(w->tmp); free(w->ffn);
+}
+
+static void cache_alloc(orc_gpt2 *m) {
+    if (m->kc) return;
+    const size_t n = (size_t)m->n_layer * m->n_head * m->n_positions * m->d_head;
+    m->kc = (double *)malloc(sizeof(double) * n);
+    m->vc = (double *)malloc(sizeof(double) * n);
+}
+
+/* wte[token] + wpe[position] (compute_transformer.rs:1320-1329) */
+static void embed_rows(const orc_gpt2 *m, const uint32_t *tokens, int new_len, int pos0, double *hid) {
+    const int d = m->n_embd;
+    for (int p = 0; p < new_len; ++p)
+        for (int j = 0; j < d; ++j)
+            hid[(size_t)p * d + j] = (double)m->wte[(size_t)tokens[p] * d + j] + (double)m->wpe[(size_t)(pos0 + p) * d + j];
+}
+
+/* One pre-LN block on rows at positions pos0.. (tests_inference.rs:3746-3850): the K and V rows go into the
+ * cache of layer L, attention runs over keys 0..pos0+s for row s. */
+static void run_block(orc_gpt2 *m, int L, orc_work *w, int new_len, int pos0) {
+    const int d = m->n_embd, H = m->n_head, dh = m->d_head, ff = m->d_ffn, P = m->n_positions;
+    double *hid = w->hid, *ln = w->ln, *qkv = w->qkv, *att = w->att, *tmp = w->tmp, *ffn = w->ffn;
+    const double scale = 1.0 / sqrt((double)dh);
+    const orc_block *b = &m->blocks[L];
+    layer_norm_d(hid, b->ln1_g, b->ln1_b, ln, new_len, d, m->eps);
+    linear_f64(ln, &b->qkv, qkv, new_len);
+    double *kc = m->kc + (size_t)L * H * P * dh, *vc = m->vc + (size_t)L * H * P * dh;
+    for (int h = 0; h < H; ++h)
+        for (int s = 0; s < new_len; ++s)
+            for (int e = 0; e < dh; ++e) {
+                kc[((size_t)h * P + pos0 + s) * dh + e] = qkv[(size_t)s * 3 * d + d + h * dh + e];
+                vc[((size_t)h * P + pos0 + s) * dh + e] = qkv[(size_t)s * 3 * d + 2 * d + h * dh + e];
+            }
+#pragma omp parallel for collapse(2) schedule(dynamic, 4)
+    for (int h = 0; h < H; ++h) {
+        for (int s = 0; s < new_len; ++s) {
+            const int vis = pos0 + s + 1; /* keys 0..pos0+s */
+            double *sc = (double *)malloc(sizeof(double) * (size_t)vis);
+            const double *qv = qkv + (size_t)s * 3 * d + h * dh;
+            double mx = -INFINITY;
+            for (int j = 0; j < vis; ++j) {
+                const double *kj = kc + ((size_t)h * P + j) * dh;
+                double dot = 0.0;
+                for (int e = 0; e < dh; ++e) dot += qv[e] * kj[e];
+                sc[j] = dot * scale;
+                if (sc[j] > mx) mx = sc[j];
+            }
+            double sum = 0.0;
+            for (int j = 0; j < vis; ++j) {
+                sc[j] = exp(sc[j] - mx);
+                sum += sc[j];
+            }
+            for (int j = 0; j < vis; ++j) sc[j] /= sum;
+            for (int e = 0; e < dh; ++e) {
+                double acc = 0.0;
+                for (int j = 0; j < vis; ++j) acc += sc[j] * vc[((size_t)h * P + j) * dh + e];
+                att[(size_t)s * d + h * dh + e] = acc;
+            }
+            free(sc);
+        }
+    }
+    linear_f64(att, &b->proj, tmp, new_len);
+    for (size_t i = 0; i < (size_t)new_len * d; ++i) hid[i] += tmp[i];
+    layer_norm_d(hid, b->ln2_g, b->ln2_b, ln, new_len, d, m->eps);
+    linear_f64(ln, &b->fc, ffn, new_len);
+    for (size_t i = 0; i < (size_t)new_len * ff; ++i) ffn[i] = gelu_tanh_f64(ffn[i]);
+    linear_f64(ffn, &b->fc_proj, tmp, new_len);
+    for (size_t i = 0; i < (size_t)new_len * d; ++i) hid[i] += tmp[i];
+}
+
+/* final LayerNorm of hid into w->ln, then logits of rows r0..r0+nr-1.  LM head: the int4 head if one was set,
+ * else an f64 dot with the wte rows (tests_inference.rs:4504-4510). */
+static void run_head(const orc_gpt2 *m, orc_work *w, int new_len, int r0, int nr, double *logits_out) {
+    const int d = m->n_embd;
+    layer_norm_d(w->hid, m->lnf_g, m->lnf_b, w->ln, new_len, d, m->eps);
+    if (!logits_out) return;
+    if (m->lm_head.w) {
+        linear_f64(w->ln + (size_t)r0 * d, &m->lm_head, logits_out, nr);
+    } else {
+#pragma omp parallel for schedule(static)
+        for (int v = 0; v < m->vocab; ++v)
+            for (int r = 0; r < nr; ++r) {
+                const double *hv = w->ln + (size_t)(r0 + r) * d;
+                double dot = 0.0;
+                for (int j = 0; j < d; ++j) dot += hv[j] * (double)m->wte[(size_t)v * d + j];
+                logits_out[(size_t)r * m->vocab + v] = dot;
+            }
+    }
+}
+
 /*
  * One forward over `new_len` tokens at positions kv_len .. kv_len+new_len-1,
  * attending to everything cached before them (gpt2.rs:712-734 control flow,
@@ -612,97 +718,20 @@ ORC_API int orc_gpt2_cache_len(const orc_gpt2 *m) { return m->kv_len; }
  *   logits_rows == 0: last row only -> logits_out[vocab]
  *   logits_rows == 1: all rows      -> logits_out[new_len, vocab]
  * hidden_out (optional, [new_len, n_embd]) receives the final-LN output.
- * LM head: int4 head if one was set, else f64 dot with wte rows
- * (tests_inference.rs:4504-4510).
  */
 ORC_API int orc_gpt2_forward(orc_gpt2 *m, const uint32_t *tokens, int new_len, int logits_rows,
                              double *logits_out, double *hidden_out) {
-    const int d = m->n_embd, H = m->n_head, dh = m->d_head, ff = m->d_ffn, P = m->n_positions;
     const int pos0 = m->kv_len, kv_total = pos0 + new_len;
-    if (kv_total > P || new_len <= 0) return -1;
-    if (!m->kc) {
-        m->kc = (double *)malloc(sizeof(double) * (size_t)m->n_layer * H * P * dh);
-        m->vc = (double *)malloc(sizeof(double) * (size_t)m->n_layer * H * P * dh);
-    }
-    double *hid = (double *)malloc(sizeof(double) * (size_t)new_len * d);
-    double *ln = (double *)malloc(sizeof(double) * (size_t)new_len * d);
-    double *qkv = (double *)malloc(sizeof(double) * (size_t)new_len * 3 * d);
-    double *att = (double *)malloc(sizeof(double) * (size_t)new_len * d);
-    double *tmp = (double *)malloc(sizeof(double) * (size_t)new_len * d);
-    double *ffn = (double *)malloc(sizeof(double) * (size_t)new_len * ff);
-
-    for (int p = 0; p < new_len; ++p)
-        for (int j = 0; j < d; ++j)
-            hid[(size_t)p * d + j] = (double)m->wte[(size_t)tokens[p] * d + j] + (double)m->wpe[(size_t)(pos0 + p) * d + j];
-
-    const double scale = 1.0 / sqrt((double)dh);
-    for (int L = 0; L < m->n_layer; ++L) {
-        const orc_block *b = &m->blocks[L];
-        layer_norm_d(hid, b->ln1_g, b->ln1_b, ln, new_len, d, m->eps);
-        linear_f64(ln, &b->qkv, qkv, new_len);
-        double *kc = m->kc + (size_t)L * H * P * dh, *vc = m->vc + (size_t)L * H * P * dh;
-        for (int h = 0; h < H; ++h)
-            for (int s = 0; s < new_len; ++s)
-                for (int e = 0; e < dh; ++e) {
-                    kc[((size_t)h * P + pos0 + s) * dh + e] = qkv[(size_t)s * 3 * d + d + h * dh + e];
-                    vc[((size_t)h * P + pos0 + s) * dh + e] = qkv[(size_t)s * 3 * d + 2 * d + h * dh + e];
-                }
-#pragma omp parallel for collapse(2) schedule(dynamic, 4)
-        for (int h = 0; h < H; ++h) {
-            for (int s = 0; s < new_len; ++s) {
-                const int vis = pos0 + s + 1; /* keys 0..pos0+s */
-                double *sc = (double *)malloc(sizeof(double) * (size_t)vis);
-                const double *qv = qkv + (size_t)s * 3 * d + h * dh;
-                double mx = -INFINITY;
-                for (int j = 0; j < vis; ++j) {
-                    const double *kj = kc + ((size_t)h * P + j) * dh;
-                    double dot = 0.0;
-                    for (int e = 0; e < dh; ++e) dot += qv[e] * kj[e];
-                    sc[j] = dot * scale;
-                    if (sc[j] > mx) mx = sc[j];
-                }
-                double sum = 0.0;
-                for (int j = 0; j < vis; ++j) {
-                    sc[j] = exp(sc[j] - mx);
-                    sum += sc[j];
-                }
-                for (int j = 0; j < vis; ++j) sc[j] /= sum;
-                for (int e = 0; e < dh; ++e) {
-                    double acc = 0.0;
-                    for (int j = 0; j < vis; ++j) acc += sc[j] * vc[((size_t)h * P + j) * dh + e];
-                    att[(size_t)s * d + h * dh + e] = acc;
-                }
-                free(sc);
-            }
-        }
-        linear_f64(att, &b->proj, tmp, new_len);
-        for (size_t i = 0; i < (size_t)new_len * d; ++i) hid[i] += tmp[i];
-        layer_norm_d(hid, b->ln2_g, b->ln2_b, ln, new_len, d, m->eps);
-        linear_f64(ln, &b->fc, ffn, new_len);
-        for (size_t i = 0; i < (size_t)new_len * ff; ++i) ffn[i] = gelu_tanh_f64(ffn[i]);
-        linear_f64(ffn, &b->fc_proj, tmp, new_len);
-        for (size_t i = 0; i < (size_t)new_len * d; ++i) hid[i] += tmp[i];
-    }
+    if (kv_total > m->n_positions || new_len <= 0) return -1;
+    cache_alloc(m);
+    orc_work w;
+    work_alloc(m, &w, new_len);
+    embed_rows(m, tokens, new_len, pos0, w.hid);
+    for (int L = 0; L < m->n_layer; ++L) run_block(m, L, &w, new_len, pos0);
     m->kv_len = kv_total;
-
-    layer_norm_d(hid, m->lnf_g, m->lnf_b, ln, new_len, d, m->eps);
-    if (hidden_out) memcpy(hidden_out, ln, sizeof(double) * (size_t)new_len * d);
-    if (logits_out) {
-        const int r0 = logits_rows ? 0 : new_len - 1, nr = logits_rows ? new_len : 1;
-        if (m->lm_head.w) {
-            linear_f64(ln + (size_t)r0 * d, &m->lm_head, logits_out, nr);
-        } else {
-#pragma omp parallel for schedule(static)
-            for (int v = 0; v < m->vocab; ++v)
-                for (int r = 0; r < nr; ++r) {
-                    const double *hv = ln + (size_t)(r0 + r) * d;
-                    double dot = 0.0;
-                    for (int j = 0; j < d; ++j) dot += hv[j] * (double)m->wte[(size_t)v * d + j];
-                    logits_out[(size_t)r * m->vocab + v] = dot;
-                }
-        }
-    }
-    free(hid); free(ln); free(qkv); free(att); free(tmp); free(ffn);
+    run_head(m, &w, new_len, logits_rows ? 0 : new_len - 1, logits_rows ? new_len : 1, logits_out);
+    if (hidden_out) memcpy(hidden_out, w.ln, sizeof(double) * (size_t)new_len * m->n_embd);
+    work_free(&w);
     return 0;
 }
 
@@ -845,6 +874,131 @@ ORC_API int orc_gpt2_generate_sampling(orc_gpt2 *m, const uint32_t *prompt, int 
         if (eos >= 0 && next == (uint32_t)eos) break;
         tokens_out[len++] = next;
     }
+    free(lf);
+    free(logits);
+    return len;
+}
+
+/* ------------------------------------------------------------------------ */
+/* early exit: softmax_max_prob, forward_early_exit, generate_cached_early_exit */
+/* ------------------------------------------------------------------------ */
+
+/* softmax_max_prob (gpt2.rs:983-988): the largest softmax probability of a row, all in f32:
+ * max by a sequential fold, sequential sum of exp(x - max), 1 / sum. */
+ORC_API float orc_softmax_max_prob(const float *logits, int n) {
+    float mx = -INFINITY;
+    for (int i = 0; i < n; ++i) mx = fmaxf(mx, logits[i]);
+    float sum = 0.0f;
+    for (int i = 0; i < n; ++i) sum += expf(logits[i] - mx);
+    return 1.0f / sum;
+}
+
+static float confidence_of(const double *logits, int n, float *scratch) {
+    for (int i = 0; i < n; ++i) scratch[i] = (float)logits[i]; /* the reference probes f32 logits */
+    return orc_softmax_max_prob(scratch, n);
+}
+
+/*
+ * forward_early_exit (gpt2.rs:797-830): uncached forward over seq_len tokens; after every block but the last,
+ * final LayerNorm + LM head on all rows and the confidence of the last row; the first layer whose confidence
+ * reaches the threshold ends the forward.  logits_out [seq_len, vocab] are the logits of the layer that ended it,
+ * *layers_used = 1..n_layer.  conf_out (optional, [n_layer - 1]) receives the confidences probed, -1 where no
+ * probe ran.
+ */
+ORC_API int orc_gpt2_forward_early_exit(orc_gpt2 *m, const uint32_t *tokens, int seq_len, float threshold,
+                                        double *logits_out, int *layers_used, float *conf_out) {
+    if (seq_len <= 0 || seq_len > m->n_positions) return -1;
+    cache_alloc(m);
+    orc_gpt2_reset_cache(m);
+    orc_work w;
+    work_alloc(m, &w, seq_len);
+    float *lf = (float *)malloc(sizeof(float) * (size_t)m->vocab);
+    for (int i = 0; conf_out && i + 1 < m->n_layer; ++i) conf_out[i] = -1.0f;
+    embed_rows(m, tokens, seq_len, 0, w.hid);
+    int used = m->n_layer;
+    for (int L = 0; L < m->n_layer; ++L) {
+        run_block(m, L, &w, seq_len, 0);
+        if (L + 1 < m->n_layer) {
+            run_head(m, &w, seq_len, 0, seq_len, logits_out);
+            const float c = confidence_of(logits_out + (size_t)(seq_len - 1) * m->vocab, m->vocab, lf);
+            if (conf_out) conf_out[L] = c;
+            if (c >= threshold) {
+                used = L + 1;
+                break;
+            }
+        }
+    }
+    if (used == m->n_layer) run_head(m, &w, seq_len, 0, seq_len, logits_out);
+    *layers_used = used;
+    free(lf);
+    work_free(&w);
+    return 0;
+}
+
+/*
+ * generate_cached_early_exit (gpt2.rs:837-922): prefill with every layer, then per token the blocks run until
+ * the confidence of an intermediate layer reaches the threshold; the layers skipped get zero K and V rows at
+ * that position; the token is the arg-max of the logits of the last layer that ran.  A token equal to `eos`
+ * ends the sequence before it is appended (eos < 0 never stops); as in the reference, the first token is produced
+ * whatever max_new_tokens is.  layers_out [max(max_new_tokens, 1)] gets the layers used per step, *steps_out their
+ * number; conf_out (optional, [max(max_new_tokens, 1), n_layer - 1]) the confidences probed (-1: no probe).
+ * Returns the total length.
+ */
+ORC_API int orc_gpt2_generate_early_exit(orc_gpt2 *m, const uint32_t *prompt, int prompt_len, int max_new_tokens,
+                                         float threshold, int eos, uint32_t *tokens_out, int *layers_out, int *steps_out,
+                                         float *conf_out) {
+    const int nl = m->n_layer, V = m->vocab, H = m->n_head, dh = m->d_head, P = m->n_positions;
+    const int rows = max_new_tokens > 1 ? max_new_tokens : 1;
+    double *logits = (double *)malloc(sizeof(double) * (size_t)V);
+    float *lf = (float *)malloc(sizeof(float) * (size_t)V);
+    int len = prompt_len, steps = 0;
+    memcpy(tokens_out, prompt, sizeof(uint32_t) * (size_t)prompt_len);
+    for (int i = 0; conf_out && i < rows * (nl - 1); ++i) conf_out[i] = -1.0f;
+    orc_gpt2_reset_cache(m);
+    *steps_out = 0;
+    if (orc_gpt2_forward(m, tokens_out, prompt_len, 0, logits, NULL) != 0) {
+        free(logits); free(lf);
+        return len;
+    }
+    layers_out[steps++] = nl;
+    uint32_t next = argmax_first_d(logits, V, NULL);
+    if (!(eos >= 0 && next == (uint32_t)eos)) {
+        tokens_out[len++] = next;
+        orc_work w;
+        work_alloc(m, &w, 1);
+        for (int t = 1; t < max_new_tokens; ++t) {
+            const int pos = m->kv_len;
+            if (pos >= P) break;
+            embed_rows(m, &next, 1, pos, w.hid);
+            int used = nl;
+            for (int L = 0; L < nl; ++L) {
+                run_block(m, L, &w, 1, pos);
+                if (L + 1 < nl) {
+                    run_head(m, &w, 1, 0, 1, logits);
+                    const float c = confidence_of(logits, V, lf);
+                    if (conf_out) conf_out[(size_t)t * (nl - 1) + L] = c;
+                    if (c >= threshold) {
+                        for (int j = L + 1; j < nl; ++j)
+                            for (int h = 0; h < H; ++h) {
+                                const size_t at = (((size_t)j * H + h) * P + pos) * dh;
+                                memset(m->kc + at, 0, sizeof(double) * (size_t)dh);
+                                memset(m->vc + at, 0, sizeof(double) * (size_t)dh);
+                            }
+                        used = L + 1;
+                        break;
+                    }
+                }
+            }
+            m->kv_len = pos + 1;
+            layers_out[steps++] = used;
+            run_head(m, &w, 1, 0, 1, logits);
+            next = argmax_first_d(logits, V, NULL);
+            if (eos >= 0 && next == (uint32_t)eos) break;
+            tokens_out[len++] = next;
+        }
+        work_free(&w);
+    }
+    *steps_out = steps;
     free(lf);
     free(logits);
     return len;

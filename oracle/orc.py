@@ -78,6 +78,10 @@ _g_gen = _sig("orc_gpt2_generate", _i, C.c_void_p, _u32p, _i, _i, _i, _i, _u32p,
 _rng_new = _sig("orc_simple_rng_new", C.c_uint64, C.c_uint64)
 _rng_f32 = _sig("orc_simple_rng_next_f32", C.c_float, C.POINTER(C.c_uint64))
 _topk = _sig("orc_top_k_sample", C.c_uint32, _f32p, _i, _i, C.c_float, C.POINTER(C.c_uint64), C.c_void_p, C.c_void_p)
+_maxprob = _sig("orc_softmax_max_prob", C.c_float, _f32p, _i)
+_g_fee = _sig("orc_gpt2_forward_early_exit", _i, C.c_void_p, _u32p, _i, C.c_float, C.c_void_p, C.POINTER(_i), C.c_void_p)
+_g_gee = _sig("orc_gpt2_generate_early_exit", _i, C.c_void_p, _u32p, _i, _i, C.c_float, _i, _u32p, C.c_void_p,
+              C.POINTER(_i), C.c_void_p)
 _g_samp = _sig("orc_gpt2_generate_sampling", _i, C.c_void_p, _u32p, _i, _i, _i, C.c_float, C.POINTER(C.c_uint64), _i, _u32p)
 
 
@@ -306,6 +310,30 @@ class Gpt2:
         n = _g_samp(self._h, prompt, prompt.size, max_new_tokens, top_k, temperature, C.byref(rng._s), eos, out)
         return out[:n].copy()
 
+    def forward_early_exit(self, tokens, threshold):
+        """forward_early_exit (gpt2.rs:797-830) -> (logits [seq, vocab] f64, layers_used, confidences [n_layer-1])."""
+        tokens = _u32(tokens)
+        logits = np.empty((tokens.size, self.vocab), np.float64)
+        conf = np.full(max(self.cfg["n_layer"] - 1, 0), -1.0, np.float32)
+        used = _i(0)
+        rc = _g_fee(self._h, tokens, tokens.size, float(threshold), logits.ctypes.data_as(C.c_void_p), C.byref(used),
+                    conf.ctypes.data_as(C.c_void_p))
+        if rc != 0:
+            raise ValueError("sequence exceeds n_positions")
+        return logits, int(used.value), conf
+
+    def generate_early_exit(self, prompt, max_new_tokens, threshold, eos=50256):
+        """generate_cached_early_exit (gpt2.rs:837-922) -> (tokens, layers per step, confidences [steps, n_layer-1])."""
+        prompt = _u32(prompt)
+        rows = max(int(max_new_tokens), 1)
+        out = np.zeros(prompt.size + rows, np.uint32)
+        layers = np.zeros(rows, np.int32)
+        conf = np.full((rows, max(self.cfg["n_layer"] - 1, 0)), -1.0, np.float32)
+        steps = _i(0)
+        n = _g_gee(self._h, prompt, prompt.size, int(max_new_tokens), float(threshold), eos, out,
+                   layers.ctypes.data_as(C.c_void_p), C.byref(steps), conf.ctypes.data_as(C.c_void_p))
+        return out[:n].copy(), layers[: steps.value].copy(), conf[: steps.value].copy()
+
     def generate(self, prompt, max_new_tokens, cached=True, eos=50256):
         prompt = _u32(prompt)
         out = np.zeros(prompt.size + max_new_tokens, np.uint32)
@@ -313,6 +341,12 @@ class Gpt2:
         n = _g_gen(self._h, prompt, prompt.size, max_new_tokens, int(cached), eos, out,
                    margins.ctypes.data_as(C.c_void_p))
         return out[:n].copy(), margins[: max(n - prompt.size, 0)].copy()
+
+
+def softmax_max_prob(logits):
+    """softmax_max_prob (gpt2.rs:983-988): the largest softmax probability, f32 arithmetic."""
+    lg = _f32(logits).ravel()
+    return float(_maxprob(lg, lg.size))
 
 
 class SimpleRng:

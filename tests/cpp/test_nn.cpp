@@ -255,6 +255,16 @@ int main() {
             SimpleRng r4(1);
             CHECK(r4.next_f32() == 0.0f && *r4.state() == 0x40822041ull);  // one xorshift64 step from 1 (13, 7, 17)
             CHECK(r4.next_f32() == (float)(1048641ull) / 16777216.0f);
+            // early exit: an unreachable threshold is greedy decoding, threshold 0 leaves after the first block
+            auto ee = model.generate_cached_early_exit(prompt, 10, 2.0f, -1);
+            CHECK(ee.first == cac && ee.second == std::vector<size_t>(10, model.config().n_layer));
+            auto e0 = model.generate_cached_early_exit(prompt, 10, 0.0f, -1);
+            CHECK(e0.first.size() == prompt.size() + 10 && e0.second.size() == 10 && e0.second[0] == model.config().n_layer);
+            for (size_t i = 1; i < e0.second.size(); ++i) CHECK(e0.second[i] == 1);
+            auto fe = model.forward_early_exit(prompt, 2.0f);
+            CHECK(fe.second == model.config().n_layer && fe.first.shape() == std::vector<size_t>({prompt.size(), model.config().vocab_size}));
+            CHECK(model.forward_early_exit(prompt, 0.0f).second == 1);
+            CHECK(model.generate_cached(prompt, 10, -1) == cac);
         }
     });
 
