@@ -23,27 +23,27 @@
 //   D: lane (cg, q) receives rows 4q..4q+3 = the four digit sums of slot q for column 4 * cg + c.
 // Whatever k index the hardware assigns to (lane group, register, byte), A and B use the same one.
 //
-// Work decomposition, cross-wave reduction and split-K are those of the VALU kernel: a workgroup owns
-// 64 columns x one K slice per tile, each wave at most two trips per tile whose loads are issued before
-// anything else (and for the next tile before the current one is reduced); waves reduce through LDS in
-// wave order; with ksplit > 1 partial sums are published write-through and the last workgroup to take a
-// ticket adds them in split order.  Rows with a NaN or infinity produce NaN outputs.
+// Work decomposition: a workgroup owns up to four tiles of 64 columns x one K slice.  Its (tile, trip) pairs are
+// dealt to the waves round robin (item i goes to wave i % W), so any number of waves shares any number of trips
+// evenly, and a wave keeps up to SETS items in flight: their loads are issued before anything else, which for
+// the wide layers (the LM head) puts most of the matrix in flight while x is still being converted.  Waves reduce
+// through LDS in wave order; with ksplit > 1 partial sums are published write-through and the last workgroup to
+// take a ticket adds them in split order.  Rows with a NaN or infinity produce NaN outputs.
 #include "linear_common.h"
 
 namespace {
 
 typedef int intx4 __attribute__((ext_vector_type(4)));
-constexpr int kMaxTilesPerPass = 4;
+constexpr int kMaxTilesPerPass = 4;  // regions of the reduction buffer
 
 struct I8Params {
     GemvArgs a;
     int trips_per_split;  // 64-k trips per workgroup
-    int trips_per_wave;   // ceil(trips_per_split / waves), 1 or even
-    int col_blocks;       // tiles of 64 columns
-    int tiles_per_pass;   // tiles a workgroup reduces together, <= kMaxTilesPerPass
+    int col_blocks;       // tiles of 64 columns; a workgroup takes tiles blockIdx.x + j * gridDim.x, at most kMaxTilesPerPass
     int chunk_shift;      // log2(group / 32): 32-k chunk index >> chunk_shift = scale row
     float *partial;       // [ksplit, M, N]
     unsigned int *counters;
+    int sets_before;      // register sets requested before x is converted; the others follow the digits
 };
 
 // Reduces N values over the workgroup at once; every thread gets the results.  scratch is [N][16] floats
@@ -66,10 +66,10 @@ __device__ __forceinline__ void block_reduce(float (&v)[N], float *scratch, int 
     }
 }
 
-// LDS: xd bytes [MT][tps][4 digits][4 q][16] | xsum float [MT][2 * tps rounded up to 4] | red float [tiles_per_pass][32][MT][64]
+// LDS: xd bytes [MT][tps][4 digits][4 q][16] | xsum float [MT][2 * tps rounded up to 4] | red float [tiles][32][MT][64]
 // (rows >= 2 W of every region of red stay zero).  x never goes through LDS as floats: thread r owns packed row r (8 values) of
 // every x row in registers through LayerNorm, the fixed-point conversion and the chunk sums.
-template <int MT, bool LN>
+template <int MT, bool LN, int SETS>
 __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
     extern __shared__ __align__(16) float smem[];
     __shared__ float s_scratch[3][MT * 16];
@@ -87,28 +87,34 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
     const int xsum_len = (2 * tps + 3) & ~3;
     float *red = xsum + MT * xsum_len;
     constexpr int n_out = MT * COLS;
-    // A wave takes trips t0 + wave + k * W, k < p.trips_per_wave, of every tile.  Two register sets hold loads in
-    // flight: set a the even k, set b the odd k (trips_per_wave is 1 or even), each refilled right after use
-    // with the wave's next trip of that parity, which may belong to the next tile.
-    const int trip_a = t0 + wave;
-    const int ntw = p.trips_per_wave;
-    uint4 wa0, wa1, wb0, wb1;  // rows 2q, 2q+1 of a trip
-    float4 sa, sb;             // scales of chunk q % 2 of a trip
+    // Items of this workgroup: (tile j, trip t) for j < my_tiles, t < ntr, numbered j * ntr + t; wave w takes the
+    // items w, w + W, ...  Two cursors walk that list: one for the loads, SETS items ahead of the one for the MFMAs.
+    const int my_tiles = blockIdx.x < p.col_blocks ? (p.col_blocks - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
+    const int ntr = t1 - t0;
+    uint4 w0s[SETS], w1s[SETS];  // rows 2q, 2q+1 of a trip
+    float4 scs[SETS];            // scales of chunk q % 2 of a trip
+    int lj = 0, lt = wave;       // load cursor: tile ordinal, trip within the slice
+    while (lt >= ntr) { lt -= ntr; ++lj; }
     // Out-of-range columns read column 0 and get a zero scale (then the weights do not matter).
-    auto load_trip = [&](int tile, int k, uint4 &w0, uint4 &w1, float4 &sc) {
-        const int trip = trip_a + k * W;
-        if (tile >= p.col_blocks || trip >= t1) return;  // wave-uniform
-        const int c_raw = tile * COLS + cg * 4;
+    auto load_next = [&](uint4 &w0, uint4 &w1, float4 &sc) {
+        if (lj >= my_tiles) return;  // wave-uniform
+        const int c_raw = (blockIdx.x + lj * gridDim.x) * COLS + cg * 4;
         const bool ok = c_raw < a.N;
         const int c0 = ok ? c_raw : 0;
+        const int trip = t0 + lt;
         const uint32_t *src = a.packed + (size_t)(8 * trip + 2 * q) * a.N + c0;
         w0 = *reinterpret_cast<const uint4 *>(src);
         w1 = *reinterpret_cast<const uint4 *>(src + a.N);
         sc = *reinterpret_cast<const float4 *>(a.scales + (size_t)((2 * trip + (q & 1)) >> p.chunk_shift) * a.N + c0);
         if (!ok) sc = make_float4(0.f, 0.f, 0.f, 0.f);
+        lt += W;
+        while (lt >= ntr) { lt -= ntr; ++lj; }
     };
-    wa0 = wa1 = wb0 = wb1 = make_uint4(0u, 0u, 0u, 0u);
-    sa = sb = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int s = 0; s < SETS; ++s) {
+        w0s[s] = w1s[s] = make_uint4(0u, 0u, 0u, 0u);
+        scs[s] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
 
     // ---- x: packed row `row` of every x row into registers ----
     // With LayerNorm the statistics need the whole row of x, so thread r owns row r of all K / 8; otherwise
@@ -143,14 +149,17 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
     }
     // The weights go out after x: a wave's loads return in order, so x would otherwise wait for them.
     __builtin_amdgcn_sched_barrier(0);
-    load_trip(blockIdx.x, 0, wa0, wa1, sa);
-    if (ntw > 1) load_trip(blockIdx.x, 1, wb0, wb1, sb);
+#pragma unroll
+    for (int s = 0; s < SETS; ++s) if (s < p.sets_before) load_next(w0s[s], w1s[s], scs[s]);
     if (tid < 16) {  // neutral columns of the reduction scratch and the unused rows of red
         if (tid >= W)
             for (int j = 0; j < 3 * MT; ++j) (&s_scratch[0][0])[j * 16 + tid] = 0.0f;
     }
-    for (int i = tid; i < p.tiles_per_pass * 32 * n_out; i += T)
-        if ((i % (32 * n_out)) >= 2 * W * n_out) red[i] = 0.0f;
+    {  // rows >= 2 W of every region of red
+        const int per = (32 - 2 * W) * n_out;
+        for (int j = 0; j < my_tiles; ++j)
+            for (int i = tid; i < per; i += T) red[j * 32 * n_out + 2 * W * n_out + i] = 0.0f;
+    }
     if constexpr (LN) {
         float st[MT];
 #pragma unroll
@@ -232,6 +241,8 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
         }
     }
     __syncthreads();
+#pragma unroll
+    for (int s = 0; s < SETS; ++s) if (s >= p.sets_before) load_next(w0s[s], w1s[s], scs[s]);
 
     // A operand addressing of this lane, D-side constants of this lane
     const int ai = lane & 15, a_slot = ai >> 2, a_m = a_slot >> 1;
@@ -246,8 +257,7 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
     const float *d_xsum = xsum + (d_ok ? d_m : 0) * xsum_len + (q & 1);
 
     float acc[4];
-    auto consume = [&](const uint4 &w0v, const uint4 &w1v, const float4 &scv, int trip) {
-        const int tl = trip - t0;
+    auto consume = [&](const uint4 &w0v, const uint4 &w1v, const float4 &scv, int tl) {
         intx4 av = {0, 0, 0, 0};
         if (a_active) av = *reinterpret_cast<const intx4 *>(a_src + (size_t)tl * 256);
         const float xs8 = d_ok ? d_xsum[2 * tl] : 0.0f;
@@ -266,93 +276,101 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
         }
     };
 
-    // Tiles blockIdx.x, blockIdx.x + gridDim.x, ... in passes of up to p.tiles_per_pass: the waves leave their
-    // sums for tile j of the pass in region j of red, and one pair of barriers serves the whole pass.
+    // The waves leave their sums for tile j in region j of red (zeros where a wave had no item of that tile), and
+    // one pair of barriers serves all tiles.
     constexpr int region = 32 * n_out;
-    const int my_tiles = blockIdx.x < p.col_blocks ? (p.col_blocks - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
-    for (int first = 0; first < my_tiles; first += p.tiles_per_pass) {
-        const int nt = min(p.tiles_per_pass, my_tiles - first);
-        // epilogue operands of this thread's first output element of the pass, fetched early
-        float e_bias = 0.0f, e_res = 0.0f;
-        if (tid < nt * n_out) {
-            const int j = tid / n_out, i = tid - j * n_out;
-            const int m = i / COLS, n = (blockIdx.x + (first + j) * gridDim.x) * COLS + (i - m * COLS);
-            if (m < a.M && n < a.N) {
-                if (a.bias) e_bias = a.bias[n];
-                if (a.residual) e_res = a.residual[(size_t)m * a.N + n];
-            }
+    const int nt = my_tiles;
+    // epilogue operands of this thread's first output element, fetched early
+    float e_bias = 0.0f, e_res = 0.0f;
+    if (tid < nt * n_out) {
+        const int j = tid / n_out, i = tid - j * n_out;
+        const int m = i / COLS, n = (blockIdx.x + j * gridDim.x) * COLS + (i - m * COLS);
+        if (m < a.M && n < a.N) {
+            if (a.bias) e_bias = a.bias[n];
+            if (a.residual) e_res = a.residual[(size_t)m * a.N + n];
         }
-        for (int j = 0; j < nt; ++j) {
-            const int tile = blockIdx.x + (first + j) * gridDim.x;
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[c] = 0.0f;
+    int cur = 0;  // tile ordinal the accumulators belong to
+    // lane groups q = 0, 1 (2, 3 for the second x row) hold the two chunks of a trip: 32 rows per region
+    auto flush_to = [&](int upto) {
+        while (cur < upto) {
+            if (d_ok)
+                *reinterpret_cast<float4 *>(red + cur * region + ((wave * 2 + (q & 1)) * MT + d_m) * COLS + cg * 4) =
+                    make_float4(acc[0], acc[1], acc[2], acc[3]);
 #pragma unroll
             for (int c = 0; c < 4; ++c) acc[c] = 0.0f;
-            for (int k = 0; k < ntw; k += 2) {
-                if (trip_a + k * W < t1) consume(wa0, wa1, sa, trip_a + k * W);
-                if (k + 2 < ntw) load_trip(tile, k + 2, wa0, wa1, sa);
-                else if (first + j + 1 < my_tiles) load_trip(tile + gridDim.x, 0, wa0, wa1, sa);
-                if (ntw > 1) {
-                    if (trip_a + (k + 1) * W < t1) consume(wb0, wb1, sb, trip_a + (k + 1) * W);
-                    if (k + 3 < ntw) load_trip(tile, k + 3, wb0, wb1, sb);
-                    else if (first + j + 1 < my_tiles) load_trip(tile + gridDim.x, 1, wb0, wb1, sb);
-                }
-            }
-            // lane groups q = 0, 1 (2, 3 for the second x row) hold the two chunks of a trip: 32 rows per region
-            if (d_ok)
-                *reinterpret_cast<float4 *>(red + j * region + ((wave * 2 + (q & 1)) * MT + d_m) * COLS + cg * 4) =
-                    make_float4(acc[0], acc[1], acc[2], acc[3]);
+            ++cur;
         }
-        __syncthreads();
-        if (ksplit > 1) {
-            // publish this workgroup's partial sums past the L2, then take one ticket per tile
-            for (int idx = tid; idx < nt * n_out; idx += T) {
-                const int j = idx / n_out, i = idx - j * n_out;
-                const int m = i / COLS, n = (blockIdx.x + (first + j) * gridDim.x) * COLS + (i - m * COLS);
-                if (m < a.M && n < a.N) {
-                    float v = 0.0f;
+    };
+    {
+        int cj = 0, ct = wave;  // MFMA cursor
+        while (ct >= ntr) { ct -= ntr; ++cj; }
+        while (cj < nt) {
 #pragma unroll
-                    for (int w = 0; w < 32; ++w) v += red[j * region + w * n_out + i];
-                    __hip_atomic_store(&p.partial[((size_t)split * a.M + m) * a.N + n], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int s = 0; s < SETS; ++s) {
+                if (cj < nt) {  // wave-uniform
+                    flush_to(cj);
+                    consume(w0s[s], w1s[s], scs[s], ct);
+                    load_next(w0s[s], w1s[s], scs[s]);
+                    ct += W;
+                    while (ct >= ntr) { ct -= ntr; ++cj; }
                 }
             }
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            __syncthreads();
-            if (tid < nt) {
-                const int tile = blockIdx.x + (first + tid) * gridDim.x;
-                const unsigned int t = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                s_last[tid] = (t == (unsigned int)(ksplit - 1));
-                if (s_last[tid]) __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            __syncthreads();
         }
+        flush_to(nt);
+    }
+    __syncthreads();
+    if (ksplit > 1) {
+        // publish this workgroup's partial sums past the L2, then take one ticket per tile
         for (int idx = tid; idx < nt * n_out; idx += T) {
             const int j = idx / n_out, i = idx - j * n_out;
-            const int m = i / COLS, n = (blockIdx.x + (first + j) * gridDim.x) * COLS + (i - m * COLS);
-            if (m < a.M && n < a.N && (ksplit == 1 || s_last[j])) {
-                float t = 0.0f;
-                if (ksplit == 1) {
+            const int m = i / COLS, n = (blockIdx.x + j * gridDim.x) * COLS + (i - m * COLS);
+            if (m < a.M && n < a.N) {
+                float v = 0.0f;
 #pragma unroll
-                    for (int w = 0; w < 32; ++w) t += red[j * region + w * n_out + i];
-                } else {
-                    const float *src = p.partial + (size_t)m * a.N + n;
-                    const size_t stride = (size_t)a.M * a.N;
-                    for (int sp0 = 0; sp0 < ksplit; sp0 += 4) {  // 4 loads in flight, summed in split order
-                        float part[4];
-#pragma unroll
-                        for (int u = 0; u < 4; ++u)
-                            part[u] = __hip_atomic_load(src + (size_t)(sp0 + u < ksplit ? sp0 + u : 0) * stride, __ATOMIC_RELAXED,
-                                                        __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-                        for (int u = 0; u < 4; ++u) t += sp0 + u < ksplit ? part[u] : 0.0f;
-                    }
-                }
-                if (idx != tid) {
-                    e_bias = a.bias ? a.bias[n] : 0.0f;
-                    e_res = a.residual ? a.residual[(size_t)m * a.N + n] : 0.0f;
-                }
-                finish_output(a, t, e_bias, e_res, m, n);
+                for (int w = 0; w < 32; ++w) v += red[j * region + w * n_out + i];
+                __hip_atomic_store(&p.partial[((size_t)split * a.M + m) * a.N + n], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
-        if (first + nt < my_tiles) __syncthreads();  // the next pass reuses red and s_last
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid < nt) {
+            const int tile = blockIdx.x + tid * gridDim.x;
+            const unsigned int t = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_last[tid] = (t == (unsigned int)(ksplit - 1));
+            if (s_last[tid]) __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+    }
+    for (int idx = tid; idx < nt * n_out; idx += T) {
+        const int j = idx / n_out, i = idx - j * n_out;
+        const int m = i / COLS, n = (blockIdx.x + j * gridDim.x) * COLS + (i - m * COLS);
+        if (m < a.M && n < a.N && (ksplit == 1 || s_last[j])) {
+            float t = 0.0f;
+            if (ksplit == 1) {
+#pragma unroll
+                for (int w = 0; w < 32; ++w) t += red[j * region + w * n_out + i];
+            } else {
+                const float *src = p.partial + (size_t)m * a.N + n;
+                const size_t stride = (size_t)a.M * a.N;
+                for (int sp0 = 0; sp0 < ksplit; sp0 += 4) {  // 4 loads in flight, summed in split order
+                    float part[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+                        part[u] = __hip_atomic_load(src + (size_t)(sp0 + u < ksplit ? sp0 + u : 0) * stride, __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) t += sp0 + u < ksplit ? part[u] : 0.0f;
+                }
+            }
+            if (idx != tid) {
+                e_bias = a.bias ? a.bias[n] : 0.0f;
+                e_res = a.residual ? a.residual[(size_t)m * a.N + n] : 0.0f;
+            }
+            finish_output(a, t, e_bias, e_res, m, n);
+        }
     }
 }
 
@@ -388,36 +406,52 @@ int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips
     if (a.ln_gamma && W < ceil_div(a.K, 512)) W = ceil_div(a.K, 512);  // ... of the whole x row with LayerNorm
     if (W > 16) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "int4_gemv: K=%d too large for one workgroup's staging", a.K);
     // A wide layer with a short K (the GPT-2 small LM head: 788 tiles of 12 trips) leaves every CU three or four
-    // tiles.  Two workgroups of 8 waves per CU keep more loads in flight than one of 12 (16 waves of preloads
-    // instead of 12) and halve the tiles each has to walk through: 8.66 us instead of 9.18 us per launch on that
-    // shape.  With more trips per tile (XL: 25) the 16-wave workgroup already fills the CU and stays faster.
+    // tiles.  Two workgroups of 8 waves per CU (16 waves of requests instead of 12, two tiles each, three items per
+    // wave) take 8.1 us per launch on that shape, one of 12 waves 9.1 us.  With more trips per tile (XL: 25) the
+    // 16-wave workgroup already fills the CU and stays faster.
     int cap = max_wgs > 0 ? max_wgs : ctx->num_cus;
     const bool paired = max_wgs <= 0 && W > 8 && W <= 12 && col_blocks >= 3 * ctx->num_cus && ksplit == 1;
     if (paired) {
         W = 8;
         cap = ceil_div(col_blocks, ceil_div(col_blocks, 2 * ctx->num_cus));  // equal tile counts, at most two workgroups per CU
     }
-    p.trips_per_wave = ceil_div(tps, W);
-    if (p.trips_per_wave > 1 && (p.trips_per_wave & 1)) ++p.trips_per_wave;
     p.trips_per_split = tps;
     p.chunk_shift = __builtin_ctz((unsigned)(a.group / 32));
     p.col_blocks = col_blocks;
     p.partial = reinterpret_cast<float *>(ctx->workspace);
     p.counters = ctx->counters;
+    // tiles per workgroup: bounded by the regions of the reduction buffer that fit the LDS
+    int max_tiles = kMaxTilesPerPass;
+    while (max_tiles > 1 && stage_bytes(tps) + sizeof(float) * (size_t)max_tiles * 32 * MT * 64 > 60 * 1024) --max_tiles;
     int gx = col_blocks;
     if (gx * ksplit > cap) gx = cap / ksplit > 0 ? cap / ksplit : 1;
+    if (gx < ceil_div(col_blocks, max_tiles)) gx = ceil_div(col_blocks, max_tiles);
     const int tiles_per_wg = ceil_div(col_blocks, gx);
-    p.tiles_per_pass = tiles_per_wg < kMaxTilesPerPass ? tiles_per_wg : kMaxTilesPerPass;
-    while (p.tiles_per_pass > 1 && stage_bytes(tps) + sizeof(float) * (size_t)p.tiles_per_pass * 32 * MT * 64 > 60 * 1024)
-        --p.tiles_per_pass;
-    const size_t lds = stage_bytes(tps) + sizeof(float) * (size_t)p.tiles_per_pass * 32 * MT * 64;
+    // equal tile counts: the slowest workgroup sets the time, idle CUs cost nothing (XL LM head, 788 tiles: 197
+    // workgroups of 4 tiles take 13.6 us, 256 of 3 or 4 take 15.0 us)
+    if (tiles_per_wg > 1) gx = ceil_div(col_blocks, tiles_per_wg);
+    const size_t lds = stage_bytes(tps) + sizeof(float) * (size_t)tiles_per_wg * 32 * MT * 64;
+    const int items_per_wave = ceil_div(tiles_per_wg * tps, W);
+    // With three or more items per wave a full request queue keeps the late waves from reaching the barriers of
+    // the x conversion before most of the matrix has arrived; one set up front and the rest after the digits was
+    // the fastest split on the LM head (8.1 us against 8.5 with two and 9.0 with all).
+    p.sets_before = items_per_wave > 2 ? 1 : 2;
     const dim3 grid(gx, ksplit), block(64 * W);
+#define AGPU_I8_LAUNCH(MTv, LNv, Sv) hipLaunchKernelGGL((int4_gemv_i8_kernel<MTv, LNv, Sv>), grid, block, lds, ctx->stream, p)
+#define AGPU_I8_SETS(MTv, LNv)                         \
+    do {                                               \
+        if (items_per_wave <= 1) AGPU_I8_LAUNCH(MTv, LNv, 1); \
+        else if (items_per_wave == 2) AGPU_I8_LAUNCH(MTv, LNv, 2); \
+        else AGPU_I8_LAUNCH(MTv, LNv, 4);              \
+    } while (0)
     if (a.ln_gamma) {
-        if (MT == 1) hipLaunchKernelGGL((int4_gemv_i8_kernel<1, true>), grid, block, lds, ctx->stream, p);
-        else hipLaunchKernelGGL((int4_gemv_i8_kernel<2, true>), grid, block, lds, ctx->stream, p);
+        if (MT == 1) AGPU_I8_SETS(1, true);
+        else AGPU_I8_SETS(2, true);
     } else {
-        if (MT == 1) hipLaunchKernelGGL((int4_gemv_i8_kernel<1, false>), grid, block, lds, ctx->stream, p);
-        else hipLaunchKernelGGL((int4_gemv_i8_kernel<2, false>), grid, block, lds, ctx->stream, p);
+        if (MT == 1) AGPU_I8_SETS(1, false);
+        else AGPU_I8_SETS(2, false);
     }
+#undef AGPU_I8_SETS
+#undef AGPU_I8_LAUNCH
     return AGPU_LAUNCH_CHECK(ctx, "int4_gemv_i8_kernel");
 }
