@@ -26,7 +26,7 @@ import __graft_entry__ as entry  # noqa: E402
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, GB/s
 # HBM bytes per launch of the roofline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
 # a device copy of known size (profiles/gemv_lm_head_pmc_traffic.md); None until measured.
-TRAFFIC_BYTES_PER_LAUNCH = 24561000
+TRAFFIC_BYTES_PER_LAUNCH = 24617000
 
 
 def step_bytes(cfg, group, context_len):
