@@ -395,8 +395,10 @@ int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips
     };
     while (tps_max > 1 && stage_bytes(tps_max) > 24 * 1024) --tps_max;
     int ksplit = ceil_div(trips_total, tps_max);
-    // a narrow layer occupies few CUs: split K further, down to one trip per wave (measured on K = 3072, N = 768)
-    if (col_blocks * ksplit < ctx->num_cus / 4 && ceil_div(trips_total, ksplit) > 16) ksplit = ceil_div(trips_total, 16);
+    // A narrow layer occupies few CUs.  Up to two trips per wave it still runs fastest unsplit (K = 1600, N = 1600:
+    // 4.4 us, 5.6 us in two slices: the tickets cost more than the second trip); beyond that, slices of one trip per
+    // wave (K = 3072, N = 768 inside the decode step: three slices 0.330 ms per step, two 0.336, four 0.337).
+    if (col_blocks * ksplit < ctx->num_cus / 4 && trips_total > 32) ksplit = ceil_div(trips_total, 16);
     const int tps = ceil_div(trips_total, ksplit);
     ksplit = ceil_div(trips_total, tps);
     if ((size_t)ksplit * a.M * a.N * sizeof(float) > kWorkspaceBytes / 2)

@@ -111,6 +111,49 @@ def test_gemv_int8_matrix_core_shapes(agpu, orc, dev, M, K, N, g):
     assert np.abs(y.cpu().numpy() - ref).max() <= TOL_LINEAR
 
 
+@pytest.mark.parametrize("M", [3, 5, 8, 9, 16])
+@pytest.mark.parametrize("K,N,g", [(32, 4, 32), (64, 132, 64), (544, 260, 32), (768, 2304, 64), (6400, 1600, 32), (3072, 768, 128),
+                                   (1600, 4800, 32), (1600, 50257 // 4 * 4, 32)])
+def test_batched_decode_shapes(agpu, orc, dev, M, K, N, g):
+    """2 < M <= 16 rows of very different magnitude: one chunk, ragged last column tile, groups spanning several
+    chunks, split K, the LM-head width; the default kernel choice and the fp32 VALU kernel against the oracle."""
+    from async_gpu_amd import ops, workloads
+    rng = np.random.default_rng(M * 131 + K + N + g)
+    packed, scales, bias = workloads.random_int4_linear(rng, K, N, g, bias=True)
+    x = (rng.standard_normal((M, K)) * np.exp(rng.uniform(-3, 3, (M, 1)))).astype(np.float32)  # rows of different size
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    y = ops.int4_linear(to_dev(x, dev), to_dev(packed, dev), to_dev(scales, dev), bias=to_dev(bias, dev),
+                        residual=to_dev(res, dev), group=g).cpu().numpy()
+    ref = orc.int4_gemm_f64(x, packed, scales, g, bias=bias) + res
+    bound = np.abs(x).astype(np.float64) @ np.abs(orc.int4_dequantize(packed, scales, g)).astype(np.float64)
+    assert np.all(np.abs(y - ref) <= 3e-6 * bound + 1e-6 * np.abs(ref) + 1e-6)
+    # and the fp32 VALU kernel on the same inputs
+    y32 = ops.int4_linear(to_dev(x, dev), to_dev(packed, dev), to_dev(scales, dev), bias=to_dev(bias, dev),
+                          residual=to_dev(res, dev), group=g, flags=agpu._lib.EPI_FORCE_FP32_GEMV).cpu().numpy()
+    assert np.all(np.abs(y32 - ref) <= 3e-6 * bound + 1e-6 * np.abs(ref) + 1e-6)
+
+
+def test_batched_decode_special_rows(agpu, orc, dev):
+    """A NaN or infinity poisons its own row only; an all-zero row gives the bias; two calls give the same bits."""
+    from async_gpu_amd import ops, workloads
+    rng = np.random.default_rng(5)
+    K, N, g = 1600, 1600, 32
+    packed, scales, bias = workloads.random_int4_linear(rng, K, N, g, bias=True)
+    dp, ds, db = to_dev(packed, dev), to_dev(scales, dev), to_dev(bias, dev)
+    x = rng.standard_normal((16, K)).astype(np.float32)
+    x[3] = 0.0
+    x[7, 900] = np.nan
+    x[12, 31] = np.inf
+    y = ops.int4_linear(to_dev(x, dev), dp, ds, bias=db, group=g).cpu().numpy()
+    y2 = ops.int4_linear(to_dev(x, dev), dp, ds, bias=db, group=g).cpu().numpy()
+    assert np.array_equal(y, y2, equal_nan=True)
+    assert np.isnan(y[7]).all() and not np.isfinite(y[12]).any()
+    assert np.array_equal(y[3], bias)
+    good = [r for r in range(16) if r not in (7, 12)]
+    ref = orc.int4_gemm_f64(x[good], packed, scales, g, bias=bias)
+    assert np.abs(y[good] - ref).max() <= TOL_LINEAR
+
+
 def test_gemv_int8_fixed_point_ranges(agpu, orc, dev):
     """The fixed-point scale follows max|x| of the row: wide dynamic range, tiny and huge rows, an all-zero
     row, and the extreme nibbles 0 and 15 everywhere keep the relative error at fp32 level; NaN poisons its row."""
