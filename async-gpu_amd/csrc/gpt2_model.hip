@@ -320,15 +320,29 @@ int32_t launch_block(agpu_gpt2 *m, int L, int B, int new_len, int max_kv) {
     return agpu_int4_linear(ctx, ffn, wo.packed, wo.scales, wo.bias, hid, hid, R, d, ff, g, 0);
 }
 
-// Final LayerNorm + LM head on `rows` rows of head_in -> m->logits.
-int32_t launch_head(agpu_gpt2 *m, const float *head_in, int rows) {
+// Final LayerNorm + LM head on `rows` rows of head_in -> m->logits.  With `feed` (single row only) the same launch
+// also picks the arg-max and feeds it back as the next token; *fed tells whether it did.
+int32_t launch_head(agpu_gpt2 *m, const float *head_in, int rows, const ArgmaxAdvance *feed = nullptr, bool *fed = nullptr) {
     agpu_ctx *ctx = m->ctx;
     const int d = m->d, g = m->cfg.group_size;
     const float eps = m->cfg.layer_norm_epsilon;
     float *logits = (float *)m->logits.p;
-    if (m->cfg.lm_head == AGPU_LM_HEAD_INT4)
+    if (fed) *fed = false;
+    if (m->cfg.lm_head == AGPU_LM_HEAD_INT4) {
+        if (feed && rows == 1) {
+            GemvArgs ga{};
+            ga.x = head_in; ga.packed = m->lm_head.packed; ga.scales = m->lm_head.scales; ga.y = logits;
+            ga.ln_gamma = m->lnf_g; ga.ln_beta = m->lnf_b; ga.ln_eps = eps;
+            ga.M = 1; ga.N = m->Vpad; ga.K = d; ga.group = g;
+            ga.am_idx_out = m->next_tok; ga.am_cols = m->V; ga.am_last = m->cfg.argmax_last; ga.am_adv = *feed;
+            if (agpu_int4_gemv_i8_supported(ga)) {
+                *fed = true;
+                return agpu_int4_gemv_launch(ctx, ga);
+            }
+        }
         return agpu_ln_int4_linear(ctx, head_in, m->lnf_g, m->lnf_b, eps, m->lm_head.packed, m->lm_head.scales, nullptr, nullptr,
                                    logits, rows, m->Vpad, d, g, 0);
+    }
     int32_t rc = agpu_layer_norm(ctx, head_in, m->lnf_g, m->lnf_b, (float *)m->lnb.p, rows, d, eps);
     if (rc == AGPU_OK) rc = agpu_gemm_f32(ctx, (float *)m->lnb.p, m->wte_t, logits, rows, m->V, d);
     return rc;
@@ -343,13 +357,15 @@ int32_t launch_gather_last(agpu_gpt2 *m, int B, int new_len) {
 // One forward over `new_len` tokens per sequence.  Every kernel reads the number of cached
 // positions from pos_dev, so the same launch sequence serves eager calls and graph replays.
 // max_kv bounds cache_len + new_len for sizing the attention key split.
-int32_t launch_forward(agpu_gpt2 *m, const uint32_t *tokens, int B, int new_len, int max_kv, bool all_rows_logits) {
+int32_t launch_forward(agpu_gpt2 *m, const uint32_t *tokens, int B, int new_len, int max_kv, bool all_rows_logits,
+                       const ArgmaxAdvance *feed = nullptr, bool *fed = nullptr) {
+    if (fed) *fed = false;
     int32_t rc = launch_embed(m, tokens, B, new_len);
     for (int L = 0; rc == AGPU_OK && L < m->cfg.n_layer; ++L) rc = launch_block(m, L, B, new_len, max_kv);
     if (rc != AGPU_OK) return rc;
     // final LayerNorm + LM head on the rows whose logits are wanted
     if (all_rows_logits) return launch_head(m, (float *)m->hid.p, B * new_len);
-    if (new_len == 1) return launch_head(m, (float *)m->hid.p, B);
+    if (new_len == 1) return launch_head(m, (float *)m->hid.p, B, B == 1 ? feed : nullptr, fed);
     if ((rc = launch_gather_last(m, B, new_len)) != AGPU_OK) return rc;
     return launch_head(m, (float *)m->last.p, B);
 }
@@ -388,10 +404,15 @@ int32_t set_counters(agpu_gpt2 *m, int pos, int step) {
     return AGPU_LAUNCH_CHECK(m->ctx, "set_counters_kernel");
 }
 
-int32_t launch_argmax_advance(agpu_gpt2 *m, int B, int delta) {
+ArgmaxAdvance token_feed(const agpu_gpt2 *m, int B, int delta) {
     ArgmaxAdvance adv{};
     adv.cur_tok = m->cur_tok; adv.out_tok = m->out_tok; adv.pos_dev = m->pos_dev; adv.step_dev = m->step_dev;
     adv.delta = delta; adv.out_capacity = m->out_capacity; adv.bump_counters = (B == 1);
+    return adv;
+}
+
+int32_t launch_argmax_advance(agpu_gpt2 *m, int B, int delta) {
+    const ArgmaxAdvance adv = token_feed(m, B, delta);
     int32_t rc = agpu_argmax_rows_strided(m->ctx, (float *)m->logits.p, m->next_tok, B, m->V, logits_stride(m),
                                           m->cfg.argmax_last, &adv);
     if (rc != AGPU_OK || B == 1) return rc;
@@ -419,8 +440,11 @@ int32_t decode_graph(agpu_gpt2 *m, int B, int bucket, hipGraphExec_t *out) {
         return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "gpt2: graph capture needs a context with its own stream (agpu_ctx_create)");
     hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
     if (e != hipSuccess) return agpu_hip(ctx, e, "hipStreamBeginCapture");
-    int32_t rc = launch_forward(m, m->cur_tok, B, 1, bucket, false);
-    if (rc == AGPU_OK) rc = launch_argmax_advance(m, B, 1);
+    // one sequence: the LM head picks and feeds the next token itself
+    const ArgmaxAdvance feed = token_feed(m, B, 1);
+    bool fed = false;
+    int32_t rc = launch_forward(m, m->cur_tok, B, 1, bucket, false, &feed, &fed);
+    if (rc == AGPU_OK && !fed) rc = launch_argmax_advance(m, B, 1);
     hipGraph_t graph = nullptr;
     e = hipStreamEndCapture(ctx->stream, &graph);
     if (rc != AGPU_OK) {

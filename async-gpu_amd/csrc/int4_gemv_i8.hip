@@ -44,7 +44,33 @@ struct I8Params {
     float *partial;       // [ksplit, M, N]
     unsigned int *counters;
     int sets_before;      // register sets requested before x is converted; the others follow the digits
+    unsigned long long *am_partial;  // fused arg-max: one candidate per workgroup, written through
 };
+
+// Order-preserving key of a float (NaN lowest, both zeros equal) with the column behind it: the larger 64-bit word wins.
+__device__ __forceinline__ unsigned long long argmax_word(float v, int n, int last) {
+    if (v != v) return 0ull;
+    const uint32_t u = v == 0.0f ? 0u : __float_as_uint(v);
+    const uint32_t key = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+    return ((unsigned long long)key << 32) | (uint32_t)(last ? n : ~n);
+}
+
+// Largest word over the workgroup (scratch: 2 x 16 uint32); every thread of wave 0 gets the result.
+__device__ __forceinline__ unsigned long long block_max_word(unsigned long long w, uint32_t *scratch, int lane, int wave, int W) {
+    uint32_t hi = (uint32_t)(w >> 32), lo = (uint32_t)w;
+    const uint32_t mh = wave_minmax_u32<true>(hi);
+    const uint32_t ml = wave_minmax_u32<true>(hi == mh ? lo : 0u);
+    if (lane == 0) {
+        scratch[wave] = mh;
+        scratch[16 + wave] = ml;
+    }
+    __syncthreads();
+    hi = (lane & 15) < W ? scratch[lane & 15] : 0u;
+    lo = (lane & 15) < W ? scratch[16 + (lane & 15)] : 0u;
+    const uint32_t gh = row16_minmax_u32<true>(hi);
+    const uint32_t gl = row16_minmax_u32<true>(hi == gh ? lo : 0u);
+    return ((unsigned long long)gh << 32) | gl;
+}
 
 // Reduces N values over the workgroup at once; every thread gets the results.  scratch is [N][16] floats
 // whose columns >= W hold 0 (the neutral element for sums and for maxima of non-negative values) and are
@@ -69,7 +95,7 @@ __device__ __forceinline__ void block_reduce(float (&v)[N], float *scratch, int 
 // LDS: xd bytes [MT][tps][4 digits][4 q][16] | xsum float [MT][2 * tps rounded up to 4] | red float [tiles][32][MT][64]
 // (rows >= 2 W of every region of red stay zero).  x never goes through LDS as floats: thread r owns packed row r (8 values) of
 // every x row in registers through LayerNorm, the fixed-point conversion and the chunk sums.
-template <int MT, bool LN, int SETS>
+template <int MT, bool LN, int SETS, bool AM = false>
 __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
     extern __shared__ __align__(16) float smem[];
     __shared__ float s_scratch[3][MT * 16];
@@ -344,6 +370,7 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
         }
         __syncthreads();
     }
+    unsigned long long best = 0ull;  // fused arg-max: this thread's candidate
     for (int idx = tid; idx < nt * n_out; idx += T) {
         const int j = idx / n_out, i = idx - j * n_out;
         const int m = i / COLS, n = (blockIdx.x + j * gridDim.x) * COLS + (i - m * COLS);
@@ -369,7 +396,49 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
                 e_bias = a.bias ? a.bias[n] : 0.0f;
                 e_res = a.residual ? a.residual[(size_t)m * a.N + n] : 0.0f;
             }
-            finish_output(a, t, e_bias, e_res, m, n);
+            const float v = finish_output(a, t, e_bias, e_res, m, n);
+            if (AM && n < a.am_cols) {
+                const unsigned long long w = argmax_word(v, n, a.am_last);
+                best = w > best ? w : best;
+            }
+        }
+    }
+    if constexpr (AM) {
+        // One candidate per workgroup goes out past the L2; the last workgroup to take a ticket picks the winner.
+        uint32_t *am_scratch = reinterpret_cast<uint32_t *>(&s_scratch[0][0]);
+        __syncthreads();  // s_scratch is free again
+        best = block_max_word(best, am_scratch, lane, wave, W);
+        if (tid == 0) {
+            __hip_atomic_store(&p.am_partial[blockIdx.x], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            const unsigned int t = __hip_atomic_fetch_add(&p.counters[kNumCounters - 1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_last[0] = (t == gridDim.x - 1);
+            if (s_last[0]) __hip_atomic_store(&p.counters[kNumCounters - 1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (s_last[0]) {
+            best = 0ull;
+            for (int i = tid; i < (int)gridDim.x; i += T) {
+                const unsigned long long w = __hip_atomic_load(&p.am_partial[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                best = w > best ? w : best;
+            }
+            __syncthreads();
+            best = block_max_word(best, am_scratch, lane, wave, W);
+            if (tid == 0) {
+                const uint32_t lo = (uint32_t)best;
+                const uint32_t win = (best >> 32) == 0ull ? 0u : (a.am_last ? lo : ~lo);  // nothing comparable: index 0
+                a.am_idx_out[0] = win;
+                const ArgmaxAdvance &adv = a.am_adv;
+                if (adv.cur_tok) {  // token feed, as in the arg-max kernel
+                    const int st = *adv.step_dev;
+                    adv.cur_tok[0] = win;
+                    if (st < adv.out_capacity) adv.out_tok[st] = win;
+                    if (adv.bump_counters) {
+                        *adv.pos_dev += adv.delta;
+                        *adv.step_dev = st + 1;
+                    }
+                }
+            }
         }
     }
 }
@@ -439,6 +508,14 @@ int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips
     // the fastest split on the LM head (8.1 us against 8.5 with two and 9.0 with all).
     p.sets_before = items_per_wave > 2 ? 1 : 2;
     const dim3 grid(gx, ksplit), block(64 * W);
+    // fused arg-max: single row, unsplit K (else the separate kernel runs afterwards)
+    const bool am = a.am_idx_out != nullptr && a.M == 1 && ksplit == 1 && (size_t)gx * sizeof(unsigned long long) <= kWorkspaceBytes / 2;
+    if (am) {
+        p.am_partial = reinterpret_cast<unsigned long long *>(ctx->workspace);
+        if (a.ln_gamma) hipLaunchKernelGGL((int4_gemv_i8_kernel<1, true, 4, true>), grid, block, lds, ctx->stream, p);
+        else hipLaunchKernelGGL((int4_gemv_i8_kernel<1, false, 4, true>), grid, block, lds, ctx->stream, p);
+        return AGPU_LAUNCH_CHECK(ctx, "int4_gemv_i8_kernel");
+    }
 #define AGPU_I8_LAUNCH(MTv, LNv, Sv) hipLaunchKernelGGL((int4_gemv_i8_kernel<MTv, LNv, Sv>), grid, block, lds, ctx->stream, p)
 #define AGPU_I8_SETS(MTv, LNv)                         \
     do {                                               \
@@ -455,5 +532,8 @@ int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips
     }
 #undef AGPU_I8_SETS
 #undef AGPU_I8_LAUNCH
-    return AGPU_LAUNCH_CHECK(ctx, "int4_gemv_i8_kernel");
+    int32_t rc = AGPU_LAUNCH_CHECK(ctx, "int4_gemv_i8_kernel");
+    if (rc == AGPU_OK && a.am_idx_out)
+        rc = agpu_argmax_rows_strided(ctx, a.y, a.am_idx_out, 1, a.am_cols, a.N, a.am_last, a.am_adv.cur_tok ? &a.am_adv : nullptr);
+    return rc;
 }

@@ -1,6 +1,7 @@
 // Pieces shared by the int4 Linear kernels: epilogue, nibble unpack, GEMV launch arguments.
 #pragma once
 #include "agpu_internal.h"
+#include "elementwise.h"
 
 // bias -> GELU -> residual, applied to one output element.
 __device__ __forceinline__ float epilogue(float v, int m, int n, int N, const float *bias, const float *residual,
@@ -45,10 +46,16 @@ struct GemvArgs {
     float *vcache;
     const int *pos_dev;
     int n_heads, n_positions;
+    // Optional arg-max of output row 0 over columns [0, am_cols), computed by the same launch (greedy decoding on
+    // the LM head; N may be padded beyond am_cols).  Ties: the smaller index wins, or the larger one with am_last;
+    // NaN never wins.  am_adv (optional) is the token feed of the arg-max kernel.  M must be 1.
+    uint32_t *am_idx_out;
+    int am_cols, am_last;
+    ArgmaxAdvance am_adv;
 };
 
 // Epilogue for one output element, plus the optional K/V scatter of a fused QKV projection.
-__device__ __forceinline__ void finish_output(const GemvArgs &a, float v, float bias, float resid, int m, int n) {
+__device__ __forceinline__ float finish_output(const GemvArgs &a, float v, float bias, float resid, int m, int n) {
     v += bias;
     if (a.flags & AGPU_EPI_GELU_TANH) v = gelu_tanh_dev(v);
     else if (a.flags & AGPU_EPI_GELU_QUICK) v = gelu_quick_dev(v);
@@ -65,6 +72,7 @@ __device__ __forceinline__ void finish_output(const GemvArgs &a, float v, float 
             dst[((size_t)(m * a.n_heads + h) * a.n_positions + *a.pos_dev) * 64 + e] = v;
         }
     }
+    return v;
 }
 
 int32_t agpu_int4_gemv_launch(agpu_ctx *ctx, const GemvArgs &a);

@@ -233,3 +233,31 @@ def test_model_from_weight_files(tiny, orc, agpu, dev, tmp_path):
         assert np.array_equal(m.forward(prompt), ref_logits)
         assert np.array_equal(m.generate_cached(prompt.reshape(1, -1), 12, eos=-1)[0][0], ref_tokens)
         m.close()
+
+
+@pytest.mark.parametrize("last", [0, 1])
+def test_decode_step_picks_the_token_itself(orc, agpu, dev, last):
+    """In a one-sequence decode step the LM-head launch also picks the next token.  All logits negative (so the zero
+    logits of the padding columns behind the vocabulary must not win) and two identical vocabulary rows (a tie that
+    the index rule decides): every generated token equals the arg-max of the step's own logits under that rule."""
+    from async_gpu_amd import gpt2, workloads
+    cfg = workloads.GPT2_TINY  # vocabulary 503: nine padding columns up to the next multiple of 256
+    w = workloads.gpt2_fp32_weights(cfg, 21, std=0.08, nonzero_bias=True, random_ln=True)
+    w["wte"] = np.abs(w["wte"]) + np.float32(0.01)
+    w["lnf_g"] = np.zeros_like(w["lnf_g"])
+    w["lnf_b"] = -np.ones_like(w["lnf_b"])  # final LayerNorm output = -1 everywhere: logit[v] = -sum(wte[v])
+    sums = w["wte"].astype(np.float64).sum(1)
+    best = int(np.argmin(sums))
+    twin = (best + 37) % cfg["vocab"]
+    w["wte"][twin] = w["wte"][best]  # the two best logits are equal
+    qz = workloads.quantize_gpt2(w, 32, lambda wt, g: orc.quantize_weight_int4(wt, g, orc.SCRIPT))
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg, argmax_last=last), qz)
+    prompt = workloads.random_prompt(cfg, 1, 5)
+    tokens = gm.generate_cached(prompt, 6, eos=-1)[0][0]
+    assert tokens.size == prompt.size + 6
+    for t in range(prompt.size, tokens.size):
+        logits = gm.forward(tokens[:t])[-1]
+        assert logits.max() < 0
+        ties = np.flatnonzero(logits == logits.max())
+        assert ties.size >= 2
+        assert tokens[t] == (ties[-1] if last else ties[0]), (t, ties)
