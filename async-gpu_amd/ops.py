@@ -51,6 +51,20 @@ def int4_linear(x, packed, scales, bias=None, residual=None, group=32, flags=0, 
     return y if x.dim() <= 2 else y.reshape(*x.shape[:-1], N)
 
 
+def int4_matmul(a, b, group=128):
+    """ops::int4_matmul (nn/ops/gemm.rs:1186-1266): B [K, N] is quantized on the fly (per column, groups of 128 along
+    K, the Rust quantizer's rounding; on the device here, on the host after a download in the reference), then
+    A [M, K] goes through the int4 Linear."""
+    if a.dim() != 2 or b.dim() != 2:
+        _shape_err("2D tensors", f"a.ndim={a.dim()}, b.ndim={b.dim()}")
+    if a.shape[1] != b.shape[0]:
+        _shape_err(f"B with {a.shape[1]} rows", f"{b.shape[0]}")
+    if a.shape[1] % 8 != 0:
+        _shape_err("K divisible by 8 for INT4 packing", f"K={a.shape[1]}")
+    packed, scales = int4_quantize(b, group, _lib.QUANT_RUST)
+    return int4_linear(a, packed, scales, group=group)
+
+
 def int4_dequantize(packed, scales, group):
     kp, N = packed.shape
     w = torch.empty((kp * 8, N), dtype=torch.float32, device=packed.device)
@@ -101,6 +115,16 @@ def add_layer_norm_dual(a, b, gamma, beta, eps=1e-5, want_sum=True):
     context(a.device.index or 0).call("agpu_add_layer_norm_dual", _f32(a), _f32(b), gamma, beta, s, n,
                                       a.numel() // d, d, eps)
     return (s, n) if want_sum else n
+
+
+def layer_norm_residual(x, residual, gamma, beta, eps=1e-5):
+    """ops::layer_norm_residual (nn/ops/norm.rs:88-237): LayerNorm(x + residual)."""
+    return add_layer_norm_dual(x, residual, gamma, beta, eps, want_sum=False)
+
+
+def layer_norm_residual_dual(x, residual, gamma, beta, eps=1e-5):
+    """ops::layer_norm_residual_dual (nn/ops/norm.rs:248-400): (x + residual, LayerNorm(x + residual))."""
+    return add_layer_norm_dual(x, residual, gamma, beta, eps, want_sum=True)
 
 
 def gelu(x, mode=_lib.GELU_TANH):
@@ -169,6 +193,29 @@ def attention(q, k, v, kv_len=None, q_offset=0, causal=True):
     context(q.device.index or 0).call("agpu_attention", _f32(q), _f32(k), _f32(v), o, H, q_len, kv_len, q_offset,
                                       kv_stride, dh, int(causal))
     return o
+
+
+def multi_head_flash_attention(q, k, v, seq_len, n_heads, d_head):
+    """ops::multi_head_flash_attention (nn/ops/attention.rs:151-202): q, k, v [H*seq, dh] head-major, causal."""
+    shape = (n_heads, seq_len, d_head)
+    if q.numel() != n_heads * seq_len * d_head or k.shape != q.shape or v.shape != q.shape:
+        _shape_err(f"q, k, v of {n_heads * seq_len} x {d_head}", f"{tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}")
+    return attention(q.view(shape), k.view(shape), v.view(shape)).view(q.shape)
+
+
+def scaled_dot_product_attention(q, k, v, causal=True):
+    """ops::scaled_dot_product_attention (nn/ops/attention.rs:17-100): one head, q, k, v [seq, dh]."""
+    if q.dim() != 2 or k.shape != q.shape or v.shape != q.shape:
+        _shape_err("q, k, v [seq, d_head]", f"{tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}")
+    return attention(q[None], k[None], v[None], causal=causal)[0]
+
+
+def scaled_dot_product_attention_kv(q, k, v, q_len, kv_len, q_offset):
+    """ops::scaled_dot_product_attention_kv (nn/ops/attention.rs:557-606): one head, q [q_len, dh] at positions
+    q_offset.., k and v [kv_stride, dh] with the first kv_len rows valid; causal."""
+    if q.dim() != 2 or q.shape[0] != q_len or k.shape != v.shape or k.shape[0] < kv_len:
+        _shape_err(f"q [{q_len}, dh], k and v [>= {kv_len}, dh]", f"{tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}")
+    return attention(q[None], k[None], v[None], kv_len=kv_len, q_offset=q_offset, causal=True)[0]
 
 
 def kv_append(src, cache, write_pos):

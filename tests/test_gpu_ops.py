@@ -480,3 +480,41 @@ def test_attention_rejects_other_head_dims(agpu, dev):
     with pytest.raises(agpu.AgpuError) as e:  # nn/ops/attention.rs:223-229
         ops.attention(t, t, t)
     assert e.value.code == agpu._lib.ERR_SHAPE_MISMATCH and "d_head" in e.value.message
+
+
+def test_reference_operator_names(agpu, orc, dev):
+    """The remaining free functions of the reference's ops module under their own names: int4_matmul (B quantized on
+    the fly, groups of 128, gemm.rs:1186-1266), layer_norm_residual(_dual) (norm.rs:88-400), multi_head_flash_attention,
+    scaled_dot_product_attention(_kv) (attention.rs:17-202, 557-606)."""
+    from async_gpu_amd import ops
+    rng = np.random.default_rng(77)
+    M, K, N = 5, 256, 72
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    b = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    c = ops.int4_matmul(to_dev(a, dev), to_dev(b, dev)).cpu().numpy()
+    packed, scales = orc.quantize_weight_int4(b, 128, orc.RUST)
+    assert np.abs(c - orc.int4_gemm_f64(a, packed, scales, 128)).max() <= TOL_LINEAR
+    assert np.abs(c - a.astype(np.float64) @ b).max() <= 0.5 * np.abs(b).max() / 7 * np.abs(a).sum(1).max()  # quantization error
+    with pytest.raises(agpu.AgpuError) as e:
+        ops.int4_matmul(to_dev(a[:, :60], dev), to_dev(b[:60], dev))
+    assert e.value.code == agpu._lib.ERR_SHAPE_MISMATCH and "K=60" in e.value.message
+    x = rng.standard_normal((7, 768)).astype(np.float32)
+    r = rng.standard_normal((7, 768)).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(768)).astype(np.float32)
+    be = (0.1 * rng.standard_normal(768)).astype(np.float32)
+    n1 = ops.layer_norm_residual(to_dev(x, dev), to_dev(r, dev), to_dev(g, dev), to_dev(be, dev)).cpu().numpy()
+    s2, n2 = ops.layer_norm_residual_dual(to_dev(x, dev), to_dev(r, dev), to_dev(g, dev), to_dev(be, dev))
+    ref = orc.layer_norm(x + r, g, be)
+    assert np.abs(n1 - ref).max() <= 1e-5 and np.array_equal(n1, n2.cpu().numpy()) and np.array_equal(s2.cpu().numpy(), x + r)
+    H, seq, dh = 3, 40, 64
+    q, k, v = (rng.standard_normal((H, seq, dh)).astype(np.float32) / 4 for _ in range(3))
+    want = orc.attention_kv(q, k, v)
+    flat = lambda t: to_dev(t.reshape(H * seq, dh), dev)
+    got = ops.multi_head_flash_attention(flat(q), flat(k), flat(v), seq, H, dh).cpu().numpy().reshape(H, seq, dh)
+    assert np.abs(got - want).max() <= 1e-5
+    one = ops.scaled_dot_product_attention(to_dev(q[1], dev), to_dev(k[1], dev), to_dev(v[1], dev)).cpu().numpy()
+    assert np.abs(one - want[1]).max() <= 1e-5
+    bid = ops.scaled_dot_product_attention(to_dev(q[1], dev), to_dev(k[1], dev), to_dev(v[1], dev), causal=False).cpu().numpy()
+    assert np.abs(bid - orc.attention_kv(q[1:2], k[1:2], v[1:2], causal=False)[0]).max() <= 1e-5 and np.abs(bid - one).max() > 1e-3
+    last = ops.scaled_dot_product_attention_kv(to_dev(q[2, -1:], dev), to_dev(k[2], dev), to_dev(v[2], dev), 1, seq, seq - 1).cpu().numpy()
+    assert np.abs(last[0] - want[2, -1]).max() <= 1e-5  # q_len = 1 at the last position = last row of the full attention
