@@ -16,6 +16,8 @@ struct AttnParams {
     // Decode kernel: fetch the first pass of K/V rows before the context length is known (hides one memory
     // round trip; reads up to 32 * waves rows whatever the length).  Set by the launcher for small launches.
     int speculate;
+    // Prefill kernel: a workgroup takes query block nb-1-x and then block x (set by the launcher).
+    int pair_blocks;
 };
 
 // max_kv_len bounds kv_len for launches that read it from pos_dev (sizes the key split).

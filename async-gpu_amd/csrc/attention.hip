@@ -30,6 +30,10 @@ __device__ __forceinline__ void resolve_positions(const AttnParams &p, int &kv_l
 // through LDS in wave order.  Query blocks are issued last-first: the causal mask makes the last blocks
 // the long ones.
 constexpr int ATT_TILE_FLOATS = 32 * KLD + 32 * DH;  // per wave: K tile (padded rows) + V tile
+// exp of the prefill kernel: v_exp_f32 on x * log2(e), relative error about 2^-22 at the arguments that matter
+// (the reference kernels use ex2.approx the same way, compute_transformer.rs:837-1065); 13 % of the kernel's time
+// against the correctly rounded expf, which the decode kernel keeps.
+#define ATT_EXP __expf
 
 __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnParams p) {
     extern __shared__ __align__(16) float att_smem[];
@@ -38,9 +42,15 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnParams p) {
     float *Ks = att_smem + wave * ATT_TILE_FLOATS;
     float *Vs = Ks + 32 * KLD;
     const int hb = blockIdx.y, b = hb / p.n_heads, h = hb % p.n_heads;
-    const int i0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * 32;
     int kv_len, q_offset;
     resolve_positions(p, kv_len, q_offset);
+    // Query blocks of this workgroup: with pairing, block nb-1-x and then block x, so that under the causal mask
+    // every workgroup walks through the same number of key tiles; otherwise one block, the long ones first.
+    const int nb = (p.q_len + 31) >> 5;
+    for (int rep = 0; rep < (p.pair_blocks ? 2 : 1); ++rep) {
+    const int qb = rep == 0 ? nb - 1 - (int)blockIdx.x : (int)blockIdx.x;
+    if (rep == 1 && qb >= nb - 1 - (int)blockIdx.x) break;  // the middle block of an odd count was done already
+    const int i0 = qb * 32;
 
     const float *kh = p.k + (size_t)hb * p.kv_stride * DH;
     const float *vh = p.v + (size_t)hb * p.kv_stride * DH;
@@ -112,11 +122,11 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnParams p) {
         const float m_new = fmaxf(m_run, tmax);
         // A wave's first tile can be fully masked for some queries (m_new = -inf): keep them empty.
         const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-        const float alpha = expf(m_run - m_use);
+        const float alpha = ATT_EXP(m_run - m_use);
         float psum = 0.0f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            sacc[r] = expf(sacc[r] - m_use);
+            sacc[r] = ATT_EXP(sacc[r] - m_use);
             psum += sacc[r];
         }
         psum += __shfl_xor(psum, 32, kWave);
@@ -174,7 +184,8 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnParams p) {
                 orow[d] = acc * inv_l;
             }
         }
-        return;
+        if (p.pair_blocks) __syncthreads();  // the tiles are reused by the second block
+        continue;
     }
     const int qi = i0 + c;
     if (qi < p.q_len) {
@@ -189,6 +200,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnParams p) {
                 make_float4(o1[4 * rb] * inv_l, o1[4 * rb + 1] * inv_l, o1[4 * rb + 2] * inv_l, o1[4 * rb + 3] * inv_l);
         }
     }
+    }  // query blocks of this workgroup
 }
 
 // Merge (m, l, o) of `other` into (m, l, o); empty partials have l == 0 and m == -inf.
@@ -308,12 +320,27 @@ int32_t agpu_attention_launch(agpu_ctx *ctx, const AttnParams &p, int max_kv_len
         hipLaunchKernelGGL(attn_decode_kernel, dim3(p.q_len, hb), dim3(64 * W), 0, ctx->stream, pd);
         return AGPU_LAUNCH_CHECK(ctx, "attn_decode_kernel");
     }
-    // key split: one wave per 4 key tiles of the longest query block, at most 3 (their tiles fill 64 KiB of LDS)
+    // key split: one wave per 4 key tiles of the longest query block, at most 4 (their tiles take 68 KiB of LDS;
+    // 6 or 8 waves leave room for one workgroup per CU only and are slower)
     const int tiles = ceil_div(max_kv_len, 32);
     int S = ceil_div(tiles, 4);
-    S = S < 1 ? 1 : (S > 3 ? 3 : S);
-    hipLaunchKernelGGL(attn_mfma_kernel, dim3(ceil_div(p.q_len, 32), hb), dim3(64 * S), sizeof(float) * ATT_TILE_FLOATS * S,
-                       ctx->stream, p);
+    S = S < 1 ? 1 : (S > 4 ? 4 : S);
+    static bool lds_raised = false;
+    if (!lds_raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)(sizeof(float) * ATT_TILE_FLOATS * 4));
+        if (e != hipSuccess) return agpu_hip(ctx, e, "hipFuncSetAttribute");
+        lds_raised = true;
+    }
+    // Under the causal mask query block i walks through i + 1 key tiles.  When there are more workgroups than CUs, the
+    // long ones share their SIMDs with others and set the time; pairing block nb-1-x with block x gives every
+    // workgroup the same nb + 1 tiles and one workgroup per CU (12 heads x 1024: 48.5 us against 58.8 us unpaired).
+    // With fewer workgroups pairing only lengthens the chains (12 heads x 256: 28 us against 20.6 us).
+    AttnParams pm = p;
+    const int nb = ceil_div(p.q_len, 32);
+    pm.pair_blocks = (p.causal && nb >= 4 && nb * hb > ctx->num_cus) ? 1 : 0;
+    hipLaunchKernelGGL(attn_mfma_kernel, dim3(pm.pair_blocks ? (nb + 1) / 2 : nb, hb), dim3(64 * S), sizeof(float) * ATT_TILE_FLOATS * S,
+                       ctx->stream, pm);
     return AGPU_LAUNCH_CHECK(ctx, "attn_mfma_kernel");
 }
 
