@@ -75,14 +75,23 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnParams p) {
 
     // rows it*4 + lane/16 of a tile, 4 floats at column 4*(lane%16): 8 x (K, V) float4 per lane
     float4 kpre[8], vpre[8];
+    const int lane_off = (lane >> 4) * DH + (lane & 15) * 4;  // this lane's place in rows 0..3 of a tile
     auto fetch = [&](int j0) {
+        const float *kt = kh + (size_t)j0 * DH + lane_off, *vt = vh + (size_t)j0 * DH + lane_off;
+        if (j0 + 32 <= kv_len) {  // a whole tile (uniform): constant offsets from one address
 #pragma unroll
-        for (int it = 0; it < 8; ++it) {
-            const int r = it * 4 + (lane >> 4), c4 = (lane & 15) * 4;
-            kpre[it] = vpre[it] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (j0 + r < kv_len) {
-                kpre[it] = *reinterpret_cast<const float4 *>(kh + (size_t)(j0 + r) * DH + c4);
-                vpre[it] = *reinterpret_cast<const float4 *>(vh + (size_t)(j0 + r) * DH + c4);
+            for (int it = 0; it < 8; ++it) {
+                kpre[it] = *reinterpret_cast<const float4 *>(kt + it * 4 * DH);
+                vpre[it] = *reinterpret_cast<const float4 *>(vt + it * 4 * DH);
+            }
+        } else {
+#pragma unroll
+            for (int it = 0; it < 8; ++it) {
+                kpre[it] = vpre[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (j0 + it * 4 + (lane >> 4) < kv_len) {
+                    kpre[it] = *reinterpret_cast<const float4 *>(kt + it * 4 * DH);
+                    vpre[it] = *reinterpret_cast<const float4 *>(vt + it * 4 * DH);
+                }
             }
         }
     };
@@ -111,13 +120,17 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnParams p) {
         }
         // register r holds key j0 + 8*(r/4) + 4*h2 + r%4 for query c
         float tmax = -INFINITY;
+        // only the tiles on the diagonal or at the end of the context hide anything (uniform over the wave)
+        if (j0 + 32 > kv_len || (p.causal && j0 + 31 > q_offset + i0)) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int j = j0 + 8 * (r >> 2) + 4 * h2 + (r & 3);
-            const bool vis = (j <= my_limit) && (j < kv_len);
-            sacc[r] = vis ? sacc[r] : -INFINITY;
-            tmax = fmaxf(tmax, sacc[r]);
+            for (int r = 0; r < 16; ++r) {
+                const int j = j0 + 8 * (r >> 2) + 4 * h2 + (r & 3);
+                const bool vis = (j <= my_limit) && (j < kv_len);
+                sacc[r] = vis ? sacc[r] : -INFINITY;
+            }
         }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, sacc[r]);
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
         const float m_new = fmaxf(m_run, tmax);
         // A wave's first tile can be fully masked for some queries (m_new = -inf): keep them empty.
