@@ -338,12 +338,13 @@ int32_t agpu_attention_launch(agpu_ctx *ctx, const AttnParams &p, int max_kv_len
     const int tiles = ceil_div(max_kv_len, 32);
     int S = ceil_div(tiles, 4);
     S = S < 1 ? 1 : (S > 4 ? 4 : S);
-    static bool lds_raised = false;
-    if (!lds_raised) {
+    static std::atomic<unsigned long long> lds_raised{0};  // one bit per device: the attribute belongs to the device's code object
+    const unsigned long long dev_bit = 1ull << (ctx->device & 63);
+    if (S > 3 && !(lds_raised.load(std::memory_order_relaxed) & dev_bit)) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)(sizeof(float) * ATT_TILE_FLOATS * 4));
         if (e != hipSuccess) return agpu_hip(ctx, e, "hipFuncSetAttribute");
-        lds_raised = true;
+        lds_raised.fetch_or(dev_bit, std::memory_order_relaxed);
     }
     // Under the causal mask query block i walks through i + 1 key tiles.  When there are more workgroups than CUs, the
     // long ones share their SIMDs with others and set the time; pairing block nb-1-x with block x gives every
