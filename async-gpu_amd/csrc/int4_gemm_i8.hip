@@ -38,6 +38,9 @@ struct GemmI8Params {
     float *y;
     int M, N, K, chunk_shift;
     uint32_t flags;
+    int blocks_per_split;    // K blocks of 128 per workgroup (gridDim.z slices of K)
+    float *partial;          // [ksplit, M, N] when gridDim.z > 1
+    unsigned int *counters;  // one ticket per output tile, left at zero
 };
 
 __global__ __launch_bounds__(64 * GI_WAVES, 4) void int4_gemm_i8_kernel(const GemmI8Params p) {
@@ -49,6 +52,8 @@ __global__ __launch_bounds__(64 * GI_WAVES, 4) void int4_gemm_i8_kernel(const Ge
     const int j = lane & 31, h = lane >> 5;
     const int m0 = blockIdx.y * GI_BM, n0 = blockIdx.x * GI_BN + wave * 32;
     const int chunks = p.K / 32, kblocks = (chunks + GI_KBC - 1) / GI_KBC;
+    const int ksplit = gridDim.z, kb0 = blockIdx.z * p.blocks_per_split, kb1 = min(kblocks, kb0 + p.blocks_per_split);
+    __shared__ int s_last;
     const int rb_count = (min(GI_BM, p.M - m0) + 7) / 8;
     const bool wave_active = n0 < p.N;
     const int col = min(n0 + j, p.N - 1);  // out-of-range columns read the last one and are not stored
@@ -128,8 +133,8 @@ __global__ __launch_bounds__(64 * GI_WAVES, 4) void int4_gemm_i8_kernel(const Ge
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[rb][t] = 0.0f;
 
-    load_x(0);
-    if (wave_active) load_b(0, 0);
+    load_x(kb0);
+    if (wave_active) load_b(kb0, 0);
     stage(0);
     __syncthreads();
 
@@ -170,9 +175,9 @@ __global__ __launch_bounds__(64 * GI_WAVES, 4) void int4_gemm_i8_kernel(const Ge
         }
     };
 
-    for (int kb = 0; kb < kblocks; ++kb) {
-        const int buf = kb & 1;
-        const bool more = kb + 1 < kblocks;
+    for (int kb = kb0; kb < kb1; ++kb) {
+        const int buf = (kb - kb0) & 1;
+        const bool more = kb + 1 < kb1;
         if (more) {
             load_x(kb + 1);
             if (wave_active) {
@@ -188,8 +193,62 @@ __global__ __launch_bounds__(64 * GI_WAVES, 4) void int4_gemm_i8_kernel(const Ge
         __syncthreads();
     }
 
-    if (!wave_active || n0 + j >= p.N) return;
     const int n = n0 + j;
+    const bool col_ok = wave_active && n < p.N;
+    if (ksplit > 1) {
+        // K slices: partial sums go out past the L2, the last workgroup of a tile to take a ticket adds them in
+        // slice order (the same sum every run) and finishes the outputs.
+        if (col_ok) {
+#pragma unroll
+            for (int rb = 0; rb < GI_BM / 8; ++rb)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int m = m0 + rb * 8 + 2 * t + h;
+                    if (m < p.M)
+                        __hip_atomic_store(&p.partial[((size_t)blockIdx.z * p.M + m) * p.N + n], acc[rb][t], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+                }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+        if (tid == 0) {
+            const unsigned int tk = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_last = (tk == (unsigned int)(ksplit - 1));
+            if (s_last) __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (!s_last) return;
+        if (col_ok) {
+            const size_t stride = (size_t)p.M * p.N;
+#pragma unroll
+            for (int rb = 0; rb < GI_BM / 8; ++rb)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) acc[rb][t] = 0.0f;
+            for (int sp0 = 0; sp0 < ksplit; sp0 += 2) {  // two slices = 32 loads in flight
+                float part[2][GI_BM / 8][4];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int sp = sp0 + u < ksplit ? sp0 + u : sp0;
+#pragma unroll
+                    for (int rb = 0; rb < GI_BM / 8; ++rb)
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) {
+                            const int m = min(m0 + rb * 8 + 2 * t + h, p.M - 1);
+                            part[u][rb][t] = __hip_atomic_load(p.partial + (size_t)sp * stride + (size_t)m * p.N + n, __ATOMIC_RELAXED,
+                                                               __HIP_MEMORY_SCOPE_AGENT);
+                        }
+                }
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int rb = 0; rb < GI_BM / 8; ++rb)
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) acc[rb][t] += sp0 + u < ksplit ? part[u][rb][t] : 0.0f;
+            }
+        }
+    }
+    if (!col_ok) return;
     const float bias = p.bias ? p.bias[n] : 0.0f;
 #pragma unroll
     for (int rb = 0; rb < GI_BM / 8; ++rb)
@@ -218,7 +277,22 @@ int32_t agpu_int4_gemm_i8_launch(agpu_ctx *ctx, const float *x, const uint32_t *
     GemmI8Params p{};
     p.x = x; p.packed = packed; p.scales = scales; p.bias = bias; p.residual = residual; p.y = y;
     p.M = M; p.N = N; p.K = K; p.chunk_shift = __builtin_ctz((unsigned)(group / 32)); p.flags = flags;
-    const dim3 grid(ceil_div(N, GI_BN), ceil_div(M, GI_BM));
+    // Few rows leave most CUs without a workgroup and every workgroup with a chain of K blocks whose loads it cannot
+    // hide: slice K over more workgroups then, at least two blocks each (K = 768, N = 2304: 128 rows 23.5 -> 15.3 us,
+    // 512 rows 25.3 -> 21.9 us; K = 6400, N = 1600, 256 rows: 176 -> 56 us).
+    const int tiles = ceil_div(N, GI_BN) * ceil_div(M, GI_BM);
+    const int kblocks = ceil_div(K, 32 * GI_KBC);
+    int ksplit = 1;
+    if (tiles < 2 * ctx->num_cus && tiles <= kNumCounters) {
+        ksplit = ceil_div(2 * ctx->num_cus, tiles);  // two workgroups per CU hide each other's waits
+        if (ksplit > ceil_div(kblocks, 2)) ksplit = ceil_div(kblocks, 2);
+        while (ksplit > 1 && (size_t)ksplit * M * N * sizeof(float) > kWorkspaceBytes / 2) --ksplit;
+    }
+    p.blocks_per_split = ceil_div(kblocks, ksplit);
+    ksplit = ceil_div(kblocks, p.blocks_per_split);
+    p.partial = reinterpret_cast<float *>(ctx->workspace);
+    p.counters = ctx->counters;
+    const dim3 grid(ceil_div(N, GI_BN), ceil_div(M, GI_BM), ksplit);
     hipLaunchKernelGGL(int4_gemm_i8_kernel, grid, dim3(64 * GI_WAVES), 0, ctx->stream, p);
     return AGPU_LAUNCH_CHECK(ctx, "int4_gemm_i8_kernel");
 }
