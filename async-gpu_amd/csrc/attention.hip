@@ -328,6 +328,9 @@ int32_t agpu_attention_launch(agpu_ctx *ctx, const AttnParams &p, int max_kv_len
         // many workgroups (batched decode: one per head and sequence) fill the chip by themselves: four waves each
         // (XL shape, 16 sequences, context 300: 15 us per layer against 18.4 us with sixteen waves)
         if (p.q_len * hb > 64 && W > 4) W = 4;
+        // up to 512 keys eight waves in two passes beat sixteen in one (XL shape, context 300: 3 % of the step);
+        // at 1024 keys sixteen waves are faster (8.0 against 9.0 us)
+        if (max_kv_len <= 512 && W > 8) W = 8;
         AttnParams pd = p;
         pd.speculate = p.q_len * hb <= 64 ? 1 : 0;  // latency matters for a few workgroups, bandwidth for many
         hipLaunchKernelGGL(attn_decode_kernel, dim3(p.q_len, hb), dim3(64 * W), 0, ctx->stream, pd);
