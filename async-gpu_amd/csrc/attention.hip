@@ -29,18 +29,57 @@ __device__ __forceinline__ void resolve_positions(const AttnParams &p, int &kv_l
 // memory into registers while the matrix cores work on the current one.  The S partials are merged
 // through LDS in wave order.  Query blocks are issued last-first: the causal mask makes the last blocks
 // the long ones.
-constexpr int ATT_TILE_FLOATS = 32 * KLD + 32 * DH;  // per wave: K tile (padded rows) + V tile
+constexpr int OLD = 33;                    // row length of a wave's O^T partial in its tile: 64 x 33 + m + l = 32 * KLD floats
+constexpr int ATT_TILE_FLOATS = 32 * KLD;  // per wave: the K tile (padded rows), then the V tile in the same place
 // exp of the prefill kernel: v_exp_f32 on x * log2(e), relative error about 2^-22 at the arguments that matter
 // (the reference kernels use ex2.approx the same way, compute_transformer.rs:837-1065); 13 % of the kernel's time
 // against the correctly rounded expf, which the decode kernel keeps.
 #define ATT_EXP __expf
 
-__global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnParams p) {
+// Sum of the S waves' partial results of one query block.  Every wave's tile holds its O^T (64 x 32, rows of OLD
+// floats), then m and l per query.  Lane = output dimension, so that a wave stores whole rows; wave w takes queries
+// w, w + S, ...  Lane x first works out the weight exp(m_v - m) / l of partial v = x % S for the wave's query number
+// x / S; the sums then take the weights from those lanes.  S is a constant here so that no read waits for another.
+template <int S>
+__device__ __noinline__ void merge_partials(const float *att_smem, int lane, int wave, int i0, int q_len, float *obase, long long o_row_stride) {
+    constexpr int NQ = (32 + S - 1) / S;
+    float wgt;
+    {
+        const int qc = min(wave + S * (lane / S), 31), v = lane % S;
+        float mv[S], lv[S], m_all = -INFINITY, l_all = 0.0f, mine = 0.0f;
+#pragma unroll
+        for (int w = 0; w < S; ++w) {
+            mv[w] = att_smem[w * ATT_TILE_FLOATS + 64 * OLD + qc];
+            lv[w] = att_smem[w * ATT_TILE_FLOATS + 64 * OLD + 32 + qc];
+        }
+#pragma unroll
+        for (int w = 0; w < S; ++w) m_all = fmaxf(m_all, mv[w]);
+#pragma unroll
+        for (int w = 0; w < S; ++w) {
+            const float f = mv[w] == -INFINITY ? 0.0f : ATT_EXP(mv[w] - m_all);
+            l_all += lv[w] * f;
+            mine = w == v ? f : mine;
+        }
+        wgt = mine / l_all;
+    }
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) {
+        const int qc = wave + S * i;
+        float acc = 0.0f;
+#pragma unroll
+        for (int w = 0; w < S; ++w)
+            acc += att_smem[w * ATT_TILE_FLOATS + lane * OLD + min(qc, 31)] *
+                   __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wgt), i * S + w));
+        if (qc < 32 && i0 + qc < q_len) obase[(size_t)(i0 + qc) * o_row_stride] = acc;
+    }
+}
+
+__global__ __launch_bounds__(512) void attn_mfma_kernel(const AttnParams p) {
     extern __shared__ __align__(16) float att_smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, S = blockDim.x >> 6;
     const int c = lane & 31, h2 = lane >> 5;
     float *Ks = att_smem + wave * ATT_TILE_FLOATS;
-    float *Vs = Ks + 32 * KLD;
+    float *Vs = Ks;  // V takes the tile's place once the wave has read K (LDS operations of one wave complete in order)
     const int hb = blockIdx.y, b = hb / p.n_heads, h = hb % p.n_heads;
     int kv_len, q_offset;
     resolve_positions(p, kv_len, q_offset);
@@ -55,20 +94,6 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnParams p) {
     const float *kh = p.k + (size_t)hb * p.kv_stride * DH;
     const float *vh = p.v + (size_t)hb * p.kv_stride * DH;
 
-    // Q fragment: lane (c, h2) holds Q[i0+c][32*h2 + s], pre-multiplied by 1/8 (exact).
-    float qreg[32];
-    {
-        const int qi = i0 + c;
-        const float *qrow = p.q + (size_t)b * p.q_batch_stride + (size_t)h * p.q_head_stride + (size_t)qi * p.q_row_stride + 32 * h2;
-#pragma unroll
-        for (int s = 0; s < 32; s += 4) {
-            float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (qi < p.q_len) t = *reinterpret_cast<const float4 *>(qrow + s);
-            qreg[s] = t.x * 0.125f; qreg[s + 1] = t.y * 0.125f; qreg[s + 2] = t.z * 0.125f; qreg[s + 3] = t.w * 0.125f;
-        }
-    }
-    floatx16 o0 = {0}, o1 = {0};
-    float m_run = -INFINITY, l_run = 0.0f;
     const int last_q = min(p.q_len, i0 + 32) - 1;
     const int jmax = p.causal ? min(kv_len, q_offset + last_q + 1) : kv_len;  // keys [0, jmax)
     const int my_limit = p.causal ? q_offset + i0 + c : 0x7fffffff;            // last visible key of my query
@@ -76,26 +101,51 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnParams p) {
     // rows it*4 + lane/16 of a tile, 4 floats at column 4*(lane%16): 8 x (K, V) float4 per lane
     float4 kpre[8], vpre[8];
     const int lane_off = (lane >> 4) * DH + (lane & 15) * 4;  // this lane's place in rows 0..3 of a tile
-    auto fetch = [&](int j0) {
-        const float *kt = kh + (size_t)j0 * DH + lane_off, *vt = vh + (size_t)j0 * DH + lane_off;
+    auto fetch_tile = [&](const float *base, float4 (&pre)[8], int j0) {
+        const float *t = base + (size_t)j0 * DH + lane_off;
         if (j0 + 32 <= kv_len) {  // a whole tile (uniform): constant offsets from one address
 #pragma unroll
-            for (int it = 0; it < 8; ++it) {
-                kpre[it] = *reinterpret_cast<const float4 *>(kt + it * 4 * DH);
-                vpre[it] = *reinterpret_cast<const float4 *>(vt + it * 4 * DH);
-            }
+            for (int it = 0; it < 8; ++it) pre[it] = *reinterpret_cast<const float4 *>(t + it * 4 * DH);
         } else {
 #pragma unroll
             for (int it = 0; it < 8; ++it) {
-                kpre[it] = vpre[it] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (j0 + it * 4 + (lane >> 4) < kv_len) {
-                    kpre[it] = *reinterpret_cast<const float4 *>(kt + it * 4 * DH);
-                    vpre[it] = *reinterpret_cast<const float4 *>(vt + it * 4 * DH);
-                }
+                pre[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (j0 + it * 4 + (lane >> 4) < kv_len) pre[it] = *reinterpret_cast<const float4 *>(t + it * 4 * DH);
             }
         }
     };
-    if (wave * 32 < jmax) fetch(wave * 32);
+    // The query block comes in like a key tile (whole rows per 16 lanes), passes through the wave's tile and leaves
+    // as the fragment: lane (c, h2) holds Q[i0+c][32*h2 + s], pre-multiplied by 1/8 (exact).  Read row by row per lane
+    // it would cost 64 cache lines per instruction.
+    float qreg[32];
+    {
+        float4 qpre[8];
+        const float *qb0 = p.q + (size_t)b * p.q_batch_stride + (size_t)h * p.q_head_stride + (lane & 15) * 4;
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int qi = i0 + it * 4 + (lane >> 4);
+            qpre[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (qi < p.q_len) qpre[it] = *reinterpret_cast<const float4 *>(qb0 + (size_t)qi * p.q_row_stride);
+        }
+        // the first tile's requests go out before the wave waits for its queries
+        if (wave * 32 < jmax) {
+            fetch_tile(kh, kpre, wave * 32);
+            fetch_tile(vh, vpre, wave * 32);
+        }
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int r = it * 4 + (lane >> 4), c4 = (lane & 15) * 4;
+            *reinterpret_cast<float4 *>(&Ks[r * KLD + c4]) = qpre[it];
+        }
+        const float *qrow = &Ks[c * KLD + 32 * h2];
+#pragma unroll
+        for (int s = 0; s < 32; s += 4) {
+            const float4 t = *reinterpret_cast<const float4 *>(qrow + s);
+            qreg[s] = t.x * 0.125f; qreg[s + 1] = t.y * 0.125f; qreg[s + 2] = t.z * 0.125f; qreg[s + 3] = t.w * 0.125f;
+        }
+    }
+    floatx16 o0 = {0}, o1 = {0};
+    float m_run = -INFINITY, l_run = 0.0f;
 
     for (int j0 = wave * 32; j0 < jmax; j0 += 32 * S) {
         // the tile is private to the wave: LDS operations of one wave complete in order, no barrier
@@ -103,9 +153,9 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnParams p) {
         for (int it = 0; it < 8; ++it) {
             const int r = it * 4 + (lane >> 4), c4 = (lane & 15) * 4;
             *reinterpret_cast<float4 *>(&Ks[r * KLD + c4]) = kpre[it];
-            *reinterpret_cast<float4 *>(&Vs[r * DH + c4]) = vpre[it];
         }
-        if (j0 + 32 * S < jmax) fetch(j0 + 32 * S);
+        const bool more = j0 + 32 * S < jmax;
+        if (more) fetch_tile(kh, kpre, j0 + 32 * S);
 
         // S^T[key][query]: A = K[key = c][32*h2 + s], B = Q[query = c][32*h2 + s]
         floatx16 sacc = {0};
@@ -118,6 +168,13 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnParams p) {
             sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(k4.z, qreg[s + 2], sacc, 0, 0, 0);
             sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(k4.w, qreg[s + 3], sacc, 0, 0, 0);
         }
+        // K has been read: V goes into the same tile, the next V into the registers it leaves
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int r = it * 4 + (lane >> 4), c4 = (lane & 15) * 4;
+            *reinterpret_cast<float4 *>(&Vs[r * DH + c4]) = vpre[it];
+        }
+        if (more) fetch_tile(vh, vpre, j0 + 32 * S);
         // register r holds key j0 + 8*(r/4) + 4*h2 + r%4 for query c
         float tmax = -INFINITY;
         // only the tiles on the diagonal or at the end of the context hide anything (uniform over the wave)
@@ -161,41 +218,29 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnParams p) {
         }
     }
 
-    // ---- merge the S partials: each wave leaves m, l and its O^T (64 x 32) in its own tile memory ----
+    // ---- merge the S partials: each wave leaves its O^T (64 x 32, rows padded to 33), m and l in its own tile ----
     // O^T element (d, query c) of lane (c, h2): o0[r] at d = 8*(r/4) + 4*h2 + r%4, o1[r] at d + 32.
     if (S > 1) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int d = 8 * (r >> 2) + 4 * h2 + (r & 3);
-            Ks[d * 32 + c] = o0[r];
-            Ks[(d + 32) * 32 + c] = o1[r];
+            Ks[d * OLD + c] = o0[r];
+            Ks[(d + 32) * OLD + c] = o1[r];
         }
         if (h2 == 0) {
-            Vs[c] = m_run;
-            Vs[32 + c] = l_run;
+            Ks[64 * OLD + c] = m_run;
+            Ks[64 * OLD + 32 + c] = l_run;
         }
         __syncthreads();
-        // thread t of the workgroup: query c, dims d = t/32, t/32 + 2S, ... (S waves x 2 halves)
-        const int qi = i0 + c;
-        float m_all = -INFINITY;
-        for (int w = 0; w < S; ++w) m_all = fmaxf(m_all, att_smem[w * ATT_TILE_FLOATS + 32 * KLD + c]);
-        float l_all = 0.0f, fac[4];
-        for (int w = 0; w < 4; ++w) {
-            fac[w] = 0.0f;
-            if (w < S) {
-                const float mw = att_smem[w * ATT_TILE_FLOATS + 32 * KLD + c];
-                fac[w] = mw == -INFINITY ? 0.0f : expf(mw - m_all);
-                l_all += att_smem[w * ATT_TILE_FLOATS + 32 * KLD + 32 + c] * fac[w];
-            }
-        }
-        if (qi < p.q_len) {
-            const float inv_l = 1.0f / l_all;
-            float *orow = p.o + (size_t)b * p.o_batch_stride + (size_t)h * p.o_head_stride + (size_t)qi * p.o_row_stride;
-            for (int d = wave * 2 + h2; d < DH; d += 2 * S) {
-                float acc = 0.0f;
-                for (int w = 0; w < S; ++w) acc += att_smem[w * ATT_TILE_FLOATS + d * 32 + c] * fac[w];
-                orow[d] = acc * inv_l;
-            }
+        float *obase = p.o + (size_t)b * p.o_batch_stride + (size_t)h * p.o_head_stride + lane;
+        switch (S) {
+            case 2: merge_partials<2>(att_smem, lane, wave, i0, p.q_len, obase, p.o_row_stride); break;
+            case 3: merge_partials<3>(att_smem, lane, wave, i0, p.q_len, obase, p.o_row_stride); break;
+            case 4: merge_partials<4>(att_smem, lane, wave, i0, p.q_len, obase, p.o_row_stride); break;
+            case 5: merge_partials<5>(att_smem, lane, wave, i0, p.q_len, obase, p.o_row_stride); break;
+            case 6: merge_partials<6>(att_smem, lane, wave, i0, p.q_len, obase, p.o_row_stride); break;
+            case 7: merge_partials<7>(att_smem, lane, wave, i0, p.q_len, obase, p.o_row_stride); break;
+            default: merge_partials<8>(att_smem, lane, wave, i0, p.q_len, obase, p.o_row_stride); break;
         }
         if (p.pair_blocks) __syncthreads();  // the tiles are reused by the second block
         continue;
@@ -336,26 +381,28 @@ int32_t agpu_attention_launch(agpu_ctx *ctx, const AttnParams &p, int max_kv_len
         hipLaunchKernelGGL(attn_decode_kernel, dim3(p.q_len, hb), dim3(64 * W), 0, ctx->stream, pd);
         return AGPU_LAUNCH_CHECK(ctx, "attn_decode_kernel");
     }
-    // key split: one wave per 4 key tiles of the longest query block, at most 4 (their tiles take 68 KiB of LDS;
-    // 6 or 8 waves leave room for one workgroup per CU only and are slower)
-    const int tiles = ceil_div(max_kv_len, 32);
-    int S = ceil_div(tiles, 4);
-    S = S < 1 ? 1 : (S > 4 ? 4 : S);
-    static std::atomic<unsigned long long> lds_raised{0};  // one bit per device: the attribute belongs to the device's code object
-    const unsigned long long dev_bit = 1ull << (ctx->device & 63);
-    if (S > 3 && !(lds_raised.load(std::memory_order_relaxed) & dev_bit)) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)(sizeof(float) * ATT_TILE_FLOATS * 4));
-        if (e != hipSuccess) return agpu_hip(ctx, e, "hipFuncSetAttribute");
-        lds_raised.fetch_or(dev_bit, std::memory_order_relaxed);
-    }
     // Under the causal mask query block i walks through i + 1 key tiles.  When there are more workgroups than CUs, the
     // long ones share their SIMDs with others and set the time; pairing block nb-1-x with block x gives every
-    // workgroup the same nb + 1 tiles and one workgroup per CU (12 heads x 1024: 48.5 us against 58.8 us unpaired).
-    // With fewer workgroups pairing only lengthens the chains (12 heads x 256: 28 us against 20.6 us).
+    // workgroup the same nb + 1 tiles (12 heads x 1024: 32.3 us against 44.2 us unpaired).  With fewer workgroups
+    // pairing only lengthens the chains (12 heads x 256: 15.6 us against 10.0 us).
     AttnParams pm = p;
     const int nb = ceil_div(p.q_len, 32);
     pm.pair_blocks = (p.causal && nb >= 4 && nb * hb > ctx->num_cus) ? 1 : 0;
+    const int wgs = (pm.pair_blocks ? (nb + 1) / 2 : nb) * hb;
+    // key split: one wave per key tile of the longest query block.  The registers allow two waves per SIMD: one
+    // workgroup of eight waves fills them when every workgroup has a CU of its own, two of four waves otherwise
+    // (25 heads x 1024, 400 workgroups: 54.4 us with four waves, 63.1 us with eight)
+    const int tiles = ceil_div(max_kv_len, 32);
+    const int cap = wgs <= ctx->num_cus ? 8 : 4;
+    const int S = tiles < 1 ? 1 : (tiles < cap ? tiles : cap);
+    static std::atomic<unsigned long long> lds_raised{0};  // one bit per device: the attribute belongs to the device's code object
+    const unsigned long long dev_bit = 1ull << (ctx->device & 63);
+    if (S > 7 && !(lds_raised.load(std::memory_order_relaxed) & dev_bit)) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)(sizeof(float) * ATT_TILE_FLOATS * 8));
+        if (e != hipSuccess) return agpu_hip(ctx, e, "hipFuncSetAttribute");
+        lds_raised.fetch_or(dev_bit, std::memory_order_relaxed);
+    }
     hipLaunchKernelGGL(attn_mfma_kernel, dim3(pm.pair_blocks ? (nb + 1) / 2 : nb, hb), dim3(64 * S), sizeof(float) * ATT_TILE_FLOATS * S,
                        ctx->stream, pm);
     return AGPU_LAUNCH_CHECK(ctx, "attn_mfma_kernel");
