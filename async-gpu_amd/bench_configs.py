@@ -19,7 +19,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 sys.path.insert(0, ROOT)
 import __graft_entry__ as entry  # noqa: E402
 
-HBM_GBS, MFMA_F32_TFLOPS = 8000.0, 157.3
+HBM_GBS, MFMA_F32_TFLOPS, MFMA_BF16_TFLOPS = 8000.0, 157.3, 2500.0
 
 
 def main():
@@ -79,7 +79,9 @@ def kernel_cases(ctx, emit, bench_linear, workloads, args=None):
         us = bench_linear(M, 768, 2304, reps=50)
         fl = 2.0 * M * 768 * 2304
         emit(case=f"config2 int4 GEMM M={M} K=768 N=2304 g=32", us=round(us, 3), flops=fl,
-             TFLOPs=round(fl / us / 1e6, 2), frac_mfma_f32=round(fl / us / 1e6 / MFMA_F32_TFLOPS, 4))
+             TFLOPs=round(fl / us / 1e6, 2), frac_mfma_f32=round(fl / us / 1e6 / MFMA_F32_TFLOPS, 4),
+             # the kernel issues 3 bf16 MFMAs per product (x = three bf16 pieces): share of the bf16 matrix rate in use
+             frac_mfma_bf16_issued=round(3 * fl / us / 1e6 / MFMA_BF16_TFLOPS, 4))
     # config 3: attention prefill and decode
     w = workloads.config3_attention()
     dq, dk, dv = ctx.upload(w["q"]), ctx.upload(w["k"]), ctx.upload(w["v"])

@@ -1,0 +1,360 @@
+// Prefill GEMM of the int4 weight-only Linear (M > 16 rows) on the bf16 matrix cores of gfx950, at fp32 accuracy.
+//
+// An fp32 x is the exact sum of three bf16 numbers (8 + 8 + 8 significant bits: x = hi + mid + lo, each the leading
+// bits of what the previous ones left), and the weights q - 8 in [-8, 7] are bf16 numbers as they are.  So
+//     sum_k x[k] * (q[k] - 8)  =  sum over the three pieces of  sum_k piece[k] * (q[k] - 8)
+// with every product exact in fp32: three v_mfma_f32_32x32x16_bf16 per 16 k replace the multiply-adds of the fp32
+// reference, and only the additions round (fp32 accumulation inside the matrix core, smallest piece first).
+// One scale group (or a 32-k part of one) is summed by itself, u = sum over its k, and then acc += scale * u in
+// fp32, which is the reference's w = q * scale, y += x * w up to the order of the roundings.
+//
+// Workgroup = 4 waves = 64 x rows x 256 columns; wave w owns columns 64w .. 64w + 63 as 2 x 2 tiles of 32 x 32.
+// K runs in blocks of 64 (two 32-k chunks).  The x pieces of a block are staged through LDS, double buffered, in
+// exactly the order the A operand wants them: thread t splits the 8 floats k = 8 * (t % 8) .. + 7 of row t / 8
+// (and of row t / 8 + 32) and writes one 16-byte fragment per piece, so an MFMA's A operand is one conflict-free
+// 1 KiB read.  B words and scales come straight from global memory, one block ahead; a word (8 nibbles of one
+// column) becomes the 8 bf16 of one B fragment in the order (0, 2, 4, 6, 1, 3, 5, 7) of its nibbles, which is the
+// order the x fragments are packed in as well.
+//   A fragment: lane (i, hh) = row i, the 8 k of half hh of a 16-k step
+//   B fragment: lane (j, hh) = column j, the same 8 k: packed row 4 * chunk + 2 * step + hh
+//   D: register r of lane (j, hh) = row 8 * (r / 4) + 4 * hh + r % 4, column j
+// With fewer tiles than the chip has room for, K is sliced over gridDim.z workgroups per tile: partial sums go
+// out past the L2, the last workgroup of a tile to take a ticket adds them in slice order.
+#include "linear_common.h"
+#include <type_traits>
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int GB_WAVES = 4, GB_BN = 64 * GB_WAVES, GB_KB = 64;  // waves, columns, k per block; rows: 32 * RB
+constexpr int GB_CHUNKS = GB_KB / 32;                                       // 32-k chunks per block
+constexpr int GB_FRAG_BYTES = 32 * 16;                                      // one half of an A operand: 32 rows x 8 bf16
+constexpr int GB_BUF_BYTES = GB_CHUNKS * 3 * 2 * 2 * 2 * GB_FRAG_BYTES;  // 24 KiB (two row blocks)
+
+struct GemmBfParams {
+    const float *x;
+    const uint32_t *packed;
+    const float *scales;
+    const float *bias;
+    const float *residual;
+    float *y;
+    int M, N, K, chunk_shift;
+    uint32_t flags;
+    int blocks_per_split;    // K blocks of 64 per workgroup (gridDim.z slices of K)
+    float *partial;          // [ksplit, M, N] when gridDim.z > 1
+    unsigned int *counters;  // one ticket per output tile, left at zero
+};
+
+// fragment [chunk][piece][step][row block][half]
+__device__ __forceinline__ int frag_offset(int chunk, int piece, int step, int rb, int hh) {
+    return ((((chunk * 3 + piece) * 2 + step) * 2 + rb) * 2 + hh) * GB_FRAG_BYTES;
+}
+
+// the leading 16 bits of two floats as one register: a in the low half
+__device__ __forceinline__ uint32_t pack_top(float a, float b) {
+    return __builtin_amdgcn_perm(__float_as_uint(b), __float_as_uint(a), 0x07060302u);
+}
+
+__device__ __forceinline__ float top_bits(float v) { return __uint_as_float(__float_as_uint(v) & 0xffff0000u); }
+
+// 8 nibbles of one column -> the bf16 numbers q - 8 in the order (0, 2, 4, 6, 1, 3, 5, 7): with the top bit of a
+// nibble flipped, q - 8 is the nibble read as a signed 4-bit field
+__device__ __forceinline__ bf16x8 nibbles_to_bf16(uint32_t w) {
+    const int s = (int)(w ^ 0x88888888u);
+    float f[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = (float)((s << (28 - 4 * e)) >> 28);
+    const uint4 v = make_uint4(pack_top(f[0], f[2]), pack_top(f[4], f[6]), pack_top(f[1], f[3]), pack_top(f[5], f[7]));
+    return __builtin_bit_cast(bf16x8, v);
+}
+
+template <int RB>  // row blocks of 32 per workgroup
+__global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const GemmBfParams p) {
+    constexpr int GB_BM = 32 * RB;
+    __shared__ __align__(16) unsigned char s_a[2][GB_BUF_BYTES];
+    __shared__ int s_last;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int j = lane & 31, hh = lane >> 5;
+    const int m0 = blockIdx.y * GB_BM, n0 = blockIdx.x * GB_BN + wave * 64;
+    const int chunks = p.K / 32, kblocks = (chunks + GB_CHUNKS - 1) / GB_CHUNKS;
+    const int ksplit = gridDim.z, kb0 = blockIdx.z * p.blocks_per_split, kb1 = min(kblocks, kb0 + p.blocks_per_split);
+    const bool wave_active = n0 < p.N;
+    const int cb_count = p.N - n0 > 32 ? 2 : 1;
+    int col[2];
+    col[0] = min(n0 + j, p.N - 1);  // out-of-range columns read the last one and are not stored
+    col[1] = min(n0 + 32 + j, p.N - 1);
+
+    // ---- staging role of this thread: rows t / 8 and t / 8 + 32, the 8 floats at 8 * (t % 8) of the block.
+    // Everything in the K loop is branch-free (clamped addresses, zeros by selection).  Registers filled by a load
+    // are first read one iteration later, where the compiler can only wait for every load in flight; so an
+    // iteration reads the old registers first and sends its own requests after that, a whole block ahead ----
+    const int si = tid >> 3, sk = tid & 7;
+    float4 xv[2][RB][2];  // [block parity][row block][8 floats]
+    auto load_x = [&](int kb, int set) {
+#pragma unroll
+        for (int ps = 0; ps < RB; ++ps) {
+            const int row = min(m0 + 32 * ps + si, p.M - 1), k = min(kb * GB_KB + 8 * sk, p.K - 8);
+            const float *src = p.x + (size_t)row * p.K + k;
+            xv[set][ps][0] = *reinterpret_cast<const float4 *>(src);
+            xv[set][ps][1] = *reinterpret_cast<const float4 *>(src + 4);
+        }
+    };
+    auto stage_half = [&](int kb, int set, int buf, int ps) {
+        const int chunk = sk >> 2, step = (sk >> 1) & 1, half = sk & 1;
+        const bool ok = m0 + 32 * ps + si < p.M && kb * GB_KB + 8 * sk < p.K;
+        const float4 lo4 = xv[set][ps][0], hi4 = xv[set][ps][1];
+        const float in[8] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w};
+        float v[8], r1[8], r2[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            v[e] = ok ? in[e] : 0.0f;
+            r1[e] = v[e] - top_bits(v[e]);    // exact: what the leading 8 bits leave
+            r2[e] = r1[e] - top_bits(r1[e]);  // exact, at most 8 significant bits
+        }
+        // row slot rotated by the fragment's k position: the 8 threads of a row write 8 different bank groups
+        unsigned char *dst = s_a[buf] + ((si + sk) & 31) * 16;
+        *reinterpret_cast<uint4 *>(dst + frag_offset(chunk, 2, step, ps, half)) =
+            make_uint4(pack_top(v[0], v[2]), pack_top(v[4], v[6]), pack_top(v[1], v[3]), pack_top(v[5], v[7]));
+        *reinterpret_cast<uint4 *>(dst + frag_offset(chunk, 1, step, ps, half)) =
+            make_uint4(pack_top(r1[0], r1[2]), pack_top(r1[4], r1[6]), pack_top(r1[1], r1[3]), pack_top(r1[5], r1[7]));
+        *reinterpret_cast<uint4 *>(dst + frag_offset(chunk, 0, step, ps, half)) =
+            make_uint4(pack_top(r2[0], r2[2]), pack_top(r2[4], r2[6]), pack_top(r2[1], r2[3]), pack_top(r2[5], r2[7]));
+    };
+
+    // ---- B side of this lane: per chunk and column tile two words (16-k steps) and one scale ----
+    uint32_t bw[2][GB_CHUNKS][2][2];  // [block parity][chunk][column tile][step]
+    float bs[2][GB_CHUNKS][2];
+    auto load_b = [&](int kb, int set) {
+#pragma unroll
+        for (int c = 0; c < GB_CHUNKS; ++c) {
+            const bool valid = kb * GB_CHUNKS + c < chunks;
+            const int chunk = valid ? kb * GB_CHUNKS + c : chunks - 1;  // past the end: a valid address and a zero scale
+#pragma unroll
+            for (int cb = 0; cb < 2; ++cb) {
+                const uint32_t *src = p.packed + (size_t)(4 * chunk + hh) * p.N + col[cb];
+                bw[set][c][cb][0] = src[0];
+                bw[set][c][cb][1] = src[2 * (size_t)p.N];
+                const float sc = p.scales[(size_t)(chunk >> p.chunk_shift) * p.N + col[cb]];
+                bs[set][c][cb] = valid ? sc : 0.0f;
+            }
+        }
+    };
+
+    floatx16 acc[RB][2];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[rb][cb][r] = 0.0f;
+
+    // A fragments of one group (chunk c, row block rb): [piece][step]; a register set is refilled for the next
+    // group as soon as its two MFMAs are out
+    auto a_frag = [&](int buf, int c, int rb, int piece, int st) {
+        return *reinterpret_cast<const bf16x8 *>(s_a[buf] + frag_offset(c, piece, st, rb, hh) + ((j + 4 * c + 2 * st + hh) & 31) * 16);
+    };
+
+    bf16x8 bf[GB_CHUNKS][2][2];  // [chunk][column tile][step]
+    float sc[GB_CHUNKS][2];
+    auto convert = [&](int set, int c) {
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb) {
+#pragma unroll
+            for (int st = 0; st < 2; ++st) bf[c][cb][st] = nibbles_to_bf16(bw[set][c][cb][st]);
+            sc[c][cb] = bs[set][c][cb];
+        }
+    };
+
+    // block b of this slice: x in xv[b & 1] and LDS buffer b & 1, words in bw[b & 1]
+    load_x(kb0, 0);
+    load_b(kb0, 0);
+    load_x(min(kb0 + 1, kblocks), 1);
+#pragma unroll
+    for (int ps = 0; ps < RB; ++ps) stage_half(kb0, 0, 0, ps);
+    convert(0, 0);
+    __syncthreads();
+
+    // One K block; P = its parity.  Reads what earlier iterations requested, then requests block + 1 (words) and
+    // block + 2 (x), then works on with the MFMAs of a group beside the vector work named at its end.
+    auto block = [&](int kb, auto parity) {
+        constexpr int P = decltype(parity)::value;
+        floatx16 gs[2][2];  // [group parity][column tile]: the sums of one chunk and row block
+        const floatx16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        bf16x8 a[3][2];
+#pragma unroll
+        for (int piece = 0; piece < 3; ++piece)
+#pragma unroll
+            for (int st = 0; st < 2; ++st) a[piece][st] = a_frag(P, 0, 0, piece, st);
+#pragma unroll
+        for (int t = 0; t < 2 * RB; ++t) {  // group t = (chunk t / RB, row block t % RB)
+            const int c = t / RB, g = t & 1;
+#pragma unroll
+            for (int piece = 0; piece < 3; ++piece)
+#pragma unroll
+                for (int st = 0; st < 2; ++st) {
+#pragma unroll
+                    for (int cb = 0; cb < 2; ++cb) {
+                        if (piece == 0 && st == 0) gs[g][cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[piece][st], bf[c][cb][st], zero, 0, 0, 0);
+                        else gs[g][cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[piece][st], bf[c][cb][st], gs[g][cb], 0, 0, 0);
+                    }
+                    if (t + 1 < 2 * RB) a[piece][st] = a_frag(P, (t + 1) / RB, (t + 1) % RB, piece, st);
+                }
+            if (t == 0) {
+                convert(P, 1);  // the first read of registers that a load of the previous iteration fills
+                __builtin_amdgcn_sched_barrier(0);
+                load_b(min(kb + 1, kblocks), P ^ 1);
+                load_x(min(kb + 2, kblocks), P);
+            } else {  // the previous group's sums, scaled, join the accumulators
+                const int pc = (t - 1) / RB, prb = (t - 1) % RB, pg = (t - 1) & 1;
+#pragma unroll
+                for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[prb][cb][r] = fmaf(sc[pc][cb], gs[pg][cb][r], acc[prb][cb][r]);
+            }
+            if (t >= 1 && t - 1 < RB) stage_half(kb + 1, P ^ 1, P ^ 1, t - 1);
+            __builtin_amdgcn_sched_barrier(0);  // a group's vector work stays beside its MFMAs
+        }
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[RB - 1][cb][r] = fmaf(sc[1][cb], gs[1][cb][r], acc[RB - 1][cb][r]);
+        convert(P ^ 1, 0);  // chunk 0 of the next block
+        __syncthreads();
+    };
+    for (int kb = kb0; kb < kb1; kb += 2) {
+        block(kb, std::integral_constant<int, 0>{});
+        if (kb + 1 < kb1) block(kb + 1, std::integral_constant<int, 1>{});
+    }
+
+    // element (rb, cb, r) of this lane: row m0 + 32 rb + 8 (r / 4) + 4 hh + r % 4, column n0 + 32 cb + j
+    auto row_of = [&](int rb, int r) { return m0 + 32 * rb + 8 * (r >> 2) + 4 * hh + (r & 3); };
+    if (ksplit > 1) {
+        // Partial sums live in the order of the registers: [slice][tile][wave][rb][cb][pair of r][lane] 8-byte
+        // words, so that a wave writes and reads whole 512-byte lines with constant offsets from one address.
+        const int tile = blockIdx.y * gridDim.x + blockIdx.x, tiles = gridDim.x * gridDim.y;
+        constexpr int kWaveWords = RB * 2 * 8 * 64;  // 8-byte words of one wave's results
+        unsigned long long *mine = reinterpret_cast<unsigned long long *>(p.partial) +
+                                   ((size_t)(blockIdx.z * tiles + tile) * GB_WAVES + wave) * kWaveWords + lane;
+        if (wave_active) {
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) {
+                        const unsigned long long v = (unsigned long long)__float_as_uint(acc[rb][cb][2 * q]) |
+                                                     ((unsigned long long)__float_as_uint(acc[rb][cb][2 * q + 1]) << 32);
+                        __hip_atomic_store(mine + ((rb * 2 + cb) * 8 + q) * 64, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned int tk = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_last = (tk == (unsigned int)(ksplit - 1));
+            if (s_last) __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (!s_last) return;
+        if (wave_active) {
+            const size_t slice_words = (size_t)tiles * GB_WAVES * kWaveWords;
+            const unsigned long long *first = mine - (size_t)blockIdx.z * slice_words;
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                for (int cb = 0; cb < 2; ++cb) acc[rb][cb] = floatx16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            for (int sp0 = 0; sp0 < ksplit; sp0 += 2) {  // slice order: the same sum every run; two slices = 64 loads in flight
+                unsigned long long part[2][RB * 16];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const unsigned long long *src = first + (size_t)(sp0 + u < ksplit ? sp0 + u : sp0) * slice_words;
+#pragma unroll
+                    for (int w = 0; w < RB * 16; ++w) part[u][w] = __hip_atomic_load(src + w * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    if (sp0 + u >= ksplit) break;  // uniform
+#pragma unroll
+                    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                        for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+                            for (int q = 0; q < 8; ++q) {
+                                const unsigned long long v = part[u][(rb * 2 + cb) * 8 + q];
+                                acc[rb][cb][2 * q] += __uint_as_float((uint32_t)v);
+                                acc[rb][cb][2 * q + 1] += __uint_as_float((uint32_t)(v >> 32));
+                            }
+                }
+            }
+        }
+    }
+    if (!wave_active) return;
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb) {
+        const int n = n0 + 32 * cb + j;
+        if (n >= p.N) continue;
+        const float bias = p.bias ? p.bias[n] : 0.0f;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = row_of(rb, r);
+                if (m < p.M) {
+                    float v = acc[rb][cb][r] + bias;
+                    if (p.flags & AGPU_EPI_GELU_TANH) v = gelu_tanh_dev(v);
+                    else if (p.flags & AGPU_EPI_GELU_QUICK) v = gelu_quick_dev(v);
+                    if (p.residual) v += p.residual[(size_t)m * p.N + n];
+                    p.y[(size_t)m * p.N + n] = v;
+                }
+            }
+    }
+}
+
+}  // namespace
+
+bool agpu_int4_gemm_bf16_supported(const void *x, int M, int N, int K, int group) {
+    (void)N;
+    return M > 16 && group % 32 == 0 && ((group / 32) & (group / 32 - 1)) == 0 && K % 32 == 0 && ((uintptr_t)x % 16) == 0;
+}
+
+int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t *packed, const float *scales, const float *bias,
+                                   const float *residual, float *y, int M, int N, int K, int group, uint32_t flags) {
+    GemmBfParams p{};
+    p.x = x; p.packed = packed; p.scales = scales; p.bias = bias; p.residual = residual; p.y = y;
+    p.M = M; p.N = N; p.K = K; p.chunk_shift = __builtin_ctz((unsigned)(group / 32)); p.flags = flags;
+    // 32 rows per workgroup; 64 (every weight fragment serves two row blocks) once that still leaves a workgroup
+    // per CU (M = 1024: N = 3072 29.4 us against 32.9 us with 64 rows, N = 6400 105.6 us against 96.5 us)
+    const int RB = ceil_div(N, GB_BN) * ceil_div(M, 64) >= ctx->num_cus ? 2 : 1;
+    const int BM = 32 * RB;
+    const int tiles = ceil_div(N, GB_BN) * ceil_div(M, BM);
+    const int kblocks = ceil_div(K, GB_KB);
+    // K slices: the one with the least estimated time, in units of one K block of one workgroup.  A workgroup costs
+    // its blocks plus about 2.2 for its start and end; workgroups beyond one per CU run in rounds, of which a part
+    // overlaps (the mean of the whole and the fractional number of rounds fits the measurements); slices cost the
+    // write, the ticket and one read-back round per two of them.
+    int ksplit = 1;
+    float best = 0.0f;
+    for (int ks = 1; ks <= kblocks && ks <= 16; ++ks) {
+        const int bps = ceil_div(kblocks, ks), ks2 = ceil_div(kblocks, bps);
+        const float w = (float)tiles * ks2 / ctx->num_cus;
+        const float rounds = 0.5f * ((float)ceil_div(tiles * ks2, ctx->num_cus) + (w > 1.0f ? w : 1.0f));
+        float c = rounds * (bps + 2.2f);
+        if (ks2 > 1) c += 0.75f + 0.18f * ks2;
+        if (ks == 1 || c < best) {
+            best = c;
+            ksplit = ks2;
+        }
+    }
+    if (tiles > kNumCounters) ksplit = 1;
+    while (ksplit > 1 && (size_t)ksplit * tiles * BM * GB_BN * sizeof(float) > kWorkspaceBytes / 2) --ksplit;
+    p.blocks_per_split = ceil_div(kblocks, ksplit);
+    ksplit = ceil_div(kblocks, p.blocks_per_split);
+    p.partial = reinterpret_cast<float *>(ctx->workspace);
+    p.counters = ctx->counters;
+    const dim3 grid(ceil_div(N, GB_BN), ceil_div(M, BM), ksplit);
+    if (RB == 1) hipLaunchKernelGGL(int4_gemm_bf16_kernel<1>, grid, dim3(64 * GB_WAVES), 0, ctx->stream, p);
+    else hipLaunchKernelGGL(int4_gemm_bf16_kernel<2>, grid, dim3(64 * GB_WAVES), 0, ctx->stream, p);
+    return AGPU_LAUNCH_CHECK(ctx, "int4_gemm_bf16_kernel");
+}

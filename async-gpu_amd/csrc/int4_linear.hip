@@ -245,8 +245,8 @@ AGPU_EXPORT int32_t agpu_ln_int4_linear(agpu_ctx *ctx, const float *x, const flo
         if (!(flags & AGPU_EPI_FORCE_FP32_GEMV) && agpu_int4_skinny_supported(a)) return agpu_int4_skinny_launch(ctx, a);
         return agpu_int4_gemv_launch(ctx, a);
     }
-    if (!(flags & AGPU_EPI_FORCE_FP32_GEMV) && agpu_int4_gemm_i8_supported(xin, M, N, K, group))
-        return agpu_int4_gemm_i8_launch(ctx, xin, packed, scales, bias, residual, y, M, N, K, group, epi);
+    if (!(flags & AGPU_EPI_FORCE_FP32_GEMV) && agpu_int4_gemm_bf16_supported(xin, M, N, K, group))
+        return agpu_int4_gemm_bf16_launch(ctx, xin, packed, scales, bias, residual, y, M, N, K, group, epi);
     const dim3 grid(ceil_div(N, GEMM_BN), ceil_div(M, GEMM_BM));
     hipLaunchKernelGGL((int4_gemm_mfma_kernel<false>), grid, dim3(256), 0, ctx->stream, xin, packed, scales,
                        (const float *)nullptr, bias, residual, y, M, N, K, group, epi);

@@ -79,10 +79,11 @@ int32_t agpu_int4_gemv_launch(agpu_ctx *ctx, const GemvArgs &a);
 // int8-MFMA variant for M <= 2 (needs group % 32 == 0, K % 64 == 0, N % 4 == 0, 16-byte aligned weights).
 bool agpu_int4_gemv_i8_supported(const GemvArgs &a);
 int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips_per_split, int max_wgs);
-// int8-MFMA GEMM for M > 16 (needs group / 32 a power of two, K % 32 == 0, 16-byte aligned x).
-bool agpu_int4_gemm_i8_supported(const void *x, int M, int N, int K, int group);
-int32_t agpu_int4_gemm_i8_launch(agpu_ctx *ctx, const float *x, const uint32_t *packed, const float *scales, const float *bias,
-                                 const float *residual, float *y, int M, int N, int K, int group, uint32_t flags);
+// bf16-MFMA GEMM for M > 16 with x split into three bf16 pieces (needs group / 32 a power of two, K % 32 == 0,
+// 16-byte aligned x).
+bool agpu_int4_gemm_bf16_supported(const void *x, int M, int N, int K, int group);
+int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t *packed, const float *scales, const float *bias,
+                                   const float *residual, float *y, int M, int N, int K, int group, uint32_t flags);
 // MFMA variant for 4 < M <= 16 (needs group % 32 == 0, K % 32 == 0, N % 4 == 0, 16-byte aligned weights).
 bool agpu_int4_skinny_supported(const GemvArgs &a);
 int32_t agpu_int4_skinny_launch(agpu_ctx *ctx, const GemvArgs &a);
