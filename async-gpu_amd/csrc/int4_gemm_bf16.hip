@@ -8,13 +8,13 @@
 // One scale group (or a 32-k part of one) is summed by itself, u = sum over its k, and then acc += scale * u in
 // fp32, which is the reference's w = q * scale, y += x * w up to the order of the roundings.
 //
-// Workgroup = 4 waves = 64 x rows x 256 columns; wave w owns columns 64w .. 64w + 63 as 2 x 2 tiles of 32 x 32.
-// K runs in blocks of 64 (two 32-k chunks).  The x pieces of a block are staged through LDS, double buffered, in
-// exactly the order the A operand wants them: thread t splits the 8 floats k = 8 * (t % 8) .. + 7 of row t / 8
-// (and of row t / 8 + 32) and writes one 16-byte fragment per piece, so an MFMA's A operand is one conflict-free
-// 1 KiB read.  B words and scales come straight from global memory, one block ahead; a word (8 nibbles of one
-// column) becomes the 8 bf16 of one B fragment in the order (0, 2, 4, 6, 1, 3, 5, 7) of its nibbles, which is the
-// order the x fragments are packed in as well.
+// Workgroup = 4 waves = 32 RB rows x 128 CB columns; wave w owns 32 CB columns as RB x CB tiles of 32 x 32
+// (RB = CB = 1, or 2 for large problems).  K runs in blocks of 64 (two 32-k chunks).  The x pieces of a block are
+// staged through LDS, double buffered, in exactly the order the A operand wants them: thread t splits the 8 floats
+// k = 8 * (t % 8) .. + 7 of row t / 8 (and of row t / 8 + 32 when RB = 2) and writes one 16-byte fragment per
+// piece, so an MFMA's A operand is one conflict-free 1 KiB read.  B words and scales come straight from global
+// memory, one block ahead; a word (8 nibbles of one column) becomes the 8 bf16 of one B fragment in the order
+// (0, 2, 4, 6, 1, 3, 5, 7) of its nibbles, which is the order the x fragments are packed in as well.
 //   A fragment: lane (i, hh) = row i, the 8 k of half hh of a 16-k step
 //   B fragment: lane (j, hh) = column j, the same 8 k: packed row 4 * chunk + 2 * step + hh
 //   D: register r of lane (j, hh) = row 8 * (r / 4) + 4 * hh + r % 4, column j
@@ -28,7 +28,7 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int GB_WAVES = 4, GB_BN = 64 * GB_WAVES, GB_KB = 64;  // waves, columns, k per block; rows: 32 * RB
+constexpr int GB_WAVES = 4, GB_KB = 64;  // waves, k per block; rows: 32 * RB, columns: 32 * CB per wave
 constexpr int GB_CHUNKS = GB_KB / 32;                                       // 32-k chunks per block
 constexpr int GB_FRAG_BYTES = 32 * 16;                                      // one half of an A operand: 32 rows x 8 bf16
 constexpr int GB_BUF_BYTES = GB_CHUNKS * 3 * 2 * 2 * 2 * GB_FRAG_BYTES;  // 24 KiB (two row blocks)
@@ -70,21 +70,20 @@ __device__ __forceinline__ bf16x8 nibbles_to_bf16(uint32_t w) {
     return __builtin_bit_cast(bf16x8, v);
 }
 
-template <int RB>  // row blocks of 32 per workgroup
+template <int RB, int CB>  // row blocks of 32 per workgroup, column blocks of 32 per wave
 __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const GemmBfParams p) {
-    constexpr int GB_BM = 32 * RB;
+    constexpr int GB_BM = 32 * RB, GB_BN = 32 * CB * GB_WAVES;
     __shared__ __align__(16) unsigned char s_a[2][GB_BUF_BYTES];
     __shared__ int s_last;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int j = lane & 31, hh = lane >> 5;
-    const int m0 = blockIdx.y * GB_BM, n0 = blockIdx.x * GB_BN + wave * 64;
+    const int m0 = blockIdx.y * GB_BM, n0 = blockIdx.x * GB_BN + wave * 32 * CB;
     const int chunks = p.K / 32, kblocks = (chunks + GB_CHUNKS - 1) / GB_CHUNKS;
     const int ksplit = gridDim.z, kb0 = blockIdx.z * p.blocks_per_split, kb1 = min(kblocks, kb0 + p.blocks_per_split);
     const bool wave_active = n0 < p.N;
-    const int cb_count = p.N - n0 > 32 ? 2 : 1;
-    int col[2];
-    col[0] = min(n0 + j, p.N - 1);  // out-of-range columns read the last one and are not stored
-    col[1] = min(n0 + 32 + j, p.N - 1);
+    int col[CB];  // out-of-range columns read the last one and are not stored
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) col[cb] = min(n0 + 32 * cb + j, p.N - 1);
 
     // ---- staging role of this thread: rows t / 8 and t / 8 + 32, the 8 floats at 8 * (t % 8) of the block.
     // Everything in the K loop is branch-free (clamped addresses, zeros by selection).  Registers filled by a load
@@ -124,15 +123,15 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
     };
 
     // ---- B side of this lane: per chunk and column tile two words (16-k steps) and one scale ----
-    uint32_t bw[2][GB_CHUNKS][2][2];  // [block parity][chunk][column tile][step]
-    float bs[2][GB_CHUNKS][2];
+    uint32_t bw[2][GB_CHUNKS][CB][2];  // [block parity][chunk][column tile][step]
+    float bs[2][GB_CHUNKS][CB];
     auto load_b = [&](int kb, int set) {
 #pragma unroll
         for (int c = 0; c < GB_CHUNKS; ++c) {
             const bool valid = kb * GB_CHUNKS + c < chunks;
             const int chunk = valid ? kb * GB_CHUNKS + c : chunks - 1;  // past the end: a valid address and a zero scale
 #pragma unroll
-            for (int cb = 0; cb < 2; ++cb) {
+            for (int cb = 0; cb < CB; ++cb) {
                 const uint32_t *src = p.packed + (size_t)(4 * chunk + hh) * p.N + col[cb];
                 bw[set][c][cb][0] = src[0];
                 bw[set][c][cb][1] = src[2 * (size_t)p.N];
@@ -142,11 +141,11 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
         }
     };
 
-    floatx16 acc[RB][2];
+    floatx16 acc[RB][CB];
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int cb = 0; cb < 2; ++cb)
+        for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[rb][cb][r] = 0.0f;
 
@@ -156,11 +155,11 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
         return *reinterpret_cast<const bf16x8 *>(s_a[buf] + frag_offset(c, piece, st, rb, hh) + ((j + 4 * c + 2 * st + hh) & 31) * 16);
     };
 
-    bf16x8 bf[GB_CHUNKS][2][2];  // [chunk][column tile][step]
-    float sc[GB_CHUNKS][2];
+    bf16x8 bf[GB_CHUNKS][CB][2];  // [chunk][column tile][step]
+    float sc[GB_CHUNKS][CB];
     auto convert = [&](int set, int c) {
 #pragma unroll
-        for (int cb = 0; cb < 2; ++cb) {
+        for (int cb = 0; cb < CB; ++cb) {
 #pragma unroll
             for (int st = 0; st < 2; ++st) bf[c][cb][st] = nibbles_to_bf16(bw[set][c][cb][st]);
             sc[c][cb] = bs[set][c][cb];
@@ -180,7 +179,7 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
     // block + 2 (x), then works on with the MFMAs of a group beside the vector work named at its end.
     auto block = [&](int kb, auto parity) {
         constexpr int P = decltype(parity)::value;
-        floatx16 gs[2][2];  // [group parity][column tile]: the sums of one chunk and row block
+        floatx16 gs[2][CB];  // [group parity][column tile]: the sums of one chunk and row block
         const floatx16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         bf16x8 a[3][2];
 #pragma unroll
@@ -195,7 +194,7 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
 #pragma unroll
                 for (int st = 0; st < 2; ++st) {
 #pragma unroll
-                    for (int cb = 0; cb < 2; ++cb) {
+                    for (int cb = 0; cb < CB; ++cb) {
                         if (piece == 0 && st == 0) gs[g][cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[piece][st], bf[c][cb][st], zero, 0, 0, 0);
                         else gs[g][cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[piece][st], bf[c][cb][st], gs[g][cb], 0, 0, 0);
                     }
@@ -209,7 +208,7 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
             } else {  // the previous group's sums, scaled, join the accumulators
                 const int pc = (t - 1) / RB, prb = (t - 1) % RB, pg = (t - 1) & 1;
 #pragma unroll
-                for (int cb = 0; cb < 2; ++cb)
+                for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) acc[prb][cb][r] = fmaf(sc[pc][cb], gs[pg][cb][r], acc[prb][cb][r]);
             }
@@ -217,7 +216,7 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
             __builtin_amdgcn_sched_barrier(0);  // a group's vector work stays beside its MFMAs
         }
 #pragma unroll
-        for (int cb = 0; cb < 2; ++cb)
+        for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[RB - 1][cb][r] = fmaf(sc[1][cb], gs[1][cb][r], acc[RB - 1][cb][r]);
         convert(P ^ 1, 0);  // chunk 0 of the next block
@@ -234,19 +233,19 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
         // Partial sums live in the order of the registers: [slice][tile][wave][rb][cb][pair of r][lane] 8-byte
         // words, so that a wave writes and reads whole 512-byte lines with constant offsets from one address.
         const int tile = blockIdx.y * gridDim.x + blockIdx.x, tiles = gridDim.x * gridDim.y;
-        constexpr int kWaveWords = RB * 2 * 8 * 64;  // 8-byte words of one wave's results
+        constexpr int kWaveWords = RB * CB * 8 * 64;  // 8-byte words of one wave's results
         unsigned long long *mine = reinterpret_cast<unsigned long long *>(p.partial) +
                                    ((size_t)(blockIdx.z * tiles + tile) * GB_WAVES + wave) * kWaveWords + lane;
         if (wave_active) {
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-                for (int cb = 0; cb < 2; ++cb)
+                for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
                     for (int q = 0; q < 8; ++q) {
                         const unsigned long long v = (unsigned long long)__float_as_uint(acc[rb][cb][2 * q]) |
                                                      ((unsigned long long)__float_as_uint(acc[rb][cb][2 * q + 1]) << 32);
-                        __hip_atomic_store(mine + ((rb * 2 + cb) * 8 + q) * 64, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        __hip_atomic_store(mine + ((rb * CB + cb) * 8 + q) * 64, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     }
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -264,14 +263,14 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-                for (int cb = 0; cb < 2; ++cb) acc[rb][cb] = floatx16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                for (int cb = 0; cb < CB; ++cb) acc[rb][cb] = floatx16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
             for (int sp0 = 0; sp0 < ksplit; sp0 += 2) {  // slice order: the same sum every run; two slices = 64 loads in flight
-                unsigned long long part[2][RB * 16];
+                unsigned long long part[2][RB * CB * 8];
 #pragma unroll
                 for (int u = 0; u < 2; ++u) {
                     const unsigned long long *src = first + (size_t)(sp0 + u < ksplit ? sp0 + u : sp0) * slice_words;
 #pragma unroll
-                    for (int w = 0; w < RB * 16; ++w) part[u][w] = __hip_atomic_load(src + w * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    for (int w = 0; w < RB * CB * 8; ++w) part[u][w] = __hip_atomic_load(src + w * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
 #pragma unroll
                 for (int u = 0; u < 2; ++u) {
@@ -279,10 +278,10 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
 #pragma unroll
                     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-                        for (int cb = 0; cb < 2; ++cb)
+                        for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
                             for (int q = 0; q < 8; ++q) {
-                                const unsigned long long v = part[u][(rb * 2 + cb) * 8 + q];
+                                const unsigned long long v = part[u][(rb * CB + cb) * 8 + q];
                                 acc[rb][cb][2 * q] += __uint_as_float((uint32_t)v);
                                 acc[rb][cb][2 * q + 1] += __uint_as_float((uint32_t)(v >> 32));
                             }
@@ -292,7 +291,7 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
     }
     if (!wave_active) return;
 #pragma unroll
-    for (int cb = 0; cb < 2; ++cb) {
+    for (int cb = 0; cb < CB; ++cb) {
         const int n = n0 + 32 * cb + j;
         if (n >= p.N) continue;
         const float bias = p.bias ? p.bias[n] : 0.0f;
@@ -324,11 +323,14 @@ int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t
     GemmBfParams p{};
     p.x = x; p.packed = packed; p.scales = scales; p.bias = bias; p.residual = residual; p.y = y;
     p.M = M; p.N = N; p.K = K; p.chunk_shift = __builtin_ctz((unsigned)(group / 32)); p.flags = flags;
-    // 32 rows per workgroup; 64 (every weight fragment serves two row blocks) once that still leaves a workgroup
-    // per CU (M = 1024: N = 3072 29.4 us against 32.9 us with 64 rows, N = 6400 105.6 us against 96.5 us)
-    const int RB = ceil_div(N, GB_BN) * ceil_div(M, 64) >= ctx->num_cus ? 2 : 1;
-    const int BM = 32 * RB;
-    const int tiles = ceil_div(N, GB_BN) * ceil_div(M, BM);
+    // Workgroup tile: 32 rows x 128 columns (one 32 x 32 tile per wave), which puts the most waves on the chip for
+    // the layer sizes of GPT-2 small; 64 x 256 (every weight fragment serves two row blocks, every x fragment two
+    // column blocks) once that still leaves a workgroup per CU.  M = 1024, K = 768, N = 2304: 25.8 us with the
+    // small tile, 28.2 us with 32 x 256, 33.1 us with 64 x 256; K = 1600, N = 6400: 96.5 us with the large tile,
+    // 105.6 us with 32 x 256.
+    const bool large = ceil_div(N, 256) * ceil_div(M, 64) >= ctx->num_cus;
+    const int BM = large ? 64 : 32, BN = large ? 256 : 128;
+    const int tiles = ceil_div(N, BN) * ceil_div(M, BM);
     const int kblocks = ceil_div(K, GB_KB);
     // K slices: the one with the least estimated time, in units of one K block of one workgroup.  A workgroup costs
     // its blocks plus about 2.2 for its start and end; workgroups beyond one per CU run in rounds, of which a part
@@ -348,13 +350,13 @@ int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t
         }
     }
     if (tiles > kNumCounters) ksplit = 1;
-    while (ksplit > 1 && (size_t)ksplit * tiles * BM * GB_BN * sizeof(float) > kWorkspaceBytes / 2) --ksplit;
+    while (ksplit > 1 && (size_t)ksplit * tiles * BM * BN * sizeof(float) > kWorkspaceBytes / 2) --ksplit;
     p.blocks_per_split = ceil_div(kblocks, ksplit);
     ksplit = ceil_div(kblocks, p.blocks_per_split);
     p.partial = reinterpret_cast<float *>(ctx->workspace);
     p.counters = ctx->counters;
-    const dim3 grid(ceil_div(N, GB_BN), ceil_div(M, BM), ksplit);
-    if (RB == 1) hipLaunchKernelGGL(int4_gemm_bf16_kernel<1>, grid, dim3(64 * GB_WAVES), 0, ctx->stream, p);
-    else hipLaunchKernelGGL(int4_gemm_bf16_kernel<2>, grid, dim3(64 * GB_WAVES), 0, ctx->stream, p);
+    const dim3 grid(ceil_div(N, BN), ceil_div(M, BM), ksplit);
+    if (large) hipLaunchKernelGGL((int4_gemm_bf16_kernel<2, 2>), grid, dim3(64 * GB_WAVES), 0, ctx->stream, p);
+    else hipLaunchKernelGGL((int4_gemm_bf16_kernel<1, 1>), grid, dim3(64 * GB_WAVES), 0, ctx->stream, p);
     return AGPU_LAUNCH_CHECK(ctx, "int4_gemm_bf16_kernel");
 }
