@@ -83,6 +83,59 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const float *a, const f
     }
 }
 
+// The same with 16-byte accesses: one wave per row, lane l owns the float4 numbers l, l + 64, ... of the row
+// (d % 4 == 0, d <= 64 * LN_CACHE, 16-byte aligned pointers).  For the many rows of a prefill.
+template <bool ADD>
+__global__ __launch_bounds__(256) void layer_norm_vec4_kernel(const float *a, const float *b, const float *__restrict__ gamma,
+                                                               const float *__restrict__ beta, float *sum_out, float *y,
+                                                               int rows, int d, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int d4 = d >> 2;
+    const float4 *ar = reinterpret_cast<const float4 *>(a + (size_t)row * d);
+    const float4 *br = ADD ? reinterpret_cast<const float4 *>(b + (size_t)row * d) : nullptr;
+    float4 *sr = (ADD && sum_out) ? reinterpret_cast<float4 *>(sum_out + (size_t)row * d) : nullptr;
+    float4 *yr = reinterpret_cast<float4 *>(y + (size_t)row * d);
+    float4 v[LN_CACHE / 4];
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < LN_CACHE / 4; ++i) {
+        const int k = lane + 64 * i;
+        float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (k < d4) {
+            t = ar[k];
+            if (ADD) {
+                const float4 u = br[k];
+                t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
+                if (sr) sr[k] = t;
+            }
+        }
+        v[i] = t;
+        s += (t.x + t.y) + (t.z + t.w);
+    }
+    const float mean = wave_sum(s) / (float)d;
+    float q = 0.0f;
+#pragma unroll
+    for (int i = 0; i < LN_CACHE / 4; ++i) {
+        if (lane + 64 * i < d4) {
+            const float dx = v[i].x - mean, dy = v[i].y - mean, dz = v[i].z - mean, dw = v[i].w - mean;
+            q += (dx * dx + dy * dy) + (dz * dz + dw * dw);
+        }
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)d + eps);
+    const float4 *g4 = reinterpret_cast<const float4 *>(gamma), *b4 = reinterpret_cast<const float4 *>(beta);
+#pragma unroll
+    for (int i = 0; i < LN_CACHE / 4; ++i) {
+        const int k = lane + 64 * i;
+        if (k < d4) {
+            const float4 g = g4[k], be = b4[k];
+            yr[k] = make_float4((v[i].x - mean) * rstd * g.x + be.x, (v[i].y - mean) * rstd * g.y + be.y,
+                                (v[i].z - mean) * rstd * g.z + be.z, (v[i].w - mean) * rstd * g.w + be.w);
+        }
+    }
+}
+
 // One 256-thread workgroup per row, for launches with few rows (decode): every load of the row is in
 // flight at once and the code stays short.  d <= 256 * LNW_CACHE.
 constexpr int LNW_CACHE = 8;
@@ -144,6 +197,10 @@ void launch_layer_norm(agpu_ctx *ctx, const float *a, const float *b, const floa
                        float *y, int rows, int d, float eps) {
     if (rows <= 512 && d <= 256 * LNW_CACHE)
         hipLaunchKernelGGL((layer_norm_row_kernel<ADD>), dim3(rows), dim3(256), 0, ctx->stream, a, b, gamma, beta, sum_out, y, d, eps);
+    else if (d % 4 == 0 && d <= 64 * LN_CACHE &&
+             (((uintptr_t)a | (uintptr_t)b | (uintptr_t)gamma | (uintptr_t)beta | (uintptr_t)sum_out | (uintptr_t)y) & 15) == 0)
+        hipLaunchKernelGGL((layer_norm_vec4_kernel<ADD>), dim3(ceil_div(rows, 4)), dim3(256), 0, ctx->stream, a, b, gamma, beta,
+                           sum_out, y, rows, d, eps);
     else
         hipLaunchKernelGGL((layer_norm_kernel<ADD>), dim3(ceil_div(rows, 4)), dim3(256), 0, ctx->stream, a, b, gamma, beta,
                            sum_out, y, rows, d, eps);

@@ -299,12 +299,17 @@ int32_t launch_block(agpu_gpt2 *m, int L, int B, int new_len, int max_kv) {
         rc = agpu_int4_skinny_supported(ga) ? agpu_int4_skinny_launch(ctx, ga) : agpu_int4_gemv_launch(ctx, ga);
         if (rc != AGPU_OK) return rc;
     } else {
-        rc = agpu_ln_int4_linear(ctx, hid, b.ln1_g, b.ln1_b, eps, wq.packed, wq.scales, wq.bias, nullptr, qkv, R, 3 * d, d, g,
-                                 0);
+        // prefill: the GEMM writes the K/V rows into the cache itself where it can
+        const KvScatter kv{kc, vc, m->pos_dev, H, P, new_len};
+        bool kv_done = false;
+        rc = agpu_ln_int4_linear_kv(ctx, hid, b.ln1_g, b.ln1_b, eps, wq.packed, wq.scales, wq.bias, nullptr, qkv, R, 3 * d, d, g, 0,
+                                    &kv, &kv_done);
         if (rc != AGPU_OK) return rc;
-        hipLaunchKernelGGL(kv_scatter_kernel, dim3((unsigned)(((size_t)R * d + 255) / 256)), dim3(256), 0, ctx->stream, qkv, kc,
-                           vc, R, new_len, H, P, m->pos_dev);
-        if ((rc = AGPU_LAUNCH_CHECK(ctx, "kv_scatter_kernel")) != AGPU_OK) return rc;
+        if (!kv_done) {
+            hipLaunchKernelGGL(kv_scatter_kernel, dim3((unsigned)(((size_t)R * d + 255) / 256)), dim3(256), 0, ctx->stream, qkv,
+                               kc, vc, R, new_len, H, P, m->pos_dev);
+            if ((rc = AGPU_LAUNCH_CHECK(ctx, "kv_scatter_kernel")) != AGPU_OK) return rc;
+        }
     }
     AttnParams ap{};
     ap.q = qkv; ap.k = kc; ap.v = vc; ap.o = att;

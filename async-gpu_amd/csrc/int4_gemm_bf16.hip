@@ -45,6 +45,7 @@ struct GemmBfParams {
     int blocks_per_split;    // K blocks of 64 per workgroup (gridDim.z slices of K)
     float *partial;          // [ksplit, M, N] when gridDim.z > 1
     unsigned int *counters;  // one ticket per output tile, left at zero
+    KvScatter kv;            // kcache == nullptr: none
 };
 
 // fragment [chunk][piece][step][row block][half]
@@ -306,6 +307,12 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
                     else if (p.flags & AGPU_EPI_GELU_QUICK) v = gelu_quick_dev(v);
                     if (p.residual) v += p.residual[(size_t)m * p.N + n];
                     p.y[(size_t)m * p.N + n] = v;
+                    if (p.kv.kcache && n >= p.N / 3) {
+                        const int dm = p.N / 3, jj = n - dm, in_v = jj >= dm ? 1 : 0, e = jj - in_v * dm;
+                        const int b = m / p.kv.new_len, s = m - b * p.kv.new_len;
+                        float *dst = in_v ? p.kv.vcache : p.kv.kcache;
+                        dst[((size_t)(b * p.kv.n_heads + (e >> 6)) * p.kv.n_positions + *p.kv.pos_dev + s) * 64 + (e & 63)] = v;
+                    }
                 }
             }
     }
@@ -319,8 +326,10 @@ bool agpu_int4_gemm_bf16_supported(const void *x, int M, int N, int K, int group
 }
 
 int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t *packed, const float *scales, const float *bias,
-                                   const float *residual, float *y, int M, int N, int K, int group, uint32_t flags) {
+                                   const float *residual, float *y, int M, int N, int K, int group, uint32_t flags,
+                                   const KvScatter *kv) {
     GemmBfParams p{};
+    if (kv) p.kv = *kv;
     p.x = x; p.packed = packed; p.scales = scales; p.bias = bias; p.residual = residual; p.y = y;
     p.M = M; p.N = N; p.K = K; p.chunk_shift = __builtin_ctz((unsigned)(group / 32)); p.flags = flags;
     // Workgroup tile: 32 rows x 128 columns (one 32 x 32 tile per wave), which puts the most waves on the chip for

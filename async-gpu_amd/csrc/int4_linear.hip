@@ -211,7 +211,15 @@ AGPU_EXPORT int32_t agpu_ln_int4_linear(agpu_ctx *ctx, const float *x, const flo
                                         float eps, const uint32_t *packed, const float *scales, const float *bias,
                                         const float *residual, float *y, int32_t M, int32_t N, int32_t K,
                                         int32_t group, uint32_t flags) {
+    return agpu_ln_int4_linear_kv(ctx, x, gamma, beta, eps, packed, scales, bias, residual, y, M, N, K, group, flags, nullptr,
+                                  nullptr);
+}
+
+int32_t agpu_ln_int4_linear_kv(agpu_ctx *ctx, const float *x, const float *gamma, const float *beta, float eps,
+                               const uint32_t *packed, const float *scales, const float *bias, const float *residual, float *y,
+                               int32_t M, int32_t N, int32_t K, int32_t group, uint32_t flags, const KvScatter *kv, bool *kv_done) {
     AGPU_REQUIRE_CTX(ctx);
+    if (kv_done) *kv_done = false;
     int32_t rc = check_linear_args(ctx, x, packed, scales, y, M, N, K, group);
     if (rc != AGPU_OK) return rc;
     if ((gamma == nullptr) != (beta == nullptr))
@@ -245,8 +253,11 @@ AGPU_EXPORT int32_t agpu_ln_int4_linear(agpu_ctx *ctx, const float *x, const flo
         if (!(flags & AGPU_EPI_FORCE_FP32_GEMV) && agpu_int4_skinny_supported(a)) return agpu_int4_skinny_launch(ctx, a);
         return agpu_int4_gemv_launch(ctx, a);
     }
-    if (!(flags & AGPU_EPI_FORCE_FP32_GEMV) && agpu_int4_gemm_bf16_supported(xin, M, N, K, group))
-        return agpu_int4_gemm_bf16_launch(ctx, xin, packed, scales, bias, residual, y, M, N, K, group, epi);
+    if (!(flags & AGPU_EPI_FORCE_FP32_GEMV) && agpu_int4_gemm_bf16_supported(xin, M, N, K, group)) {
+        const bool with_kv = kv && kv->kcache && N % 3 == 0 && (N / 3) % 64 == 0;
+        if (with_kv && kv_done) *kv_done = true;
+        return agpu_int4_gemm_bf16_launch(ctx, xin, packed, scales, bias, residual, y, M, N, K, group, epi, with_kv ? kv : nullptr);
+    }
     const dim3 grid(ceil_div(N, GEMM_BN), ceil_div(M, GEMM_BM));
     hipLaunchKernelGGL((int4_gemm_mfma_kernel<false>), grid, dim3(256), 0, ctx->stream, xin, packed, scales,
                        (const float *)nullptr, bias, residual, y, M, N, K, group, epi);

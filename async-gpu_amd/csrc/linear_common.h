@@ -79,11 +79,24 @@ int32_t agpu_int4_gemv_launch(agpu_ctx *ctx, const GemvArgs &a);
 // int8-MFMA variant for M <= 2 (needs group % 32 == 0, K % 64 == 0, N % 4 == 0, 16-byte aligned weights).
 bool agpu_int4_gemv_i8_supported(const GemvArgs &a);
 int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips_per_split, int max_wgs);
+// K/V scatter of a fused QKV projection over rows (sequence b = m / new_len, step s = m % new_len), N = 3*d_model:
+// columns [d, 2d) also go to kcache[(b*n_heads + h), *pos_dev + s, e], columns [2d, 3d) to vcache.
+struct KvScatter {
+    float *kcache;
+    float *vcache;
+    const int *pos_dev;
+    int n_heads, n_positions, new_len;
+};
 // bf16-MFMA GEMM for M > 16 with x split into three bf16 pieces (needs group / 32 a power of two, K % 32 == 0,
-// 16-byte aligned x).
+// 16-byte aligned x).  kv (optional): the K/V scatter above, done by the same launch.
 bool agpu_int4_gemm_bf16_supported(const void *x, int M, int N, int K, int group);
 int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t *packed, const float *scales, const float *bias,
-                                   const float *residual, float *y, int M, int N, int K, int group, uint32_t flags);
+                                   const float *residual, float *y, int M, int N, int K, int group, uint32_t flags,
+                                   const KvScatter *kv = nullptr);
+// LayerNorm (optional) + Linear like agpu_ln_int4_linear; *kv_done tells whether the launch did the K/V scatter.
+int32_t agpu_ln_int4_linear_kv(agpu_ctx *ctx, const float *x, const float *gamma, const float *beta, float eps,
+                               const uint32_t *packed, const float *scales, const float *bias, const float *residual, float *y,
+                               int32_t M, int32_t N, int32_t K, int32_t group, uint32_t flags, const KvScatter *kv, bool *kv_done);
 // MFMA variant for 4 < M <= 16 (needs group % 32 == 0, K % 32 == 0, N % 4 == 0, 16-byte aligned weights).
 bool agpu_int4_skinny_supported(const GemvArgs &a);
 int32_t agpu_int4_skinny_launch(agpu_ctx *ctx, const GemvArgs &a);

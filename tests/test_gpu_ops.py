@@ -327,7 +327,8 @@ def _ln_inputs(rows=4, d=768):
     return x, gamma, beta
 
 
-@pytest.mark.parametrize("rows,d", [(4, 768), (1, 768), (16, 1600), (64, 768), (3, 100), (2, 4100)])
+@pytest.mark.parametrize("rows,d", [(4, 768), (1, 768), (16, 1600), (64, 768), (3, 100), (2, 4100), (1027, 768), (600, 1600),
+                                    (515, 102)])
 def test_layer_norm(agpu, orc, dev, rows, d):
     from async_gpu_amd import ops
     x, gamma, beta = _ln_inputs(rows, d)
@@ -337,9 +338,10 @@ def test_layer_norm(agpu, orc, dev, rows, d):
     assert np.abs(y - orc.layer_norm(x, gamma, beta, 1e-5)).max() <= 1e-5  # reference tolerance: 1e-3
 
 
-def test_add_layer_norm_dual(agpu, orc, dev):
+@pytest.mark.parametrize("rows", [5, 700])
+def test_add_layer_norm_dual(agpu, orc, dev, rows):
     from async_gpu_amd import ops
-    x, gamma, beta = _ln_inputs(5, 768)
+    x, gamma, beta = _ln_inputs(rows, 768)
     b = (np.random.default_rng(1).standard_normal(x.shape)).astype(np.float32)
     s, n = ops.add_layer_norm_dual(to_dev(x, dev), to_dev(b, dev), to_dev(gamma, dev), to_dev(beta, dev))
     so, no = orc.add_layer_norm_dual(x, b, gamma, beta)
