@@ -4,7 +4,7 @@ configurations other than the headline one, which bench.py covers): isolated int
 attention prefill / decode, and GPT-2 XL-shaped decode at batch 1 and 16.  Prints one JSON line per
 case.  Kernel cases are timed as graph replays with HIP events on the context's stream.
 
-    python3 async-gpu_amd/bench_configs.py [--xl-layers 48] [--skip-xl] [--skip-kernels]
+    python3 async-gpu_amd/bench_configs.py [--xl-layers 48] [--skip-xl] [--skip-kernels] [--prefill-only]
 """
 import argparse
 import ctypes as C
@@ -27,6 +27,7 @@ def main():
     ap.add_argument("--xl-layers", type=int, default=48)
     ap.add_argument("--skip-xl", action="store_true")
     ap.add_argument("--skip-kernels", action="store_true")
+    ap.add_argument("--prefill-only", action="store_true", help="only the whole-model prefill of GPT-2 small (for kernel traces)")
     ap.add_argument("--cpu", action="store_true", help="also time the CPU oracle on configs 1-3 (single thread, as the reference CPU path)")
     args = ap.parse_args()
     entry.load_package()
@@ -50,11 +51,42 @@ def main():
             ctx.free(p)
         return us.value
 
+    if args.prefill_only:
+        prefill_cases(ctx, emit, _lib, gpt2, workloads, lengths=(1024,))
+        return
     if not args.skip_kernels:
         kernel_cases(ctx, emit, bench_linear, workloads, args)
+        prefill_cases(ctx, emit, _lib, gpt2, workloads)
     if args.skip_xl:
         return
     xl_cases(ctx, emit, args, _lib, gpt2, workloads)
+
+
+def prefill_cases(ctx, emit, _lib, gpt2, workloads, lengths=(1024, 512, 128, 32)):
+    """Whole-model prefill of GPT-2 small (int4 g32, tied int4 head): tokens in, logits of the last row out; wall
+    clock around launch + synchronise, best of 5 after one untimed pass."""
+    from async_gpu_amd import ops
+    cfg = workloads.GPT2_SMALL
+    weights = workloads.gpt2_fp32_weights(cfg, seed=3)
+    qz = workloads.quantize_gpt2(weights, 32, lambda wt, g: ops.int4_quantize_host(wt, g, _lib.QUANT_SCRIPT))
+    model = gpt2.Int4Gpt2Model.from_quantized(gpt2.Gpt2Config.small(group_size=32), qz, ctx=ctx)
+    lg = ctx.malloc(cfg["vocab"] * 4)
+    for n in lengths:
+        tokens = np.atleast_2d(workloads.random_prompt(cfg, 1, n).astype(np.uint32))
+        p = ctx.upload(tokens)
+        ts = []
+        for _ in range(6):
+            model.reset_cache()
+            ctx.sync()
+            t0 = time.perf_counter()
+            model._call("agpu_gpt2_forward_cached", p, 1, n, lg, 0)
+            ctx.sync()
+            ts.append((time.perf_counter() - t0) * 1e3)
+        ms = min(ts[1:])
+        emit(case=f"GPT-2 small int4 prefill, {n} tokens, last-row logits", ms=round(ms, 4), tok_s=round(n / ms * 1e3, 0))
+        ctx.free(p)
+    ctx.free(lg)
+    model.close()
 
 
 def kernel_cases(ctx, emit, bench_linear, workloads, args=None):
