@@ -9,7 +9,7 @@
 // fp32, which is the reference's w = q * scale, y += x * w up to the order of the roundings.
 //
 // Workgroup = 4 waves = 32 RB rows x 128 CB columns; wave w owns 32 CB columns as RB x CB tiles of 32 x 32
-// (RB = CB = 1, or 2 for large problems).  K runs in blocks of 64 (two 32-k chunks).  The x pieces of a block are
+// (RB = CB = 1, or 2 for large problems).  K runs in blocks of 64 or 128 (NCH 32-k chunks).  The x pieces of a block are
 // staged through LDS, double buffered, in exactly the order the A operand wants them: thread t splits the 8 floats
 // k = 8 * (t % 8) .. + 7 of row t / 8 (and of row t / 8 + 32 when RB = 2) and writes one 16-byte fragment per
 // piece, so an MFMA's A operand is one conflict-free 1 KiB read.  B words and scales come straight from global
@@ -28,10 +28,8 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int GB_WAVES = 4, GB_KB = 64;  // waves, k per block; rows: 32 * RB, columns: 32 * CB per wave
-constexpr int GB_CHUNKS = GB_KB / 32;                                       // 32-k chunks per block
+constexpr int GB_WAVES = 4;  // waves; rows: 32 * RB, columns: 32 * CB per wave, k per block: 32 * NCH
 constexpr int GB_FRAG_BYTES = 32 * 16;                                      // one half of an A operand: 32 rows x 8 bf16
-constexpr int GB_BUF_BYTES = GB_CHUNKS * 3 * 2 * 2 * 2 * GB_FRAG_BYTES;  // 24 KiB (two row blocks)
 
 struct GemmBfParams {
     const float *x;
@@ -49,8 +47,9 @@ struct GemmBfParams {
 };
 
 // fragment [chunk][piece][step][row block][half]
+template <int RB>
 __device__ __forceinline__ int frag_offset(int chunk, int piece, int step, int rb, int hh) {
-    return ((((chunk * 3 + piece) * 2 + step) * 2 + rb) * 2 + hh) * GB_FRAG_BYTES;
+    return ((((chunk * 3 + piece) * 2 + step) * RB + rb) * 2 + hh) * GB_FRAG_BYTES;
 }
 
 // the leading 16 bits of two floats as one register: a in the low half
@@ -71,39 +70,42 @@ __device__ __forceinline__ bf16x8 nibbles_to_bf16(uint32_t w) {
     return __builtin_bit_cast(bf16x8, v);
 }
 
-template <int RB, int CB>  // row blocks of 32 per workgroup, column blocks of 32 per wave
+template <int RB, int CB, int NCH>  // row blocks of 32 per workgroup, column blocks of 32 per wave, 32-k chunks per K block
 __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const GemmBfParams p) {
-    constexpr int GB_BM = 32 * RB, GB_BN = 32 * CB * GB_WAVES;
-    __shared__ __align__(16) unsigned char s_a[2][GB_BUF_BYTES];
+    static_assert(NCH % 2 == 0, "staging works on 64-k halves");
+    constexpr int GB_BM = 32 * RB, GB_BN = 32 * CB * GB_WAVES, GB_KB = 32 * NCH, NP = RB * NCH / 2;
+    __shared__ __align__(16) unsigned char s_a[2][NCH * RB * 3 * 2 * 2 * GB_FRAG_BYTES];  // 6 KiB per (chunk, row block)
     __shared__ int s_last;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int j = lane & 31, hh = lane >> 5;
     const int m0 = blockIdx.y * GB_BM, n0 = blockIdx.x * GB_BN + wave * 32 * CB;
-    const int chunks = p.K / 32, kblocks = (chunks + GB_CHUNKS - 1) / GB_CHUNKS;
+    const int chunks = p.K / 32, kblocks = (chunks + NCH - 1) / NCH;
     const int ksplit = gridDim.z, kb0 = blockIdx.z * p.blocks_per_split, kb1 = min(kblocks, kb0 + p.blocks_per_split);
     const bool wave_active = n0 < p.N;
     int col[CB];  // out-of-range columns read the last one and are not stored
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) col[cb] = min(n0 + 32 * cb + j, p.N - 1);
 
-    // ---- staging role of this thread: rows t / 8 and t / 8 + 32, the 8 floats at 8 * (t % 8) of the block.
+    // ---- staging role of this thread: row t / 8 of a row block, the 8 floats at 8 * (t % 8) of a 64-k half of the
+    // block; pass ps of NP = (row block ps % RB, half ps / RB).
     // Everything in the K loop is branch-free (clamped addresses, zeros by selection).  Registers filled by a load
     // are first read one iteration later, where the compiler can only wait for every load in flight; so an
     // iteration reads the old registers first and sends its own requests after that, a whole block ahead ----
     const int si = tid >> 3, sk = tid & 7;
-    float4 xv[2][RB][2];  // [block parity][row block][8 floats]
+    float4 xv[2][NP][2];  // [block parity][pass][8 floats]
     auto load_x = [&](int kb, int set) {
 #pragma unroll
-        for (int ps = 0; ps < RB; ++ps) {
-            const int row = min(m0 + 32 * ps + si, p.M - 1), k = min(kb * GB_KB + 8 * sk, p.K - 8);
+        for (int ps = 0; ps < NP; ++ps) {
+            const int row = min(m0 + 32 * (ps % RB) + si, p.M - 1), k = min(kb * GB_KB + 64 * (ps / RB) + 8 * sk, p.K - 8);
             const float *src = p.x + (size_t)row * p.K + k;
             xv[set][ps][0] = *reinterpret_cast<const float4 *>(src);
             xv[set][ps][1] = *reinterpret_cast<const float4 *>(src + 4);
         }
     };
     auto stage_half = [&](int kb, int set, int buf, int ps) {
-        const int chunk = sk >> 2, step = (sk >> 1) & 1, half = sk & 1;
-        const bool ok = m0 + 32 * ps + si < p.M && kb * GB_KB + 8 * sk < p.K;
+        const int rb = ps % RB, kh = ps / RB;
+        const int chunk = 2 * kh + (sk >> 2), step = (sk >> 1) & 1, half = sk & 1;
+        const bool ok = m0 + 32 * rb + si < p.M && kb * GB_KB + 64 * kh + 8 * sk < p.K;
         const float4 lo4 = xv[set][ps][0], hi4 = xv[set][ps][1];
         const float in[8] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w};
         float v[8], r1[8], r2[8];
@@ -114,23 +116,23 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
             r2[e] = r1[e] - top_bits(r1[e]);  // exact, at most 8 significant bits
         }
         // row slot rotated by the fragment's k position: the 8 threads of a row write 8 different bank groups
-        unsigned char *dst = s_a[buf] + ((si + sk) & 31) * 16;
-        *reinterpret_cast<uint4 *>(dst + frag_offset(chunk, 2, step, ps, half)) =
+        unsigned char *dst = s_a[buf] + ((si + 8 * kh + sk) & 31) * 16;
+        *reinterpret_cast<uint4 *>(dst + frag_offset<RB>(chunk, 2, step, rb, half)) =
             make_uint4(pack_top(v[0], v[2]), pack_top(v[4], v[6]), pack_top(v[1], v[3]), pack_top(v[5], v[7]));
-        *reinterpret_cast<uint4 *>(dst + frag_offset(chunk, 1, step, ps, half)) =
+        *reinterpret_cast<uint4 *>(dst + frag_offset<RB>(chunk, 1, step, rb, half)) =
             make_uint4(pack_top(r1[0], r1[2]), pack_top(r1[4], r1[6]), pack_top(r1[1], r1[3]), pack_top(r1[5], r1[7]));
-        *reinterpret_cast<uint4 *>(dst + frag_offset(chunk, 0, step, ps, half)) =
+        *reinterpret_cast<uint4 *>(dst + frag_offset<RB>(chunk, 0, step, rb, half)) =
             make_uint4(pack_top(r2[0], r2[2]), pack_top(r2[4], r2[6]), pack_top(r2[1], r2[3]), pack_top(r2[5], r2[7]));
     };
 
     // ---- B side of this lane: per chunk and column tile two words (16-k steps) and one scale ----
-    uint32_t bw[2][GB_CHUNKS][CB][2];  // [block parity][chunk][column tile][step]
-    float bs[2][GB_CHUNKS][CB];
+    uint32_t bw[2][NCH][CB][2];  // [block parity][chunk][column tile][step]
+    float bs[2][NCH][CB];
     auto load_b = [&](int kb, int set) {
 #pragma unroll
-        for (int c = 0; c < GB_CHUNKS; ++c) {
-            const bool valid = kb * GB_CHUNKS + c < chunks;
-            const int chunk = valid ? kb * GB_CHUNKS + c : chunks - 1;  // past the end: a valid address and a zero scale
+        for (int c = 0; c < NCH; ++c) {
+            const bool valid = kb * NCH + c < chunks;
+            const int chunk = valid ? kb * NCH + c : chunks - 1;  // past the end: a valid address and a zero scale
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
                 const uint32_t *src = p.packed + (size_t)(4 * chunk + hh) * p.N + col[cb];
@@ -153,17 +155,17 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
     // A fragments of one group (chunk c, row block rb): [piece][step]; a register set is refilled for the next
     // group as soon as its two MFMAs are out
     auto a_frag = [&](int buf, int c, int rb, int piece, int st) {
-        return *reinterpret_cast<const bf16x8 *>(s_a[buf] + frag_offset(c, piece, st, rb, hh) + ((j + 4 * c + 2 * st + hh) & 31) * 16);
+        return *reinterpret_cast<const bf16x8 *>(s_a[buf] + frag_offset<RB>(c, piece, st, rb, hh) + ((j + 4 * c + 2 * st + hh) & 31) * 16);
     };
 
-    bf16x8 bf[GB_CHUNKS][CB][2];  // [chunk][column tile][step]
-    float sc[GB_CHUNKS][CB];
+    bf16x8 bf[2][CB][2];  // [chunk parity][column tile][step]: chunk c + 1 is converted while chunk c is in use
+    float sc[2][CB];
     auto convert = [&](int set, int c) {
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
 #pragma unroll
-            for (int st = 0; st < 2; ++st) bf[c][cb][st] = nibbles_to_bf16(bw[set][c][cb][st]);
-            sc[c][cb] = bs[set][c][cb];
+            for (int st = 0; st < 2; ++st) bf[c & 1][cb][st] = nibbles_to_bf16(bw[set][c][cb][st]);
+            sc[c & 1][cb] = bs[set][c][cb];
         }
     };
 
@@ -172,7 +174,7 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
     load_b(kb0, 0);
     load_x(min(kb0 + 1, kblocks), 1);
 #pragma unroll
-    for (int ps = 0; ps < RB; ++ps) stage_half(kb0, 0, 0, ps);
+    for (int ps = 0; ps < NP; ++ps) stage_half(kb0, 0, 0, ps);
     convert(0, 0);
     __syncthreads();
 
@@ -188,7 +190,7 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
 #pragma unroll
             for (int st = 0; st < 2; ++st) a[piece][st] = a_frag(P, 0, 0, piece, st);
 #pragma unroll
-        for (int t = 0; t < 2 * RB; ++t) {  // group t = (chunk t / RB, row block t % RB)
+        for (int t = 0; t < NCH * RB; ++t) {  // group t = (chunk t / RB, row block t % RB)
             const int c = t / RB, g = t & 1;
 #pragma unroll
             for (int piece = 0; piece < 3; ++piece)
@@ -196,30 +198,34 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
                 for (int st = 0; st < 2; ++st) {
 #pragma unroll
                     for (int cb = 0; cb < CB; ++cb) {
-                        if (piece == 0 && st == 0) gs[g][cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[piece][st], bf[c][cb][st], zero, 0, 0, 0);
-                        else gs[g][cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[piece][st], bf[c][cb][st], gs[g][cb], 0, 0, 0);
+                        if (piece == 0 && st == 0) gs[g][cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[piece][st], bf[c & 1][cb][st], zero, 0, 0, 0);
+                        else gs[g][cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[piece][st], bf[c & 1][cb][st], gs[g][cb], 0, 0, 0);
                     }
-                    if (t + 1 < 2 * RB) a[piece][st] = a_frag(P, (t + 1) / RB, (t + 1) % RB, piece, st);
+                    if (t + 1 < NCH * RB) a[piece][st] = a_frag(P, (t + 1) / RB, (t + 1) % RB, piece, st);
                 }
-            if (t == 0) {
-                convert(P, 1);  // the first read of registers that a load of the previous iteration fills
-                __builtin_amdgcn_sched_barrier(0);
-                load_b(min(kb + 1, kblocks), P ^ 1);
-                load_x(min(kb + 2, kblocks), P);
-            } else {  // the previous group's sums, scaled, join the accumulators
+            // vector work beside these MFMAs: first the previous group's sums, scaled, join the accumulators
+            if (t > 0) {
                 const int pc = (t - 1) / RB, prb = (t - 1) % RB, pg = (t - 1) & 1;
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) acc[prb][cb][r] = fmaf(sc[pc][cb], gs[pg][cb][r], acc[prb][cb][r]);
+                    for (int r = 0; r < 16; ++r) acc[prb][cb][r] = fmaf(sc[pc & 1][cb], gs[pg][cb][r], acc[prb][cb][r]);
             }
-            if (t >= 1 && t - 1 < RB) stage_half(kb + 1, P ^ 1, P ^ 1, t - 1);
+            // then the words of the next chunk become fragments (in place of those of the chunk before this one)
+            if (t % RB == 0 && c + 1 < NCH) convert(P, c + 1);
+            if (t == 0) {  // that was the first read of registers that a load of the previous iteration fills
+                __builtin_amdgcn_sched_barrier(0);
+                load_b(min(kb + 1, kblocks), P ^ 1);
+                load_x(min(kb + 2, kblocks), P);
+            }
+            if (t >= 1 && t - 1 < NP) stage_half(kb + 1, P ^ 1, P ^ 1, t - 1);
             __builtin_amdgcn_sched_barrier(0);  // a group's vector work stays beside its MFMAs
         }
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[RB - 1][cb][r] = fmaf(sc[1][cb], gs[1][cb][r], acc[RB - 1][cb][r]);
+            for (int r = 0; r < 16; ++r)
+                acc[RB - 1][cb][r] = fmaf(sc[(NCH - 1) & 1][cb], gs[(NCH * RB - 1) & 1][cb][r], acc[RB - 1][cb][r]);
         convert(P ^ 1, 0);  // chunk 0 of the next block
         __syncthreads();
     };
@@ -340,8 +346,13 @@ int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t
     const bool large = ceil_div(N, 256) * ceil_div(M, 64) >= ctx->num_cus;
     const int BM = large ? 64 : 32, BN = large ? 256 : 128;
     const int tiles = ceil_div(N, BN) * ceil_div(M, BM);
-    const int kblocks = ceil_div(K, GB_KB);
-    // K slices: the one with the least estimated time, in units of one K block of one workgroup.  A workgroup costs
+    // K per block: 64; 128 for the small tile on small problems (fewer barriers and loop ends per k, but 159
+    // registers against 126, three waves per SIMD against four: M = 512, K = 768, N = 2304: 17.5 us against 18.7 us;
+    // M = 1024: 27.3 us against 25.8 us)
+    const bool long_blocks = !large && (long long)tiles * ceil_div(K, 64) <= 5000;
+    const int KB = long_blocks ? 128 : 64;
+    const int kblocks = ceil_div(K, KB);
+    // K slices: the one with the least estimated time, in units of 64 k of one workgroup.  A workgroup costs
     // its blocks plus about 2.2 for its start and end; workgroups beyond one per CU run in rounds, of which a part
     // overlaps (the mean of the whole and the fractional number of rounds fits the measurements); slices cost the
     // write, the ticket and one read-back round per two of them.
@@ -351,7 +362,7 @@ int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t
         const int bps = ceil_div(kblocks, ks), ks2 = ceil_div(kblocks, bps);
         const float w = (float)tiles * ks2 / ctx->num_cus;
         const float rounds = 0.5f * ((float)ceil_div(tiles * ks2, ctx->num_cus) + (w > 1.0f ? w : 1.0f));
-        float c = rounds * (bps + 2.2f);
+        float c = rounds * (bps * (KB / 64) + 2.2f);
         if (ks2 > 1) c += 0.75f + 0.18f * ks2;
         if (ks == 1 || c < best) {
             best = c;
@@ -365,7 +376,8 @@ int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t
     p.partial = reinterpret_cast<float *>(ctx->workspace);
     p.counters = ctx->counters;
     const dim3 grid(ceil_div(N, BN), ceil_div(M, BM), ksplit);
-    if (large) hipLaunchKernelGGL((int4_gemm_bf16_kernel<2, 2>), grid, dim3(64 * GB_WAVES), 0, ctx->stream, p);
-    else hipLaunchKernelGGL((int4_gemm_bf16_kernel<1, 1>), grid, dim3(64 * GB_WAVES), 0, ctx->stream, p);
+    if (large) hipLaunchKernelGGL((int4_gemm_bf16_kernel<2, 2, 2>), grid, dim3(64 * GB_WAVES), 0, ctx->stream, p);
+    else if (long_blocks) hipLaunchKernelGGL((int4_gemm_bf16_kernel<1, 1, 4>), grid, dim3(64 * GB_WAVES), 0, ctx->stream, p);
+    else hipLaunchKernelGGL((int4_gemm_bf16_kernel<1, 1, 2>), grid, dim3(64 * GB_WAVES), 0, ctx->stream, p);
     return AGPU_LAUNCH_CHECK(ctx, "int4_gemm_bf16_kernel");
 }
