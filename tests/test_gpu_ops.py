@@ -188,6 +188,31 @@ def test_gemv_int8_fixed_point_ranges(agpu, orc, dev):
     assert not np.isfinite(y[0]).any() and np.isfinite(y[1]).all()
 
 
+def test_gemm_error_bound_over_the_dynamic_range(agpu, orc, dev):
+    """The bf16 matrix-core GEMM (x as three exact bf16 pieces, exact weights) keeps the error of every output below
+    4e-7 * sum |x| |w|, whatever the range of x: extreme nibbles, rows of very different magnitudes side by side."""
+    from async_gpu_amd import ops, workloads
+    rng = np.random.default_rng(13)
+    K, N, g, M = 768, 300, 32, 40
+    packed, scales, _ = workloads.random_int4_linear(rng, K, N, g)
+    packed[::2] = 0xFFFFFFFF  # nibble 15 -> +7
+    packed[1::2] = 0x00000000  # nibble 0 -> -8
+    dp, ds = to_dev(packed, dev), to_dev(scales, dev)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    x[0:8] *= np.exp(rng.uniform(-12, 4, (8, K))).astype(np.float32)
+    x[8:12] *= np.float32(1e-20)
+    x[12:16] *= np.float32(1e-33)
+    x[16:20] *= np.float32(1e30)
+    x[20] = np.where(np.arange(K) == 5, np.float32(3e4), x[20])
+    x[21] = 0.0
+    y = ops.int4_linear(to_dev(x, dev), dp, ds, group=g).cpu().numpy()
+    ref = orc.int4_gemm_f64(x, packed, scales, g)
+    bound = np.abs(x).astype(np.float64) @ np.abs(orc.int4_dequantize(packed, scales, g)).astype(np.float64)
+    err = np.abs(y - ref)
+    assert np.all(err <= 4e-7 * bound + 1e-27), float((err / (bound + 1e-300)).max())
+    assert np.all(y[21] == 0.0)
+
+
 @pytest.mark.parametrize("M", [128, 512, 1024, 17, 100])
 def test_config2_gemm(agpu, orc, dev, M):
     """BASELINE config 2: K=768, N=2304, group 32, seed 1, M in {128, 512, 1024} (+ ragged M)."""
