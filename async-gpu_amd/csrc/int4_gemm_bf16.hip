@@ -28,7 +28,6 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int GB_WAVES = 4;  // waves; rows: 32 * RB, columns: 32 * CB per wave, k per block: 32 * NCH
 constexpr int GB_FRAG_BYTES = 32 * 16;                                      // one half of an A operand: 32 rows x 8 bf16
 
 struct GemmBfParams {
@@ -70,7 +69,9 @@ __device__ __forceinline__ bf16x8 nibbles_to_bf16(uint32_t w) {
     return __builtin_bit_cast(bf16x8, v);
 }
 
-template <int RB, int CB, int NCH>  // row blocks of 32 per workgroup, column blocks of 32 per wave, 32-k chunks per K block
+// RB row blocks of 32 per workgroup, CB column blocks of 32 per wave, NCH 32-k chunks per K block, GB_WAVES waves (4 or
+// 8; the first four stage x)
+template <int RB, int CB, int NCH, int GB_WAVES>
 __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const GemmBfParams p) {
     static_assert(NCH % 2 == 0, "staging works on 64-k halves");
     constexpr int GB_BM = 32 * RB, GB_BN = 32 * CB * GB_WAVES, GB_KB = 32 * NCH, NP = RB * NCH / 2;
@@ -93,7 +94,9 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
     // iteration reads the old registers first and sends its own requests after that, a whole block ahead ----
     const int si = tid >> 3, sk = tid & 7;
     float4 xv[2][NP][2];  // [block parity][pass][8 floats]
+    const bool stager = GB_WAVES == 4 || tid < 256;  // wave-uniform
     auto load_x = [&](int kb, int set) {
+        if (!stager) return;
 #pragma unroll
         for (int ps = 0; ps < NP; ++ps) {
             const int row = min(m0 + 32 * (ps % RB) + si, p.M - 1), k = min(kb * GB_KB + 64 * (ps / RB) + 8 * sk, p.K - 8);
@@ -103,6 +106,7 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
         }
     };
     auto stage_half = [&](int kb, int set, int buf, int ps) {
+        if (!stager) return;
         const int rb = ps % RB, kh = ps / RB;
         const int chunk = 2 * kh + (sk >> 2), step = (sk >> 1) & 1, half = sk & 1;
         const bool ok = m0 + 32 * rb + si < p.M && kb * GB_KB + 64 * kh + 8 * sk < p.K;
@@ -344,12 +348,15 @@ int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t
     // small tile, 28.2 us with 32 x 256, 33.1 us with 64 x 256; K = 1600, N = 6400: 96.5 us with the large tile,
     // 105.6 us with 32 x 256.
     const bool large = ceil_div(N, 256) * ceil_div(M, 64) >= ctx->num_cus;
-    const int BM = large ? 64 : 32, BN = large ? 256 : 128;
-    const int tiles = ceil_div(N, BN) * ceil_div(M, BM);
     // K per block: 64; 128 for the small tile on small problems (fewer barriers and loop ends per k, but 159
     // registers against 126, three waves per SIMD against four: M = 512, K = 768, N = 2304: 17.5 us against 18.7 us;
     // M = 1024: 27.3 us against 25.8 us)
-    const bool long_blocks = !large && (long long)tiles * ceil_div(K, 64) <= 5000;
+    const bool long_blocks = !large && (long long)ceil_div(N, 128) * ceil_div(M, 32) * ceil_div(K, 64) <= 5000;
+    // With a long K the split of x weighs more: eight waves share one 32-row x tile over 256 columns, the first four
+    // stage it (M = 1024, K = 1600, N = 1600: 32.8 us against 38.1 us; K = 768, N = 2304: 27.3 us against 25.2 us)
+    const bool wide = !large && !long_blocks && K >= 1536;
+    const int BM = large ? 64 : 32, BN = large || wide ? 256 : 128;
+    const int tiles = ceil_div(N, BN) * ceil_div(M, BM);
     const int KB = long_blocks ? 128 : 64;
     const int kblocks = ceil_div(K, KB);
     // K slices: the one with the least estimated time, in units of 64 k of one workgroup.  A workgroup costs
@@ -376,8 +383,9 @@ int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t
     p.partial = reinterpret_cast<float *>(ctx->workspace);
     p.counters = ctx->counters;
     const dim3 grid(ceil_div(N, BN), ceil_div(M, BM), ksplit);
-    if (large) hipLaunchKernelGGL((int4_gemm_bf16_kernel<2, 2, 2>), grid, dim3(64 * GB_WAVES), 0, ctx->stream, p);
-    else if (long_blocks) hipLaunchKernelGGL((int4_gemm_bf16_kernel<1, 1, 4>), grid, dim3(64 * GB_WAVES), 0, ctx->stream, p);
-    else hipLaunchKernelGGL((int4_gemm_bf16_kernel<1, 1, 2>), grid, dim3(64 * GB_WAVES), 0, ctx->stream, p);
+    if (large) hipLaunchKernelGGL((int4_gemm_bf16_kernel<2, 2, 2, 4>), grid, dim3(256), 0, ctx->stream, p);
+    else if (wide) hipLaunchKernelGGL((int4_gemm_bf16_kernel<1, 1, 2, 8>), grid, dim3(512), 0, ctx->stream, p);
+    else if (long_blocks) hipLaunchKernelGGL((int4_gemm_bf16_kernel<1, 1, 4, 4>), grid, dim3(256), 0, ctx->stream, p);
+    else hipLaunchKernelGGL((int4_gemm_bf16_kernel<1, 1, 2, 4>), grid, dim3(256), 0, ctx->stream, p);
     return AGPU_LAUNCH_CHECK(ctx, "int4_gemm_bf16_kernel");
 }
