@@ -18,6 +18,11 @@ struct AttnParams {
     int speculate;
     // Prefill kernel: a workgroup takes query block nb-1-x and then block x (set by the launcher).
     int pair_blocks;
+    // Decode kernel with the keys split over gridDim.z workgroups (set by the launcher): keys per workgroup, where
+    // the partial results go, and the tickets (one per query row and head, left at zero).
+    int kv_chunk;
+    float *kv_partial;
+    unsigned int *counters;
 };
 
 // max_kv_len bounds kv_len for launches that read it from pos_dev (sizes the key split).

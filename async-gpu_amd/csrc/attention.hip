@@ -278,7 +278,11 @@ __device__ __forceinline__ void merge_partial(float &m, float &l, float4 &o, flo
 // loaded for every slot below kv_stride before the context length (possibly a device-side counter) is
 // known, and masked afterwards; dot products reduce with DPP; the 4W lane-group partials are brought to
 // the common maximum first (one exp each) and then just added, in a fixed order.
+// With gridDim.z > 1 (long contexts, few workgroups) workgroup z takes the keys [z * kv_chunk, (z + 1) * kv_chunk):
+// more CUs pull the cache in.  Each writes (o, m, l) past the L2 and takes a ticket; the last one of a row adds the
+// partial results in the order of z.
 constexpr int PASS = 8;
+constexpr int kMaxKeySplits = 8;
 
 __global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
     __shared__ float sm[64], sl[64];
@@ -294,7 +298,8 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
     const float *qrow = p.q + (size_t)b * p.q_batch_stride + (size_t)h * p.q_head_stride + (size_t)qi * p.q_row_stride;
     float4 q4 = *reinterpret_cast<const float4 *>(qrow + 4 * sub);
     const int stride = 4 * W;  // keys between two consecutive keys of one lane group
-    const int first = wave * 4 + gq;
+    const int Z = gridDim.z, lo = (int)blockIdx.z * p.kv_chunk;  // kv_chunk = 0 without a split
+    const int first = lo + wave * 4 + gq;
     float4 k4[PASS], v4[PASS];
     auto fetch = [&](int base, int limit) {  // rows below kv_stride exist whatever the context length is; others read row 0
 #pragma unroll
@@ -308,7 +313,8 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
     if (p.speculate) fetch(first, p.kv_stride);
     int kv_len, q_offset;
     resolve_positions(p, kv_len, q_offset);
-    const int vis = p.causal ? min(kv_len, q_offset + qi + 1) : kv_len;  // keys [0, vis)
+    const int vis_all = p.causal ? min(kv_len, q_offset + qi + 1) : kv_len;  // keys [0, vis_all)
+    const int vis = Z > 1 ? min(vis_all, lo + p.kv_chunk) : vis_all;          // this workgroup's keys: [lo, vis)
     if (!p.speculate && first < vis) fetch(first, vis);
     q4.x *= 0.125f; q4.y *= 0.125f; q4.z *= 0.125f; q4.w *= 0.125f;
 
@@ -344,8 +350,8 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
     if (sub == 0) sm[g] = m;
     if (tid >= 4 * W && tid < 64) sm[tid] = -INFINITY;
     __syncthreads();
-    const float m_all = wave_max(sm[lane]);  // finite: key 0 is visible
-    const float fac = expf(m - m_all);       // 0 for an empty partial
+    const float m_all = wave_max(sm[lane]);  // finite when the workgroup has a key (without a split: key 0)
+    const float fac = m_all == -INFINITY ? 0.0f : expf(m - m_all);  // 0 for an empty partial
     if (sub == 0) sl[g] = l * fac;
     if (tid >= 4 * W && tid < 64) sl[tid] = 0.0f;
     *reinterpret_cast<float4 *>(&so[g][4 * sub]) = make_float4(o.x * fac, o.y * fac, o.z * fac, o.w * fac);
@@ -358,7 +364,47 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
         float acc = 0.0f;
         for (int w = 0; w < W; ++w) acc += so2[w][lane];
         float *orow = p.o + (size_t)b * p.o_batch_stride + (size_t)h * p.o_head_stride + (size_t)qi * p.o_row_stride;
-        orow[lane] = acc / l_all;
+        if (Z == 1) {
+            orow[lane] = acc / l_all;
+            return;
+        }
+        const int row = qi * gridDim.y + hb;
+        float *part = p.kv_partial + (size_t)row * kMaxKeySplits * 66;
+        __hip_atomic_store(part + blockIdx.z * 66 + lane, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) {
+            __hip_atomic_store(part + blockIdx.z * 66 + 64, m_all, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(part + blockIdx.z * 66 + 65, l_all, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        unsigned int tk = 0;
+        if (lane == 0) {
+            tk = __hip_atomic_fetch_add(&p.counters[row], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (tk == (unsigned int)(Z - 1)) __hip_atomic_store(&p.counters[row], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        tk = __builtin_amdgcn_readfirstlane(tk);
+        if (tk != (unsigned int)(Z - 1)) return;
+        float mz[kMaxKeySplits], lz[kMaxKeySplits], oz[kMaxKeySplits];
+#pragma unroll
+        for (int zz = 0; zz < kMaxKeySplits; ++zz) {
+            mz[zz] = -INFINITY;
+            lz[zz] = oz[zz] = 0.0f;
+            if (zz < Z) {
+                oz[zz] = __hip_atomic_load(part + zz * 66 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                mz[zz] = __hip_atomic_load(part + zz * 66 + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                lz[zz] = __hip_atomic_load(part + zz * 66 + 65, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        float mm = -INFINITY;
+#pragma unroll
+        for (int zz = 0; zz < kMaxKeySplits; ++zz) mm = fmaxf(mm, mz[zz]);
+        float lsum = 0.0f, osum = 0.0f;
+#pragma unroll
+        for (int zz = 0; zz < kMaxKeySplits; ++zz) {
+            const float f = mz[zz] == -INFINITY ? 0.0f : expf(mz[zz] - mm);
+            lsum += lz[zz] * f;
+            osum += oz[zz] * f;
+        }
+        orow[lane] = osum / lsum;
     }
 }
 
@@ -378,7 +424,19 @@ int32_t agpu_attention_launch(agpu_ctx *ctx, const AttnParams &p, int max_kv_len
         if (max_kv_len <= 512 && W > 8) W = 8;
         AttnParams pd = p;
         pd.speculate = p.q_len * hb <= 64 ? 1 : 0;  // latency matters for a few workgroups, bandwidth for many
-        hipLaunchKernelGGL(attn_decode_kernel, dim3(p.q_len, hb), dim3(64 * W), 0, ctx->stream, pd);
+        // Beyond 512 keys a few workgroups cannot pull the cache in fast enough: 256 keys per workgroup, eight waves
+        // (12 heads, 1024 keys: 6.3 us against 8.0 us with one workgroup of sixteen waves per head; 128 keys each: 6.4 us)
+        int Z = 1;
+        if (p.q_len * hb <= 64 && max_kv_len > 512 && p.q_len * hb <= kNumCounters) {
+            Z = ceil_div(max_kv_len, 256);
+            if (Z > kMaxKeySplits) Z = kMaxKeySplits;
+            pd.kv_chunk = ceil_div(max_kv_len, Z);
+            pd.kv_partial = reinterpret_cast<float *>(ctx->workspace);
+            pd.counters = ctx->counters;
+            W = ceil_div(pd.kv_chunk, 32);
+            W = W > 16 ? 16 : W;
+        }
+        hipLaunchKernelGGL(attn_decode_kernel, dim3(p.q_len, hb, Z), dim3(64 * W), 0, ctx->stream, pd);
         return AGPU_LAUNCH_CHECK(ctx, "attn_decode_kernel");
     }
     // Under the causal mask query block i walks through i + 1 key tiles.  When there are more workgroups than CUs, the

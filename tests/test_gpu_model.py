@@ -68,6 +68,30 @@ def test_tiny_chunked_cached_forward(tiny):
     assert np.abs(d[0] - full[29]).max() <= 1e-5
 
 
+def test_long_context_decode(orc, agpu, dev):
+    """Decode steps at a context beyond 512 positions: the attention splits the keys over several workgroups per
+    head there and merges their partial results; logits must still match the oracle, step by step."""
+    from async_gpu_amd import gpt2, workloads
+    cfg = dict(workloads.GPT2_TINY, n_positions=1024, n_layer=2)
+    w, qz = _quantized(orc, cfg, 21, nonzero_bias=True, random_ln=True)
+    om = build_oracle_model(cfg, qz)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg), qz)
+    tokens = workloads.random_prompt(cfg, 4, 800)
+    om.reset_cache()
+    gm.reset_cache()
+    ref = om.forward(tokens[:790], all_rows=False)
+    got = gm.forward_cached(tokens[:790].reshape(1, -1), all_rows=False)[0]
+    assert np.abs(got - ref).max() <= TOL_LOGITS
+    for i in range(790, 796):  # context 791 .. 796: bucket of 1024 keys, four key ranges of 256
+        ref = om.forward(tokens[i:i + 1], all_rows=False)
+        got = gm.forward_cached(tokens[i:i + 1].reshape(1, -1), all_rows=False)[0]
+        assert np.abs(got - ref).max() <= TOL_LOGITS
+    ref_out, margins = om.generate(tokens[:600], 8, cached=True, eos=-1)
+    (out,), _ = gm.generate_cached(tokens[:600], 8, eos=-1)  # the replayed decode graph at a long context
+    _assert_tokens_match(out, ref_out, margins, 600, "generate_cached at context 600")
+    gm.close()
+
+
 def test_tiny_generate_matches_oracle(tiny):
     from async_gpu_amd import workloads
     cfg, w, qz, om, gm = tiny
