@@ -8,8 +8,9 @@
 // One scale group (or a 32-k part of one) is summed by itself, u = sum over its k, and then acc += scale * u in
 // fp32, which is the reference's w = q * scale, y += x * w up to the order of the roundings.
 //
-// Workgroup = 4 waves = 32 RB rows x 128 CB columns; wave w owns 32 CB columns as RB x CB tiles of 32 x 32
-// (RB = CB = 1, or 2 for large problems).  K runs in blocks of 64 or 128 (NCH 32-k chunks).  The x pieces of a block are
+// Workgroup = 4 or 8 waves = 32 RB rows x (32 CB columns per wave); a wave owns RB x CB tiles of 32 x 32.  Built as
+// 32 x 128 (4 waves, RB = CB = 1), 32 x 256 (8 waves), 64 x 256 (4 waves, RB = CB = 2); the launcher picks by problem
+// size.  K runs in blocks of 64 or 128 (NCH 32-k chunks).  The x pieces of a block are
 // staged through LDS, double buffered, in exactly the order the A operand wants them: thread t splits the 8 floats
 // k = 8 * (t % 8) .. + 7 of row t / 8 (and of row t / 8 + 32 when RB = 2) and writes one 16-byte fragment per
 // piece, so an MFMA's A operand is one conflict-free 1 KiB read.  B words and scales come straight from global
