@@ -284,6 +284,7 @@ __device__ __forceinline__ void merge_partial(float &m, float &l, float4 &o, flo
 constexpr int PASS = 8;
 constexpr int kMaxKeySplits = 8;
 
+template <bool SPLIT>  // keys split over gridDim.z workgroups
 __global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
     __shared__ float sm[64], sl[64];
     __shared__ __align__(16) float so[64][DH];  // one row per lane group
@@ -298,7 +299,7 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
     const float *qrow = p.q + (size_t)b * p.q_batch_stride + (size_t)h * p.q_head_stride + (size_t)qi * p.q_row_stride;
     float4 q4 = *reinterpret_cast<const float4 *>(qrow + 4 * sub);
     const int stride = 4 * W;  // keys between two consecutive keys of one lane group
-    const int Z = gridDim.z, lo = (int)blockIdx.z * p.kv_chunk;  // kv_chunk = 0 without a split
+    const int Z = SPLIT ? (int)gridDim.z : 1, lo = SPLIT ? (int)blockIdx.z * p.kv_chunk : 0;
     const int first = lo + wave * 4 + gq;
     float4 k4[PASS], v4[PASS];
     auto fetch = [&](int base, int limit) {  // rows below kv_stride exist whatever the context length is; others read row 0
@@ -314,7 +315,7 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
     int kv_len, q_offset;
     resolve_positions(p, kv_len, q_offset);
     const int vis_all = p.causal ? min(kv_len, q_offset + qi + 1) : kv_len;  // keys [0, vis_all)
-    const int vis = Z > 1 ? min(vis_all, lo + p.kv_chunk) : vis_all;          // this workgroup's keys: [lo, vis)
+    const int vis = SPLIT ? min(vis_all, lo + p.kv_chunk) : vis_all;          // this workgroup's keys: [lo, vis)
     if (!p.speculate && first < vis) fetch(first, vis);
     q4.x *= 0.125f; q4.y *= 0.125f; q4.z *= 0.125f; q4.w *= 0.125f;
 
@@ -351,7 +352,7 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
     if (tid >= 4 * W && tid < 64) sm[tid] = -INFINITY;
     __syncthreads();
     const float m_all = wave_max(sm[lane]);  // finite when the workgroup has a key (without a split: key 0)
-    const float fac = m_all == -INFINITY ? 0.0f : expf(m - m_all);  // 0 for an empty partial
+    const float fac = SPLIT && m_all == -INFINITY ? 0.0f : expf(m - m_all);  // 0 for an empty partial
     if (sub == 0) sl[g] = l * fac;
     if (tid >= 4 * W && tid < 64) sl[tid] = 0.0f;
     *reinterpret_cast<float4 *>(&so[g][4 * sub]) = make_float4(o.x * fac, o.y * fac, o.z * fac, o.w * fac);
@@ -364,7 +365,7 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
         float acc = 0.0f;
         for (int w = 0; w < W; ++w) acc += so2[w][lane];
         float *orow = p.o + (size_t)b * p.o_batch_stride + (size_t)h * p.o_head_stride + (size_t)qi * p.o_row_stride;
-        if (Z == 1) {
+        if constexpr (!SPLIT) {
             orow[lane] = acc / l_all;
             return;
         }
@@ -436,7 +437,8 @@ int32_t agpu_attention_launch(agpu_ctx *ctx, const AttnParams &p, int max_kv_len
             W = ceil_div(pd.kv_chunk, 32);
             W = W > 16 ? 16 : W;
         }
-        hipLaunchKernelGGL(attn_decode_kernel, dim3(p.q_len, hb, Z), dim3(64 * W), 0, ctx->stream, pd);
+        if (Z > 1) hipLaunchKernelGGL(attn_decode_kernel<true>, dim3(p.q_len, hb, Z), dim3(64 * W), 0, ctx->stream, pd);
+        else hipLaunchKernelGGL(attn_decode_kernel<false>, dim3(p.q_len, hb), dim3(64 * W), 0, ctx->stream, pd);
         return AGPU_LAUNCH_CHECK(ctx, "attn_decode_kernel");
     }
     // Under the causal mask query block i walks through i + 1 key tiles.  When there are more workgroups than CUs, the
