@@ -8,7 +8,7 @@ _SO = os.path.join(_HERE, "libagpu_hip.so")
 
 # error codes of include/agpu.h
 ERR_SHAPE_MISMATCH, ERR_DIM_OUT_OF_RANGE, ERR_KERNEL_NOT_FOUND = -1, -2, -3
-ERR_NULL_POINTER, ERR_UNSUPPORTED, ERR_WORKSPACE = -4, -5, -6
+ERR_NULL_POINTER, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_DEVICE_WAIT, ERR_BUSY = -4, -5, -6, -7, -8
 
 EPI_NONE, EPI_GELU_TANH, EPI_GELU_QUICK, EPI_FORCE_LITERAL, EPI_FORCE_FP32_GEMV = 0, 1, 2, 0x100, 0x200
 QUANT_RUST, QUANT_SCRIPT = 0, 1
@@ -53,7 +53,11 @@ SIGNATURES = {
     "agpu_timer_stop": (_i32, [_vp, _vp]),
     "agpu_kernel_lookup": (_i32, [_vp, C.c_char_p, C.POINTER(C.c_char_p)]),
     "agpu_int4_linear": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32]),
-    "agpu_int4_gemv_tune": (None, [_i32, _i32, _i32]),
+    "agpu_int4_gemv_tune": (_i32, [_vp, _i32, _i32, _i32]),
+    "agpu_ctx_workspace_bytes": (C.c_size_t, [_vp]),
+    "agpu_int4_linear_workspace_bytes": (C.c_size_t, [_i32, _i32, _i32, _i32]),
+    "agpu_ctx_set_workspace": (_i32, [_vp, _vp, C.c_size_t]),
+    "agpu_ctx_test_hold": (_i32, [_vp, _i32]),
     "agpu_ln_int4_linear": (_i32, [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32]),
     "agpu_bench_int4_linear": (_i32, [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32,
                                       _i32, C.c_int64, C.c_int64, _i32, _vp]),

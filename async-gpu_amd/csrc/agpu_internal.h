@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <atomic>
+#include <pthread.h>
 
 #include <cstdarg>
 #include <cstdint>
@@ -12,16 +13,29 @@
 #define AGPU_EXPORT extern "C" __attribute__((visibility("default")))
 
 constexpr int kWave = 64;                                  // CDNA4 wavefront width
-constexpr size_t kWorkspaceBytes = size_t(96) << 20;       // split-K partials, attention partials
-constexpr int kNumCounters = 1 << 16;                      // arrival tickets (always left at zero)
+constexpr size_t kWorkspaceBytes = size_t(96) << 20;       // default scratch of a context: split-K / attention partials, LayerNorm rows
+constexpr size_t kMinWorkspaceBytes = size_t(1) << 20;     // smallest scratch a caller may bring
+constexpr int kNumCounters = 1 << 16;                      // arrival tickets of a context (always left at zero)
 
 struct agpu_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
     bool owns_stream = false;
     int num_cus = 256;
-    char *workspace = nullptr;      // kWorkspaceBytes of device scratch
-    unsigned int *counters = nullptr;  // kNumCounters zeroed uint32; kernels restore zero
+    // Device scratch: the first half holds split-K and attention partials, the second half LayerNorm rows and, in
+    // its last 8 KiB, the candidates of agpu_top_k_sample.  The context's own, or the caller's (agpu_ctx_set_workspace).
+    char *workspace = nullptr;
+    size_t ws_bytes = 0;
+    bool owns_workspace = false;
+    unsigned int *counters = nullptr;  // n_counters zeroed uint32; kernels restore zero.  The last one is the arg-max ticket.
+    int n_counters = 0;
+    bool owns_counters = false;
+    // launch-shape overrides of the decode GEMV (agpu_int4_gemv_tune); 0 = default
+    int tune_target_wgs = 0, tune_max_waves = 0, tune_rows_per_split = 256;
+    unsigned long long ws_epoch = 0;   // bumped whenever the scratch moves: models drop graphs captured before
+    // the one-thread-at-a-time guard: the thread inside a call, and how deep its calls are nested
+    std::atomic<uintptr_t> owner{0};
+    int depth = 0;
     hipEvent_t t0 = nullptr, t1 = nullptr;  // agpu_timer_*
     char err[512] = {0};
     std::atomic<int> refs{1};  // the handle itself + one per model created on the context
@@ -45,10 +59,34 @@ inline int32_t agpu_hip(agpu_ctx *ctx, hipError_t e, const char *what) {
     return agpu_fail(ctx, (int32_t)e, "%s: %s", what, hipGetErrorString(e));
 }
 
-#define AGPU_REQUIRE_CTX(ctx) \
-    do {                      \
-        if (!(ctx)) return AGPU_ERR_NULL_POINTER; \
-    } while (0)
+// Marks the calling thread as the one inside a call on the context; a second thread is turned away (ok == false).
+// Calls nest (entry points call each other), so the same thread may enter again.
+struct agpu_ctx_guard {
+    agpu_ctx *c;
+    bool ok;
+    explicit agpu_ctx_guard(agpu_ctx *ctx) : c(ctx), ok(false) {
+        const uintptr_t me = (uintptr_t)pthread_self();
+        if (c->owner.load(std::memory_order_relaxed) == me) {
+            ++c->depth;
+            ok = true;
+            return;
+        }
+        uintptr_t none = 0;
+        ok = c->owner.compare_exchange_strong(none, me, std::memory_order_acquire);
+        if (ok) c->depth = 1;
+    }
+    ~agpu_ctx_guard() {
+        if (ok && --c->depth == 0) c->owner.store(0, std::memory_order_release);
+    }
+    agpu_ctx_guard(const agpu_ctx_guard &) = delete;
+    agpu_ctx_guard &operator=(const agpu_ctx_guard &) = delete;
+};
+
+// First statement of every entry point that takes a context.
+#define AGPU_REQUIRE_CTX(ctx)                                      \
+    if (!(ctx)) return AGPU_ERR_NULL_POINTER;                      \
+    agpu_ctx_guard agpu_guard_(const_cast<agpu_ctx *>(ctx));       \
+    if (!agpu_guard_.ok) return AGPU_ERR_BUSY
 
 #define AGPU_REQUIRE_PTR(ctx, p)                                                         \
     do {                                                                                 \

@@ -429,7 +429,7 @@ int32_t agpu_attention_launch(agpu_ctx *ctx, const AttnParams &p, int max_kv_len
         // (12 heads, 1024 keys: 6.3 us against 8.0 us with one workgroup of sixteen waves per head; 128 keys each: 6.4 us;
         // at 512 keys two workgroups per head take 6.1 us against 5.7 us for one)
         int Z = 1;
-        if (p.q_len * hb <= 64 && max_kv_len > 512 && p.q_len * hb <= kNumCounters) {
+        if (p.q_len * hb <= 64 && max_kv_len > 512 && p.q_len * hb <= ctx->n_counters) {
             Z = ceil_div(max_kv_len, 256);
             if (Z > kMaxKeySplits) Z = kMaxKeySplits;
             pd.kv_chunk = ceil_div(max_kv_len, Z);

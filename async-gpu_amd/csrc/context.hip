@@ -1,6 +1,8 @@
 // Context, device memory and the kernel-name table of libagpu_hip.so.
+#include <chrono>
 #include <cstring>
 #include <new>
+#include <thread>
 
 #include "agpu_internal.h"
 
@@ -11,8 +13,12 @@ static int32_t ctx_init(agpu_ctx *c) {
     c->num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
     e = hipMalloc((void **)&c->workspace, kWorkspaceBytes);
     if (e != hipSuccess) return agpu_hip(c, e, "hipMalloc(workspace)");
+    c->ws_bytes = kWorkspaceBytes;
+    c->owns_workspace = true;
     e = hipMalloc((void **)&c->counters, kNumCounters * sizeof(unsigned int));
     if (e != hipSuccess) return agpu_hip(c, e, "hipMalloc(counters)");
+    c->n_counters = kNumCounters;
+    c->owns_counters = true;
     e = hipMemset(c->counters, 0, kNumCounters * sizeof(unsigned int));
     if (e != hipSuccess) return agpu_hip(c, e, "hipMemset(counters)");
     return AGPU_OK;
@@ -72,10 +78,58 @@ void agpu_ctx_release(agpu_ctx *ctx) {
     if (ctx->stream || !ctx->owns_stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->t0) (void)hipEventDestroy(ctx->t0);
     if (ctx->t1) (void)hipEventDestroy(ctx->t1);
-    if (ctx->workspace) (void)hipFree(ctx->workspace);
-    if (ctx->counters) (void)hipFree(ctx->counters);
+    if (ctx->workspace && ctx->owns_workspace) (void)hipFree(ctx->workspace);
+    if (ctx->counters && ctx->owns_counters) (void)hipFree(ctx->counters);
     if (ctx->owns_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
+}
+
+AGPU_EXPORT size_t agpu_ctx_workspace_bytes(const agpu_ctx *ctx) { return ctx ? ctx->ws_bytes : 0; }
+
+AGPU_EXPORT int32_t agpu_ctx_set_workspace(agpu_ctx *ctx, void *workspace, size_t bytes) {
+    AGPU_REQUIRE_CTX(ctx);
+    hipError_t e = hipStreamSynchronize(ctx->stream);  // nothing in flight may still use the old scratch
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipStreamSynchronize");
+    if (!workspace) {
+        // back to a scratch of the context's own
+        if (ctx->owns_workspace) return AGPU_OK;
+        char *own = nullptr;
+        e = hipMalloc((void **)&own, kWorkspaceBytes);
+        if (e != hipSuccess) return agpu_hip(ctx, e, "hipMalloc(workspace)");
+        ctx->workspace = own;
+        ctx->ws_bytes = kWorkspaceBytes;
+        ctx->owns_workspace = true;
+        ++ctx->ws_epoch;
+        return AGPU_OK;
+    }
+    if (bytes < kMinWorkspaceBytes || ((uintptr_t)workspace & 255u) != 0)
+        return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "ctx_set_workspace: need at least %zu bytes, 256-byte aligned (got %zu at %p)",
+                         kMinWorkspaceBytes, bytes, workspace);
+    if (ctx->owns_workspace && ctx->workspace) (void)hipFree(ctx->workspace);
+    ctx->workspace = static_cast<char *>(workspace);
+    ctx->ws_bytes = bytes & ~(size_t)511;  // both halves stay 256-byte aligned
+    ctx->owns_workspace = false;
+    ++ctx->ws_epoch;
+    return AGPU_OK;
+}
+
+AGPU_EXPORT int32_t agpu_ctx_test_hold(agpu_ctx *ctx, int32_t ms) {
+    AGPU_REQUIRE_CTX(ctx);
+    std::this_thread::sleep_for(std::chrono::milliseconds(ms > 0 ? ms : 0));
+    return AGPU_OK;
+}
+
+// Scratch a Linear call of this shape can use at most: the partial sums of the deepest K split any of the kernels
+// would choose (one slice per 64 k) in the first half, one LayerNorm copy of x in the second.
+AGPU_EXPORT size_t agpu_int4_linear_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t with_layer_norm) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    const size_t slices = (size_t)(K + 63) / 64;
+    const size_t rows = M <= 16 ? (size_t)M : ((size_t)M + 63) / 64 * 64, cols = ((size_t)N + 255) / 256 * 256;
+    size_t partial = slices * rows * cols * sizeof(float);
+    const size_t ln = with_layer_norm ? (size_t)M * K * sizeof(float) : 0;
+    size_t half = partial > ln ? partial : ln;
+    if (half < kMinWorkspaceBytes / 2) half = kMinWorkspaceBytes / 2;
+    return 2 * ((half + 255) & ~(size_t)255);
 }
 
 AGPU_EXPORT const char *agpu_last_error_string(const agpu_ctx *ctx) { return ctx ? ctx->err : "null context"; }

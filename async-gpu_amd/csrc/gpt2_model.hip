@@ -61,6 +61,7 @@ struct agpu_gpt2 {
     int out_capacity = 0;  // steps recorded in out_tok
     int *pos_dev = nullptr, *step_dev = nullptr;
     std::map<long long, hipGraphExec_t> graphs;  // key: batch << 32 | kv bucket
+    unsigned long long ws_epoch = 0;             // the context's scratch the graphs were captured with
     hipEvent_t ev0 = nullptr, ev1 = nullptr, ev2 = nullptr;
     // early exit: per block one (confidence, arg-max) pair in host-visible memory and one event
     float *probe_conf_host = nullptr, *probe_conf_dev = nullptr;
@@ -75,12 +76,15 @@ constexpr int DH = 64;
 __global__ __launch_bounds__(256) void embed_rows_kernel(const uint32_t *__restrict__ tokens,
                                                           const float *__restrict__ wte,
                                                           const float *__restrict__ wpe, float *out, int rows,
-                                                          int new_len, int d, const int *pos_dev) {
+                                                          int new_len, int d, const int *pos_dev, int vocab, int n_positions) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= (size_t)rows * d) return;
     const int r = (int)(i / d), j = (int)(i % d);
-    const int pos = *pos_dev + (r % new_len);
-    out[i] = wte[(size_t)tokens[r] * d + j] + wpe[(size_t)pos * d + j];
+    // ids and positions are checked on the host wherever the host knows them; a bad one on the device reads the
+    // last row instead of faulting
+    const int pos = min(*pos_dev + (r % new_len), n_positions - 1);
+    const uint32_t tok = min(tokens[r], (uint32_t)(vocab - 1));
+    out[i] = wte[(size_t)tok * d + j] + wpe[(size_t)pos * d + j];
 }
 
 // K and V columns of qkv [rows, 3d] -> cache[(b*H + h), pos + s, :]
@@ -260,10 +264,36 @@ int32_t check_layer(agpu_gpt2 *m, int layer, int which, int K, int N) {
     return AGPU_OK;
 }
 
+// Token ids the host can see are checked before anything is launched.
+int32_t check_token_ids(agpu_gpt2 *m, const uint32_t *ids_host, size_t n, const char *who) {
+    for (size_t i = 0; i < n; ++i)
+        if (ids_host[i] >= (uint32_t)m->V)
+            return agpu_fail(m->ctx, AGPU_ERR_DIM_OUT_OF_RANGE, "%s: token id %u at index %zu is outside the vocabulary of %d", who,
+                             ids_host[i], i, m->V);
+    return AGPU_OK;
+}
+
+// LayerNorm + Linear.  Rows the decode kernels do not normalise themselves are normalised into the model's own
+// buffer first (sized with the other activations), so no prefill shape depends on the context's scratch.
+int32_t ln_linear(agpu_gpt2 *m, const float *x, const float *gamma, const float *beta, const Int4Lin &w, const float *residual,
+                  float *y, int R, int N, uint32_t flags, const KvScatter *kv = nullptr, bool *kv_done = nullptr) {
+    agpu_ctx *ctx = m->ctx;
+    const float eps = m->cfg.layer_norm_epsilon;
+    const int g = m->cfg.group_size;
+    if (!agpu_int4_gemv_can_fuse_ln(R, w.K)) {
+        float *lnb = (float *)m->lnb.p;
+        int32_t rc = agpu_layer_norm_impl(ctx, x, gamma, beta, lnb, R, w.K, eps);
+        if (rc != AGPU_OK) return rc;
+        return agpu_ln_int4_linear_kv(ctx, lnb, nullptr, nullptr, eps, w.packed, w.scales, w.bias, residual, y, R, N, w.K, g, flags, kv,
+                                      kv_done);
+    }
+    return agpu_ln_int4_linear_kv(ctx, x, gamma, beta, eps, w.packed, w.scales, w.bias, residual, y, R, N, w.K, g, flags, kv, kv_done);
+}
+
 int32_t launch_embed(agpu_gpt2 *m, const uint32_t *tokens, int B, int new_len) {
     const int R = B * new_len, d = m->d;
     hipLaunchKernelGGL(embed_rows_kernel, dim3((unsigned)(((size_t)R * d + 255) / 256)), dim3(256), 0, m->ctx->stream, tokens,
-                       m->wte, m->wpe, (float *)m->hid.p, R, new_len, d, m->pos_dev);
+                       m->wte, m->wpe, (float *)m->hid.p, R, new_len, d, m->pos_dev, m->V, m->P);
     return AGPU_LAUNCH_CHECK(m->ctx, "embed_rows_kernel");
 }
 
@@ -302,8 +332,7 @@ int32_t launch_block(agpu_gpt2 *m, int L, int B, int new_len, int max_kv) {
         // prefill: the GEMM writes the K/V rows into the cache itself where it can
         const KvScatter kv{kc, vc, m->pos_dev, H, P, new_len};
         bool kv_done = false;
-        rc = agpu_ln_int4_linear_kv(ctx, hid, b.ln1_g, b.ln1_b, eps, wq.packed, wq.scales, wq.bias, nullptr, qkv, R, 3 * d, d, g, 0,
-                                    &kv, &kv_done);
+        rc = ln_linear(m, hid, b.ln1_g, b.ln1_b, wq, nullptr, qkv, R, 3 * d, 0, &kv, &kv_done);
         if (rc != AGPU_OK) return rc;
         if (!kv_done) {
             hipLaunchKernelGGL(kv_scatter_kernel, dim3((unsigned)(((size_t)R * d + 255) / 256)), dim3(256), 0, ctx->stream, qkv,
@@ -320,8 +349,7 @@ int32_t launch_block(agpu_gpt2 *m, int L, int B, int new_len, int max_kv) {
     if ((rc = agpu_attention_launch(ctx, ap, max_kv)) != AGPU_OK) return rc;
     rc = agpu_int4_linear(ctx, att, wp.packed, wp.scales, wp.bias, hid, hid, R, d, d, g, 0);
     if (rc != AGPU_OK) return rc;
-    rc = agpu_ln_int4_linear(ctx, hid, b.ln2_g, b.ln2_b, eps, wf.packed, wf.scales, wf.bias, nullptr, ffn, R, ff, d, g, gelu_flag);
-    if (rc != AGPU_OK) return rc;
+    if ((rc = ln_linear(m, hid, b.ln2_g, b.ln2_b, wf, nullptr, ffn, R, ff, gelu_flag)) != AGPU_OK) return rc;
     return agpu_int4_linear(ctx, ffn, wo.packed, wo.scales, wo.bias, hid, hid, R, d, ff, g, 0);
 }
 
@@ -345,8 +373,7 @@ int32_t launch_head(agpu_gpt2 *m, const float *head_in, int rows, const ArgmaxAd
                 return agpu_int4_gemv_launch(ctx, ga);
             }
         }
-        return agpu_ln_int4_linear(ctx, head_in, m->lnf_g, m->lnf_b, eps, m->lm_head.packed, m->lm_head.scales, nullptr, nullptr,
-                                   logits, rows, m->Vpad, d, g, 0);
+        return ln_linear(m, head_in, m->lnf_g, m->lnf_b, m->lm_head, nullptr, logits, rows, m->Vpad, 0);
     }
     int32_t rc = agpu_layer_norm(ctx, head_in, m->lnf_g, m->lnf_b, (float *)m->lnb.p, rows, d, eps);
     if (rc == AGPU_OK) rc = agpu_gemm_f32(ctx, (float *)m->lnb.p, m->wte_t, logits, rows, m->V, d);
@@ -385,7 +412,7 @@ int32_t ensure_buffers(agpu_gpt2 *m, int B, int new_len, bool all_rows_logits) {
     if ((rc = ensure(m, m->qkv, R * 3 * d * 4)) != AGPU_OK) return rc;
     if ((rc = ensure(m, m->att, R * d * 4)) != AGPU_OK) return rc;
     if ((rc = ensure(m, m->ffn, R * m->ff * 4)) != AGPU_OK) return rc;
-    if ((rc = ensure(m, m->lnb, Rl * d * 4)) != AGPU_OK) return rc;
+    if ((rc = ensure(m, m->lnb, (R > Rl ? R : Rl) * d * 4)) != AGPU_OK) return rc;
     if ((rc = ensure(m, m->last, (size_t)B * d * 4)) != AGPU_OK) return rc;
     if ((rc = ensure(m, m->logits, Rl * logits_stride(m) * 4)) != AGPU_OK) return rc;
     return AGPU_OK;
@@ -435,6 +462,10 @@ int kv_bucket(const agpu_gpt2 *m, int kv_len) {
 // The captured decode step for (batch, kv bucket); captured on first use.
 int32_t decode_graph(agpu_gpt2 *m, int B, int bucket, hipGraphExec_t *out) {
     const long long key = ((long long)B << 32) | (unsigned)bucket;
+    if (m->ws_epoch != m->ctx->ws_epoch) {  // the scratch moved: captured launches point at the old one
+        drop_graphs(m);
+        m->ws_epoch = m->ctx->ws_epoch;
+    }
     auto it = m->graphs.find(key);
     if (it != m->graphs.end()) {
         *out = it->second;
@@ -657,6 +688,7 @@ AGPU_EXPORT int32_t agpu_gpt2_set_embeddings(agpu_gpt2 *m, const float *wte, con
                                              const float *lnf_b, int32_t on_device) {
     if (!m) return AGPU_ERR_NULL_POINTER;
     agpu_ctx *ctx = m->ctx;
+    AGPU_REQUIRE_CTX(ctx);
     int32_t rc = set_vec(ctx, &m->wte, wte, (size_t)m->V * m->d, on_device);
     if (rc == AGPU_OK) rc = set_vec(ctx, &m->wpe, wpe, (size_t)m->P * m->d, on_device);
     if (rc == AGPU_OK) rc = set_vec(ctx, &m->lnf_g, lnf_g, m->d, on_device);
@@ -711,6 +743,7 @@ AGPU_EXPORT int32_t agpu_gpt2_quantize_linear(agpu_gpt2 *m, int32_t layer, int32
     if (rc != AGPU_OK) return rc;
     if (!weight_t) return agpu_fail(m->ctx, AGPU_ERR_NULL_POINTER, "gpt2_quantize_linear: null pointer");
     agpu_ctx *ctx = m->ctx;
+    AGPU_REQUIRE_CTX(ctx);
     const int g = m->cfg.group_size, ng = ceil_div(K, g);
     float *w_dev = nullptr;
     uint32_t *p_dev = nullptr;
@@ -761,6 +794,7 @@ AGPU_EXPORT int32_t agpu_gpt2_forward_cached(agpu_gpt2 *m, const uint32_t *token
                                              float *logits, int32_t all_rows) {
     if (!m) return AGPU_ERR_NULL_POINTER;
     agpu_ctx *ctx = m->ctx;
+    AGPU_REQUIRE_CTX(ctx);
     if (!tokens) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "gpt2_forward_cached: null tokens");
     if (batch <= 0 || batch > m->cfg.max_batch)
         return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_forward_cached: batch %d not in 1..%d", batch, m->cfg.max_batch);
@@ -793,6 +827,7 @@ AGPU_EXPORT int32_t agpu_gpt2_forward_cached(agpu_gpt2 *m, const uint32_t *token
 AGPU_EXPORT int32_t agpu_gpt2_decode_steps(agpu_gpt2 *m, int32_t batch, int32_t steps, float *ms_total_out_host) {
     if (!m) return AGPU_ERR_NULL_POINTER;
     agpu_ctx *ctx = m->ctx;
+    AGPU_REQUIRE_CTX(ctx);
     if (batch <= 0 || batch > m->cfg.max_batch || steps < 0)
         return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_decode_steps: bad batch/steps");
     if (m->cache_len == 0) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "gpt2_decode_steps: run a prefill first");
@@ -818,6 +853,7 @@ AGPU_EXPORT int32_t agpu_gpt2_generate_cached(agpu_gpt2 *m, const uint32_t *prom
                                               int32_t *lengths_out_host, float *timing_ms_out_host) {
     if (!m) return AGPU_ERR_NULL_POINTER;
     agpu_ctx *ctx = m->ctx;
+    AGPU_REQUIRE_CTX(ctx);
     if (!prompt_host || !tokens_out_host || !lengths_out_host)
         return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "gpt2_generate_cached: null pointer");
     if (batch <= 0 || batch > m->cfg.max_batch || prompt_len <= 0 || max_new_tokens < 0)
@@ -826,14 +862,15 @@ AGPU_EXPORT int32_t agpu_gpt2_generate_cached(agpu_gpt2 *m, const uint32_t *prom
     if (prompt_len + (max_new_tokens > 0 ? max_new_tokens - 1 : 0) > m->P)
         return agpu_fail(ctx, AGPU_ERR_DIM_OUT_OF_RANGE, "gpt2_generate_cached: prompt %d + %d new tokens exceed n_positions %d",
                          prompt_len, max_new_tokens, m->P);
+    int32_t rc = check_token_ids(m, prompt_host, (size_t)batch * prompt_len, "gpt2_generate_cached");
+    if (rc != AGPU_OK) return rc;
     const int total = prompt_len + max_new_tokens;
     for (int b = 0; b < batch; ++b) {
         std::memcpy(tokens_out_host + (size_t)b * total, prompt_host + (size_t)b * prompt_len, (size_t)prompt_len * 4);
         lengths_out_host[b] = prompt_len;
     }
     if (max_new_tokens == 0) return AGPU_OK;
-    int32_t rc = check_ready(m);
-    if (rc != AGPU_OK) return rc;
+    if ((rc = check_ready(m)) != AGPU_OK) return rc;
     if ((rc = ensure(m, m->tok_in, (size_t)batch * prompt_len * 4)) != AGPU_OK) return rc;
     if ((rc = ensure_buffers(m, batch, prompt_len, false)) != AGPU_OK) return rc;
     if ((rc = ensure_out_tokens(m, max_new_tokens, batch)) != AGPU_OK) return rc;
@@ -877,6 +914,7 @@ AGPU_EXPORT int32_t agpu_gpt2_generate_cached_sampling(agpu_gpt2 *m, const uint3
                                                        int32_t *length_out_host) {
     if (!m) return AGPU_ERR_NULL_POINTER;
     agpu_ctx *ctx = m->ctx;
+    AGPU_REQUIRE_CTX(ctx);
     if (!prompt_host || !tokens_out_host || !length_out_host || !rng_state)
         return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "gpt2_generate_cached_sampling: null pointer");
     if (prompt_len <= 0 || max_new_tokens < 0 || top_k <= 0)
@@ -885,12 +923,13 @@ AGPU_EXPORT int32_t agpu_gpt2_generate_cached_sampling(agpu_gpt2 *m, const uint3
         return agpu_fail(ctx, AGPU_ERR_DIM_OUT_OF_RANGE,
                          "gpt2_generate_cached_sampling: prompt %d + %d new tokens exceed n_positions %d", prompt_len,
                          max_new_tokens, m->P);
+    int32_t rc = check_token_ids(m, prompt_host, (size_t)prompt_len, "gpt2_generate_cached_sampling");
+    if (rc != AGPU_OK) return rc;
     std::memcpy(tokens_out_host, prompt_host, (size_t)prompt_len * 4);
     int len = prompt_len;
     *length_out_host = len;
     if (max_new_tokens == 0) return AGPU_OK;
-    int32_t rc = check_ready(m);
-    if (rc != AGPU_OK) return rc;
+    if ((rc = check_ready(m)) != AGPU_OK) return rc;
     const int k = top_k < m->V ? top_k : m->V;
     if (k > 1024) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "gpt2_generate_cached_sampling: top_k = %d exceeds 1024", top_k);
     uint32_t *idx_dev = nullptr;
@@ -931,6 +970,7 @@ AGPU_EXPORT int32_t agpu_gpt2_forward_early_exit(agpu_gpt2 *m, const uint32_t *t
                                                  float *logits_out, int32_t *layers_used_out_host) {
     if (!m) return AGPU_ERR_NULL_POINTER;
     agpu_ctx *ctx = m->ctx;
+    AGPU_REQUIRE_CTX(ctx);
     if (!tokens || !layers_used_out_host) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "gpt2_forward_early_exit: null pointer");
     if (seq_len <= 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_forward_early_exit: seq_len must be positive");
     if (seq_len > m->P)
@@ -975,6 +1015,7 @@ AGPU_EXPORT int32_t agpu_gpt2_generate_cached_early_exit(agpu_gpt2 *m, const uin
                                                          int32_t *layers_out_host, int32_t *steps_out_host) {
     if (!m) return AGPU_ERR_NULL_POINTER;
     agpu_ctx *ctx = m->ctx;
+    AGPU_REQUIRE_CTX(ctx);
     if (!prompt_host || !tokens_out_host || !length_out_host || !layers_out_host || !steps_out_host)
         return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "gpt2_generate_cached_early_exit: null pointer");
     if (prompt_len <= 0 || max_new_tokens < 0)
@@ -983,11 +1024,13 @@ AGPU_EXPORT int32_t agpu_gpt2_generate_cached_early_exit(agpu_gpt2 *m, const uin
         return agpu_fail(ctx, AGPU_ERR_DIM_OUT_OF_RANGE,
                          "gpt2_generate_cached_early_exit: prompt %d + %d new tokens exceed n_positions %d", prompt_len,
                          max_new_tokens, m->P);
+    int32_t rc = check_token_ids(m, prompt_host, (size_t)prompt_len, "gpt2_generate_cached_early_exit");
+    if (rc != AGPU_OK) return rc;
     std::memcpy(tokens_out_host, prompt_host, (size_t)prompt_len * 4);
     int len = prompt_len, steps = 0;
     *length_out_host = len;
     *steps_out_host = 0;
-    int32_t rc = check_ready(m);
+    rc = check_ready(m);
     if (rc == AGPU_OK) rc = ensure_probes(m);
     if (rc == AGPU_OK) rc = ensure(m, m->tok_in, (size_t)prompt_len * 4);
     if (rc == AGPU_OK) rc = ensure_buffers(m, 1, prompt_len, false);
@@ -1019,14 +1062,16 @@ AGPU_EXPORT int32_t agpu_gpt2_generate(agpu_gpt2 *m, const uint32_t *prompt_host
                                        int32_t eos, uint32_t *tokens_out_host, int32_t *length_out_host) {
     if (!m) return AGPU_ERR_NULL_POINTER;
     agpu_ctx *ctx = m->ctx;
+    AGPU_REQUIRE_CTX(ctx);
     if (!prompt_host || !tokens_out_host || !length_out_host)
         return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "gpt2_generate: null pointer");
     if (prompt_len <= 0 || max_new_tokens < 0)
         return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_generate: bad prompt_len/max_new_tokens");
+    int32_t rc = check_token_ids(m, prompt_host, (size_t)prompt_len, "gpt2_generate");
+    if (rc != AGPU_OK) return rc;
     std::memcpy(tokens_out_host, prompt_host, (size_t)prompt_len * 4);
     int len = prompt_len;
-    int32_t rc = check_ready(m);
-    if (rc != AGPU_OK) return rc;
+    if ((rc = check_ready(m)) != AGPU_OK) return rc;
     for (int step = 0; step < max_new_tokens; ++step) {
         if (len > m->P) {
             rc = agpu_fail(ctx, AGPU_ERR_DIM_OUT_OF_RANGE, "gpt2_generate: sequence length %d exceeds n_positions %d", len, m->P);

@@ -378,8 +378,8 @@ int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t
             ksplit = ks2;
         }
     }
-    if (tiles > kNumCounters) ksplit = 1;
-    while (ksplit > 1 && (size_t)ksplit * tiles * BM * BN * sizeof(float) > kWorkspaceBytes / 2) --ksplit;
+    if (tiles > ctx->n_counters) ksplit = 1;
+    while (ksplit > 1 && (size_t)ksplit * tiles * BM * BN * sizeof(float) > ctx->ws_bytes / 2) --ksplit;
     p.blocks_per_split = ceil_div(kblocks, ksplit);
     ksplit = ceil_div(kblocks, p.blocks_per_split);
     p.partial = reinterpret_cast<float *>(ctx->workspace);

@@ -367,19 +367,16 @@ int32_t launch_m(agpu_ctx *ctx, const GemvParams &p, int MT, dim3 grid, int W, s
     }
 }
 
-int g_tune_target_wgs = 0;    // 0: default
-int g_tune_max_waves = 0;         // 0: the launch bound of the instantiation
-int g_tune_rows_per_split = 256;  // packed rows a workgroup takes at most
-
 }  // namespace
 
 bool agpu_int4_gemv_can_fuse_ln(int M, int K) { return M <= 2 && (size_t)M * K * sizeof(float) <= 32 * 1024; }
 
-AGPU_EXPORT void agpu_int4_gemv_tune(int32_t max_wgs, int32_t min_rows_per_wave, int32_t max_waves) {
-    g_tune_max_waves = max_waves;
-    const int32_t target_wgs = max_wgs;
-    g_tune_target_wgs = target_wgs;
-    g_tune_rows_per_split = min_rows_per_wave > 0 ? min_rows_per_wave : 256;
+AGPU_EXPORT int32_t agpu_int4_gemv_tune(agpu_ctx *ctx, int32_t max_wgs, int32_t max_rows_per_wg, int32_t max_waves) {
+    AGPU_REQUIRE_CTX(ctx);
+    ctx->tune_max_waves = max_waves > 0 ? max_waves : 0;
+    ctx->tune_target_wgs = max_wgs > 0 ? max_wgs : 0;
+    ctx->tune_rows_per_split = max_rows_per_wg > 0 ? max_rows_per_wg : 256;
+    return AGPU_OK;
 }
 
 int32_t agpu_int4_gemv_launch(agpu_ctx *ctx, const GemvArgs &a) {
@@ -388,18 +385,18 @@ int32_t agpu_int4_gemv_launch(agpu_ctx *ctx, const GemvArgs &a) {
     if (a.ln_gamma && !agpu_int4_gemv_can_fuse_ln(a.M, a.K))
         return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "int4_gemv: fused LayerNorm needs M <= 2 and M*K <= 8192");
     if (!(a.flags & AGPU_EPI_FORCE_FP32_GEMV) && agpu_int4_gemv_i8_supported(a))
-        return agpu_int4_gemv_i8_launch(ctx, a, g_tune_rows_per_split / 8, g_tune_target_wgs);
+        return agpu_int4_gemv_i8_launch(ctx, a, ctx->tune_rows_per_split / 8, ctx->tune_target_wgs);
     const int kp_total = a.K / 8;
     const int MT = a.M <= 1 ? 1 : a.M <= 2 ? 2 : a.M <= 4 ? 4 : a.M <= 8 ? 8 : 16;
     const bool aligned16 = (a.N % 4 == 0) && (((uintptr_t)a.packed | (uintptr_t)a.scales) % 16 == 0);
     const int cpl = aligned16 ? 4 : 1;
     const int col_blocks = ceil_div(a.N, 16 * cpl);
-    if (col_blocks > kNumCounters) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_gemv: N=%d too large", a.N);
+    if (col_blocks > ctx->n_counters) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_gemv: N=%d too large", a.N);
 
     // K split over workgroups: a workgroup of 16 waves covers 64 packed rows per trip and keeps two
     // trips in flight, so up to 4 trips (256 rows) per workgroup cost two memory round trips.
-    int ksplit = ceil_div(kp_total, g_tune_rows_per_split);
-    while (ksplit > 1 && (size_t)ksplit * a.M * a.N * sizeof(float) > kWorkspaceBytes / 2) --ksplit;
+    int ksplit = ceil_div(kp_total, ctx->tune_rows_per_split);
+    while (ksplit > 1 && (size_t)ksplit * a.M * a.N * sizeof(float) > ctx->ws_bytes / 2) --ksplit;
     auto stage_floats = [&](int ks) {
         const int rps = ceil_div(kp_total, ks);
         const size_t xs_len = a.ln_gamma ? (size_t)a.K : (size_t)rps * 8;
@@ -411,12 +408,12 @@ int32_t agpu_int4_gemv_launch(agpu_ctx *ctx, const GemvArgs &a) {
     ksplit = ceil_div(kp_total, p.rows_per_split);
     if (stage_floats(ksplit) * sizeof(float) > kLdsBudget)
         return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "int4_gemv: staged x does not fit in LDS (M=%d K=%d)", a.M, a.K);
-    if ((size_t)ksplit * a.M * a.N * sizeof(float) > kWorkspaceBytes / 2)
+    if ((size_t)ksplit * a.M * a.N * sizeof(float) > ctx->ws_bytes / 2)
         return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_gemv: split-K partials exceed the workspace (M=%d N=%d K=%d)", a.M, a.N, a.K);
-    // waves: one per 4*g_tune_min_rows rows of the slice, bounded by the launch bound of the
+    // waves: one per 8 packed rows of the slice, bounded by the launch bound of the
     // instantiation and by the LDS the cross-wave reduction needs
     int max_w = MT == 1 ? 16 : 8;
-    if (g_tune_max_waves > 0 && g_tune_max_waves < max_w) max_w = g_tune_max_waves;
+    if (ctx->tune_max_waves > 0 && ctx->tune_max_waves < max_w) max_w = ctx->tune_max_waves;
     int W = ceil_div(p.rows_per_split, 8);  // two trips of 4 rows per wave
     W = W < 1 ? 1 : (W > max_w ? max_w : W);
     while (W > 1 && ((size_t)W * MT * 16 * cpl + stage_floats(ksplit)) * sizeof(float) > 64 * 1024) --W;
@@ -427,7 +424,7 @@ int32_t agpu_int4_gemv_launch(agpu_ctx *ctx, const GemvArgs &a) {
     p.col_blocks = col_blocks;
     // at most one workgroup per CU (measured best for the LM head); each strides over the column tiles
     int gx = col_blocks;
-    const int cap = g_tune_target_wgs > 0 ? g_tune_target_wgs : ctx->num_cus;
+    const int cap = ctx->tune_target_wgs > 0 ? ctx->tune_target_wgs : ctx->num_cus;
     if (gx * ksplit > cap) gx = cap / ksplit > 0 ? cap / ksplit : 1;
     const dim3 grid(gx, ksplit);
     return cpl == 4 ? launch_m<4>(ctx, p, MT, grid, W, lds) : launch_m<1>(ctx, p, MT, grid, W, lds);

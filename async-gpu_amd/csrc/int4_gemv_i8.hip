@@ -45,6 +45,7 @@ struct I8Params {
     unsigned int *counters;
     int sets_before;      // register sets requested before x is converted; the others follow the digits
     unsigned long long *am_partial;  // fused arg-max: one candidate per workgroup, written through
+    unsigned int *am_counter;        // ... and the ticket the workgroups take after it
 };
 
 // Order-preserving key of a float (NaN lowest, both zeros equal) with the column behind it: the larger 64-bit word wins.
@@ -411,9 +412,9 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
         if (tid == 0) {
             __hip_atomic_store(&p.am_partial[blockIdx.x], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            const unsigned int t = __hip_atomic_fetch_add(&p.counters[kNumCounters - 1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const unsigned int t = __hip_atomic_fetch_add(&p.am_counter[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             s_last[0] = (t == gridDim.x - 1);
-            if (s_last[0]) __hip_atomic_store(&p.counters[kNumCounters - 1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (s_last[0]) __hip_atomic_store(&p.am_counter[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         __syncthreads();
         if (s_last[0]) {
@@ -457,7 +458,7 @@ int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips
     const int MT = a.M <= 1 ? 1 : 2;
     const int trips_total = a.K / 64;
     const int col_blocks = ceil_div(a.N, 64);
-    if (col_blocks > kNumCounters) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_gemv: N=%d too large", a.N);
+    if (col_blocks > ctx->n_counters - 1) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_gemv: N=%d too large", a.N);
     int tps_max = max_trips_per_split < 1 ? 1 : (max_trips_per_split > 128 ? 128 : max_trips_per_split);
     auto stage_bytes = [&](int tps) {
         return (size_t)MT * tps * 256 + sizeof(float) * (size_t)MT * ((2 * tps + 3) & ~3);
@@ -470,7 +471,7 @@ int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips
     if (col_blocks * ksplit < ctx->num_cus / 4 && trips_total > 32) ksplit = ceil_div(trips_total, 16);
     const int tps = ceil_div(trips_total, ksplit);
     ksplit = ceil_div(trips_total, tps);
-    if ((size_t)ksplit * a.M * a.N * sizeof(float) > kWorkspaceBytes / 2)
+    if ((size_t)ksplit * a.M * a.N * sizeof(float) > ctx->ws_bytes / 2)
         return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_gemv: split-K partials exceed the workspace (M=%d N=%d K=%d)", a.M, a.N, a.K);
     int W = tps <= 16 ? tps : 16;
     if (W < ceil_div(8 * tps, 64)) W = ceil_div(8 * tps, 64);          // one thread per packed row of the slice
@@ -509,9 +510,10 @@ int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips
     p.sets_before = items_per_wave > 2 ? 1 : 2;
     const dim3 grid(gx, ksplit), block(64 * W);
     // fused arg-max: single row, unsplit K (else the separate kernel runs afterwards)
-    const bool am = a.am_idx_out != nullptr && a.M == 1 && ksplit == 1 && (size_t)gx * sizeof(unsigned long long) <= kWorkspaceBytes / 2;
+    const bool am = a.am_idx_out != nullptr && a.M == 1 && ksplit == 1 && (size_t)gx * sizeof(unsigned long long) <= ctx->ws_bytes / 2;
     if (am) {
         p.am_partial = reinterpret_cast<unsigned long long *>(ctx->workspace);
+        p.am_counter = ctx->counters + (ctx->n_counters - 1);
         if (a.ln_gamma) hipLaunchKernelGGL((int4_gemv_i8_kernel<1, true, 4, true>), grid, block, lds, ctx->stream, p);
         else hipLaunchKernelGGL((int4_gemv_i8_kernel<1, false, 4, true>), grid, block, lds, ctx->stream, p);
         return AGPU_LAUNCH_CHECK(ctx, "int4_gemv_i8_kernel");

@@ -231,9 +231,9 @@ int32_t agpu_ln_int4_linear_kv(agpu_ctx *ctx, const float *x, const float *gamma
     if (gamma && (literal || M > 16 || !agpu_int4_gemv_can_fuse_ln(M, K))) {
         // LayerNorm into the workspace tail, then the plain kernels.
         const size_t need = (size_t)M * K * sizeof(float);
-        if (need > kWorkspaceBytes / 2)
+        if (need > ctx->ws_bytes / 2)
             return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "ln_int4_linear: M*K=%zu floats exceed the workspace", (size_t)M * K);
-        float *tmp = reinterpret_cast<float *>(ctx->workspace + kWorkspaceBytes / 2);
+        float *tmp = reinterpret_cast<float *>(ctx->workspace + ctx->ws_bytes / 2);
         rc = agpu_layer_norm_impl(ctx, x, gamma, beta, tmp, M, K, eps);
         if (rc != AGPU_OK) return rc;
         xin = tmp;

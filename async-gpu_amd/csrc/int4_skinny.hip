@@ -189,10 +189,10 @@ int32_t agpu_int4_skinny_launch(agpu_ctx *ctx, const GemvArgs &a) {
     const int tps_max = 16 / tpg * tpg;     // at most 2 trips per wave, 8 waves
     const int ksplit = ceil_div(trips_total, tps_max);
     const int tps = ceil_div(ceil_div(trips_total, ksplit), tpg) * tpg;
-    if ((size_t)ksplit * a.M * a.N * sizeof(float) > kWorkspaceBytes / 2)
+    if ((size_t)ksplit * a.M * a.N * sizeof(float) > ctx->ws_bytes / 2)
         return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_skinny: split-K partials exceed the workspace (M=%d N=%d K=%d)", a.M, a.N, a.K);
     const int col_blocks = ceil_div(a.N, 64);
-    if (col_blocks > kNumCounters) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_skinny: N=%d too large", a.N);
+    if (col_blocks > ctx->n_counters) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_skinny: N=%d too large", a.N);
     p.trips_per_split = tps;
     p.xs_stride = tps * 32 + 4;
     const int W = tps < 8 ? tps : 8;

@@ -169,8 +169,8 @@ AGPU_EXPORT int32_t agpu_top_k_sample(agpu_ctx *ctx, const float *logits, int32_
     if (!logits || !rng_state || !token_out_host) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "top_k_sample: null pointer");
     if (k > n) k = n;
     if (k <= 0 || k > TK_MAX_K) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "top_k_sample: k = %d outside 1..%d", k, TK_MAX_K);
-    uint32_t *idx_dev = reinterpret_cast<uint32_t *>(ctx->workspace + kWorkspaceBytes - 2 * TK_MAX_K * 4);
-    float *val_dev = reinterpret_cast<float *>(ctx->workspace + kWorkspaceBytes - TK_MAX_K * 4);
+    uint32_t *idx_dev = reinterpret_cast<uint32_t *>(ctx->workspace + ctx->ws_bytes - 2 * TK_MAX_K * 4);
+    float *val_dev = reinterpret_cast<float *>(ctx->workspace + ctx->ws_bytes - TK_MAX_K * 4);
     int32_t rc = agpu_top_k_launch(ctx, logits, 1, n, n, k, temperature, idx_dev, val_dev);
     if (rc != AGPU_OK) return rc;
     std::vector<uint32_t> idx((size_t)k);

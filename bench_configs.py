@@ -4,7 +4,7 @@ configurations other than the headline one, which bench.py covers): isolated int
 attention prefill / decode, and GPT-2 XL-shaped decode at batch 1 and 16.  Prints one JSON line per
 case.  Kernel cases are timed as graph replays with HIP events on the context's stream.
 
-    python3 async-gpu_amd/bench_configs.py [--xl-layers 48] [--skip-xl] [--skip-kernels] [--prefill-only]
+    python3 bench_configs.py [--xl-layers 48] [--skip-xl] [--skip-kernels] [--prefill-only]
 """
 import argparse
 import ctypes as C
@@ -15,7 +15,7 @@ import time
 
 import numpy as np
 
-ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 import __graft_entry__ as entry  # noqa: E402
 

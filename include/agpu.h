@@ -18,7 +18,10 @@
  *     allocates or synchronises, so a sequence of calls may be captured in a HIP graph;
  *   - return value: 0 ok; <0 argument/shape error found on the host before any
  *     launch; >0 a hipError_t.  agpu_last_error_string() describes the last failure.
- *   - a context is used by one thread at a time; different contexts are independent.
+ *   - a context has ONE stream and is used by one thread at a time; different contexts are independent.
+ *     A call that arrives while another thread is inside a call on the same context returns
+ *     AGPU_ERR_BUSY and does nothing.  Work that must overlap goes to a second context (its own
+ *     stream, its own scratch); the scratch of one context is never shared between streams.
  */
 #ifndef AGPU_H
 #define AGPU_H
@@ -37,6 +40,7 @@ extern "C" {
 #define AGPU_ERR_NULL_POINTER (-4)
 #define AGPU_ERR_UNSUPPORTED (-5)
 #define AGPU_ERR_WORKSPACE (-6)        /* split-K scratch too small for the request */
+#define AGPU_ERR_BUSY (-8)             /* another thread is inside a call on this context */
 
 typedef struct agpu_ctx agpu_ctx;
 
@@ -52,6 +56,28 @@ int32_t agpu_ctx_create_on_stream(int32_t device, void *hip_stream, agpu_ctx **o
 int32_t agpu_ctx_destroy(agpu_ctx *ctx);
 const char *agpu_last_error_string(const agpu_ctx *ctx);
 void *agpu_ctx_stream(const agpu_ctx *ctx);
+
+/*
+ * Scratch of a context.  The reference's operators allocate what they need per call (alloc_zeros,
+ * nn/layers/int4_linear.rs:94-95); the launchers here never allocate, so partial sums of a K split over
+ * workgroups, partial attention results and LayerNorm rows of a prefill Linear live in one scratch buffer per
+ * context: 96 MiB of the context's own by default, or memory the caller brings.
+ *   agpu_ctx_workspace_bytes          size of the scratch in use
+ *   agpu_int4_linear_workspace_bytes  an upper bound of what agpu_int4_linear / agpu_ln_int4_linear can use for
+ *                                     this shape (with less the kernels split K less deeply, or the call
+ *                                     returns AGPU_ERR_WORKSPACE when even the unsplit form does not fit)
+ *   agpu_ctx_set_workspace            use `bytes` (>= 1 MiB) at `workspace` (device memory, 256-byte aligned)
+ *                                     from now on; the context's own scratch is freed.  NULL returns to a
+ *                                     scratch of the context's own.  Synchronises the stream first.  The
+ *                                     caller keeps ownership and must not touch the memory while calls on the
+ *                                     context are in flight.  Graphs captured before the change still point at
+ *                                     the old scratch: models drop theirs on their next call.
+ */
+size_t agpu_ctx_workspace_bytes(const agpu_ctx *ctx);
+size_t agpu_int4_linear_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t with_layer_norm);
+int32_t agpu_ctx_set_workspace(agpu_ctx *ctx, void *workspace, size_t bytes);
+/* Test hook of the one-thread-at-a-time guard: stays inside a call on the context for `ms` milliseconds. */
+int32_t agpu_ctx_test_hold(agpu_ctx *ctx, int32_t ms);
 
 int32_t agpu_malloc(agpu_ctx *ctx, size_t bytes, void **out);              /* alloc_zeros: memory is zeroed */
 int32_t agpu_free(agpu_ctx *ctx, void *ptr);
@@ -93,6 +119,16 @@ int32_t agpu_kernel_lookup(const agpu_ctx *ctx, const char *name, const char **e
  *   scales [ceil(K/group), N] f32;  w = (float)(nibble-8) * scale[k/group, n]
  * bias and residual may be NULL; residual may alias y.  K % 8 == 0 is required
  * (nn/ops/quantize.rs:109); otherwise AGPU_ERR_SHAPE_MISMATCH.
+ *
+ * Arithmetic for M <= 2 with group = 32 * 2^n, K % 64 == 0 and 16-byte aligned pointers (the decode shapes):
+ * each x row is converted to 32-bit fixed point, X = rint(x * 2^s) with s chosen from the row's max |x| so
+ * that |X| < 2^30, and the products with the nibbles are summed exactly in int32 per 32-k chunk; only the
+ * per-group scale and the additions across groups round (fp32).  Consequences a caller can observe: an element
+ * smaller than max|x| * 2^-31 of its row contributes as zero (the reference's fp32 fma chain would keep it, at a
+ * weight below the chain's own rounding error); a row whose max |x| is below 2^-97 gives the bias / residual
+ * alone; a row holding NaN or Inf gives NaN in every output of that row.  Results stay within
+ * 4e-7 * sum_k |x_k| |w_kn| of the exact dot product, tighter than the reference's fp32 chain.
+ * AGPU_EPI_FORCE_FP32_GEMV selects the plain fp32 kernels instead.
  */
 int32_t agpu_int4_linear(agpu_ctx *ctx, const float *x, const uint32_t *packed, const float *scales,
                          const float *bias, const float *residual, float *y, int32_t M, int32_t N,
@@ -102,8 +138,9 @@ int32_t agpu_int4_linear(agpu_ctx *ctx, const float *x, const uint32_t *packed, 
  * the default; each workgroup strides over the column tiles) and the most packed rows (8 k each)
  * one workgroup takes before K is split over workgroups (0 = 256, the default), and the most waves per
  * workgroup (0 = 16 for M = 1, 8 otherwise).
- * Process-wide; results stay deterministic for any setting. */
-void agpu_int4_gemv_tune(int32_t max_wgs, int32_t max_rows_per_wg, int32_t max_waves_per_wg);
+ * Per context (benchmark sweeps on one context do not change what another computes); results stay deterministic
+ * for any setting, but the summation order, and with it the last bits, follow the launch shape. */
+int32_t agpu_int4_gemv_tune(agpu_ctx *ctx, int32_t max_wgs, int32_t max_rows_per_wg, int32_t max_waves_per_wg);
 
 /* Same with LayerNorm(x; gamma, beta, eps) over K applied to each input row first
  * (ops::layer_norm followed by Int4Linear::forward, gpt2.rs:1307-1316,1329-1331). */
