@@ -98,6 +98,33 @@ def quantize_gpt2(weights, group, quantize_fn, lm_head_int4=True):
     return q
 
 
+def gpt2_quantized_layerwise(cfg, seed, group, quantize_fn, std=0.02, workers=8):
+    """The dict of quantize_gpt2 for a random-init GPT-2 (weights, wte, wpe ~ N(0, std); LN gain 1, every bias 0),
+    built one layer at a time by a pool of threads, so that a model of XL size never holds its 6 GB of fp32 weights
+    at once and does not take minutes to draw.  Layer L draws from its own generator seeded (seed, L), the embeddings
+    from (seed, n_layer): the values differ from gpt2_fp32_weights(cfg, seed)."""
+    from concurrent.futures import ThreadPoolExecutor
+    d, ff, V, P, nl = cfg["n_embd"], 4 * cfg["n_embd"], cfg["vocab"], cfg["n_positions"], cfg["n_layer"]
+
+    def layer(L):
+        rng = np.random.default_rng([seed, L])
+        e = dict(ln1_g=np.ones(d, np.float32), ln1_b=np.zeros(d, np.float32), ln2_g=np.ones(d, np.float32),
+                 ln2_b=np.zeros(d, np.float32))
+        for name, (k, n) in zip(LINEAR_NAMES, ((d, 3 * d), (d, d), (d, ff), (ff, d))):
+            w = rng.standard_normal((k, n), dtype=np.float32) * np.float32(std)
+            packed, scales = quantize_fn(w, group)
+            e[name] = (packed, scales, np.zeros(n, np.float32))
+        return e
+
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        layers = list(pool.map(layer, range(nl)))
+    rng = np.random.default_rng([seed, nl])
+    wte = rng.standard_normal((V, d), dtype=np.float32) * np.float32(std)
+    wpe = rng.standard_normal((P, d), dtype=np.float32) * np.float32(std)
+    return dict(group=group, wte=wte, wpe=wpe, lnf_g=np.ones(d, np.float32), lnf_b=np.zeros(d, np.float32), layers=layers,
+                lm_head=quantize_fn(np.ascontiguousarray(wte.T), group))
+
+
 def random_prompt(cfg, seed, length, batch=None):
     rng = np.random.default_rng(seed + 1000)
     shape = (length,) if batch is None else (batch, length)

@@ -36,6 +36,20 @@ def dev():
     return torch.device("cuda:0")
 
 
+def progress(msg):
+    """A line for long GPU tests: printed, and appended to gpurun_out/test_progress.log so that a run whose output
+    pytest captures still shows signs of life on the GPU box."""
+    import time
+    line = f"[{time.strftime('%H:%M:%S')}] {msg}"
+    print(line, flush=True)
+    try:
+        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+        with open(os.path.join(ROOT, "gpurun_out", "test_progress.log"), "a") as f:
+            f.write(line + "\n")
+    except OSError:
+        pass
+
+
 def to_dev(a, dev):
     import torch
 
