@@ -53,6 +53,7 @@ SIGNATURES = {
     "agpu_timer_stop": (_i32, [_vp, _vp]),
     "agpu_kernel_lookup": (_i32, [_vp, C.c_char_p, C.POINTER(C.c_char_p)]),
     "agpu_int4_linear": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32]),
+    "agpu_int4_linear_static": (_i32, [_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32, C.c_char_p, _i32]),
     "agpu_int4_gemv_tune": (_i32, [_vp, _i32, _i32, _i32]),
     "agpu_ctx_workspace_bytes": (C.c_size_t, [_vp]),
     "agpu_int4_linear_workspace_bytes": (C.c_size_t, [_i32, _i32, _i32, _i32]),

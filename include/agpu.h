@@ -134,6 +134,25 @@ int32_t agpu_int4_linear(agpu_ctx *ctx, const float *x, const uint32_t *packed, 
                          const float *bias, const float *residual, float *y, int32_t M, int32_t N,
                          int32_t K, int32_t group, uint32_t flags);
 
+/*
+ * agpu_int4_linear for callers that cannot allocate.  No counterpart in the reference.  It is for code under HIP
+ * graph capture, tight serving loops and harnesses that forbid hipMalloc: it needs no context (creating one allocates
+ * the 96 MiB scratch) and calls no hipMalloc, hipFree or allocating library routine.  The partial sums and tickets of
+ * a K split over workgroups live in a fixed array inside the library's device image (8 MiB + 16 KiB per GPU, held
+ * until the process ends); the kernels and results are those of agpu_int4_linear (bit-identical for M <= 16; the
+ * prefill GEMM may split K less deeply, which only reorders its additions).
+ *   device      GPU the pointers belong to; hip_stream a hipStream_t of that GPU (NULL = the default stream).
+ *   Limits      M * N * 4 bytes <= 4 MiB and N <= 262080, else AGPU_ERR_WORKSPACE; a K split that does not fit the
+ *               4 MiB is made shallower, and the call returns AGPU_ERR_WORKSPACE where the kernel cannot do that.
+ *   err_out     optional buffer of err_cap bytes for the message of a failed call.
+ * Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams, two threads) race.
+ * The first call on a GPU looks up the array's address (hipGetSymbolAddress) and the CU count; make it outside
+ * graph capture.
+ */
+int32_t agpu_int4_linear_static(int32_t device, void *hip_stream, const float *x, const uint32_t *packed, const float *scales,
+                                const float *bias, const float *residual, float *y, int32_t M, int32_t N, int32_t K,
+                                int32_t group, uint32_t flags, char *err_out, int32_t err_cap);
+
 /* Tuning hook of the decode GEMV (M <= 16): the most workgroups a launch uses (0 = one per CU,
  * the default; each workgroup strides over the column tiles) and the most packed rows (8 k each)
  * one workgroup takes before K is split over workgroups (0 = 256, the default), and the most waves per
