@@ -20,6 +20,7 @@
 #include "../../include/agpu_gpt2.h"
 #include "agpu_internal.h"
 #include "attention.h"
+#include "decode_persistent.h"
 #include "elementwise.h"
 #include "linear_common.h"
 
@@ -67,6 +68,13 @@ struct agpu_gpt2 {
     float *probe_conf_host = nullptr, *probe_conf_dev = nullptr;
     uint32_t *probe_tok_host = nullptr, *probe_tok_dev = nullptr;
     std::vector<hipEvent_t> probe_ev;
+    // one-launch decode step (single sequence): plan built on first use, dropped with the graphs
+    PkPlan pk;
+    std::vector<PkLayer> pk_layers;
+    bool pk_tried = false;
+    bool pk_failed = false;   // a wait of the one-launch step gave up once: this model keeps to the per-stage path
+    int pk_spin_limit = 0;    // test hook: poll rounds a wait may take (0 = default)
+    int decode_mode = AGPU_DECODE_AUTO;
 };
 
 namespace {
@@ -186,6 +194,9 @@ void free_lin(Int4Lin &l) {
 void drop_graphs(agpu_gpt2 *m) {
     for (auto &kv : m->graphs) (void)hipGraphExecDestroy(kv.second);
     m->graphs.clear();
+    // the plan of the one-launch step holds the same addresses
+    agpu_pk_plan_free(&m->pk);
+    m->pk_tried = false;
 }
 
 // Grow a buffer; existing graphs hold the old address, so they are dropped.
@@ -459,6 +470,48 @@ int kv_bucket(const agpu_gpt2 *m, int kv_len) {
     return b < m->P ? b : m->P;
 }
 
+// The model as the one-launch decode step sees it (sequence 0 of the cache).
+PkModel pk_view(agpu_gpt2 *m) {
+    const size_t layer_stride = (size_t)m->cfg.max_batch * m->H * m->P * DH;
+    m->pk_layers.resize((size_t)m->cfg.n_layer);
+    auto lin = [](const Int4Lin &l) { return PkLinear{l.packed, l.scales, l.bias, l.K, l.N, l.Npad}; };
+    for (int L = 0; L < m->cfg.n_layer; ++L) {
+        const Block &b = m->blocks[L];
+        PkLayer &y = m->pk_layers[L];
+        y.ln1_g = b.ln1_g; y.ln1_b = b.ln1_b; y.ln2_g = b.ln2_g; y.ln2_b = b.ln2_b;
+        y.qkv = lin(b.lin[AGPU_LINEAR_QKV]); y.proj = lin(b.lin[AGPU_LINEAR_PROJ]);
+        y.fc = lin(b.lin[AGPU_LINEAR_FC]); y.fc_proj = lin(b.lin[AGPU_LINEAR_FC_PROJ]);
+        y.kcache = m->kcache + L * layer_stride;
+        y.vcache = m->vcache + L * layer_stride;
+    }
+    PkModel v{};
+    v.d = m->d; v.H = m->H; v.ff = m->ff; v.V = m->V; v.P = m->P; v.group = m->cfg.group_size; v.n_layer = m->cfg.n_layer;
+    v.eps = m->cfg.layer_norm_epsilon;
+    v.gelu_quick = m->cfg.gelu == AGPU_GELU_QUICK;
+    v.argmax_last = m->cfg.argmax_last;
+    v.wte = m->wte; v.wpe = m->wpe; v.lnf_g = m->lnf_g; v.lnf_b = m->lnf_b;
+    v.head = lin(m->lm_head);
+    v.layers = m->pk_layers.data();
+    v.logits = (float *)m->logits.p;
+    v.cur_tok = m->cur_tok; v.out_tok = m->out_tok; v.next_tok = m->next_tok;
+    v.pos_dev = m->pos_dev; v.step_dev = m->step_dev; v.out_capacity = m->out_capacity;
+    return v;
+}
+
+// Whether single-sequence decode steps run as one launch; builds the plan on first use (never inside a capture).
+bool pk_ready(agpu_gpt2 *m) {
+    if (m->decode_mode == AGPU_DECODE_PER_STAGE || m->pk_failed || m->cfg.lm_head != AGPU_LM_HEAD_INT4) return false;
+    if (m->pk.stages_dev) return true;
+    if (m->pk_tried) return false;
+    m->pk_tried = true;
+    if (!m->logits.p || !m->out_tok) return false;
+    const PkModel v = pk_view(m);
+    if (!agpu_pk_supported(m->ctx, v)) return false;
+    if (agpu_pk_plan_build(m->ctx, v, &m->pk) != AGPU_OK) return false;
+    m->pk.spin_limit = m->pk_spin_limit;
+    return true;
+}
+
 // The captured decode step for (batch, kv bucket); captured on first use.
 int32_t decode_graph(agpu_gpt2 *m, int B, int bucket, hipGraphExec_t *out) {
     const long long key = ((long long)B << 32) | (unsigned)bucket;
@@ -474,13 +527,20 @@ int32_t decode_graph(agpu_gpt2 *m, int B, int bucket, hipGraphExec_t *out) {
     agpu_ctx *ctx = m->ctx;
     if (ctx->stream == nullptr)
         return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "gpt2: graph capture needs a context with its own stream (agpu_ctx_create)");
+    const bool one_launch = B == 1 && pk_ready(m);  // builds the plan: before the capture begins
     hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
     if (e != hipSuccess) return agpu_hip(ctx, e, "hipStreamBeginCapture");
-    // one sequence: the LM head picks and feeds the next token itself
-    const ArgmaxAdvance feed = token_feed(m, B, 1);
-    bool fed = false;
-    int32_t rc = launch_forward(m, m->cur_tok, B, 1, bucket, false, &feed, &fed);
-    if (rc == AGPU_OK && !fed) rc = launch_argmax_advance(m, B, 1);
+    int32_t rc;
+    if (one_launch) {
+        // one sequence: the whole step, arg-max and token feed included, is one launch
+        rc = agpu_pk_launch(ctx, pk_view(m), m->pk, 0);
+    } else {
+        // the LM head picks and feeds the next token itself where it can
+        const ArgmaxAdvance feed = token_feed(m, B, 1);
+        bool fed = false;
+        rc = launch_forward(m, m->cur_tok, B, 1, bucket, false, &feed, &fed);
+        if (rc == AGPU_OK && !fed) rc = launch_argmax_advance(m, B, 1);
+    }
     hipGraph_t graph = nullptr;
     e = hipStreamEndCapture(ctx->stream, &graph);
     if (rc != AGPU_OK) {
@@ -520,6 +580,26 @@ int32_t run_decode_steps(agpu_gpt2 *m, int B, int steps) {
         hipError_t e = hipGraphLaunch(exec, m->ctx->stream);
         if (e != hipSuccess) return agpu_hip(m->ctx, e, "hipGraphLaunch");
         m->cache_len += 1;
+    }
+    return AGPU_OK;
+}
+
+// After a synchronisation: whether a wait inside a one-launch decode step gave up since the last check.
+int32_t pk_check(agpu_gpt2 *m) {
+    if (!m->pk.stages_dev) return AGPU_OK;
+    unsigned int err = 0u;
+    int32_t rc = agpu_pk_take_error(m->ctx, m->pk, &err);
+    if (rc != AGPU_OK) return rc;
+    if (err != 0u) {
+        // The steps since the last check are void.  Nothing is known about why the wait gave up (the workgroups of the
+        // step must all be resident at once: another process on the device can prevent that), so this model keeps to
+        // the per-stage path from now on; the caller resets the cache and runs again.
+        m->pk_failed = true;
+        drop_graphs(m);
+        return agpu_fail(m->ctx, AGPU_ERR_DEVICE_WAIT,
+                         "gpt2: a wait of the one-launch decode step gave up (stage %u); the steps since the last check are invalid, "
+                         "decode steps run per stage from now on",
+                         err & 0xfffu);
     }
     return AGPU_OK;
 }
@@ -662,7 +742,7 @@ AGPU_EXPORT int32_t agpu_gpt2_create(agpu_ctx *ctx, const agpu_gpt2_config *cfg,
 AGPU_EXPORT int32_t agpu_gpt2_destroy(agpu_gpt2 *m) {
     if (!m) return AGPU_OK;
     if (m->ctx) (void)hipStreamSynchronize(m->ctx->stream);
-    drop_graphs(m);
+    drop_graphs(m);  // also frees the plan of the one-launch step
     for (auto &b : m->blocks) {
         for (float *p : {b.ln1_g, b.ln1_b, b.ln2_g, b.ln2_b})
             if (p) (void)hipFree(p);
@@ -782,6 +862,30 @@ AGPU_EXPORT int64_t agpu_gpt2_quantized_memory_bytes(const agpu_gpt2 *m) {
     return total;
 }
 
+AGPU_EXPORT int32_t agpu_gpt2_set_decode_mode(agpu_gpt2 *m, int32_t mode) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    if (mode != AGPU_DECODE_AUTO && mode != AGPU_DECODE_PER_STAGE)
+        return agpu_fail(m->ctx, AGPU_ERR_DIM_OUT_OF_RANGE, "gpt2_set_decode_mode: unknown mode %d", mode);
+    if (mode != m->decode_mode) {
+        (void)hipStreamSynchronize(m->ctx->stream);
+        drop_graphs(m);
+        m->decode_mode = mode;
+    }
+    return AGPU_OK;
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_decode_is_one_launch(agpu_gpt2 *m) { return m && m->pk.stages_dev ? 1 : 0; }
+
+AGPU_EXPORT int32_t agpu_gpt2_set_decode_wait_limit(agpu_gpt2 *m, int32_t poll_rounds) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    if (poll_rounds < 0) return agpu_fail(m->ctx, AGPU_ERR_DIM_OUT_OF_RANGE, "gpt2_set_decode_wait_limit: negative limit");
+    (void)hipStreamSynchronize(m->ctx->stream);
+    m->pk_spin_limit = poll_rounds;
+    m->pk.spin_limit = poll_rounds;
+    drop_graphs(m);  // captured launches carry the old limit
+    return AGPU_OK;
+}
+
 AGPU_EXPORT int32_t agpu_gpt2_reset_cache(agpu_gpt2 *m) {
     if (!m) return AGPU_ERR_NULL_POINTER;
     m->cache_len = 0;
@@ -845,7 +949,59 @@ AGPU_EXPORT int32_t agpu_gpt2_decode_steps(agpu_gpt2 *m, int32_t batch, int32_t 
     if ((rc = agpu_hip(ctx, hipEventRecord(m->ev1, ctx->stream), "hipEventRecord")) != AGPU_OK) return rc;
     if ((rc = agpu_hip(ctx, hipEventSynchronize(m->ev1), "hipEventSynchronize")) != AGPU_OK) return rc;
     if (ms_total_out_host) (void)hipEventElapsedTime(ms_total_out_host, m->ev0, m->ev1);
-    return AGPU_OK;
+    return pk_check(m);
+}
+
+#ifdef AGPU_PK_TRACE
+// Debug builds only: one step of the one-launch decode with time stamps, [grid][n_stages][4] ticks of 10 ns.
+AGPU_EXPORT int32_t agpu_gpt2_decode_trace(agpu_gpt2 *m, int32_t mode, unsigned long long *out_host, int32_t *grid_out, int32_t *stages_out) {
+    if (!pk_ready(m)) return AGPU_ERR_UNSUPPORTED;
+    const size_t n = (size_t)m->pk.grid * m->pk.n_stages * 8;
+    unsigned long long *dev = nullptr;
+    if (hipMalloc((void **)&dev, n * 8) != hipSuccess) return AGPU_ERR_WORKSPACE;
+    (void)hipMemset(dev, 0, n * 8);
+    int32_t rc = agpu_pk_launch(m->ctx, pk_view(m), m->pk, mode, dev);
+    (void)hipStreamSynchronize(m->ctx->stream);
+    (void)hipMemcpy(out_host, dev, n * 8, hipMemcpyDeviceToHost);
+    (void)hipFree(dev);
+    *grid_out = m->pk.grid;
+    *stages_out = m->pk.n_stages;
+    if (mode == 0) m->cache_len += 1;
+    return rc;
+}
+#endif
+
+AGPU_EXPORT int32_t agpu_gpt2_last_logits(agpu_gpt2 *m, int32_t batch, float *logits_out_host) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    agpu_ctx *ctx = m->ctx;
+    if (!logits_out_host) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "gpt2_last_logits: null pointer");
+    if (batch <= 0 || batch > m->cfg.max_batch) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_last_logits: bad batch");
+    const size_t stride = logits_stride(m);
+    if (!m->logits.p || m->logits.bytes < (size_t)batch * stride * 4)
+        return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "gpt2_last_logits: no forward has run for this batch");
+    hipError_t e = hipMemcpy2DAsync(logits_out_host, (size_t)m->V * 4, m->logits.p, stride * 4, (size_t)m->V * 4, (size_t)batch,
+                                    hipMemcpyDeviceToHost, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    return agpu_hip(ctx, e, "gpt2_last_logits");
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_decode_floor(agpu_gpt2 *m, int32_t steps, float *ms_total_out_host) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    agpu_ctx *ctx = m->ctx;
+    if (steps < 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_decode_floor: bad steps");
+    int32_t rc = check_ready(m);
+    if (rc != AGPU_OK) return rc;
+    if ((rc = ensure_buffers(m, 1, 1, false)) != AGPU_OK) return rc;
+    if ((rc = ensure_out_tokens(m, 1, 1)) != AGPU_OK) return rc;
+    if (!pk_ready(m)) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "gpt2_decode_floor: this model does not take the one-launch decode step");
+    const PkModel v = pk_view(m);
+    if ((rc = agpu_hip(ctx, hipEventRecord(m->ev0, ctx->stream), "hipEventRecord")) != AGPU_OK) return rc;
+    for (int s = 0; s < steps; ++s)
+        if ((rc = agpu_pk_launch(ctx, v, m->pk, 1)) != AGPU_OK) return rc;
+    if ((rc = agpu_hip(ctx, hipEventRecord(m->ev1, ctx->stream), "hipEventRecord")) != AGPU_OK) return rc;
+    if ((rc = agpu_hip(ctx, hipEventSynchronize(m->ev1), "hipEventSynchronize")) != AGPU_OK) return rc;
+    if (ms_total_out_host) (void)hipEventElapsedTime(ms_total_out_host, m->ev0, m->ev1);
+    return pk_check(m);
 }
 
 AGPU_EXPORT int32_t agpu_gpt2_generate_cached(agpu_gpt2 *m, const uint32_t *prompt_host, int32_t batch, int32_t prompt_len,
@@ -886,6 +1042,7 @@ AGPU_EXPORT int32_t agpu_gpt2_generate_cached(agpu_gpt2 *m, const uint32_t *prom
     std::vector<uint32_t> gen((size_t)max_new_tokens * batch);
     rc = agpu_memcpy_d2h(ctx, gen.data(), m->out_tok, gen.size() * 4);
     if (rc != AGPU_OK) return rc;
+    if ((rc = pk_check(m)) != AGPU_OK) return rc;
     if (timing_ms_out_host) {
         (void)hipEventElapsedTime(&timing_ms_out_host[0], m->ev0, m->ev1);
         (void)hipEventElapsedTime(&timing_ms_out_host[1], m->ev1, m->ev2);
@@ -963,6 +1120,7 @@ AGPU_EXPORT int32_t agpu_gpt2_generate_cached_sampling(agpu_gpt2 *m, const uint3
     (void)hipFree(idx_dev);
     (void)hipFree(val_dev);
     *length_out_host = len;
+    if (rc == AGPU_OK) rc = pk_check(m);
     return rc;
 }
 

@@ -241,3 +241,28 @@ class Int4Gpt2Model:
         ms = C.c_float(0)
         self._call("agpu_gpt2_decode_steps", batch, steps, C.addressof(ms))
         return float(ms.value)
+
+    DECODE_AUTO, DECODE_PER_STAGE = 0, 1
+
+    def set_decode_mode(self, mode):
+        """DECODE_AUTO: single-sequence steps run as one launch where the shape allows; DECODE_PER_STAGE: one launch per stage."""
+        self._call("agpu_gpt2_set_decode_mode", mode)
+
+    def decode_is_one_launch(self):
+        return bool(self._lib.agpu_gpt2_decode_is_one_launch(self.handle))
+
+    def set_decode_wait_limit(self, poll_rounds):
+        """Test hook: poll rounds a wait inside the one-launch step may take (0 = default)."""
+        self._call("agpu_gpt2_set_decode_wait_limit", poll_rounds)
+
+    def decode_floor(self, steps):
+        """The one-launch step's stage chain with empty bodies, `steps` times; returns the total milliseconds."""
+        ms = C.c_float(0)
+        self._call("agpu_gpt2_decode_floor", steps, C.addressof(ms))
+        return float(ms.value)
+
+    def last_logits(self, batch=1):
+        """[batch, vocab] logits of the last position as the most recent forward or decode step left them."""
+        out = np.empty((batch, self.config.vocab_size), np.float32)
+        self._call("agpu_gpt2_last_logits", batch, out)
+        return out

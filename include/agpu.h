@@ -41,6 +41,7 @@ extern "C" {
 #define AGPU_ERR_UNSUPPORTED (-5)
 #define AGPU_ERR_WORKSPACE (-6)        /* split-K scratch too small for the request */
 #define AGPU_ERR_BUSY (-8)             /* another thread is inside a call on this context */
+#define AGPU_ERR_DEVICE_WAIT (-7)      /* a bounded wait inside a kernel gave up; the results of that call are invalid */
 
 typedef struct agpu_ctx agpu_ctx;
 

@@ -139,6 +139,41 @@ int32_t agpu_gpt2_generate_cached_early_exit(agpu_gpt2 *m, const uint32_t *promp
                                              int32_t *layers_out_host, int32_t *steps_out_host);
 
 /*
+ * How single-sequence decode steps run.  No counterpart in the reference, whose host loop launches every kernel
+ * of every step (gpt2.rs:760-780).
+ *   AGPU_DECODE_AUTO       one launch per token where the model's shape allows it (int4 head, head_dim 64, group a
+ *                          power of two >= 8, vocab < 65536, K <= 8192), else as below
+ *   AGPU_DECODE_PER_STAGE  one launch per stage (5 per block + 1), replayed as a HIP graph
+ * Both give the same greedy tokens wherever the arg-max is not within rounding of a tie; logits differ by
+ * summation order only (both within 2e-4 of the f64 forward).  The one-launch step keeps one workgroup resident on
+ * every CU for the duration of the step: nothing else should run on the device meanwhile.  Its waits are bounded;
+ * a wait that gives up makes the call that ran the step return AGPU_ERR_DEVICE_WAIT: the tokens of that call are
+ * void, the model then keeps to the per-stage path, and the caller may simply run the call again.
+ */
+#define AGPU_DECODE_AUTO 0
+#define AGPU_DECODE_PER_STAGE 1
+int32_t agpu_gpt2_set_decode_mode(agpu_gpt2 *m, int32_t mode);
+/* 1 once a single-sequence decode step has been planned as one launch, else 0. */
+int32_t agpu_gpt2_decode_is_one_launch(agpu_gpt2 *m);
+/* Test hook: the number of poll rounds a wait inside the one-launch step may take before it gives up (0 = the
+ * default, tens of milliseconds).  With a limit of a few rounds every wait gives up, the kernel still runs to its end,
+ * and the call that ran the step returns AGPU_ERR_DEVICE_WAIT: the error path without a hung device. */
+int32_t agpu_gpt2_set_decode_wait_limit(agpu_gpt2 *m, int32_t poll_rounds);
+/*
+ * Benchmark hook: the latency floor of the one-launch decode step.  Runs `steps` launches of the same stage chain
+ * with empty bodies (every tagged store and every wait, no weights, no arithmetic; cache, tokens and counters are
+ * left alone) and reports the total time.  AGPU_ERR_UNSUPPORTED when the model does not take the one-launch step.
+ */
+int32_t agpu_gpt2_decode_floor(agpu_gpt2 *m, int32_t steps, float *ms_total_out_host);
+
+/*
+ * Test hook: the logits the most recent forward or decode step left on the device, rows [batch, vocab_size] of
+ * the last position (HOST pointer).  The reference returns them from forward_cached (gpt2.rs:712-734); the
+ * replayed decode loop keeps them on the device and only consumes their arg-max.
+ */
+int32_t agpu_gpt2_last_logits(agpu_gpt2 *m, int32_t batch, float *logits_out_host);
+
+/*
  * Benchmark hook: replay `steps` decode steps (one token per sequence per step) starting from the
  * current cache state and the device-resident current tokens, without any host round trip, and
  * report the time per step measured with HIP events on the context's stream.  The cache advances by

@@ -1,0 +1,109 @@
+"""The one-launch decode step (single sequence): same tokens as the per-stage path and the f64 oracle, logits within
+2e-4, across context lengths that change the number of key ranges per head, with the model's options; its bounded
+waits give up cleanly when the host makes them."""
+import numpy as np
+import pytest
+
+from conftest import build_oracle_model, gpu_config
+
+pytestmark = pytest.mark.gpu
+
+TOL_LOGITS = 2e-4
+
+
+def _quantized(orc, cfg, seed, **kw):
+    from async_gpu_amd import workloads
+    w = workloads.gpt2_fp32_weights(cfg, seed, std=0.08, **kw)
+    return workloads.quantize_gpt2(w, 32, lambda wt, g: orc.quantize_weight_int4(wt, g, orc.SCRIPT))
+
+
+def _match(got, ref, margins, prompt_len, what):
+    n = min(len(got), len(ref))
+    diff = [i for i in range(n) if got[i] != ref[i]]
+    if diff or len(got) != len(ref):
+        i = diff[0] if diff else n
+        gap = margins[i - prompt_len] if prompt_len <= i < prompt_len + len(margins) else float("nan")
+        pytest.fail(f"{what}: tokens diverge at index {i}; oracle top-1/top-2 gap there {gap:.3e}")
+
+
+@pytest.mark.parametrize("options", [dict(), dict(gelu=1), dict(argmax_last=1)])
+def test_one_launch_equals_per_stage_and_oracle(orc, agpu, dev, options):
+    from async_gpu_amd import gpt2, workloads
+    cfg = workloads.GPT2_TINY
+    qz = _quantized(orc, cfg, 31, nonzero_bias=True, random_ln=True)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg, **options), qz)
+    prompt = workloads.random_prompt(cfg, 8, 7)
+    gm.set_decode_mode(gm.DECODE_PER_STAGE)
+    (a,), _ = gm.generate_cached(prompt, 40, eos=-1)
+    la = gm.last_logits()
+    assert not gm.decode_is_one_launch()
+    gm.set_decode_mode(gm.DECODE_AUTO)
+    (b,), _ = gm.generate_cached(prompt, 40, eos=-1)
+    lb = gm.last_logits()
+    assert gm.decode_is_one_launch()
+    assert np.array_equal(a, b)
+    assert np.abs(la - lb).max() <= 1e-5
+    (b2,), _ = gm.generate_cached(prompt, 40, eos=-1)
+    assert np.array_equal(b, b2) and np.array_equal(lb, gm.last_logits())  # bit-identical run to run
+    if not options:
+        om = build_oracle_model(cfg, qz)
+        ref, margins = om.generate(prompt, 40, cached=True, eos=-1)
+        _match(b, ref, margins, 7, "one-launch step")
+        om.reset_cache()
+        om.forward(ref[:-2], all_rows=False)
+        lo = om.forward(ref[-2:-1], all_rows=False)
+        assert np.abs(lb[0] - lo[0]).max() <= TOL_LOGITS
+    assert gm.decode_floor(8) > 0.0
+
+
+@pytest.mark.parametrize("prompt_len", [250, 505, 760])
+def test_one_launch_across_key_range_counts(orc, agpu, dev, prompt_len):
+    """Beyond 256, 512 and 768 cached positions a head's keys go to two, three and four workgroups."""
+    from async_gpu_amd import gpt2, workloads
+    cfg = dict(n_layer=2, n_embd=128, n_head=2, vocab=503, n_positions=1024)
+    qz = _quantized(orc, cfg, 32, nonzero_bias=True, random_ln=True)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg), qz)
+    om = build_oracle_model(cfg, qz)
+    prompt = workloads.random_prompt(cfg, prompt_len, prompt_len)
+    ref, margins = om.generate(prompt, 24, cached=True, eos=-1)
+    (got,), _ = gm.generate_cached(prompt, 24, eos=-1)
+    assert gm.decode_is_one_launch()
+    _match(got, ref, margins, prompt_len, f"one-launch step from {prompt_len} positions")
+    lb = gm.last_logits()
+    gm.set_decode_mode(gm.DECODE_PER_STAGE)
+    (per,), _ = gm.generate_cached(prompt, 24, eos=-1)
+    assert np.array_equal(per, got)
+    assert np.abs(gm.last_logits() - lb).max() <= 1e-5
+
+
+def test_wait_that_gives_up_is_reported_and_the_model_recovers(orc, agpu, dev):
+    """With a limit of two poll rounds every wait inside the step gives up: the kernel still ends, the call reports
+    AGPU_ERR_DEVICE_WAIT, and the model serves the same request per stage afterwards."""
+    from async_gpu_amd import _lib, gpt2, workloads
+    cfg = workloads.GPT2_TINY
+    qz = _quantized(orc, cfg, 33)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg), qz)
+    prompt = workloads.random_prompt(cfg, 9, 5)
+    (good,), _ = gm.generate_cached(prompt, 12, eos=-1)
+    assert gm.decode_is_one_launch()
+    gm.set_decode_wait_limit(2)
+    with pytest.raises(_lib.AgpuError) as e:
+        gm.generate_cached(prompt, 12, eos=-1)
+    assert e.value.code == _lib.ERR_DEVICE_WAIT
+    assert not gm.decode_is_one_launch()
+    (again,), _ = gm.generate_cached(prompt, 12, eos=-1)
+    assert not gm.decode_is_one_launch()
+    assert np.array_equal(again, good)
+
+
+def test_sampling_runs_on_the_one_launch_step(orc, agpu, dev):
+    from async_gpu_amd import gpt2, ops, workloads
+    cfg = workloads.GPT2_TINY
+    qz = _quantized(orc, cfg, 34)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg), qz)
+    prompt = workloads.random_prompt(cfg, 10, 6)
+    a = gm.generate_cached_sampling(prompt, 20, 5, 0.9, ops.SimpleRng(7), eos=-1)
+    assert gm.decode_is_one_launch()
+    gm.set_decode_mode(gm.DECODE_PER_STAGE)
+    b = gm.generate_cached_sampling(prompt, 20, 5, 0.9, ops.SimpleRng(7), eos=-1)
+    assert np.array_equal(a, b)
