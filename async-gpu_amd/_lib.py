@@ -45,6 +45,8 @@ SIGNATURES = {
     "agpu_ctx_stream": (_vp, [_vp]),
     "agpu_malloc": (_i32, [_vp, _sz, C.POINTER(_vp)]),
     "agpu_free": (_i32, [_vp, _vp]),
+    "agpu_host_alloc_mapped": (_i32, [_vp, _sz, C.POINTER(_vp), C.POINTER(_vp)]),
+    "agpu_host_free_mapped": (_i32, [_vp, _vp]),
     "agpu_memcpy_h2d": (_i32, [_vp, _vp, _vp, _sz]),
     "agpu_memcpy_d2h": (_i32, [_vp, _vp, _vp, _sz]),
     "agpu_memcpy_d2d": (_i32, [_vp, _vp, _vp, _sz]),

@@ -21,3 +21,6 @@ echo "built $(cd .. && pwd)/libagpu_hip.so"
 g++ -O1 -std=c++17 -I../../include ../../tests/cpp/test_nn.cpp -o ../../tests/cpp/test_nn \
     -L.. -lagpu_hip -Wl,-rpath,'$ORIGIN/../../async-gpu_amd' -Wl,-rpath,/opt/rocm/lib -L/opt/rocm/lib -lamdhip64
 echo "built tests/cpp/test_nn"
+g++ -O1 -std=c++17 -I../../include ../../tests/cpp/test_gpu_array_host.cpp -o ../../tests/cpp/test_gpu_array_host \
+    -L.. -lagpu_hip -Wl,-rpath,'$ORIGIN/../../async-gpu_amd' -Wl,-rpath,/opt/rocm/lib -L/opt/rocm/lib -lamdhip64
+echo "built tests/cpp/test_gpu_array_host"

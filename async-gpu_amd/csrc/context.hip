@@ -155,6 +155,34 @@ AGPU_EXPORT int32_t agpu_free(agpu_ctx *ctx, void *ptr) {
     return agpu_hip(ctx, hipFree(ptr), "hipFree");
 }
 
+AGPU_EXPORT int32_t agpu_host_alloc_mapped(agpu_ctx *ctx, size_t bytes, void **host_out, void **dev_out) {
+    AGPU_REQUIRE_CTX(ctx);
+    AGPU_REQUIRE_PTR(ctx, host_out);
+    AGPU_REQUIRE_PTR(ctx, dev_out);
+    *host_out = *dev_out = nullptr;
+    if (bytes == 0) return AGPU_OK;
+    void *h = nullptr, *d = nullptr;
+    hipError_t e = hipHostMalloc(&h, bytes, hipHostMallocMapped);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipHostMalloc");
+    e = hipHostGetDevicePointer(&d, h, 0);
+    if (e != hipSuccess) {
+        (void)hipHostFree(h);
+        return agpu_hip(ctx, e, "hipHostGetDevicePointer");
+    }
+    std::memset(h, 0, bytes);
+    *host_out = h;
+    *dev_out = d;
+    return AGPU_OK;
+}
+
+AGPU_EXPORT int32_t agpu_host_free_mapped(agpu_ctx *ctx, void *host) {
+    AGPU_REQUIRE_CTX(ctx);
+    if (!host) return AGPU_OK;
+    hipError_t e = hipStreamSynchronize(ctx->stream);  // a kernel may still be reading or writing the memory
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipStreamSynchronize");
+    return agpu_hip(ctx, hipHostFree(host), "hipHostFree");
+}
+
 AGPU_EXPORT int32_t agpu_memcpy_h2d(agpu_ctx *ctx, void *dst, const void *src_host, size_t bytes) {
     AGPU_REQUIRE_CTX(ctx);
     if (bytes == 0) return AGPU_OK;

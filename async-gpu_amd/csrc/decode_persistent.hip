@@ -640,9 +640,8 @@ __device__ __forceinline__ void head_finish(const Params &p, const Stage &st, co
 }
 
 // ---- relay ----
-// Every input vector of a Linear, in the order the step produces them: awaited in memory, copied into this XCD's
-// mirror.  Thread t owns the element pairs t, t + T, ...; nothing orders the threads among themselves, every
-// pair carries its own tags.
+// One vector: awaited in memory, copied into this XCD's mirror.  Thread t owns the element pairs t, t + T, ...; nothing
+// orders the threads among themselves, every pair carries its own tags.
 __device__ __forceinline__ void relay_copy(const Params &p, Ctl &c, u64 *mirror, int off, int n_elems, int tid, int phase) {
     const int n_pairs = n_elems >> 1;
     const u64 *src = p.arena + off;
@@ -681,9 +680,7 @@ __device__ __forceinline__ void relay_copy(const Params &p, Ctl &c, u64 *mirror,
     PK_STAMP(1);
 }
 
-// Every input vector of a Linear, in the order the step produces them: awaited in memory, copied into this XCD's
-// mirror.  Thread t owns the element pairs t, t + T, ...; nothing orders the threads
-// among themselves, every pair carries its own tags.
+// Every input vector of a Linear, in the order the step produces them.
 __device__ __forceinline__ void relay_role(const Params &p, const Stage *tab, Ctl &c, u64 *mirror, int tid, int phase) {
     for (int s = 0; s < p.n_stages; ++s) {
         c.stage = s;

@@ -87,6 +87,12 @@ int32_t agpu_memcpy_d2h(agpu_ctx *ctx, void *dst_host, const void *src, size_t b
 int32_t agpu_memcpy_d2d(agpu_ctx *ctx, void *dst, const void *src, size_t bytes);      /* clone_tensor, tensor.rs:270-282 */
 int32_t agpu_sync(agpu_ctx *ctx);                                                       /* dev.synchronize() */
 
+/* Pinned host memory that the device reads and writes in place (MappedBuffer, crates/core/gpu-host/src/memory.rs, the
+ * zero-copy backend of GpuArray below 64 KiB, gpu_array.rs:45-51,174-176): *host_out is the host address, *dev_out the
+ * address kernels use for the same bytes.  The memory is zeroed.  Free it with agpu_host_free_mapped(host address). */
+int32_t agpu_host_alloc_mapped(agpu_ctx *ctx, size_t bytes, void **host_out, void **dev_out);
+int32_t agpu_host_free_mapped(agpu_ctx *ctx, void *host);
+
 /* Stage timing as Gpt2Model::forward_profiled does it (synchronize + clock around a stage,
  * nn/models/gpt2.rs:529-568), with HIP events on the context's stream instead of a host clock:
  * agpu_timer_start records an event; agpu_timer_stop records a second one, waits for it and

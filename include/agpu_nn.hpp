@@ -4,6 +4,7 @@
 //   NnError            nn/error.rs:7-29
 //   KernelRegistry     nn/registry.rs:26-144
 //   GpuTensor          nn/tensor.rs:45-282
+//   GpuArray, Residency  gpu_array.rs:42-385 (crates/core/gpu-host/src/gpu_array.rs)
 //   ops::*             nn/ops/{gemm,norm,activation,reshape,attention,quantize}.rs
 //   Module, Int4Linear, Linear, LayerNorm, Gelu, Embedding   nn/layers/*.rs
 //   Gpt2Config, Int4Gpt2Model                                nn/models/gpt2.rs:20-93,1341-1580,712-783
@@ -13,11 +14,13 @@
 #pragma once
 
 #include <cstdint>
+#include <cstring>
 #include <memory>
 #include <numeric>
 #include <optional>
 #include <stdexcept>
 #include <string>
+#include <type_traits>
 #include <utility>
 #include <vector>
 
@@ -154,6 +157,151 @@ public:
 private:
     GpuTensor t_;
     size_t n_ = 0;
+};
+
+// ---- GpuArray (gpu_array.rs:42-385): a host vector with a device copy made on demand -----------
+// Residency (gpu_array.rs:55-69).
+enum class Residency {
+    HostOnly,    // data on the host only; no device storage yet
+    Synced,      // host and device hold the same data
+    DeviceOnly,  // a kernel wrote the device copy: the host copy is stale until read() syncs it back
+    HostDirty,   // the host copy was modified: the device copy is stale until ensure_device uploads it
+};
+
+// Below this size the device side is pinned host memory that kernels access in place, at or above it separate device
+// memory with explicit copies (SIZE_THRESHOLD_BYTES, gpu_array.rs:45-51).
+constexpr size_t kGpuArrayMappedThresholdBytes = 64 * 1024;
+
+template <class T>
+class GpuArray {
+    static_assert(std::is_trivially_copyable<T>::value, "GpuArray elements are copied byte for byte");
+
+public:
+    // GpuArray::from_vec (gpu_array.rs:138-150): HostOnly, nothing allocated on the device.
+    static GpuArray from_vec(std::vector<T> data) {
+        GpuArray a;
+        a.len_ = data.size();
+        a.host_ = std::move(data);
+        return a;
+    }
+    static GpuArray from_slice(const T *data, size_t n) { return from_vec(std::vector<T>(data, data + n)); }
+    static GpuArray zeroed(size_t n) { return from_vec(std::vector<T>(n, T{})); }  // gpu_array.rs:344-351
+
+    GpuArray() = default;
+    GpuArray(GpuArray &&o) noexcept { *this = std::move(o); }
+    GpuArray &operator=(GpuArray &&o) noexcept {
+        if (this != &o) {
+            release();
+            host_ = std::move(o.host_);
+            len_ = o.len_;
+            residency_ = o.residency_;
+            reg_ = std::move(o.reg_);
+            dev_ptr_ = o.dev_ptr_;
+            mapped_host_ = o.mapped_host_;
+            o.dev_ptr_ = o.mapped_host_ = nullptr;
+            o.len_ = 0;
+            o.residency_ = Residency::HostOnly;
+        }
+        return *this;
+    }
+    GpuArray(const GpuArray &) = delete;  // the reference type is not Clone
+    GpuArray &operator=(const GpuArray &) = delete;
+    ~GpuArray() { release(); }
+
+    size_t len() const { return len_; }
+    bool is_empty() const { return len_ == 0; }
+    Residency residency() const { return residency_; }
+    bool should_use_mapped() const { return len_ * sizeof(T) < kGpuArrayMappedThresholdBytes; }  // gpu_array.rs:174-176
+    bool is_mapped() const { return mapped_host_ != nullptr; }
+
+    // Deref (gpu_array.rs:353-370): the host data, synced back from the device first if a kernel wrote it.
+    const std::vector<T> &read() const {
+        if (residency_ == Residency::DeviceOnly) sync_to_host();
+        return host_;
+    }
+    const T &operator[](size_t i) const { return read()[i]; }
+    // DerefMut (gpu_array.rs:372-385): as read(), then the host copy is the newer one.
+    std::vector<T> &write() {
+        if (residency_ == Residency::DeviceOnly) sync_to_host();
+        residency_ = Residency::HostDirty;
+        return host_;
+    }
+
+    // mark_device_dirty (gpu_array.rs:227-240): a kernel wrote the device copy.
+    void mark_device_dirty() const {
+        if (residency_ == Residency::Synced) residency_ = Residency::DeviceOnly;
+    }
+
+    // ensure_device (gpu_array.rs:241-340): the device address of the data, uploaded if the host copy is newer.
+    // HostOnly: allocates (mapped below the threshold) and uploads -> Synced.  HostDirty: uploads -> Synced.
+    // Synced / DeviceOnly: nothing to do.  An empty array has no storage and the address 0.
+    uint64_t ensure_device(const Registry &reg) const {
+        switch (residency_) {
+            case Residency::HostOnly: {
+                if (len_ == 0) {
+                    residency_ = Residency::Synced;
+                    return 0;
+                }
+                const size_t bytes = len_ * sizeof(T);
+                reg_ = reg;
+                if (should_use_mapped()) {
+                    reg->check(agpu_host_alloc_mapped(reg->device(), bytes, &mapped_host_, &dev_ptr_));
+                    std::memcpy(mapped_host_, host_.data(), bytes);
+                } else {
+                    reg->check(agpu_malloc(reg->device(), bytes, &dev_ptr_));
+                    reg->check(agpu_memcpy_h2d(reg->device(), dev_ptr_, host_.data(), bytes));
+                }
+                residency_ = Residency::Synced;
+                return (uint64_t)(uintptr_t)dev_ptr_;
+            }
+            case Residency::HostDirty: {
+                if (len_ == 0 || !dev_ptr_) {  // modified before the first upload: nothing on the device yet
+                    residency_ = Residency::HostOnly;
+                    return ensure_device(reg);
+                }
+                const size_t bytes = len_ * sizeof(T);
+                if (mapped_host_) {
+                    reg_->check(agpu_sync(reg_->device()));  // no kernel may still be reading the old contents
+                    std::memcpy(mapped_host_, host_.data(), bytes);
+                } else {
+                    reg_->check(agpu_memcpy_h2d(reg_->device(), dev_ptr_, host_.data(), bytes));
+                }
+                residency_ = Residency::Synced;
+                return (uint64_t)(uintptr_t)dev_ptr_;
+            }
+            default: return (uint64_t)(uintptr_t)dev_ptr_;
+        }
+    }
+    // The typed device pointer for the C ABI (after ensure_device).
+    T *device_ptr(const Registry &reg) const { return reinterpret_cast<T *>((uintptr_t)ensure_device(reg)); }
+
+private:
+    void sync_to_host() const {  // gpu_array.rs:178-218
+        if (len_ != 0 && dev_ptr_) {
+            const size_t bytes = len_ * sizeof(T);
+            if (mapped_host_) {
+                reg_->check(agpu_sync(reg_->device()));  // the kernel that wrote the memory has finished
+                std::memcpy(host_.data(), mapped_host_, bytes);
+            } else {
+                reg_->check(agpu_memcpy_d2h(reg_->device(), host_.data(), dev_ptr_, bytes));
+            }
+        }
+        residency_ = Residency::Synced;
+    }
+    void release() {
+        if (reg_) {
+            if (mapped_host_) agpu_host_free_mapped(reg_->device(), mapped_host_);
+            else if (dev_ptr_) agpu_free(reg_->device(), dev_ptr_);
+        }
+        dev_ptr_ = mapped_host_ = nullptr;
+    }
+
+    mutable std::vector<T> host_;
+    size_t len_ = 0;
+    mutable Residency residency_ = Residency::HostOnly;
+    mutable Registry reg_;
+    mutable void *dev_ptr_ = nullptr;      // device address of the data (either backend)
+    mutable void *mapped_host_ = nullptr;  // host address of the pinned mapped backend, else null
 };
 
 // ---- ops (nn/ops/*.rs) ------------------------------------------------------------------------

@@ -1,0 +1,182 @@
+//! Gpt2Config and Int4Gpt2Model (nn/models/gpt2.rs:20-93, 1341-1580) with the cached control flow of
+//! Gpt2Model::{forward_cached, generate_cached} (gpt2.rs:712-783), over the model driver of libagpu_hip.so: weights
+//! and the KV cache live on the device, a decode step needs no host round trip.
+use std::ffi::c_void;
+use std::sync::Arc;
+
+use agpu_sys as sys;
+
+use crate::error::{NnError, Result};
+use crate::registry::KernelRegistry;
+
+/// Gpt2Config (gpt2.rs:20-93).
+#[derive(Clone, Copy, Debug, PartialEq)]
+pub struct Gpt2Config {
+    pub vocab_size: usize,
+    pub n_positions: usize,
+    pub n_embd: usize,
+    pub n_layer: usize,
+    pub n_head: usize,
+    pub layer_norm_epsilon: f32,
+}
+
+impl Gpt2Config {
+    pub fn small() -> Self {
+        Gpt2Config { vocab_size: 50257, n_positions: 1024, n_embd: 768, n_layer: 12, n_head: 12, layer_norm_epsilon: 1e-5 }
+    }
+    pub fn medium() -> Self {
+        Gpt2Config { n_embd: 1024, n_layer: 24, n_head: 16, ..Self::small() }
+    }
+    pub fn large() -> Self {
+        Gpt2Config { n_embd: 1280, n_layer: 36, n_head: 20, ..Self::small() }
+    }
+    pub fn xl() -> Self {
+        Gpt2Config { n_embd: 1600, n_layer: 48, n_head: 25, ..Self::small() }
+    }
+    pub fn head_dim(&self) -> usize {
+        self.n_embd / self.n_head
+    }
+    pub fn ffn_dim(&self) -> usize {
+        4 * self.n_embd
+    }
+}
+
+/// fp32 weights of one block, Conv1D layout [in, out] (model.rs:308-378).
+pub struct Gpt2LayerWeights {
+    pub ln1_g: Vec<f32>,
+    pub ln1_b: Vec<f32>,
+    pub ln2_g: Vec<f32>,
+    pub ln2_b: Vec<f32>,
+    pub qkv_w: Vec<f32>,
+    pub qkv_b: Vec<f32>,
+    pub proj_w: Vec<f32>,
+    pub proj_b: Vec<f32>,
+    pub fc_w: Vec<f32>,
+    pub fc_b: Vec<f32>,
+    pub fc_proj_w: Vec<f32>,
+    pub fc_proj_b: Vec<f32>,
+}
+
+pub struct Gpt2Weights {
+    pub wte: Vec<f32>,
+    pub wpe: Vec<f32>,
+    pub lnf_g: Vec<f32>,
+    pub lnf_b: Vec<f32>,
+    pub layers: Vec<Gpt2LayerWeights>,
+}
+
+pub struct Int4Gpt2Model {
+    handle: *mut sys::agpu_gpt2,
+    config: Gpt2Config,
+    registry: Arc<KernelRegistry>,
+}
+
+unsafe impl Send for Int4Gpt2Model {}
+
+impl Int4Gpt2Model {
+    /// DEFAULT_GROUP_SIZE (gpt2.rs:1358).
+    pub const DEFAULT_GROUP_SIZE: usize = 128;
+
+    /// Int4Gpt2Model::from_weights (gpt2.rs:1362-1433): every Linear is quantized at load, on the device.
+    pub fn from_weights(weights: &Gpt2Weights, config: &Gpt2Config, group_size: usize, registry: &Arc<KernelRegistry>) -> Result<Self> {
+        let mut cfg = sys::agpu_gpt2_config::default();
+        cfg.n_layer = config.n_layer as i32;
+        cfg.n_embd = config.n_embd as i32;
+        cfg.n_head = config.n_head as i32;
+        cfg.vocab_size = config.vocab_size as i32;
+        cfg.n_positions = config.n_positions as i32;
+        cfg.layer_norm_epsilon = config.layer_norm_epsilon;
+        cfg.group_size = group_size as i32;
+        cfg.max_batch = 1;
+        cfg.lm_head = sys::AGPU_LM_HEAD_F32; // the reference model keeps an f32 head over wte (gpt2.rs:1415-1422)
+        cfg.gelu = sys::AGPU_GELU_QUICK; // ops::gelu
+        cfg.argmax_last = 1; // Iterator::max_by keeps the last maximum (gpt2.rs:991-997)
+        let mut handle: *mut sys::agpu_gpt2 = std::ptr::null_mut();
+        registry.check(unsafe { sys::agpu_gpt2_create(registry.raw(), &cfg, &mut handle) })?;
+        let model = Int4Gpt2Model { handle, config: *config, registry: Arc::clone(registry) };
+        let (d, ff) = (config.n_embd as i32, config.ffn_dim() as i32);
+        registry.check(unsafe {
+            sys::agpu_gpt2_set_embeddings(handle, weights.wte.as_ptr(), weights.wpe.as_ptr(), weights.lnf_g.as_ptr(), weights.lnf_b.as_ptr(), 0)
+        })?;
+        for (l, w) in weights.layers.iter().enumerate() {
+            let l = l as i32;
+            registry.check(unsafe {
+                sys::agpu_gpt2_set_layer_norms(handle, l, w.ln1_g.as_ptr(), w.ln1_b.as_ptr(), w.ln2_g.as_ptr(), w.ln2_b.as_ptr(), 0)
+            })?;
+            for (which, wt, b, k, n) in [
+                (sys::AGPU_LINEAR_QKV, &w.qkv_w, &w.qkv_b, d, 3 * d),
+                (sys::AGPU_LINEAR_PROJ, &w.proj_w, &w.proj_b, d, d),
+                (sys::AGPU_LINEAR_FC, &w.fc_w, &w.fc_b, d, ff),
+                (sys::AGPU_LINEAR_FC_PROJ, &w.fc_proj_w, &w.fc_proj_b, ff, d),
+            ] {
+                registry.check(unsafe {
+                    sys::agpu_gpt2_quantize_linear(handle, l, which, wt.as_ptr(), b.as_ptr(), k, n, sys::AGPU_QUANT_RUST, 0)
+                })?;
+            }
+        }
+        Ok(model)
+    }
+
+    pub fn config(&self) -> &Gpt2Config {
+        &self.config
+    }
+
+    /// memory of the quantized Linears (quantized_memory_bytes, gpt2.rs:1436-1446).
+    pub fn quantized_memory_bytes(&self) -> usize {
+        unsafe { sys::agpu_gpt2_quantized_memory_bytes(self.handle) as usize }
+    }
+
+    /// Int4Gpt2Model::forward (gpt2.rs:1522-1533): logits [seq, vocab] of one sequence, no cache.
+    pub fn forward(&self, tokens: &[u32]) -> Result<Vec<f32>> {
+        let reg = &self.registry;
+        reg.check(unsafe { sys::agpu_gpt2_reset_cache(self.handle) })?;
+        let v = self.config.vocab_size;
+        let (mut dtok, mut dlog): (*mut c_void, *mut c_void) = (std::ptr::null_mut(), std::ptr::null_mut());
+        reg.check(unsafe { sys::agpu_malloc(reg.raw(), tokens.len() * 4, &mut dtok) })?;
+        reg.check(unsafe { sys::agpu_malloc(reg.raw(), tokens.len() * v * 4, &mut dlog) })?;
+        let mut out = vec![0f32; tokens.len() * v];
+        let rc = (|| -> Result<()> {
+            reg.check(unsafe { sys::agpu_memcpy_h2d(reg.raw(), dtok, tokens.as_ptr() as *const c_void, tokens.len() * 4) })?;
+            reg.check(unsafe { sys::agpu_gpt2_forward_cached(self.handle, dtok as *const u32, 1, tokens.len() as i32, dlog as *mut f32, 1) })?;
+            reg.check(unsafe { sys::agpu_memcpy_d2h(reg.raw(), out.as_mut_ptr() as *mut c_void, dlog, out.len() * 4) })
+        })();
+        unsafe {
+            sys::agpu_free(reg.raw(), dtok);
+            sys::agpu_free(reg.raw(), dlog);
+        }
+        rc.map(|_| out)
+    }
+
+    /// Int4Gpt2Model::generate (gpt2.rs:1535-1560): greedy, the whole sequence recomputed per token, stops before
+    /// appending the end-of-text token 50256.
+    pub fn generate(&self, prompt: &[u32], max_new_tokens: usize) -> Result<Vec<u32>> {
+        let mut out = vec![0u32; prompt.len() + max_new_tokens];
+        let mut len: i32 = 0;
+        self.registry.check(unsafe {
+            sys::agpu_gpt2_generate(self.handle, prompt.as_ptr(), prompt.len() as i32, max_new_tokens as i32, 50256, out.as_mut_ptr(), &mut len)
+        })?;
+        out.truncate(len as usize);
+        Ok(out)
+    }
+
+    /// generate_cached (gpt2.rs:736-783): prefill once, then one KV-cached step per token, all on the device.
+    pub fn generate_cached(&self, prompt: &[u32], max_new_tokens: usize) -> Result<Vec<u32>> {
+        if prompt.is_empty() {
+            return Err(NnError::ShapeMismatch { expected: "a non-empty prompt".to_string(), actual: "0 tokens".to_string() });
+        }
+        let mut out = vec![0u32; prompt.len() + max_new_tokens];
+        let mut len: i32 = 0;
+        self.registry.check(unsafe {
+            sys::agpu_gpt2_generate_cached(self.handle, prompt.as_ptr(), 1, prompt.len() as i32, max_new_tokens as i32, 50256, out.as_mut_ptr(),
+                                           &mut len, std::ptr::null_mut())
+        })?;
+        out.truncate(len as usize);
+        Ok(out)
+    }
+}
+
+impl Drop for Int4Gpt2Model {
+    fn drop(&mut self) {
+        unsafe { sys::agpu_gpt2_destroy(self.handle) };
+    }
+}

@@ -81,6 +81,44 @@ int main() {
         CHECK(throws_kind(NnError::Kind::DimOutOfRange, [&] { t.dim(3); }));
     });
 
+    run("gpu_array_residency", [&] {  // gpu_array.rs:516-640: upload on demand, kernel output synced back on read
+        for (size_t n : {size_t(100), size_t(16384 + 77)}) {  // pinned mapped backend, then device memory
+            std::vector<float> h(n);
+            for (size_t i = 0; i < n; ++i) h[i] = ((float)(i % 41) - 20.0f) * 0.125f;
+            auto in = GpuArray<float>::from_vec(h);
+            auto out = GpuArray<float>::zeroed(n);
+            CHECK(in.residency() == Residency::HostOnly);
+            const float *din = in.device_ptr(reg);
+            float *dout = out.device_ptr(reg);
+            CHECK(in.residency() == Residency::Synced && out.residency() == Residency::Synced);
+            CHECK(in.is_mapped() == (n * 4 < kGpuArrayMappedThresholdBytes));
+            CHECK(in.device_ptr(reg) == din);  // Synced: no new storage, no copy
+            // y = x + x through the device copies; the kernel's output is marked, the next read syncs it back
+            reg->check(agpu_memcpy_d2d(reg->device(), dout, din, n * sizeof(float)));
+            reg->check(agpu_add_inplace(reg->device(), dout, din, n));
+            out.mark_device_dirty();
+            CHECK(out.residency() == Residency::DeviceOnly);
+            bool ok = true;
+            for (size_t i = 0; i < n; ++i) ok = ok && out[i] == 2.0f * h[i];
+            CHECK(ok);
+            CHECK(out.residency() == Residency::Synced);
+            // a host write makes the device copy stale; the next ensure_device uploads into the same storage
+            in.write()[3] = 1000.0f;
+            CHECK(in.residency() == Residency::HostDirty);
+            CHECK(in.device_ptr(reg) == din && in.residency() == Residency::Synced);
+            reg->check(agpu_memcpy_d2d(reg->device(), dout, din, n * sizeof(float)));
+            out.mark_device_dirty();
+            CHECK(out[3] == 1000.0f && out[4] == h[4]);
+            // a write while the device copy is the newer one syncs back first, so the kernel's results are kept
+            reg->check(agpu_add_inplace(reg->device(), dout, din, n));
+            out.mark_device_dirty();
+            out.write()[0] = -1.0f;
+            CHECK(out.residency() == Residency::HostDirty && out[3] == 2000.0f && out[0] == -1.0f);
+        }
+        auto empty = GpuArray<float>::from_vec({});
+        CHECK(empty.ensure_device(reg) == 0 && empty.residency() == Residency::Synced);  // gpu_array.rs:262-266
+    });
+
     run("quantize_weight_int4_roundtrip", [&] {  // quantize.rs:217-267
         const size_t k = 8, n = 4;
         std::vector<float> w(k * n);
