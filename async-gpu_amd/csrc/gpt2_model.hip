@@ -500,7 +500,7 @@ PkModel pk_view(agpu_gpt2 *m) {
 
 // Whether single-sequence decode steps run as one launch; builds the plan on first use (never inside a capture).
 bool pk_ready(agpu_gpt2 *m) {
-    if (m->decode_mode == AGPU_DECODE_PER_STAGE || m->pk_failed || m->cfg.lm_head != AGPU_LM_HEAD_INT4) return false;
+    if (m->decode_mode != AGPU_DECODE_AUTO || m->pk_failed || m->cfg.lm_head != AGPU_LM_HEAD_INT4) return false;
     if (m->pk.stages_dev) return true;
     if (m->pk_tried) return false;
     m->pk_tried = true;
@@ -510,6 +510,15 @@ bool pk_ready(agpu_gpt2 *m) {
     if (agpu_pk_plan_build(m->ctx, v, &m->pk) != AGPU_OK) return false;
     m->pk.spin_limit = m->pk_spin_limit;
     return true;
+}
+
+// One decode step as one launch per stage; the LM head picks and feeds the next token itself where it can.
+int32_t launch_step_per_stage(agpu_gpt2 *m, int B, int bucket) {
+    const ArgmaxAdvance feed = token_feed(m, B, 1);
+    bool fed = false;
+    int32_t rc = launch_forward(m, m->cur_tok, B, 1, bucket, false, &feed, &fed);
+    if (rc == AGPU_OK && !fed) rc = launch_argmax_advance(m, B, 1);
+    return rc;
 }
 
 // The captured decode step for (batch, kv bucket); captured on first use.
@@ -535,11 +544,7 @@ int32_t decode_graph(agpu_gpt2 *m, int B, int bucket, hipGraphExec_t *out) {
         // one sequence: the whole step, arg-max and token feed included, is one launch
         rc = agpu_pk_launch(ctx, pk_view(m), m->pk, 0);
     } else {
-        // the LM head picks and feeds the next token itself where it can
-        const ArgmaxAdvance feed = token_feed(m, B, 1);
-        bool fed = false;
-        rc = launch_forward(m, m->cur_tok, B, 1, bucket, false, &feed, &fed);
-        if (rc == AGPU_OK && !fed) rc = launch_argmax_advance(m, B, 1);
+        rc = launch_step_per_stage(m, B, bucket);
     }
     hipGraph_t graph = nullptr;
     e = hipStreamEndCapture(ctx->stream, &graph);
@@ -574,11 +579,17 @@ int32_t ensure_out_tokens(agpu_gpt2 *m, int steps, int B) {
 // Replays `steps` decode steps; the host only tracks the position to pick the graph.
 int32_t run_decode_steps(agpu_gpt2 *m, int B, int steps) {
     for (int s = 0; s < steps; ++s) {
-        hipGraphExec_t exec;
-        int32_t rc = decode_graph(m, B, kv_bucket(m, m->cache_len + 1), &exec);
-        if (rc != AGPU_OK) return rc;
-        hipError_t e = hipGraphLaunch(exec, m->ctx->stream);
-        if (e != hipSuccess) return agpu_hip(m->ctx, e, "hipGraphLaunch");
+        const int bucket = kv_bucket(m, m->cache_len + 1);
+        if (m->decode_mode == AGPU_DECODE_EAGER) {
+            const int32_t rc = launch_step_per_stage(m, B, bucket);
+            if (rc != AGPU_OK) return rc;
+        } else {
+            hipGraphExec_t exec;
+            const int32_t rc = decode_graph(m, B, bucket, &exec);
+            if (rc != AGPU_OK) return rc;
+            const hipError_t e = hipGraphLaunch(exec, m->ctx->stream);
+            if (e != hipSuccess) return agpu_hip(m->ctx, e, "hipGraphLaunch");
+        }
         m->cache_len += 1;
     }
     return AGPU_OK;
@@ -864,7 +875,7 @@ AGPU_EXPORT int64_t agpu_gpt2_quantized_memory_bytes(const agpu_gpt2 *m) {
 
 AGPU_EXPORT int32_t agpu_gpt2_set_decode_mode(agpu_gpt2 *m, int32_t mode) {
     if (!m) return AGPU_ERR_NULL_POINTER;
-    if (mode != AGPU_DECODE_AUTO && mode != AGPU_DECODE_PER_STAGE)
+    if (mode != AGPU_DECODE_AUTO && mode != AGPU_DECODE_PER_STAGE && mode != AGPU_DECODE_EAGER)
         return agpu_fail(m->ctx, AGPU_ERR_DIM_OUT_OF_RANGE, "gpt2_set_decode_mode: unknown mode %d", mode);
     if (mode != m->decode_mode) {
         (void)hipStreamSynchronize(m->ctx->stream);
@@ -942,7 +953,7 @@ AGPU_EXPORT int32_t agpu_gpt2_decode_steps(agpu_gpt2 *m, int32_t batch, int32_t 
     if (rc != AGPU_OK) return rc;
     // capture outside the timed region
     hipGraphExec_t exec;
-    for (int s = 0; s < steps; ++s)
+    for (int s = 0; s < steps && m->decode_mode != AGPU_DECODE_EAGER; ++s)
         if ((rc = decode_graph(m, batch, kv_bucket(m, m->cache_len + 1 + s), &exec)) != AGPU_OK) return rc;
     if ((rc = agpu_hip(ctx, hipEventRecord(m->ev0, ctx->stream), "hipEventRecord")) != AGPU_OK) return rc;
     if ((rc = run_decode_steps(m, batch, steps)) != AGPU_OK) return rc;

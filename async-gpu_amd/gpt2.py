@@ -242,10 +242,11 @@ class Int4Gpt2Model:
         self._call("agpu_gpt2_decode_steps", batch, steps, C.addressof(ms))
         return float(ms.value)
 
-    DECODE_AUTO, DECODE_PER_STAGE = 0, 1
+    DECODE_AUTO, DECODE_PER_STAGE, DECODE_EAGER = 0, 1, 2
 
     def set_decode_mode(self, mode):
-        """DECODE_AUTO: single-sequence steps run as one launch where the shape allows; DECODE_PER_STAGE: one launch per stage."""
+        """DECODE_AUTO: single-sequence steps run as one launch where the shape allows; DECODE_PER_STAGE: one launch per stage,
+        replayed as a HIP graph; DECODE_EAGER: the same launches without a graph."""
         self._call("agpu_gpt2_set_decode_mode", mode)
 
     def decode_is_one_launch(self):

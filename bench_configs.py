@@ -28,6 +28,7 @@ def main():
     ap.add_argument("--skip-xl", action="store_true")
     ap.add_argument("--skip-kernels", action="store_true")
     ap.add_argument("--prefill-only", action="store_true", help="only the whole-model prefill of GPT-2 small (for kernel traces)")
+    ap.add_argument("--eager", action="store_true", help="XL-shaped decode at batch 16 without HIP graphs (for kernel traces)")
     ap.add_argument("--cpu", action="store_true", help="also time the CPU oracle on configs 1-3 (single thread, as the reference CPU path)")
     args = ap.parse_args()
     entry.load_package()
@@ -182,6 +183,7 @@ def xl_cases(ctx, emit, args, _lib, gpt2, workloads):
     per_w = 0.5 + 4.0 / 32
     wbytes = cfg["n_layer"] * (12 * d * d * per_w + (3 * d + d + ff + d) * 4 + 4 * d * 4) + d * V * per_w
     for B in (1, 16):
+        model.set_decode_mode(model.DECODE_EAGER if args.eager and B > 1 else model.DECODE_AUTO)
         prompts = workloads.random_prompt(cfg, 4, 256, batch=B)
         model.reset_cache()
         t0 = time.time()
@@ -196,6 +198,7 @@ def xl_cases(ctx, emit, args, _lib, gpt2, workloads):
         emit(case=f"config5 GPT-2 XL-shaped ({cfg['n_layer']} layers) int4 decode B={B}, prompt 256", ms_per_step=round(ms / steps, 4),
              tok_s=round(B * steps / (ms / 1e3), 1), algorithmic_bytes_per_step=int(bytes_step),
              GBps=round(bytes_step / (ms / steps) / 1e6, 1), frac_hbm=round(bytes_step / (ms / steps) / 1e6 / HBM_GBS, 4),
+             decode_path="one launch per token" if B == 1 and model.decode_is_one_launch() else ("one launch per stage, no graph" if args.eager else "one launch per stage"),
              prefill_wall_s=round(prefill_s, 3), model_build_s=round(build_s, 1))
 
 

@@ -144,6 +144,8 @@ int32_t agpu_gpt2_generate_cached_early_exit(agpu_gpt2 *m, const uint32_t *promp
  *   AGPU_DECODE_AUTO       one launch per token where the model's shape allows it (int4 head, head_dim 64, group a
  *                          power of two >= 8, vocab < 65536, K <= 8192), else as below
  *   AGPU_DECODE_PER_STAGE  one launch per stage (5 per block + 1), replayed as a HIP graph
+ *   AGPU_DECODE_EAGER      the same launches issued one by one, without a graph (for profilers that cannot follow
+ *                          graph replays, and for callers whose stream is under a capture of their own)
  * Both give the same greedy tokens wherever the arg-max is not within rounding of a tie; logits differ by
  * summation order only (both within 2e-4 of the f64 forward).  The one-launch step keeps one workgroup resident on
  * every CU for the duration of the step: nothing else should run on the device meanwhile.  Its waits are bounded;
@@ -152,6 +154,7 @@ int32_t agpu_gpt2_generate_cached_early_exit(agpu_gpt2 *m, const uint32_t *promp
  */
 #define AGPU_DECODE_AUTO 0
 #define AGPU_DECODE_PER_STAGE 1
+#define AGPU_DECODE_EAGER 2
 int32_t agpu_gpt2_set_decode_mode(agpu_gpt2 *m, int32_t mode);
 /* 1 once a single-sequence decode step has been planned as one launch, else 0. */
 int32_t agpu_gpt2_decode_is_one_launch(agpu_gpt2 *m);

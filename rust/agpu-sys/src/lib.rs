@@ -65,6 +65,7 @@ pub const AGPU_LINEAR_FC: i32 = 2;
 pub const AGPU_LINEAR_FC_PROJ: i32 = 3;
 pub const AGPU_DECODE_AUTO: i32 = 0;
 pub const AGPU_DECODE_PER_STAGE: i32 = 1;
+pub const AGPU_DECODE_EAGER: i32 = 2;
 
 extern "C" {
     // ---- include/agpu.h ----

@@ -56,6 +56,24 @@ def test_one_launch_equals_per_stage_and_oracle(orc, agpu, dev, options):
     assert gm.decode_floor(8) > 0.0
 
 
+@pytest.mark.parametrize("batch", [1, 3])
+def test_eager_steps_equal_graph_replays(orc, agpu, dev, batch):
+    """The per-stage step launched kernel by kernel gives the bits of its graph replay."""
+    from async_gpu_amd import gpt2, workloads
+    cfg = workloads.GPT2_TINY
+    qz = _quantized(orc, cfg, 33, nonzero_bias=True)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg, max_batch=4), qz)
+    prompt = workloads.random_prompt(cfg, 9, 6, batch=batch)
+    gm.set_decode_mode(gm.DECODE_PER_STAGE)
+    a, _ = gm.generate_cached(prompt, 30, eos=-1)
+    la = gm.last_logits(batch)
+    gm.set_decode_mode(gm.DECODE_EAGER)
+    b, _ = gm.generate_cached(prompt, 30, eos=-1)
+    assert not gm.decode_is_one_launch()
+    assert all(np.array_equal(x, y) for x, y in zip(a, b))
+    assert np.array_equal(la, gm.last_logits(batch))
+
+
 @pytest.mark.parametrize("prompt_len", [250, 505, 760])
 def test_one_launch_across_key_range_counts(orc, agpu, dev, prompt_len):
     """Beyond 256, 512 and 768 cached positions a head's keys go to two, three and four workgroups."""

@@ -286,11 +286,13 @@ def test_linear_epilogues_and_ln_prologue(agpu, orc, dev, M):
     xn = orc.layer_norm(x, gamma, beta, 1e-5)
     ref = orc.gelu(orc.int4_gemm_f64(xn, packed, scales, g, bias=bias)) + res
     assert np.abs(y.cpu().numpy() - ref).max() <= TOL_LINEAR
-    # quick GELU, residual aliasing the output
+    # quick GELU, residual aliasing the output.  The unnormalised x above (std 2, mean 0.5) gives outputs of magnitude 10,
+    # where fp32 itself resolves 1e-6 per term: at the N(0, 1) input scale the bound is stated for, 1e-4 holds.
+    x1 = rng.standard_normal((M, K)).astype(np.float32)
     out = to_dev(res, dev).clone()
-    ops.int4_linear(to_dev(x, dev), dp, ds, bias=db, residual=out, group=g, flags=agpu._lib.EPI_GELU_QUICK, out=out)
-    ref2 = orc.gelu(orc.int4_gemm_f64(x, packed, scales, g, bias=bias), mode=1) + res
-    assert np.abs(out.cpu().numpy() - ref2).max() <= 2e-4  # |y| reaches ~10 here; 1e-4 is held at unit scale above
+    ops.int4_linear(to_dev(x1, dev), dp, ds, bias=db, residual=out, group=g, flags=agpu._lib.EPI_GELU_QUICK, out=out)
+    ref2 = orc.gelu(orc.int4_gemm_f64(x1, packed, scales, g, bias=bias), mode=1) + res
+    assert np.abs(out.cpu().numpy() - ref2).max() <= TOL_LINEAR
 
 
 def test_linear_shape_rules_and_errors(agpu, orc, dev):
