@@ -291,7 +291,8 @@ int32_t ln_linear(agpu_gpt2 *m, const float *x, const float *gamma, const float 
     agpu_ctx *ctx = m->ctx;
     const float eps = m->cfg.layer_norm_epsilon;
     const int g = m->cfg.group_size;
-    if (!agpu_int4_gemv_can_fuse_ln(R, w.K)) {
+    const bool skinny_ln = g % 32 == 0 && w.K % 32 == 0 && N % 4 == 0 && agpu_int4_skinny_can_fuse_ln(R, N, w.K);
+    if (!agpu_int4_gemv_can_fuse_ln(R, w.K) && !skinny_ln) {
         float *lnb = (float *)m->lnb.p;
         int32_t rc = agpu_layer_norm_impl(ctx, x, gamma, beta, lnb, R, w.K, eps);
         if (rc != AGPU_OK) return rc;
@@ -331,12 +332,17 @@ int32_t launch_block(agpu_gpt2 *m, int L, int B, int new_len, int max_kv) {
         ga.kcache = kc; ga.vcache = vc; ga.pos_dev = m->pos_dev; ga.n_heads = H; ga.n_positions = P;
         if ((rc = agpu_int4_gemv_launch(ctx, ga)) != AGPU_OK) return rc;
     } else if (new_len == 1 && R <= 16 && g % 8 == 0) {
-        // batched decode: LayerNorm on its own, then the QKV projection writes the K/V rows itself
-        if ((rc = agpu_layer_norm_impl(ctx, hid, b.ln1_g, b.ln1_b, (float *)m->lnb.p, R, d, eps)) != AGPU_OK) return rc;
+        // batched decode: the QKV projection normalises the rows where it can and writes the K/V rows itself
         GemvArgs ga{};
-        ga.x = (const float *)m->lnb.p; ga.packed = wq.packed; ga.scales = wq.scales; ga.bias = wq.bias; ga.y = qkv;
+        ga.x = hid; ga.packed = wq.packed; ga.scales = wq.scales; ga.bias = wq.bias; ga.y = qkv;
+        ga.ln_gamma = b.ln1_g; ga.ln_beta = b.ln1_b; ga.ln_eps = eps;
         ga.M = R; ga.N = 3 * d; ga.K = d; ga.group = g; ga.flags = 0;
         ga.kcache = kc; ga.vcache = vc; ga.pos_dev = m->pos_dev; ga.n_heads = H; ga.n_positions = P;
+        if (!agpu_int4_skinny_supported(ga)) {
+            if ((rc = agpu_layer_norm_impl(ctx, hid, b.ln1_g, b.ln1_b, (float *)m->lnb.p, R, d, eps)) != AGPU_OK) return rc;
+            ga.x = (const float *)m->lnb.p;
+            ga.ln_gamma = ga.ln_beta = nullptr;
+        }
         rc = agpu_int4_skinny_supported(ga) ? agpu_int4_skinny_launch(ctx, ga) : agpu_int4_gemv_launch(ctx, ga);
         if (rc != AGPU_OK) return rc;
     } else {

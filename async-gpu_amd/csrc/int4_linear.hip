@@ -228,7 +228,10 @@ int32_t agpu_ln_int4_linear_kv(agpu_ctx *ctx, const float *x, const float *gamma
     const bool literal = (flags & AGPU_EPI_FORCE_LITERAL) || (group % 8 != 0 && M <= 16);
     const uint32_t epi = flags & (AGPU_EPI_GELU_TANH | AGPU_EPI_GELU_QUICK);
     const float *xin = x;
-    if (gamma && (literal || M > 16 || !agpu_int4_gemv_can_fuse_ln(M, K))) {
+    const bool skinny_ln = gamma && !literal && !(flags & AGPU_EPI_FORCE_FP32_GEMV) && group % 32 == 0 && K % 32 == 0 && N % 4 == 0 &&
+                           agpu_int4_skinny_can_fuse_ln(M, N, K) &&
+                           (((uintptr_t)packed | (uintptr_t)scales | (uintptr_t)x | (uintptr_t)gamma | (uintptr_t)beta) % 16) == 0;
+    if (gamma && !skinny_ln && (literal || M > 16 || !agpu_int4_gemv_can_fuse_ln(M, K))) {
         // LayerNorm into the workspace tail, then the plain kernels.
         const size_t need = (size_t)M * K * sizeof(float);
         if (need > ctx->ws_bytes / 2)

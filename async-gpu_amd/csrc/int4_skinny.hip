@@ -1,40 +1,107 @@
-// Decode Linear for 4 < M <= 16 rows (batched decode) on fp32 MFMA, gfx950.
+// Decode Linear for 4 < M <= 16 rows (batched decode) on the bf16 matrix cores of gfx950, at fp32 accuracy.
 //
-// With several rows the per-nibble work of the VALU GEMV grows with M; here every nibble is
-// converted once (v_cvt_f32_ubyteN) and v_mfma_f32_16x16x4_f32 applies it to all 16 rows.
-// Lane mapping is the decode GEMV's: 4 row slots x 16 column groups of 4 columns, one
-// global_load_dwordx4 per lane per trip (4 packed rows = 32 k = one scale group when group % 32 == 0).
-//   MFMA 16x16x4: lane l supplies A[i = l%16][k = l/16] and B[k = l/16][j = l%16];
+// An fp32 x is the exact sum of three bf16 numbers (x = hi + mid + lo, each the leading 8 bits of what the previous ones
+// left), and 16 + nibble is a bf16 number whose bit pattern is 0x4180 | nibble << 3, so a packed word becomes the four
+// registers of a B operand with 8 instructions and no conversion.  Per trip (32 k = one scale group or a part of one):
+//     u[row][col] = sum_k x[row][k] * (16 + n[k][col])  -  24 * sum_k x[row][k]   =   sum_k x[row][k] * (n[k][col] - 8)
+// with every product exact; the second term is three MFMAs of its own against the constant -24 (per trip, not per
+// column), whose result is the accumulator the column MFMAs start from, so only the additions inside the matrix core
+// round.  Then acc += scale * u in fp32, as the reference's w = q * scale, y += x * w up to the order of the roundings.
+//   v_mfma_f32_16x16x32_bf16: lane l supplies A[row l%16][k 8*(l/16) .. +7] and B[k 8*(l/16) .. +7][col l%16];
 //   register r of the result holds D[4*(l/16) + r][l%16].
-// For column c of the lane's four and nibble s of its word, the MFMA k index is the row slot:
-//   A = x[row = l%16][8*(4t + rs) + s],  B = (float)nibble_s(word[c]),  8 steps per trip and column,
-// so D_c = sum over the trip's 32 k of x*nibble for rows 0..15 and columns 4*cg + c.  The trip's
-// contribution is scale[c] * (D_c - 8*sum_k x), with 8*sum_k x per (row, trip) precomputed in LDS.
-// Waves take trips round-robin; cross-wave and split-K reductions are those of the decode GEMV
-// (LDS in wave order, then write-through partials + ticket, summed in split order).
+// Lane (rs = l/16, cg = l%16) loads packed row 4t + rs of trip t for CPL = 4 or 2 adjacent columns (one 16- or 8-byte
+// load); MFMA c of the trip works on the columns {CPL cg + c}.  The k order inside a register set is (0,4,1,5,2,6,3,7),
+// that of the nibble pairs a mask leaves in the two halves of a register; the x pieces are staged in LDS in the same order.
+//
+// Work decomposition: a workgroup owns a tile of 64 columns (32 while that still leaves every workgroup a CU of its
+// own) and up to 52 trips: K <= 1664 (every GPT-2 width) is one workgroup per tile, no split, and the workgroup may then
+// normalise the rows itself (LayerNorm fused: mean and variance of the whole rows in registers, one or two rows per
+// wave, while the weights are on their way).  Longer K is split over gridDim.y workgroups: write-through partial sums +
+// ticket, summed in split order by the last workgroup.  Waves take trips round-robin and meet in LDS in wave order.
+// In-kernel time stamps (K = 1600, N = 1600, 16 rows, 25 workgroups of 64 columns): pieces staged 2.7 us after the start
+// (1.6 us until the first wave is done), MFMAs 2.4 us (750 per workgroup), reduction and stores 0.8 us; with 32 columns
+// per workgroup the MFMAs take half of that.
 #include "linear_common.h"
+
+#include <atomic>
 
 namespace {
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int SK_MAX_TRIPS = 52;  // trips of a workgroup at most: three piece planes of 16 rows in 160 KiB of LDS
+
+#ifdef AGPU_SK_TRACE
+// Debug builds: wall-clock stamps (10 ns ticks) of thread 0 of the first workgroups, read back by agpu_dev_skinny_trace.
+__device__ unsigned long long sk_trace[8][8];
+#define SK_STAMP(slot)                                                                                        \
+    do {                                                                                                      \
+        if (threadIdx.x == 0 && blockIdx.x + gridDim.x * blockIdx.y < 8)                                      \
+            sk_trace[blockIdx.x + gridDim.x * blockIdx.y][slot] = wall_clock64();                             \
+    } while (0)
+#else
+#define SK_STAMP(slot) \
+    do {               \
+    } while (0)
+#endif
 
 struct SkinnyParams {
     GemvArgs a;
-    int trips_per_split;  // 4-row trips per workgroup, at most 2 per wave
-    int xs_stride;        // floats between rows of the staged x (padded)
+    int trips_per_split;  // 32-k trips per workgroup
+    int row_bytes;        // bytes between the rows of a staged piece plane (padded)
     float *partial;
     unsigned int *counters;
 };
 
-// One workgroup = one tile of 64 columns x one K split.  Every wave owns at most two trips and issues
-// their weight and scale loads before x is staged, so a workgroup pays the memory latency once.
-// LDS: xs [16][xs_stride] | xsum [trips_per_split][16]; after the MFMA loop the same memory holds
+// the leading 16 bits of two floats as one register: a in the low half
+__device__ __forceinline__ uint32_t sk_pack_top(float a, float b) {
+    return __builtin_amdgcn_perm(__float_as_uint(b), __float_as_uint(a), 0x07060302u);
+}
+__device__ __forceinline__ float sk_top_bits(float v) { return __uint_as_float(__float_as_uint(v) & 0xffff0000u); }
+
+// 8 nibbles of one column -> the bf16 numbers 16 + n, pairs (0,4) (1,5) (2,6) (3,7)
+__device__ __forceinline__ bf16x8 sk_nibbles_plus16(uint32_t w) {
+    constexpr uint32_t M = 0x00780078u, C = 0x41804180u;
+    const uint4 v = make_uint4(((w << 3) & M) | C, ((w >> 1) & M) | C, ((w >> 5) & M) | C, ((w >> 9) & M) | C);
+    return __builtin_bit_cast(bf16x8, v);
+}
+
+// 8 consecutive k of one row -> the three piece planes, in the k order of the B operand
+__device__ __forceinline__ void sk_store_pieces(unsigned char *dst, size_t plane, const float (&v)[8]) {
+    float r1[8], r2[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        r1[e] = v[e] - sk_top_bits(v[e]);    // exact: what the leading 8 bits leave
+        r2[e] = r1[e] - sk_top_bits(r1[e]);  // exact, at most 8 significant bits
+    }
+    *reinterpret_cast<uint4 *>(dst) =
+        make_uint4(sk_pack_top(r2[0], r2[4]), sk_pack_top(r2[1], r2[5]), sk_pack_top(r2[2], r2[6]), sk_pack_top(r2[3], r2[7]));
+    *reinterpret_cast<uint4 *>(dst + plane) =
+        make_uint4(sk_pack_top(r1[0], r1[4]), sk_pack_top(r1[1], r1[5]), sk_pack_top(r1[2], r1[6]), sk_pack_top(r1[3], r1[7]));
+    *reinterpret_cast<uint4 *>(dst + 2 * plane) =
+        make_uint4(sk_pack_top(v[0], v[4]), sk_pack_top(v[1], v[5]), sk_pack_top(v[2], v[6]), sk_pack_top(v[3], v[7]));
+}
+
+// One workgroup = one tile of 64 columns x one K split.  Every wave issues the weight and scale loads of its trips
+// before anything else, so a workgroup pays the memory latency once.
+// LDS: three planes [16][row_bytes] of bf16 pieces (lo, mid, hi); after the MFMA loop the same memory holds
 // red [W][16][64], the per-wave results.
-__global__ __launch_bounds__(512) void int4_skinny_mfma_kernel(const SkinnyParams p) {
-    extern __shared__ __align__(16) float smem[];
+// WHOLE: the workgroup covers all of K (K <= 32 SK_MAX_TRIPS, no split): a wave stages whole rows from registers, with
+// LN after taking their mean and variance there (two passes, nn/cpu_ref.rs:38-47).  Otherwise K is split over
+// gridDim.y workgroups and every thread stages 8-element items of the slice.
+// NW waves at most; a wave holds up to TPW = ceil(SK_MAX_TRIPS / NW) trips.  The normalising variant runs with 8 waves: it
+// needs more registers than a workgroup of 16 waves leaves a lane.
+// CPL columns per lane: a tile is 16 CPL columns wide (64, or 32 when that still leaves the chip room for every workgroup).
+template <bool WHOLE, bool LN, int NW, int CPL>
+__global__ __launch_bounds__(64 * NW) void int4_skinny_bf16_kernel(const SkinnyParams p) {
+    static_assert(WHOLE || !LN, "rows are normalised by the workgroup that holds all of them");
+    static_assert(CPL == 2 || CPL == 4, "a lane loads 8 or 16 bytes of a packed row");
+    constexpr int TPW = (SK_MAX_TRIPS + NW - 1) / NW;
+    extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int s_last;
     const GemvArgs &a = p.a;
-    constexpr int COLS = 64, MT = 16;
+    constexpr int COLS = 16 * CPL, MT = 16;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6, T = blockDim.x;
     const int rs = lane >> 4, cg = lane & 15;
     const int tile = blockIdx.x, ksplit = gridDim.y, split = blockIdx.y;
@@ -42,91 +109,197 @@ __global__ __launch_bounds__(512) void int4_skinny_mfma_kernel(const SkinnyParam
     const int t0 = split * p.trips_per_split;
     const int t1 = min(trips_total, t0 + p.trips_per_split);
     const int k0 = t0 * 32, kslice = (t1 - t0) * 32;
-    float *xs = smem;
-    float *xsum = smem + MT * p.xs_stride;
-    float *red = smem;
+    const size_t plane = (size_t)MT * p.row_bytes;
+    float *red = reinterpret_cast<float *>(smem);
     constexpr int n_out = MT * COLS;
 
-    const int c0 = tile * COLS + cg * 4;
+    SK_STAMP(0);
+    const int c0 = tile * COLS + cg * CPL;
     const bool col_ok = c0 < a.N;
-    const int trip[2] = {t0 + wave, t0 + wave + W};
-    uint4 w4[2];
-    float4 sc4[2];
+    uint32_t w4[TPW][CPL];
+    float sc4[TPW][CPL];
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-        w4[u] = make_uint4(0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u);
-        sc4[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (col_ok && trip[u] < t1) {
-            w4[u] = *reinterpret_cast<const uint4 *>(a.packed + (size_t)(4 * trip[u] + rs) * a.N + c0);
-            sc4[u] = *reinterpret_cast<const float4 *>(a.scales + (size_t)((trip[u] * 32) / a.group) * a.N + c0);
+    for (int u = 0; u < TPW; ++u) {
+        const int trip = t0 + wave + u * W;
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) {
+            w4[u][c] = 0u;
+            sc4[u][c] = 0.0f;  // absent columns and trips: whatever the products are, they count zero times
+        }
+        if (col_ok && trip < t1) {
+            const uint32_t *wp = a.packed + (size_t)(4 * trip + rs) * a.N + c0;
+            const float *sp = a.scales + (size_t)((trip * 32) / a.group) * a.N + c0;
+            if (CPL == 4) {
+                const uint4 wv = *reinterpret_cast<const uint4 *>(wp);
+                const float4 sv = *reinterpret_cast<const float4 *>(sp);
+                w4[u][0] = wv.x; w4[u][1] = wv.y; w4[u][CPL - 2] = wv.z; w4[u][CPL - 1] = wv.w;
+                sc4[u][0] = sv.x; sc4[u][1] = sv.y; sc4[u][CPL - 2] = sv.z; sc4[u][CPL - 1] = sv.w;
+            } else {
+                const uint2 wv = *reinterpret_cast<const uint2 *>(wp);
+                const float2 sv = *reinterpret_cast<const float2 *>(sp);
+                w4[u][0] = wv.x; w4[u][1] = wv.y;
+                sc4[u][0] = sv.x; sc4[u][1] = sv.y;
+            }
+        }
+    }
+    // epilogue operands of this thread's first output, requested early (the residual may be the output itself: nothing
+    // writes an output element before the thread that read it here does)
+    float e_bias = 0.0f, e_res = 0.0f;
+    if (tid < n_out) {
+        const int m = tid / COLS, n = tile * COLS + (tid - m * COLS);
+        if (m < a.M && n < a.N) {
+            if (a.bias) e_bias = a.bias[n];
+            if (a.residual) e_res = a.residual[(size_t)m * a.N + n];
         }
     }
 
-    // ---- stage x as float4 (rows beyond M are zero), four loads in flight per thread ----
-    const int q4 = kslice >> 2, total4 = MT * q4;
-    for (int base = tid; base < total4; base += 4 * T) {
-        float4 v[4];
+    if (WHOLE) {
+        // ---- a wave stages whole rows: lane l holds the blocks of 8 elements l, l + 64, ... (K <= 2048) ----
+        const int n8 = a.K >> 3;
+        constexpr int RPW = MT / NW;  // rows of a wave whose loads are in flight together
+        for (int mb = wave; mb < MT; mb += RPW * W) {  // rows mb, mb + W, ...; rows beyond M are zero
+            float v[RPW][4][8];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int i = base + u * T;
-            const int m = i / q4, j = i - m * q4;
-            v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (i < total4 && m < a.M) v[u] = *reinterpret_cast<const float4 *>(a.x + (size_t)m * a.K + k0 + 4 * j);
+            for (int h = 0; h < RPW; ++h) {
+                const int m = mb + h * W;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int blk = lane + 64 * i;
+                    float4 x0 = make_float4(0.f, 0.f, 0.f, 0.f), x1 = x0;
+                    if (m < a.M && blk < n8) {
+                        const float *src = a.x + (size_t)m * a.K + 8 * blk;
+                        x0 = *reinterpret_cast<const float4 *>(src);
+                        x1 = *reinterpret_cast<const float4 *>(src + 4);
+                    }
+                    v[h][i][0] = x0.x; v[h][i][1] = x0.y; v[h][i][2] = x0.z; v[h][i][3] = x0.w;
+                    v[h][i][4] = x1.x; v[h][i][5] = x1.y; v[h][i][6] = x1.z; v[h][i][7] = x1.w;
+                }
+            }
+            // gamma and beta of the lane's blocks (the same for every row)
+            float4 gb[4][4];
+            auto load_gb = [&](int i, int set) {
+                const int blk = lane + 64 * i;
+                gb[set][0] = gb[set][1] = gb[set][2] = gb[set][3] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (LN && blk < n8) {
+                    gb[set][0] = *reinterpret_cast<const float4 *>(a.ln_gamma + 8 * blk);
+                    gb[set][1] = *reinterpret_cast<const float4 *>(a.ln_gamma + 8 * blk + 4);
+                    gb[set][2] = *reinterpret_cast<const float4 *>(a.ln_beta + 8 * blk);
+                    gb[set][3] = *reinterpret_cast<const float4 *>(a.ln_beta + 8 * blk + 4);
+                }
+            };
+            float mean[RPW], rstd[RPW];
+            if (LN) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) load_gb(i, i);
+#pragma unroll
+                for (int h = 0; h < RPW; ++h) {
+                    float sm = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        sm += ((v[h][i][0] + v[h][i][1]) + (v[h][i][2] + v[h][i][3])) + ((v[h][i][4] + v[h][i][5]) + (v[h][i][6] + v[h][i][7]));
+                    mean[h] = wave_sum(sm) / (float)a.K;
+                    float q = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (lane + 64 * i < n8) {
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) {
+                                const float df = v[h][i][e] - mean[h];
+                                q = fmaf(df, df, q);
+                            }
+                        }
+                    rstd[h] = 1.0f / sqrtf(wave_sum(q) / (float)a.K + a.ln_eps);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int blk = lane + 64 * i;
+                float g[8], be[8];
+                if (LN) {
+                    const float4 *q4 = gb[i];
+                    g[0] = q4[0].x; g[1] = q4[0].y; g[2] = q4[0].z; g[3] = q4[0].w; g[4] = q4[1].x; g[5] = q4[1].y; g[6] = q4[1].z; g[7] = q4[1].w;
+                    be[0] = q4[2].x; be[1] = q4[2].y; be[2] = q4[2].z; be[3] = q4[2].w; be[4] = q4[3].x; be[5] = q4[3].y; be[6] = q4[3].z; be[7] = q4[3].w;
+                }
+#pragma unroll
+                for (int h = 0; h < RPW; ++h) {
+                    const int m = mb + h * W;
+                    if (m >= MT) break;  // wave-uniform
+                    if (LN) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) v[h][i][e] = m < a.M ? (v[h][i][e] - mean[h]) * rstd[h] * g[e] + be[e] : 0.0f;
+                    }
+                    if (blk < n8) sk_store_pieces(smem + (size_t)m * p.row_bytes + 16 * blk, plane, v[h][i]);
+                }
+            }
         }
+    } else {
+        // ---- every thread stages items of 8 consecutive k of one row: item i = (row i % 16, block i / 16), so that four
+        // lanes of a wave read 128 contiguous bytes of a row ----
+        const int total = MT * (kslice >> 3);
+        for (int base = tid; base < total; base += 4 * T) {
+            float4 xa[4][2];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int i = base + u * T;
-            const int m = i / q4, j = i - m * q4;
-            if (i < total4) *reinterpret_cast<float4 *>(xs + m * p.xs_stride + 4 * j) = v[u];
+            for (int h = 0; h < 4; ++h) {
+                const int i = base + h * T;
+                const int m = i & 15, j = i >> 4;
+                xa[h][0] = xa[h][1] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (i < total && m < a.M) {
+                    const float *src = a.x + (size_t)m * a.K + k0 + 8 * j;
+                    xa[h][0] = *reinterpret_cast<const float4 *>(src);
+                    xa[h][1] = *reinterpret_cast<const float4 *>(src + 4);
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < 4; ++h) {
+                const int i = base + h * T;
+                if (i >= total) break;
+                const int m = i & 15, j = i >> 4;
+                const float v[8] = {xa[h][0].x, xa[h][0].y, xa[h][0].z, xa[h][0].w, xa[h][1].x, xa[h][1].y, xa[h][1].z, xa[h][1].w};
+                sk_store_pieces(smem + (size_t)m * p.row_bytes + 16 * j, plane, v);
+            }
         }
     }
+    SK_STAMP(1);
     __syncthreads();
-    for (int i = tid; i < MT * (t1 - t0); i += T) {
-        const int t = i / MT, m = i - t * MT;
-        const float *src = xs + m * p.xs_stride + t * 32;
-        float s = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 32; j += 4) {
-            const float4 v = *reinterpret_cast<const float4 *>(src + j);
-            s += (v.x + v.y) + (v.z + v.w);
-        }
-        xsum[t * MT + m] = 8.0f * s;
-    }
-    __syncthreads();
+    SK_STAMP(2);
 
-    floatx4 acc[4];
+    floatx4 acc[CPL];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) acc[c] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < CPL; ++c) acc[c] = floatx4{0.f, 0.f, 0.f, 0.f};
+    const uint4 m24 = make_uint4(0xC1C0C1C0u, 0xC1C0C1C0u, 0xC1C0C1C0u, 0xC1C0C1C0u);  // -24 eight times
+    const bf16x8 b24 = __builtin_bit_cast(bf16x8, m24);
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-        if (trip[u] >= t1) break;  // wave-uniform
-        const int tl = trip[u] - t0;
-        const float *xr = xs + (lane & 15) * p.xs_stride + (tl * 4 + rs) * 8;
-        const float4 xa = *reinterpret_cast<const float4 *>(xr);
-        const float4 xb = *reinterpret_cast<const float4 *>(xr + 4);
-        const float xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
-        const float4 xs8 = *reinterpret_cast<const float4 *>(xsum + tl * MT + 4 * rs);
-        const uint32_t w[4] = {w4[u].x, w4[u].y, w4[u].z, w4[u].w};
-        const float sc[4] = {sc4[u].x, sc4[u].y, sc4[u].z, sc4[u].w};
+    for (int u = 0; u < TPW; ++u) {
+        const int tl = wave + u * W;
+        if (t0 + tl >= t1) break;  // wave-uniform
+        const unsigned char *ap = smem + (size_t)(lane & 15) * p.row_bytes + 64 * tl + 16 * rs;
+        const bf16x8 a_lo = *reinterpret_cast<const bf16x8 *>(ap);
+        const bf16x8 a_mid = *reinterpret_cast<const bf16x8 *>(ap + plane);
+        const bf16x8 a_hi = *reinterpret_cast<const bf16x8 *>(ap + 2 * plane);
+        floatx4 z = {0.f, 0.f, 0.f, 0.f};
+        z = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, b24, z, 0, 0, 0);
+        z = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_mid, b24, z, 0, 0, 0);
+        z = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, b24, z, 0, 0, 0);  // -24 * sum of the trip's x, rows 4 rs .. + 3
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            float nf[8];
-            unpack_u8(w[c], nf);
-            floatx4 d = {0.f, 0.f, 0.f, 0.f};
+        for (int c = 0; c < CPL; ++c) {
+            const bf16x8 b = sk_nibbles_plus16(w4[u][c]);
+            floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, b, z, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_mid, b, d, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, b, d, 0, 0, 0);
 #pragma unroll
-            for (int s = 0; s < 8; ++s) d = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[s], nf[s], d, 0, 0, 0);
-            acc[c][0] = fmaf(sc[c], d[0] - xs8.x, acc[c][0]);
-            acc[c][1] = fmaf(sc[c], d[1] - xs8.y, acc[c][1]);
-            acc[c][2] = fmaf(sc[c], d[2] - xs8.z, acc[c][2]);
-            acc[c][3] = fmaf(sc[c], d[3] - xs8.w, acc[c][3]);
+            for (int r = 0; r < 4; ++r) acc[c][r] = fmaf(sc4[u][c], d[r], acc[c][r]);
         }
     }
-    // acc[c][r] is the wave's partial of y[row 4*rs + r][column 4*cg + c]
-    __syncthreads();  // every wave is done with xs / xsum: reuse the memory
+    // acc[c][r] is the wave's partial of y[row 4*rs + r][column CPL*cg + c]
+    SK_STAMP(3);
+    __syncthreads();  // every wave is done with the pieces: reuse the memory
+    SK_STAMP(4);
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-        *reinterpret_cast<float4 *>(red + (wave * MT + 4 * rs + r) * COLS + cg * 4) =
-            make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]);
+    for (int r = 0; r < 4; ++r) {
+        float *dst = red + (wave * MT + 4 * rs + r) * COLS + cg * CPL;
+        if (CPL == 4) *reinterpret_cast<float4 *>(dst) = make_float4(acc[0][r], acc[1][r], acc[CPL - 2][r], acc[CPL - 1][r]);
+        else *reinterpret_cast<float2 *>(dst) = make_float2(acc[0][r], acc[1][r]);
+    }
     __syncthreads();
     for (int i = tid; i < n_out; i += T) {
         const int m = i / COLS, n = tile * COLS + (i - m * COLS);
@@ -134,26 +307,32 @@ __global__ __launch_bounds__(512) void int4_skinny_mfma_kernel(const SkinnyParam
             float v = 0.0f;
             for (int w2 = 0; w2 < W; ++w2) v += red[w2 * n_out + i];
             if (ksplit == 1) {
-                finish_output(a, v, a.bias ? a.bias[n] : 0.0f, a.residual ? a.residual[(size_t)m * a.N + n] : 0.0f, m, n);
+                const bool early = i == tid;  // this thread's first output: its operands are here already
+                finish_output(a, v, early ? e_bias : (a.bias ? a.bias[n] : 0.0f),
+                              early ? e_res : (a.residual ? a.residual[(size_t)m * a.N + n] : 0.0f), m, n);
             } else {
                 __hip_atomic_store(&p.partial[((size_t)split * a.M + m) * a.N + n], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
     }
+    SK_STAMP(5);
     if (ksplit == 1) return;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    SK_STAMP(6);
     if (tid == 0) {
         const unsigned int tk = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_last = (tk == (unsigned int)(ksplit - 1));
     }
     __syncthreads();
+    SK_STAMP(7);
     if (!s_last) return;  // uniform over the workgroup
-    for (int i = tid; i < n_out; i += T) {
+    for (int i = tid; i < n_out; i += T) {  // one round with 16 waves
         const int m = i / COLS, n = tile * COLS + (i - m * COLS);
         if (m < a.M && n < a.N) {
-            const float bias = a.bias ? a.bias[n] : 0.0f;
-            const float res = a.residual ? a.residual[(size_t)m * a.N + n] : 0.0f;
+            const bool early = i == tid;
+            const float bias = early ? e_bias : (a.bias ? a.bias[n] : 0.0f);
+            const float res = early ? e_res : (a.residual ? a.residual[(size_t)m * a.N + n] : 0.0f);
             const float *src = p.partial + (size_t)m * a.N + n;
             const size_t stride = (size_t)a.M * a.N;
             float v = 0.0f;
@@ -176,31 +355,66 @@ __global__ __launch_bounds__(512) void int4_skinny_mfma_kernel(const SkinnyParam
 
 }  // namespace
 
+bool agpu_int4_skinny_can_fuse_ln(int M, int N, int K) {
+    // the workgroup of a column tile holds whole rows and normalises them itself; with very many tiles a launch that
+    // normalises once is cheaper than every tile reading all the rows
+    return M > 4 && M <= 16 && K % 32 == 0 && K <= 32 * SK_MAX_TRIPS && N <= 16384;
+}
+
 bool agpu_int4_skinny_supported(const GemvArgs &a) {
-    return a.M > 4 && a.M <= 16 && !a.ln_gamma && a.group % 32 == 0 && a.group <= 512 && a.K % 32 == 0 && a.N % 4 == 0 &&
+    if (a.ln_gamma && (!agpu_int4_skinny_can_fuse_ln(a.M, a.N, a.K) || (((uintptr_t)a.ln_gamma | (uintptr_t)a.ln_beta) % 16) != 0)) return false;
+    return a.M > 4 && a.M <= 16 && a.group % 32 == 0 && a.group <= 512 && a.K % 32 == 0 && a.N % 4 == 0 &&
            (((uintptr_t)a.packed | (uintptr_t)a.scales | (uintptr_t)a.x) % 16 == 0);
 }
+
+namespace {
+template <bool WHOLE, bool LN, int NW, int CPL>
+int32_t skinny_go(agpu_ctx *ctx, const SkinnyParams &p, dim3 grid, size_t lds) {
+    const int W = p.trips_per_split < NW ? p.trips_per_split : NW;
+    static std::atomic<unsigned long long> lds_raised{0};  // one bit per device: the attribute belongs to the device's code object
+    const unsigned long long dev_bit = 1ull << (ctx->device & 63);
+    if (lds > 48 * 1024 && !(lds_raised.load(std::memory_order_relaxed) & dev_bit)) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(int4_skinny_bf16_kernel<WHOLE, LN, NW, CPL>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 3 * 16 * (SK_MAX_TRIPS * 64 + 16));
+        if (e != hipSuccess) return agpu_hip(ctx, e, "hipFuncSetAttribute");
+        lds_raised.fetch_or(dev_bit, std::memory_order_relaxed);
+    }
+    hipLaunchKernelGGL((int4_skinny_bf16_kernel<WHOLE, LN, NW, CPL>), grid, dim3(64 * W), lds, ctx->stream, p);
+    return AGPU_LAUNCH_CHECK(ctx, "int4_skinny_bf16_kernel");
+}
+}  // namespace
 
 int32_t agpu_int4_skinny_launch(agpu_ctx *ctx, const GemvArgs &a) {
     SkinnyParams p{};
     p.a = a;
     const int trips_total = a.K / 32;
-    const int tpg = a.group / 32;           // trips per scale group; a split covers whole groups
-    const int tps_max = 16 / tpg * tpg;     // at most 2 trips per wave, 8 waves
+    const int tpg = a.group / 32;  // trips per scale group; a split covers whole groups
+    const int tps_max = SK_MAX_TRIPS / tpg * tpg;
     const int ksplit = ceil_div(trips_total, tps_max);
     const int tps = ceil_div(ceil_div(trips_total, ksplit), tpg) * tpg;
-    if ((size_t)ksplit * a.M * a.N * sizeof(float) > ctx->ws_bytes / 2)
+    if (ksplit > 1 && (size_t)ksplit * a.M * a.N * sizeof(float) > ctx->ws_bytes / 2)
         return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_skinny: split-K partials exceed the workspace (M=%d N=%d K=%d)", a.M, a.N, a.K);
-    const int col_blocks = ceil_div(a.N, 64);
+    // tiles of 32 columns while every workgroup still has a CU of its own: half the MFMAs per workgroup
+    const bool narrow = ceil_div(a.N, 32) * ksplit <= ctx->num_cus;
+    const int cols = narrow ? 32 : 64;
+    const int col_blocks = ceil_div(a.N, cols);
     if (col_blocks > ctx->n_counters) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_skinny: N=%d too large", a.N);
+    if (a.ln_gamma && ksplit > 1) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "int4_skinny: LayerNorm needs K <= %d", 32 * SK_MAX_TRIPS);
     p.trips_per_split = tps;
-    p.xs_stride = tps * 32 + 4;
-    const int W = tps < 8 ? tps : 8;
-    const size_t stage = sizeof(float) * ((size_t)16 * p.xs_stride + (size_t)tps * 16);
-    const size_t red = sizeof(float) * (size_t)W * 16 * 64;
+    p.row_bytes = tps * 64 + 16;
+    const size_t stage = (size_t)3 * 16 * p.row_bytes;
+    const size_t red = sizeof(float) * (size_t)(tps < 16 ? tps : 16) * 16 * cols;
     const size_t lds = stage > red ? stage : red;
     p.partial = reinterpret_cast<float *>(ctx->workspace);
     p.counters = ctx->counters;
-    hipLaunchKernelGGL(int4_skinny_mfma_kernel, dim3(col_blocks, ksplit), dim3(64 * W), lds, ctx->stream, p);
-    return AGPU_LAUNCH_CHECK(ctx, "int4_skinny_mfma_kernel");
+    const dim3 grid(col_blocks, ksplit);
+    if (a.ln_gamma) return narrow ? skinny_go<true, true, 8, 2>(ctx, p, grid, lds) : skinny_go<true, true, 8, 4>(ctx, p, grid, lds);
+    if (ksplit == 1) return narrow ? skinny_go<true, false, 16, 2>(ctx, p, grid, lds) : skinny_go<true, false, 16, 4>(ctx, p, grid, lds);
+    return narrow ? skinny_go<false, false, 16, 2>(ctx, p, grid, lds) : skinny_go<false, false, 16, 4>(ctx, p, grid, lds);
 }
+
+#ifdef AGPU_SK_TRACE
+AGPU_EXPORT int32_t agpu_dev_skinny_trace(unsigned long long *out_host) {
+    return (int32_t)hipMemcpyFromSymbol(out_host, HIP_SYMBOL(sk_trace), sizeof(unsigned long long) * 64);
+}
+#endif

@@ -98,7 +98,9 @@ int32_t agpu_ln_int4_linear_kv(agpu_ctx *ctx, const float *x, const float *gamma
                                const uint32_t *packed, const float *scales, const float *bias, const float *residual, float *y,
                                int32_t M, int32_t N, int32_t K, int32_t group, uint32_t flags, const KvScatter *kv, bool *kv_done);
 // MFMA variant for 4 < M <= 16 (needs group % 32 == 0, K % 32 == 0, N % 4 == 0, 16-byte aligned weights).
+// With a.ln_gamma the kernel normalises the rows itself; agpu_int4_skinny_can_fuse_ln says for which shapes.
 bool agpu_int4_skinny_supported(const GemvArgs &a);
+bool agpu_int4_skinny_can_fuse_ln(int M, int N, int K);
 int32_t agpu_int4_skinny_launch(agpu_ctx *ctx, const GemvArgs &a);
 // Whether the GEMV can apply LayerNorm itself for this shape (otherwise normalise first).
 bool agpu_int4_gemv_can_fuse_ln(int M, int K);

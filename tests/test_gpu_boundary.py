@@ -48,17 +48,17 @@ def test_workspace_query_and_caller_provided_scratch(orc, agpu, dev):
     for (M, K, N), (bufs, ref, first) in base.items():
         got = _run_linear(ctx, bufs, M, K, N)
         assert np.abs(got - ref).max() <= 1e-4, (M, K, N)
-    # 16 rows x 50432 columns split four ways needs 12.9 MB of partial sums: refused, nothing launched
-    w, bufs, ref = _linear_case(orc, agpu, ctx, 16, 1600, 50432, 8)
+    # 16 rows x 4800 columns with K = 6400 split four ways needs 1.2 MB of partial sums: refused, nothing launched
+    w, bufs, ref = _linear_case(orc, agpu, ctx, 16, 6400, 4800, 8)
     with pytest.raises(_lib.AgpuError) as e:
-        _run_linear(ctx, bufs, 16, 1600, 50432)
+        _run_linear(ctx, bufs, 16, 6400, 4800)
     assert e.value.code == _lib.ERR_WORKSPACE
     with pytest.raises(_lib.AgpuError) as e:
         ctx.call("agpu_ctx_set_workspace", mine, 4096)
     assert e.value.code == _lib.ERR_WORKSPACE
     ctx.call("agpu_ctx_set_workspace", None, 0)
     assert lib.agpu_ctx_workspace_bytes(ctx.handle) == 96 << 20
-    got = _run_linear(ctx, bufs, 16, 1600, 50432)
+    got = _run_linear(ctx, bufs, 16, 6400, 4800)
     assert np.abs(got - ref).max() <= 1e-4
     for (M, K, N), (b2, ref, first) in base.items():
         assert np.array_equal(_run_linear(ctx, b2, M, K, N), first)  # same scratch size, same launch shape, same bits

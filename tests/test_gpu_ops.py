@@ -133,6 +133,25 @@ def test_batched_decode_shapes(agpu, orc, dev, M, K, N, g):
     assert np.all(np.abs(y32 - ref) <= 3e-6 * bound + 1e-6 * np.abs(ref) + 1e-6)
 
 
+@pytest.mark.parametrize("M", [5, 11, 16])
+@pytest.mark.parametrize("K,N,g", [(1600, 4800, 32), (768, 3072, 64), (2048, 260, 32), (3072, 768, 32), (1600, 50257 // 4 * 4, 32)])
+def test_batched_decode_layer_norm(agpu, orc, dev, M, K, N, g):
+    """LayerNorm in front of the batched decode Linear: normalised by the Linear kernel itself up to K = 2048 and a few
+    thousand columns, by a launch of its own beyond (K = 3072, the LM-head width); rows with different means and sizes."""
+    from async_gpu_amd import ops, workloads
+    rng = np.random.default_rng(M * 17 + K + N + g)
+    packed, scales, bias = workloads.random_int4_linear(rng, K, N, g, bias=True)
+    x = (rng.standard_normal((M, K)) * np.exp(rng.uniform(-2, 2, (M, 1))) + rng.uniform(-3, 3, (M, 1))).astype(np.float32)
+    gamma = (1 + 0.2 * rng.standard_normal(K)).astype(np.float32)
+    beta = (0.2 * rng.standard_normal(K)).astype(np.float32)
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    y = ops.int4_linear(to_dev(x, dev), to_dev(packed, dev), to_dev(scales, dev), bias=to_dev(bias, dev), residual=to_dev(res, dev),
+                        group=g, ln=(to_dev(gamma, dev), to_dev(beta, dev), 1e-5)).cpu().numpy()
+    xn = orc.layer_norm(x, gamma, beta, 1e-5)
+    ref = orc.int4_gemm_f64(xn, packed, scales, g, bias=bias) + res
+    assert np.abs(y - ref).max() <= TOL_LINEAR
+
+
 def test_batched_decode_special_rows(agpu, orc, dev):
     """A NaN or infinity poisons its own row only; an all-zero row gives the bias; two calls give the same bits."""
     from async_gpu_amd import ops, workloads

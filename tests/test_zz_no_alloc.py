@@ -61,8 +61,9 @@ def test_static_scratch_entry_point_matches_the_allocating_one(orc, agpu, dev):
     d, _ = _case(orc, ctx, 32, 64, 50432, 39, False)
     rc = fn(0, stream, d["x"], d["p"], d["s"], None, None, d["y1"], 32, 50432, 64, 32, 0, err, 256)
     assert rc == _lib.ERR_WORKSPACE and b"4 MiB" in err.value
-    d, _ = _case(orc, ctx, 16, 1600, 50432, 40, False)
-    rc = fn(0, stream, d["x"], d["p"], d["s"], None, None, d["y1"], 16, 50432, 1600, 32, 0, err, 256)
+    # within the entry point's own limits, but the K split of this shape needs 5.1 MB of partial sums
+    d, _ = _case(orc, ctx, 16, 6400, 20000, 40, False)
+    rc = fn(0, stream, d["x"], d["p"], d["s"], None, None, d["y1"], 16, 20000, 6400, 32, 0, err, 256)
     assert rc == _lib.ERR_WORKSPACE and len(err.value) > 0
     ctx.sync()
     ctx.close()
