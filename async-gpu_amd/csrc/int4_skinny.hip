@@ -175,8 +175,10 @@ __global__ __launch_bounds__(64 * NW) void int4_skinny_bf16_kernel(const SkinnyP
                     v[h][i][4] = x1.x; v[h][i][5] = x1.y; v[h][i][6] = x1.z; v[h][i][7] = x1.w;
                 }
             }
-            // gamma and beta of the lane's blocks (the same for every row)
-            float4 gb[4][4];
+            // gamma and beta of the lane's blocks (the same for every row); with 16 waves there are registers for three of
+            // the four, the last one is requested once the first is used up
+            constexpr int GBH = NW == 16 ? 2 : 4;
+            float4 gb[GBH][4];
             auto load_gb = [&](int i, int set) {
                 const int blk = lane + 64 * i;
                 gb[set][0] = gb[set][1] = gb[set][2] = gb[set][3] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -190,7 +192,7 @@ __global__ __launch_bounds__(64 * NW) void int4_skinny_bf16_kernel(const SkinnyP
             float mean[RPW], rstd[RPW];
             if (LN) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) load_gb(i, i);
+                for (int i = 0; i < GBH; ++i) load_gb(i, i);
 #pragma unroll
                 for (int h = 0; h < RPW; ++h) {
                     float sm = 0.0f;
@@ -216,7 +218,7 @@ __global__ __launch_bounds__(64 * NW) void int4_skinny_bf16_kernel(const SkinnyP
                 const int blk = lane + 64 * i;
                 float g[8], be[8];
                 if (LN) {
-                    const float4 *q4 = gb[i];
+                    const float4 *q4 = gb[i % GBH];
                     g[0] = q4[0].x; g[1] = q4[0].y; g[2] = q4[0].z; g[3] = q4[0].w; g[4] = q4[1].x; g[5] = q4[1].y; g[6] = q4[1].z; g[7] = q4[1].w;
                     be[0] = q4[2].x; be[1] = q4[2].y; be[2] = q4[2].z; be[3] = q4[2].w; be[4] = q4[3].x; be[5] = q4[3].y; be[6] = q4[3].z; be[7] = q4[3].w;
                 }
@@ -230,6 +232,7 @@ __global__ __launch_bounds__(64 * NW) void int4_skinny_bf16_kernel(const SkinnyP
                     }
                     if (blk < n8) sk_store_pieces(smem + (size_t)m * p.row_bytes + 16 * blk, plane, v[h][i]);
                 }
+                if (LN && i + GBH < 4) load_gb(i + GBH, i);
             }
         }
     } else {
@@ -408,7 +411,7 @@ int32_t agpu_int4_skinny_launch(agpu_ctx *ctx, const GemvArgs &a) {
     p.partial = reinterpret_cast<float *>(ctx->workspace);
     p.counters = ctx->counters;
     const dim3 grid(col_blocks, ksplit);
-    if (a.ln_gamma) return narrow ? skinny_go<true, true, 8, 2>(ctx, p, grid, lds) : skinny_go<true, true, 8, 4>(ctx, p, grid, lds);
+    if (a.ln_gamma) return narrow ? skinny_go<true, true, 16, 2>(ctx, p, grid, lds) : skinny_go<true, true, 8, 4>(ctx, p, grid, lds);
     if (ksplit == 1) return narrow ? skinny_go<true, false, 16, 2>(ctx, p, grid, lds) : skinny_go<true, false, 16, 4>(ctx, p, grid, lds);
     return narrow ? skinny_go<false, false, 16, 2>(ctx, p, grid, lds) : skinny_go<false, false, 16, 4>(ctx, p, grid, lds);
 }
