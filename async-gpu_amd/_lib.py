@@ -60,6 +60,7 @@ SIGNATURES = {
     "agpu_ctx_workspace_bytes": (C.c_size_t, [_vp]),
     "agpu_int4_linear_workspace_bytes": (C.c_size_t, [_i32, _i32, _i32, _i32]),
     "agpu_ctx_set_workspace": (_i32, [_vp, _vp, C.c_size_t]),
+    "agpu_ctx_set_strict_sync": (_i32, [_vp, _i32]),
     "agpu_ctx_test_hold": (_i32, [_vp, _i32]),
     "agpu_ln_int4_linear": (_i32, [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32]),
     "agpu_bench_int4_linear": (_i32, [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32,

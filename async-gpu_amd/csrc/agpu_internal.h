@@ -32,6 +32,7 @@ struct agpu_ctx {
     bool owns_counters = false;
     // launch-shape overrides of the decode GEMV (agpu_int4_gemv_tune); 0 = default
     int tune_target_wgs = 0, tune_max_waves = 0, tune_rows_per_split = 256;
+    int strict_sync = 0;  // agpu_ctx_set_strict_sync: split-K hand-overs with release/acquire fences (verification aid)
     unsigned long long ws_epoch = 0;   // bumped whenever the scratch moves: models drop graphs captured before
     // the one-thread-at-a-time guard: the thread inside a call, and how deep its calls are nested
     std::atomic<uintptr_t> owner{0};
@@ -96,6 +97,25 @@ struct agpu_ctx_guard {
 #define AGPU_LAUNCH_CHECK(ctx, name) agpu_hip((ctx), hipGetLastError(), name)
 
 // ---- device helpers ---------------------------------------------------------------
+
+// Hand-over of partial results between workgroups (split K, split keys, arg-max candidates).  A workgroup writes its
+// partials with relaxed agent-scope stores (write-through on gfx950), calls partials_published, takes a ticket; the
+// workgroup that draws the last ticket reads every partial with relaxed agent-scope loads.  The fast form rests on a
+// property of the hardware: s_waitcnt vmcnt(0) returns for a write-through store only once the store is visible to
+// the whole device.  With `strict` the same steps are also expressed to the memory model, as a release fence before
+// and an acquire fence after an acq_rel ticket; results must be the same bits either way.
+__device__ __forceinline__ void partials_published(int strict) {
+    if (strict) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+__device__ __forceinline__ unsigned int take_ticket(unsigned int *counter, int strict) {
+    if (strict) {
+        const unsigned int t = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        return t;
+    }
+    return __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 // Cross-lane moves as DPP modifiers of ordinary VALU instructions (a few cycles each; a ds_bpermute
 // round trip through the LDS crossbar costs on the order of a hundred).

@@ -23,6 +23,7 @@ struct AttnParams {
     int kv_chunk;
     float *kv_partial;
     unsigned int *counters;
+    int strict;  // the context's strict_sync
 };
 
 // max_kv_len bounds kv_len for launches that read it from pos_dev (sizes the key split).

@@ -376,10 +376,10 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
             __hip_atomic_store(part + blockIdx.z * 66 + 64, m_all, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(part + blockIdx.z * 66 + 65, l_all, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        partials_published(p.strict);
         unsigned int tk = 0;
         if (lane == 0) {
-            tk = __hip_atomic_fetch_add(&p.counters[row], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            tk = take_ticket(&p.counters[row], p.strict);
             if (tk == (unsigned int)(Z - 1)) __hip_atomic_store(&p.counters[row], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         tk = __builtin_amdgcn_readfirstlane(tk);
@@ -435,6 +435,7 @@ int32_t agpu_attention_launch(agpu_ctx *ctx, const AttnParams &p, int max_kv_len
             pd.kv_chunk = ceil_div(max_kv_len, Z);
             pd.kv_partial = reinterpret_cast<float *>(ctx->workspace);
             pd.counters = ctx->counters;
+            pd.strict = ctx->strict_sync;
             W = ceil_div(pd.kv_chunk, 32);
             W = W > 16 ? 16 : W;
         }

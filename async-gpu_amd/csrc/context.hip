@@ -132,6 +132,12 @@ AGPU_EXPORT size_t agpu_int4_linear_workspace_bytes(int32_t M, int32_t N, int32_
     return 2 * ((half + 255) & ~(size_t)255);
 }
 
+AGPU_EXPORT int32_t agpu_ctx_set_strict_sync(agpu_ctx *ctx, int32_t on) {
+    AGPU_REQUIRE_CTX(ctx);
+    ctx->strict_sync = on ? 1 : 0;
+    return AGPU_OK;
+}
+
 AGPU_EXPORT const char *agpu_last_error_string(const agpu_ctx *ctx) { return ctx ? ctx->err : "null context"; }
 
 AGPU_EXPORT void *agpu_ctx_stream(const agpu_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }

@@ -45,6 +45,7 @@ struct GemmBfParams {
     float *partial;          // [ksplit, M, N] when gridDim.z > 1
     unsigned int *counters;  // one ticket per output tile, left at zero
     KvScatter kv;            // kcache == nullptr: none
+    int strict;              // the context's strict_sync
 };
 
 // fragment [chunk][piece][step][row block][half]
@@ -261,10 +262,10 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
                         __hip_atomic_store(mine + ((rb * CB + cb) * 8 + q) * 64, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     }
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        partials_published(p.strict);
         __syncthreads();
         if (tid == 0) {
-            const unsigned int tk = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const unsigned int tk = take_ticket(&p.counters[tile], p.strict);
             s_last = (tk == (unsigned int)(ksplit - 1));
             if (s_last) __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
@@ -342,6 +343,7 @@ int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t
                                    const KvScatter *kv) {
     GemmBfParams p{};
     if (kv) p.kv = *kv;
+    p.strict = ctx->strict_sync;
     p.x = x; p.packed = packed; p.scales = scales; p.bias = bias; p.residual = residual; p.y = y;
     p.M = M; p.N = N; p.K = K; p.chunk_shift = __builtin_ctz((unsigned)(group / 32)); p.flags = flags;
     // Workgroup tile: 32 rows x 128 columns (one 32 x 32 tile per wave), which puts the most waves on the chip for

@@ -29,6 +29,7 @@ namespace {
 
 struct GemvParams {
     GemvArgs a;
+    int strict;          // the context's strict_sync
     int rows_per_split;  // packed rows per workgroup (grid.y slices of K)
     int col_blocks;      // column tiles of 16*CPL columns; a workgroup strides over them
     float *partial;      // [ksplit, M, N], only with ksplit > 1
@@ -274,10 +275,10 @@ __global__ __launch_bounds__(MT == 1 ? 1024 : 512) void int4_gemv_kernel(const G
                 __hip_atomic_store(&p.partial[((size_t)split * a.M + m) * a.N + n], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        partials_published(p.strict);
         __syncthreads();
         if (tid == 0) {
-            const unsigned int t = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const unsigned int t = take_ticket(&p.counters[tile], p.strict);
             s_last = (t == (unsigned int)(ksplit - 1));
         }
         __syncthreads();
@@ -382,6 +383,7 @@ AGPU_EXPORT int32_t agpu_int4_gemv_tune(agpu_ctx *ctx, int32_t max_wgs, int32_t 
 int32_t agpu_int4_gemv_launch(agpu_ctx *ctx, const GemvArgs &a) {
     GemvParams p{};
     p.a = a;
+    p.strict = ctx->strict_sync;
     if (a.ln_gamma && !agpu_int4_gemv_can_fuse_ln(a.M, a.K))
         return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "int4_gemv: fused LayerNorm needs M <= 2 and M*K <= 8192");
     if (!(a.flags & AGPU_EPI_FORCE_FP32_GEMV) && agpu_int4_gemv_i8_supported(a))

@@ -46,6 +46,7 @@ struct I8Params {
     int sets_before;      // register sets requested before x is converted; the others follow the digits
     unsigned long long *am_partial;  // fused arg-max: one candidate per workgroup, written through
     unsigned int *am_counter;        // ... and the ticket the workgroups take after it
+    int strict;                      // the context's strict_sync
 };
 
 // Order-preserving key of a float (NaN lowest, both zeros equal) with the column behind it: the larger 64-bit word wins.
@@ -361,11 +362,11 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
                 __hip_atomic_store(&p.partial[((size_t)split * a.M + m) * a.N + n], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        partials_published(p.strict);
         __syncthreads();
         if (tid < nt) {
             const int tile = blockIdx.x + tid * gridDim.x;
-            const unsigned int t = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const unsigned int t = take_ticket(&p.counters[tile], p.strict);
             s_last[tid] = (t == (unsigned int)(ksplit - 1));
             if (s_last[tid]) __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
@@ -411,8 +412,8 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
         best = block_max_word(best, am_scratch, lane, wave, W);
         if (tid == 0) {
             __hip_atomic_store(&p.am_partial[blockIdx.x], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            const unsigned int t = __hip_atomic_fetch_add(&p.am_counter[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            partials_published(p.strict);
+            const unsigned int t = take_ticket(&p.am_counter[0], p.strict);
             s_last[0] = (t == gridDim.x - 1);
             if (s_last[0]) __hip_atomic_store(&p.am_counter[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
@@ -455,6 +456,7 @@ bool agpu_int4_gemv_i8_supported(const GemvArgs &a) {
 int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips_per_split, int max_wgs) {
     I8Params p{};
     p.a = a;
+    p.strict = ctx->strict_sync;
     const int MT = a.M <= 1 ? 1 : 2;
     const int trips_total = a.K / 64;
     const int col_blocks = ceil_div(a.N, 64);

@@ -52,6 +52,7 @@ struct SkinnyParams {
     int row_bytes;        // bytes between the rows of a staged piece plane (padded)
     float *partial;
     unsigned int *counters;
+    int strict;           // the context's strict_sync
 };
 
 // the leading 16 bits of two floats as one register: a in the low half
@@ -320,11 +321,11 @@ __global__ __launch_bounds__(64 * NW) void int4_skinny_bf16_kernel(const SkinnyP
     }
     SK_STAMP(5);
     if (ksplit == 1) return;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    partials_published(p.strict);
     __syncthreads();
     SK_STAMP(6);
     if (tid == 0) {
-        const unsigned int tk = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned int tk = take_ticket(&p.counters[tile], p.strict);
         s_last = (tk == (unsigned int)(ksplit - 1));
     }
     __syncthreads();
@@ -390,6 +391,7 @@ int32_t skinny_go(agpu_ctx *ctx, const SkinnyParams &p, dim3 grid, size_t lds) {
 int32_t agpu_int4_skinny_launch(agpu_ctx *ctx, const GemvArgs &a) {
     SkinnyParams p{};
     p.a = a;
+    p.strict = ctx->strict_sync;
     const int trips_total = a.K / 32;
     const int tpg = a.group / 32;  // trips per scale group; a split covers whole groups
     const int tps_max = SK_MAX_TRIPS / tpg * tpg;

@@ -77,6 +77,14 @@ void *agpu_ctx_stream(const agpu_ctx *ctx);
 size_t agpu_ctx_workspace_bytes(const agpu_ctx *ctx);
 size_t agpu_int4_linear_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t with_layer_norm);
 int32_t agpu_ctx_set_workspace(agpu_ctx *ctx, void *workspace, size_t bytes);
+/*
+ * Verification aid, no counterpart in the reference.  Kernels that split a reduction over workgroups hand their partial
+ * results over through write-through stores, a wait for their acknowledgement and a ticket; that is a property of
+ * gfx950 rather than of the memory model.  With `on` != 0 the launches of this context also issue a release fence
+ * before and an acquire fence after the ticket (slower, same result bits); models replay what was captured before
+ * the switch until their graphs are dropped (agpu_gpt2_set_decode_mode does that).
+ */
+int32_t agpu_ctx_set_strict_sync(agpu_ctx *ctx, int32_t on);
 /* Test hook of the one-thread-at-a-time guard: stays inside a call on the context for `ms` milliseconds. */
 int32_t agpu_ctx_test_hold(agpu_ctx *ctx, int32_t ms);
 

@@ -77,6 +77,7 @@ extern "C" {
     pub fn agpu_ctx_workspace_bytes(ctx: *const agpu_ctx) -> usize;
     pub fn agpu_int4_linear_workspace_bytes(M: i32, N: i32, K: i32, with_layer_norm: i32) -> usize;
     pub fn agpu_ctx_set_workspace(ctx: *mut agpu_ctx, workspace: *mut c_void, bytes: usize) -> i32;
+    pub fn agpu_ctx_set_strict_sync(ctx: *mut agpu_ctx, on: i32) -> i32;
     pub fn agpu_ctx_test_hold(ctx: *mut agpu_ctx, ms: i32) -> i32;
     pub fn agpu_malloc(ctx: *mut agpu_ctx, bytes: usize, out: *mut *mut c_void) -> i32;
     pub fn agpu_free(ctx: *mut agpu_ctx, ptr: *mut c_void) -> i32;

@@ -65,6 +65,57 @@ def test_workspace_query_and_caller_provided_scratch(orc, agpu, dev):
     ctx.close()
 
 
+def test_strict_hand_over_gives_the_same_bits(orc, agpu, dev):
+    """Every kernel that splits a reduction over workgroups, once with its fast hand-over (write-through stores, a wait
+    for their acknowledgement, a relaxed ticket) and once with release/acquire fences around the ticket: same bits."""
+    import torch
+    from async_gpu_amd import _lib, ops, workloads, gpt2
+    lib = _lib.cdll()
+    ctx = ops.context(0)
+    rng = np.random.default_rng(77)
+    to = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+    def linear(M, K, N, flags=0):
+        packed, scales, bias = workloads.random_int4_linear(np.random.default_rng(M + K + N), K, N, 32, bias=True)
+        x = np.random.default_rng(M * K).standard_normal((M, K)).astype(np.float32)
+        return lambda: ops.int4_linear(to(x), to(packed), to(scales), bias=to(bias), group=32, flags=flags).cpu().numpy()
+
+    H, kv = 12, 1024
+    q = rng.standard_normal((H, 1, 64)).astype(np.float32) / 8
+    k = rng.standard_normal((H, kv, 64)).astype(np.float32) / 8
+    v = rng.standard_normal((H, kv, 64)).astype(np.float32) / 8
+    cases = {
+        "decode GEMV on the int8 matrix cores, K split": linear(1, 3072, 768),
+        "decode GEMV, fp32, K split": linear(3, 3072, 768, agpu._lib.EPI_FORCE_FP32_GEMV),
+        "batched decode Linear, K split": linear(16, 6400, 1600),
+        "prefill GEMM, K sliced": linear(64, 3072, 768),
+        "decode attention, keys split": lambda: ops.attention(to(q), to(k), to(v), q_offset=kv - 1).cpu().numpy(),
+    }
+    fast = {name: run() for name, run in cases.items()}
+    ctx.call("agpu_ctx_set_strict_sync", 1)
+    try:
+        for name, run in cases.items():
+            assert np.array_equal(run(), fast[name]), name
+    finally:
+        ctx.call("agpu_ctx_set_strict_sync", 0)
+    # the LM head's fused arg-max (candidates of all workgroups, one ticket) through the model, per stage
+    cfg = workloads.GPT2_TINY
+    w = workloads.gpt2_fp32_weights(cfg, 5, std=0.08)
+    qz = workloads.quantize_gpt2(w, 32, lambda wt, g: orc.quantize_weight_int4(wt, g, orc.SCRIPT))
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg), qz)
+    prompt = workloads.random_prompt(cfg, 6, 9)
+    gm.set_decode_mode(gm.DECODE_PER_STAGE)
+    (a,), _ = gm.generate_cached(prompt, 24, eos=-1)
+    la = gm.last_logits()
+    gm.ctx.call("agpu_ctx_set_strict_sync", 1)
+    try:
+        gm.set_decode_mode(gm.DECODE_EAGER)  # drops the graphs captured with the fast form
+        (b,), _ = gm.generate_cached(prompt, 24, eos=-1)
+        assert np.array_equal(a, b) and np.array_equal(la, gm.last_logits())
+    finally:
+        gm.ctx.call("agpu_ctx_set_strict_sync", 0)
+
+
 def test_second_thread_on_a_context_is_turned_away(agpu, dev):
     from async_gpu_amd import _lib
     lib = _lib.cdll()
