@@ -15,9 +15,10 @@
 //     only ever delay a tag, never deliver a wrong value.  Every vector of the step has its own place in the arena,
 //     so nothing is overwritten while the step runs.
 //   * The eight XCDs have an L2 each, and a load that is coherent across them goes to memory (about 0.5 us a round
-//     trip, and a thousand workgroup-sized polls of a vector at once saturate that path).  So one workgroup per XCD
-//     does nothing but relay: it polls each input vector of a Linear in memory and copies it into a mirror that only
-//     its own XCD reads, where the other workgroups of the XCD poll it through their common L2.
+//     trip, and a thousand workgroup-sized polls of a vector at once saturate that path).  So a few workgroups per XCD
+//     do nothing but relay: they poll each input vector of a Linear in memory, 16 bytes (two pairs) per load, and copy
+//     it into a mirror that only their own XCD reads, where the other workgroups of the XCD poll it through their common
+//     L2.  An XCD none of whose workgroups has a tile of a Linear leaves that Linear's input alone.
 //   * A few workgroups per XCD do nothing but attention: (head, key range) each, with the cached K and V rows of the
 //     next layer requested into registers as soon as this layer's are used up.  All others do the Linears: every
 //     wave requests its share of the next Linear's weights into registers before it starts waiting for that
@@ -61,7 +62,8 @@ constexpr int SMAX = 4;         // key ranges per head at most
 constexpr int PSTRIDE = 68;     // floats per partial attention result: o[64], m, l
 constexpr int kSpinLimit = 1 << 16;  // poll rounds a wait may take by default (tens of milliseconds)
 constexpr int DH = 64;
-constexpr int NRELAY = 4;       // relay workgroups per XCD: they poll the same words out of step, the first to see a pair copies it
+constexpr int NRELAY = 4;       // relay workgroups per XCD: they poll a short vector out of step (the first to see a pair copies it)
+                                // and share out a long one
 
 enum : int { F_LN = 1, F_GELU_TANH = 2, F_GELU_QUICK = 4, F_HEAD = 8, F_SCATTER = 16 };
 
@@ -144,6 +146,63 @@ __device__ __forceinline__ void ld_pair_l2_x4(const u64 *p0, const u64 *p1, cons
     o1 = make_uint4(v1.x, v1.y, v1.z, v1.w);
     o2 = make_uint4(v2.x, v2.y, v2.z, v2.w);
     o3 = make_uint4(v3.x, v3.y, v3.z, v3.w);
+}
+// Coherent across the XCDs: four times two pairs from memory, in flight at once.
+__device__ __forceinline__ void ld_pair_mem_x4(const u64 *p0, const u64 *p1, const u64 *p2, const u64 *p3, uint4 &o0, uint4 &o1,
+                                               uint4 &o2, uint4 &o3) {
+    u32x4 v0, v1, v2, v3;
+    asm volatile(
+        "global_load_dwordx4 %0, %4, off sc1\n\t"
+        "global_load_dwordx4 %1, %5, off sc1\n\t"
+        "global_load_dwordx4 %2, %6, off sc1\n\t"
+        "global_load_dwordx4 %3, %7, off sc1\n\t"
+        "s_waitcnt vmcnt(0)"
+        : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3)
+        : "v"(p0), "v"(p1), "v"(p2), "v"(p3)
+        : "memory");
+    o0 = make_uint4(v0.x, v0.y, v0.z, v0.w);
+    o1 = make_uint4(v1.x, v1.y, v1.z, v1.w);
+    o2 = make_uint4(v2.x, v2.y, v2.z, v2.w);
+    o3 = make_uint4(v3.x, v3.y, v3.z, v3.w);
+}
+// Two and six such loads in flight (the attention's q, and q with the new k and v).
+__device__ __forceinline__ void ld_pair_mem_x2(const u64 *p0, const u64 *p1, uint4 &o0, uint4 &o1) {
+    u32x4 v0, v1;
+    asm volatile(
+        "global_load_dwordx4 %0, %2, off sc1\n\t"
+        "global_load_dwordx4 %1, %3, off sc1\n\t"
+        "s_waitcnt vmcnt(0)"
+        : "=&v"(v0), "=&v"(v1)
+        : "v"(p0), "v"(p1)
+        : "memory");
+    o0 = make_uint4(v0.x, v0.y, v0.z, v0.w);
+    o1 = make_uint4(v1.x, v1.y, v1.z, v1.w);
+}
+__device__ __forceinline__ void ld_pair_mem_x6(const u64 *p0, const u64 *p1, const u64 *p2, const u64 *p3, const u64 *p4, const u64 *p5,
+                                               uint4 (&o)[6]) {
+    u32x4 v0, v1, v2, v3, v4, v5;
+    asm volatile(
+        "global_load_dwordx4 %0, %6, off sc1\n\t"
+        "global_load_dwordx4 %1, %7, off sc1\n\t"
+        "global_load_dwordx4 %2, %8, off sc1\n\t"
+        "global_load_dwordx4 %3, %9, off sc1\n\t"
+        "global_load_dwordx4 %4, %10, off sc1\n\t"
+        "global_load_dwordx4 %5, %11, off sc1\n\t"
+        "s_waitcnt vmcnt(0)"
+        : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3), "=&v"(v4), "=&v"(v5)
+        : "v"(p0), "v"(p1), "v"(p2), "v"(p3), "v"(p4), "v"(p5)
+        : "memory");
+    o[0] = make_uint4(v0.x, v0.y, v0.z, v0.w);
+    o[1] = make_uint4(v1.x, v1.y, v1.z, v1.w);
+    o[2] = make_uint4(v2.x, v2.y, v2.z, v2.w);
+    o[3] = make_uint4(v3.x, v3.y, v3.z, v3.w);
+    o[4] = make_uint4(v4.x, v4.y, v4.z, v4.w);
+    o[5] = make_uint4(v5.x, v5.y, v5.z, v5.w);
+}
+__device__ __forceinline__ uint4 ld_pair_mem(const u64 *p) {
+    u32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(p) : "memory");
+    return make_uint4(v.x, v.y, v.z, v.w);
 }
 __device__ __forceinline__ bool pair_ok(const uint4 &v, uint32_t epoch) { return v.y == epoch && v.w == epoch; }
 
@@ -643,49 +702,71 @@ __device__ __forceinline__ void head_finish(const Params &p, const Stage &st, co
 // One vector: awaited in memory, copied into this XCD's mirror.  Thread t owns the element pairs t, t + T, ...; nothing
 // orders the threads among themselves, every pair carries its own tags.
 __device__ __forceinline__ void relay_copy(const Params &p, Ctl &c, u64 *mirror, int off, int n_elems, int tid, int phase) {
-    const int n_pairs = n_elems >> 1;
+    int n_pairs = n_elems >> 1;
     const u64 *src = p.arena + off;
     u64 *dst = mirror + off;
-    // The relays of an XCD finish a vector together, when it arrives; each starts on the next one (which is at
+    // A vector of more pairs than a relay has threads is shared out among the relays of the XCD (a quarter each, one
+    // load per thread and round); a shorter one is polled by all of them out of step, which finds it sooner.
+    if (n_pairs > T) {
+        const int share = ((n_pairs + NRELAY - 1) / NRELAY + 1) & ~1;
+        const int lo = min(n_pairs, phase * share), hi = min(n_pairs, lo + share);
+        src += 2 * lo;
+        dst += 2 * lo;
+        n_pairs = hi - lo;
+        phase = 0;
+    }
+    // The relays of an XCD finish a short vector together, when it arrives; each starts on the next one (which is at
     // least a stage away) with its own delay, so that their polls stay out of step: a poll's round trip is
     // about 0.55 us = 20 sleeps of 64 clocks.
     for (int i = 0; i < phase * (20 / NRELAY); ++i) __builtin_amdgcn_s_sleep(1);
-    bool need[PMAX];
-#pragma unroll
-    for (int i = 0; i < PMAX; ++i) need[i] = tid + i * T < n_pairs;
     int spins = 0;
     PK_STAMP(0);
-    while (!c.dead) {
-        u64 a[PMAX], b[PMAX];
+    // 16 bytes = two pairs per load; four loads in flight where a thread owns several
 #pragma unroll
-        for (int i = 0; i < PMAX; ++i)
-            if (need[i]) {
-                a[i] = ld_tag(src + 2 * (tid + i * T));
-                b[i] = ld_tag(src + 2 * (tid + i * T) + 1);
-            }
-        bool ok = true;
+    for (int b4 = 0; b4 < PMAX; b4 += 4) {
+        if (b4 * T >= n_pairs) break;  // workgroup-uniform
+        const u64 *ptr[4];
+        bool need[4];
 #pragma unroll
-        for (int i = 0; i < PMAX; ++i)
-            if (need[i]) {
-                if (tag_ok(a[i], c.epoch) && tag_ok(b[i], c.epoch)) {
-                    *reinterpret_cast<uint4 *>(dst + 2 * (tid + i * T)) =
-                        make_uint4((uint32_t)a[i], (uint32_t)(a[i] >> 32), (uint32_t)b[i], (uint32_t)(b[i] >> 32));
-                    need[i] = false;
-                } else {
-                    ok = false;
+        for (int k = 0; k < 4; ++k) {
+            const int pr = tid + (b4 + k) * T;
+            need[k] = pr < n_pairs;
+            ptr[k] = src + 2 * (need[k] ? pr : 0);
+        }
+        if (n_pairs <= (b4 + 1) * T) {
+            // one pair of pairs per thread at most: the common case
+            while (need[0] && !c.dead) {
+                const uint4 v = ld_pair_mem(ptr[0]);
+                if (pair_ok(v, c.epoch)) {
+                    *reinterpret_cast<uint4 *>(dst + 2 * (tid + b4 * T)) = v;
+                    break;
                 }
+                if (spin_fail(c, spins)) break;
             }
-        if (ok || spin_fail(c, spins)) break;
+        } else {
+            while (!c.dead) {
+                uint4 t0, t1, t2, t3;
+                ld_pair_mem_x4(ptr[0], ptr[1], ptr[2], ptr[3], t0, t1, t2, t3);
+                bool ok = true;
+                if (need[0]) { if (pair_ok(t0, c.epoch)) { *reinterpret_cast<uint4 *>(dst + 2 * (tid + (b4 + 0) * T)) = t0; need[0] = false; } else ok = false; }
+                if (need[1]) { if (pair_ok(t1, c.epoch)) { *reinterpret_cast<uint4 *>(dst + 2 * (tid + (b4 + 1) * T)) = t1; need[1] = false; } else ok = false; }
+                if (need[2]) { if (pair_ok(t2, c.epoch)) { *reinterpret_cast<uint4 *>(dst + 2 * (tid + (b4 + 2) * T)) = t2; need[2] = false; } else ok = false; }
+                if (need[3]) { if (pair_ok(t3, c.epoch)) { *reinterpret_cast<uint4 *>(dst + 2 * (tid + (b4 + 3) * T)) = t3; need[3] = false; } else ok = false; }
+                if (ok || spin_fail(c, spins)) break;
+            }
+        }
     }
     PK_STAMP(1);
 }
 
-// Every input vector of a Linear, in the order the step produces them.
-__device__ __forceinline__ void relay_role(const Params &p, const Stage *tab, Ctl &c, u64 *mirror, int tid, int phase) {
+// Every input vector of a Linear, in the order the step produces them, that a workgroup of this XCD reads: the tiles of
+// a layer's Linear go to the Linear workgroups XCD by XCD (`first_rank` is the first of this XCD's), the head to everybody.
+__device__ __forceinline__ void relay_role(const Params &p, const Stage *tab, Ctl &c, u64 *mirror, int tid, int phase, int first_rank) {
     for (int s = 0; s < p.n_stages; ++s) {
         c.stage = s;
         const int in_off = rfl(tab[s].in_off), K = rfl(tab[s].K);
-        if (in_off >= 0) relay_copy(p, c, mirror, in_off, K, tid, phase);
+        const bool wanted = (rfl(tab[s].flags) & F_HEAD) || first_rank < rfl(tab[s].n_tiles);
+        if (in_off >= 0 && wanted) relay_copy(p, c, mirror, in_off, K, tid, phase);
     }
 }
 
@@ -755,36 +836,28 @@ __device__ __forceinline__ void attn_role(const Params &p, const Stage *tab, Ctl
             // q of this head, and for one wave the new key and value, straight from the QKV vector in memory (a dozen
             // workgroups poll it: relaying it through the mirrors was measured and is slower)
             const u64 *qsrc = p.arena + st.out_off + h * DH + 4 * e4;
-            u64 qw[4], kw[4], vw[4];
+            // (value, tag) pairs, two per 16-byte load: q, then the new k and v; every load of a round is issued before
+            // the first tag is looked at
+            uint4 w6[6];
 #pragma unroll
-            for (int k = 0; k < 4; ++k) qw[k] = kw[k] = vw[k] = 0ull;
+            for (int k = 0; k < 6; ++k) w6[k] = make_uint4(0u, 0u, 0u, 0u);
             int spins = 0;
             while (true) {
-                // every load of the round is issued before the first tag is looked at
-#pragma unroll
-                for (int k = 0; k < 4; ++k) qw[k] = ld_tag(qsrc + k);
+                bool ok;
                 if (with_new) {
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        kw[k] = ld_tag(qsrc + p.d + k);
-                        vw[k] = ld_tag(qsrc + 2 * p.d + k);
-                    }
-                }
-                bool ok = true;
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    ok = ok && tag_ok(qw[k], c.epoch);
-                    if (with_new) ok = ok && tag_ok(kw[k], c.epoch) && tag_ok(vw[k], c.epoch);
+                    ld_pair_mem_x6(qsrc, qsrc + 2, qsrc + p.d, qsrc + p.d + 2, qsrc + 2 * p.d, qsrc + 2 * p.d + 2, w6);
+                    ok = pair_ok(w6[0], c.epoch) && pair_ok(w6[1], c.epoch) && pair_ok(w6[2], c.epoch) && pair_ok(w6[3], c.epoch) &&
+                         pair_ok(w6[4], c.epoch) && pair_ok(w6[5], c.epoch);
+                } else {
+                    ld_pair_mem_x2(qsrc, qsrc + 2, w6[0], w6[1]);
+                    ok = pair_ok(w6[0], c.epoch) && pair_ok(w6[1], c.epoch);
                 }
                 if (ok || c.dead) break;
                 if (spin_fail(c, spins)) break;
             }
-            q = make_float4(tag_val(qw[0]), tag_val(qw[1]), tag_val(qw[2]), tag_val(qw[3]));
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                kn[k] = tag_val(kw[k]);
-                vn[k] = tag_val(vw[k]);
-            }
+            q = make_float4(__uint_as_float(w6[0].x), __uint_as_float(w6[0].z), __uint_as_float(w6[1].x), __uint_as_float(w6[1].z));
+            kn[0] = __uint_as_float(w6[2].x); kn[1] = __uint_as_float(w6[2].z); kn[2] = __uint_as_float(w6[3].x); kn[3] = __uint_as_float(w6[3].z);
+            vn[0] = __uint_as_float(w6[4].x); vn[1] = __uint_as_float(w6[4].z); vn[2] = __uint_as_float(w6[5].x); vn[3] = __uint_as_float(w6[5].z);
             m = ninf;
             l = 0.0f;
             o = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -992,7 +1065,7 @@ __global__ __launch_bounds__(T) void decode_step_kernel(const Params p) {
     const int per_xcd = G >> 3;
     u64 *mirror = p.arena + (size_t)(1 + xcd) * p.arena_elems;
     if (in_xcd < NRELAY) {
-        relay_role(p, tab, c, mirror, tid, in_xcd);
+        relay_role(p, tab, c, mirror, tid, in_xcd, xcd * (per_xcd - NRELAY - p.att_per_xcd));
         PK_DUMP();
         return;
     }
