@@ -528,8 +528,10 @@ int32_t launch_step_per_stage(agpu_gpt2 *m, int B, int bucket) {
 }
 
 // The captured decode step for (batch, kv bucket); captured on first use.
-int32_t decode_graph(agpu_gpt2 *m, int B, int bucket, hipGraphExec_t *out) {
-    const long long key = ((long long)B << 32) | (unsigned)bucket;
+// The one-launch step reads the position on the device and does not depend on the bucket: `reps` > 1 captures that many
+// of its launches in a row (one graph launch then costs its overhead once for `reps` tokens).
+int32_t decode_graph(agpu_gpt2 *m, int B, int bucket, hipGraphExec_t *out, int reps = 1) {
+    const long long key = reps > 1 ? ((1ll << 62) | reps) : (((long long)B << 32) | (unsigned)bucket);
     if (m->ws_epoch != m->ctx->ws_epoch) {  // the scratch moved: captured launches point at the old one
         drop_graphs(m);
         m->ws_epoch = m->ctx->ws_epoch;
@@ -548,7 +550,11 @@ int32_t decode_graph(agpu_gpt2 *m, int B, int bucket, hipGraphExec_t *out) {
     int32_t rc;
     if (one_launch) {
         // one sequence: the whole step, arg-max and token feed included, is one launch
-        rc = agpu_pk_launch(ctx, pk_view(m), m->pk, 0);
+        const PkModel view = pk_view(m);
+        rc = AGPU_OK;
+        for (int r = 0; r < reps && rc == AGPU_OK; ++r) rc = agpu_pk_launch(ctx, view, m->pk, 0);
+    } else if (reps > 1) {
+        rc = agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "gpt2: several steps per graph need the one-launch step");
     } else {
         rc = launch_step_per_stage(m, B, bucket);
     }
@@ -584,7 +590,19 @@ int32_t ensure_out_tokens(agpu_gpt2 *m, int steps, int B) {
 
 // Replays `steps` decode steps; the host only tracks the position to pick the graph.
 int32_t run_decode_steps(agpu_gpt2 *m, int B, int steps) {
-    for (int s = 0; s < steps; ++s) {
+    constexpr int kStepsPerGraph = 16;  // agpu_gpt2_decode_steps captures the same number ahead of its timed region
+    int s = 0;
+    if (B == 1 && steps >= kStepsPerGraph && pk_ready(m)) {
+        for (; s + kStepsPerGraph <= steps; s += kStepsPerGraph) {
+            hipGraphExec_t exec;
+            const int32_t rc = decode_graph(m, 1, 0, &exec, kStepsPerGraph);
+            if (rc != AGPU_OK) return rc;
+            const hipError_t e = hipGraphLaunch(exec, m->ctx->stream);
+            if (e != hipSuccess) return agpu_hip(m->ctx, e, "hipGraphLaunch");
+            m->cache_len += kStepsPerGraph;
+        }
+    }
+    for (; s < steps; ++s) {
         const int bucket = kv_bucket(m, m->cache_len + 1);
         if (m->decode_mode == AGPU_DECODE_EAGER) {
             const int32_t rc = launch_step_per_stage(m, B, bucket);
@@ -959,6 +977,7 @@ AGPU_EXPORT int32_t agpu_gpt2_decode_steps(agpu_gpt2 *m, int32_t batch, int32_t 
     if (rc != AGPU_OK) return rc;
     // capture outside the timed region
     hipGraphExec_t exec;
+    if (batch == 1 && steps >= 16 && pk_ready(m) && (rc = decode_graph(m, 1, 0, &exec, 16)) != AGPU_OK) return rc;
     for (int s = 0; s < steps && m->decode_mode != AGPU_DECODE_EAGER; ++s)
         if ((rc = decode_graph(m, batch, kv_bucket(m, m->cache_len + 1 + s), &exec)) != AGPU_OK) return rc;
     if ((rc = agpu_hip(ctx, hipEventRecord(m->ev0, ctx->stream), "hipEventRecord")) != AGPU_OK) return rc;
