@@ -43,6 +43,8 @@ struct PkPlan {
     int att_per_xcd = 0;  // workgroups per XCD that only do attention
     int smax = 1;         // key ranges per head at most
     size_t lds_bytes = 0;
+    int kmax = 0;         // longest input vector of a Linear: sizes the staging buffers
+    int head_slots = 0;   // slots of the head's second chunk that wait in LDS (0: fetched when their turn comes)
     int spin_limit = 0;   // poll rounds a wait inside the kernel may take; 0 = the default
 };
 

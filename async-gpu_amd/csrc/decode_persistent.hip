@@ -55,7 +55,6 @@ constexpr int KR = 4 * W;       // keys per round: four per wave
 constexpr int XMAX = 8192;      // longest input vector of a Linear stage (staged in LDS)
 constexpr int GS = 36;          // floats between the groups of 32 in LDS: lanes that read different groups 16 bytes at a
                                 // time then fall on different banks
-constexpr int XBUF = XMAX / 32 * GS;  // floats of one staging buffer
 constexpr int PMAX = XMAX / (2 * T);  // pairs of input elements a thread polls at most
 constexpr int LNP = 2048 / (2 * T);  // ... of a stage with LayerNorm (K <= 2048)
 constexpr int SMAX = 4;         // key ranges per head at most
@@ -102,6 +101,8 @@ struct Params {
     int att_per_xcd;  // attention workgroups per XCD
     int smax;         // key ranges per head at most
     int spin_limit;   // poll rounds a wait may take
+    int xbuf;         // floats of one staging buffer: GS per group of the longest input vector
+    int head_slots;   // slots of the head's second chunk kept in LDS ahead of the head stage (0: none)
     unsigned long long *trace;  // optional time stamps (debug builds)
 };
 
@@ -271,6 +272,48 @@ struct Regs {
     float sc[SL];
 };
 
+// The eight nibbles of a word as floats (two masks, then the byte converts).
+__device__ __forceinline__ void unpack_bytes(uint32_t w, float (&nf)[8]) {
+    const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+    asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(nf[0]) : "v"(lo));
+    asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(nf[1]) : "v"(hi));
+    asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(nf[2]) : "v"(lo));
+    asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(nf[3]) : "v"(hi));
+    asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(nf[4]) : "v"(lo));
+    asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(nf[5]) : "v"(hi));
+    asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(nf[6]) : "v"(lo));
+    asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(nf[7]) : "v"(hi));
+}
+
+// One slot: the lane's group of 32 inputs against its four packed words.  All eight LDS reads are issued before the
+// first product (left to itself the compiler reads two at a time and waits for each pair: 0.17 against 0.25 us per slot
+// and workgroup).  Reading the next slot's inputs ahead of this slot's products as well was slower.
+__device__ __forceinline__ float slot_dot(const uint32_t (&w)[4], const float *xs, const float *xsum, int g) {
+    const float4 *xg = reinterpret_cast<const float4 *>(xs + GS * g);
+    float4 xr[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) xr[i] = xg[i];
+    const float sx = xsum[g];
+    __builtin_amdgcn_sched_barrier(0);
+    float dq[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {  // one chain of eight products per packed word
+        float nf[8];
+        unpack_bytes(w[q], nf);
+        const float4 xa = xr[2 * q], xb = xr[2 * q + 1];
+        float dot = xa.x * nf[0];
+        dot = fmaf(xa.y, nf[1], dot);
+        dot = fmaf(xa.z, nf[2], dot);
+        dot = fmaf(xa.w, nf[3], dot);
+        dot = fmaf(xb.x, nf[4], dot);
+        dot = fmaf(xb.y, nf[5], dot);
+        dot = fmaf(xb.z, nf[6], dot);
+        dot = fmaf(xb.w, nf[7], dot);
+        dq[q] = dot;
+    }
+    return ((dq[0] + dq[1]) + (dq[2] + dq[3])) - 8.0f * sx;
+}
+
 // ---- what a wave requests ahead of a Linear stage ----
 // Slot s of a chunk = (tile tt, round u), tile-major.  Round u of wave w covers groups (u W + w) gpw + j,
 // gpw = 4 >> tws groups per wave-wide load; lane (col, j) takes group j of the round for column col of the tile.
@@ -319,25 +362,7 @@ __device__ __forceinline__ void compute_chunk(const Stage &st, const Regs &r, co
         {
             int g = (u * W + wave) * gpw + j;
             g = g < st.n_groups ? g : st.n_groups - 1;  // beyond the last group the words and the scale are zero
-            const float4 *xg = reinterpret_cast<const float4 *>(xs + GS * g);
-            float dq[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {  // one chain of eight products per packed word
-                float nf[8];
-                unpack_u8(r.w[s][q], nf);
-                const float4 xa = xg[2 * q], xb = xg[2 * q + 1];
-                float dot = xa.x * nf[0];
-                dot = fmaf(xa.y, nf[1], dot);
-                dot = fmaf(xa.z, nf[2], dot);
-                dot = fmaf(xa.w, nf[3], dot);
-                dot = fmaf(xb.x, nf[4], dot);
-                dot = fmaf(xb.y, nf[5], dot);
-                dot = fmaf(xb.z, nf[6], dot);
-                dot = fmaf(xb.w, nf[7], dot);
-                dq[q] = dot;
-            }
-            const float dot = (dq[0] + dq[1]) + (dq[2] + dq[3]);
-            acc = fmaf(r.sc[s], dot - 8.0f * xsum[g], acc);
+            acc = fmaf(r.sc[s], slot_dot(r.w[s], xs, xsum, g), acc);
             if (u == st.nl - 1) {  // wave-uniform: the tile is complete
                 const float tot = reduce_groups(acc, st.tws);
                 if (lane < tw) red[(tt * W + wave) * 64 + col] = tot;
@@ -352,19 +377,6 @@ __device__ __forceinline__ void compute_chunk(const Stage &st, const Regs &r, co
 }
 
 // ---- the Linears of the layers: one tile per workgroup ----
-// The eight nibbles of a word as floats (two masks, then the byte converts).
-__device__ __forceinline__ void unpack_bytes(uint32_t w, float (&nf)[8]) {
-    const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
-    asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(nf[0]) : "v"(lo));
-    asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(nf[1]) : "v"(hi));
-    asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(nf[2]) : "v"(lo));
-    asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(nf[3]) : "v"(hi));
-    asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(nf[4]) : "v"(lo));
-    asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(nf[5]) : "v"(hi));
-    asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(nf[6]) : "v"(lo));
-    asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(nf[7]) : "v"(hi));
-}
-
 // Lane (col, j) of wave w holds, in slot u, group (u W + w) gpw + j of column col of the workgroup's tile
 // (gpw = 4 >> tws groups per wave-wide load): a wave-wide load reads runs of 64 to 256 contiguous bytes.
 template <int MODE>
@@ -403,25 +415,7 @@ __device__ __forceinline__ float lay_compute(const Stage &st, const Regs &r, con
         if (u >= st.nl) break;  // wave-uniform
         int g = (u * W + wave) * gpw + j;
         g = g < st.n_groups ? g : st.n_groups - 1;  // beyond the last group the words and the scale are zero
-        const float4 *xg = reinterpret_cast<const float4 *>(xs + GS * g);
-        float dq[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {  // one chain of eight products per packed word
-            float nf[8];
-            unpack_bytes(r.w[u][q], nf);
-            const float4 xa = xg[2 * q], xb = xg[2 * q + 1];
-            float dot = xa.x * nf[0];
-            dot = fmaf(xa.y, nf[1], dot);
-            dot = fmaf(xa.z, nf[2], dot);
-            dot = fmaf(xa.w, nf[3], dot);
-            dot = fmaf(xb.x, nf[4], dot);
-            dot = fmaf(xb.y, nf[5], dot);
-            dot = fmaf(xb.z, nf[6], dot);
-            dot = fmaf(xb.w, nf[7], dot);
-            dq[q] = dot;
-        }
-        const float dot = (dq[0] + dq[1]) + (dq[2] + dq[3]);
-        acc = fmaf(r.sc[u], dot - 8.0f * xsum[g], acc);
+        acc = fmaf(r.sc[u], slot_dot(r.w[u], xs, xsum, g), acc);
     }
     return reduce_groups(acc, st.tws);
 }
@@ -454,12 +448,13 @@ __device__ __forceinline__ u64 block_max48(u64 w, uint32_t *scratch, int lane, i
 }
 
 struct Lds {
-    float *xs;       // [2][XBUF]: the staged input, stages in turn
+    float *xs;       // [2][xbuf]: the staged input, stages in turn
     float *xsum;     // [2][XMAX / 32]: sum of every group of 32 inputs
     float *red;      // [2][SL][W][64]: per-wave sums, chunks in turn; attention: per-wave partial results
     float4 *stat;    // [W]: LayerNorm statistics per wave
     float *fin;      // attention: [PSTRIDE] + [SMAX][PSTRIDE]
     uint32_t *scr;   // [2 W]
+    uint32_t *hl;    // [head_slots][5][T]: the head's second chunk as the registers will hold it
 };
 
 #ifdef AGPU_PK_TRACE
@@ -1009,6 +1004,50 @@ __device__ __forceinline__ void attn_role(const Params &p, const Stage *tab, Ctl
     }
 }
 
+// ---- the head's second chunk, fetched into LDS while the layers run ----
+// The head's weights depend on nothing, HBM idles during the layers, and what a thread's registers do not hold of
+// the workgroup's share fits in LDS for the smaller models: slot by slot, whenever the workgroup has just published a
+// stage (one slot's five words are requested, the previous slot's are written to LDS), and the rest in one go before
+// the head.  Every thread writes and later reads its own words: no barrier.
+struct HeadAhead {
+    int n_slots;  // slots of chunk 1 this workgroup has (0: nothing to do)
+    int s, tt, u; // next slot to request, as (tile of the chunk, round)
+    int pending;  // slot whose words are in v, -1: none
+    uint32_t v[5];
+};
+__device__ __forceinline__ void head_ahead_step(const Stage *th, HeadAhead &ha, uint32_t *hl, int rank, int wave, int lane, int tid) {
+    if (ha.pending >= 0) {
+#pragma unroll
+        for (int q = 0; q < 5; ++q) hl[(size_t)(ha.pending * 5 + q) * T + tid] = ha.v[q];
+        ha.pending = -1;
+    }
+    if (ha.s >= ha.n_slots) return;  // workgroup-uniform
+    const int tws = rfl(th->tws), nl = rfl(th->nl), tpc = rfl(th->tpc), n_wgs = rfl(th->n_wgs);
+    const int n_groups = rfl(th->n_groups), stride = rfl(th->stride);
+    const uint32_t *packed = rflp(th->packed);
+    const float *scales = rflp(th->scales);
+    const int tw = 16 << tws, gpw = 4 >> tws;
+    const int col = lane & (tw - 1), j = lane >> (4 + tws);
+    const int tile = rank + (tpc + ha.tt) * n_wgs;  // chunk 1
+    const int g = (ha.u * W + wave) * gpw + j, n = tile * tw + col;
+#pragma unroll
+    for (int q = 0; q < 5; ++q) ha.v[q] = 0u;
+    if (g < n_groups && n < stride) {
+        const uint32_t *wp = packed + (size_t)(4 * g) * stride + n;
+        ha.v[0] = wp[0];
+        ha.v[1] = wp[stride];
+        ha.v[2] = wp[2 * (size_t)stride];
+        ha.v[3] = wp[3 * (size_t)stride];
+        ha.v[4] = __float_as_uint(scales[(size_t)g * stride + n]);
+    }
+    ha.pending = ha.s;
+    ++ha.s;
+    if (++ha.u == nl) {
+        ha.u = 0;
+        ++ha.tt;
+    }
+}
+
 // First stage from `from` on, before the head, in which workgroup `rank` has a tile; the head (n_lay) if none.
 __device__ __forceinline__ int next_active(const Stage *tab, int from, int rank, int n_lay) {
     int s = from;
@@ -1037,12 +1076,13 @@ __global__ __launch_bounds__(T) void decode_step_kernel(const Params p) {
     }
     Lds L;
     L.xs = smem + (size_t)p.n_stages * (sizeof(Stage) / 4);
-    L.xsum = L.xs + 2 * XBUF;
+    L.xsum = L.xs + 2 * p.xbuf;
     L.red = L.xsum + 2 * (XMAX / 32);
     L.stat = reinterpret_cast<float4 *>(L.red + 2 * SL * W * 64);
     L.fin = L.red + 2 * SL * W * 64 + 4 * W;
     L.scr = reinterpret_cast<uint32_t *>(L.fin + (SMAX + 1) * PSTRIDE);
-    u64 *tr_lds = reinterpret_cast<u64 *>(L.scr + 2 * W);
+    L.hl = L.scr + 2 * W;
+    u64 *tr_lds = reinterpret_cast<u64 *>(L.hl + (size_t)p.head_slots * 5 * T);
 #ifdef AGPU_PK_TRACE
     for (int i = tid; i < p.n_stages * 8; i += T) tr_lds[i] = 0ull;
 #endif
@@ -1092,15 +1132,25 @@ __global__ __launch_bounds__(T) void decode_step_kernel(const Params p) {
     int n_enter = 0;  // staging buffers are used in turn
     Stage st = load_stage(tab + s);
     if (s < n_lay) lay_prefetch<MODE>(st, regs, rank, wave, lane);
+    HeadAhead ha;
+    ha.n_slots = ha.s = ha.tt = ha.u = 0;
+    ha.pending = -1;
+    if (MODE == 0 && p.head_slots > 0 && !is_att) {
+        const Stage *th = tab + n_lay;
+        const int n_tiles = rfl(th->n_tiles), n_wgs = rfl(th->n_wgs), tpc = rfl(th->tpc);
+        const int my_tiles = rank < n_tiles ? (n_tiles - rank + n_wgs - 1) / n_wgs : 0;
+        ha.n_slots = min(p.head_slots, min(tpc, max(0, my_tiles - tpc)) * rfl(th->nl));
+    }
     while (s < n_lay) {
         c.stage = s;
-        lay_stage<MODE>(p, st, c, regs, L.xs + (n_enter & 1) * XBUF, L.xsum + (n_enter & 1) * (XMAX / 32), L.stat,
+        lay_stage<MODE>(p, st, c, regs, L.xs + (n_enter & 1) * p.xbuf, L.xsum + (n_enter & 1) * (XMAX / 32), L.stat,
                         L.red + (n_enter & 1) * (SL * W * 64), mirror, pos, tok, rank, tid);
         // the outputs are on their way: now the next stage this workgroup takes part in, and its weights
         ++n_enter;
         s = next_active(tab, s + 1, rank, n_lay);
         st = load_stage(tab + s);
         if (s < n_lay) lay_prefetch<MODE>(st, regs, rank, wave, lane);
+        if (MODE == 0) head_ahead_step(tab + n_lay, ha, L.hl, rank, wave, lane, tid);
         PK_STAMP(5);
     }
     // the head: tiles dealt round robin, in chunks of SL slots
@@ -1110,7 +1160,10 @@ __global__ __launch_bounds__(T) void decode_step_kernel(const Params p) {
         int my_tiles, n_chunks;
         head_share(st, rank, my_tiles, n_chunks);
         prefetch_lin<MODE>(st, regs, 0, rank, wave, lane);
-        float *xs = L.xs + (n_enter & 1) * XBUF, *xsum = L.xsum + (n_enter & 1) * (XMAX / 32);
+        // what is left of the second chunk goes to LDS now (a workgroup without a tile in the layers has had no other occasion)
+        if (MODE == 0)
+            while (ha.pending >= 0 || ha.s < ha.n_slots) head_ahead_step(tab + n_lay, ha, L.hl, rank, wave, lane, tid);
+        float *xs = L.xs + (n_enter & 1) * p.xbuf, *xsum = L.xsum + (n_enter & 1) * (XMAX / 32);
         if (my_tiles > 0) {  // workgroup-uniform
             PK_STAMP(0);
             stage_input<MODE>(p, st, c, xs, xsum, L.stat, mirror, pos, tok, tid, [] {});
@@ -1118,10 +1171,27 @@ __global__ __launch_bounds__(T) void decode_step_kernel(const Params p) {
                 const int tiles = min(st.tpc, my_tiles - ch * st.tpc);
                 float *red = L.red + (ch & 1) * (SL * W * 64);
                 if (MODE == 0) compute_chunk(st, regs, xs, xsum, red, tiles, wave, lane);
+                if (ch == 0) PK_STAMP(4);
+                if (ch == 1) PK_STAMP(6);
                 // the next chunk is requested before this one's outputs are written (they wait for no load)
-                if (ch + 1 < n_chunks) prefetch_lin<MODE>(st, regs, ch + 1, rank, wave, lane);
+                if (ch + 1 < n_chunks) {
+                    if (ch == 0 && ha.n_slots > 0 && MODE == 0) {
+                        // the second chunk is in LDS, as the registers hold a chunk; slots beyond it are not looked at
+#pragma unroll
+                        for (int sl = 0; sl < SL; ++sl) {
+                            if (sl >= ha.n_slots) break;  // workgroup-uniform
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) regs.w[sl][q] = L.hl[(size_t)(sl * 5 + q) * T + tid];
+                            regs.sc[sl] = __uint_as_float(L.hl[(size_t)(sl * 5 + 4) * T + tid]);
+                        }
+                    } else {
+                        prefetch_lin<MODE>(st, regs, ch + 1, rank, wave, lane);
+                    }
+                }
                 __syncthreads();
                 head_finish<MODE>(p, st, L.red + (ch & 1) * (SL * W * 64), rank, ch, tiles, tid, best);
+                if (ch == 0) PK_STAMP(5);
+                if (ch == 1) PK_STAMP(7);
             }
             PK_STAMP(3);
         }
@@ -1221,10 +1291,17 @@ Roles plan_roles(const agpu_ctx *ctx, int H) {
     return r;
 }
 
-size_t lds_bytes_for(int n_stages) {
-    return (size_t)n_stages * sizeof(Stage) +
-           (size_t)(2 * XBUF + 2 * (XMAX / 32) + 2 * SL * W * 64 + 4 * W + (SMAX + 1) * PSTRIDE + 2 * W) * 4 +
-           (size_t)n_stages * 8 * sizeof(u64);  // time stamps (debug builds)
+// floats of one staging buffer for input vectors of up to kmax elements
+int xbuf_floats(int kmax) { return kmax / 32 * GS; }
+
+size_t lds_bytes_for(int n_stages, int kmax, int head_slots) {
+    size_t b = (size_t)n_stages * sizeof(Stage) +
+               (size_t)(2 * xbuf_floats(kmax) + 2 * (XMAX / 32) + 2 * SL * W * 64 + 4 * W + (SMAX + 1) * PSTRIDE + 2 * W) * 4 +
+               (size_t)head_slots * 5 * T * 4;
+#ifdef AGPU_PK_TRACE
+    b += (size_t)n_stages * 8 * sizeof(u64);  // time stamps
+#endif
+    return b;
 }
 
 }  // namespace
@@ -1248,7 +1325,7 @@ bool agpu_pk_supported(const agpu_ctx *ctx, const PkModel &m) {
             if (!plan_linear(s, *l, r.n_lin, false)) return false;
     }
     if (!m.lnf_g || !m.lnf_b || !m.wte || !m.wpe) return false;
-    if (lds_bytes_for(4 * m.n_layer + 1) > (size_t)160 * 1024) return false;
+    if (lds_bytes_for(4 * m.n_layer + 1, std::max(m.d, m.ff), 0) > (size_t)160 * 1024) return false;
     return true;
 }
 
@@ -1307,7 +1384,15 @@ int32_t agpu_pk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
     if (e == hipSuccess) e = hipMemset(plan->arena, 0, arena_bytes);
     if (e == hipSuccess) e = hipMemset(plan->state, 0, 64);
     // one workgroup per CU: the request is sized so that two never share a CU
-    plan->lds_bytes = std::max(lds_bytes_for(plan->n_stages), (size_t)96 * 1024);
+    // the head's second chunk in LDS where the workgroups have one and LDS has the room
+    {
+        const Stage &hs = st.back();
+        const int tiles_max = ceil_div(hs.n_tiles, hs.n_wgs);
+        const int want = std::min(SL, std::min(hs.tpc, std::max(0, tiles_max - hs.tpc)) * hs.nl);
+        plan->head_slots = want > 0 && lds_bytes_for(plan->n_stages, std::max(d, ff), want) <= (size_t)160 * 1024 ? want : 0;
+    }
+    plan->kmax = std::max(d, ff);
+    plan->lds_bytes = std::max(lds_bytes_for(plan->n_stages, plan->kmax, plan->head_slots), (size_t)96 * 1024);
     if (e == hipSuccess)
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(decode_step_kernel<0>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)plan->lds_bytes);
@@ -1344,6 +1429,8 @@ int32_t agpu_pk_launch(agpu_ctx *ctx, const PkModel &m, const PkPlan &plan, int 
     p.att_per_xcd = plan.att_per_xcd;
     p.smax = plan.smax;
     p.spin_limit = plan.spin_limit > 0 ? plan.spin_limit : kSpinLimit;
+    p.xbuf = xbuf_floats(plan.kmax);
+    p.head_slots = plan.head_slots;
     p.trace = trace;
     if (mode == 0) hipLaunchKernelGGL(decode_step_kernel<0>, dim3(plan.grid), dim3(T), plan.lds_bytes, ctx->stream, p);
     else hipLaunchKernelGGL(decode_step_kernel<1>, dim3(plan.grid), dim3(T), plan.lds_bytes, ctx->stream, p);
