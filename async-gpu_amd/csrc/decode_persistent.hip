@@ -79,7 +79,8 @@ struct Stage {
     int flags;
     int tpc;                               // tiles per chunk of SL slots: SL / nl
     float inv_k;                           // 1 / K
-    int pad_[2];
+    int rank0;                             // layers: the Linear workgroup that has tile 0 (tile t: rank0 + t, modulo their number)
+    int pad_;
 };
 static_assert(sizeof(Stage) % 16 == 0, "stage table is copied in 16-byte pieces");
 
@@ -130,6 +131,19 @@ __device__ __forceinline__ uint4 ld_pair_l2(const u64 *p) {
     asm volatile("global_load_dwordx4 %0, %1, off nt\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(p) : "memory");
     return make_uint4(v.x, v.y, v.z, v.w);
 }
+// Two such loads in flight at once.
+__device__ __forceinline__ void ld_pair_l2_x2(const u64 *p0, const u64 *p1, uint4 &o0, uint4 &o1) {
+    u32x4 v0, v1;
+    asm volatile(
+        "global_load_dwordx4 %0, %2, off nt\n\t"
+        "global_load_dwordx4 %1, %3, off nt\n\t"
+        "s_waitcnt vmcnt(0)"
+        : "=&v"(v0), "=&v"(v1)
+        : "v"(p0), "v"(p1)
+        : "memory");
+    o0 = make_uint4(v0.x, v0.y, v0.z, v0.w);
+    o1 = make_uint4(v1.x, v1.y, v1.z, v1.w);
+}
 // Four such loads in flight at once.
 __device__ __forceinline__ void ld_pair_l2_x4(const u64 *p0, const u64 *p1, const u64 *p2, const u64 *p3, uint4 &o0, uint4 &o1,
                                               uint4 &o2, uint4 &o3) {
@@ -147,6 +161,31 @@ __device__ __forceinline__ void ld_pair_l2_x4(const u64 *p0, const u64 *p1, cons
     o1 = make_uint4(v1.x, v1.y, v1.z, v1.w);
     o2 = make_uint4(v2.x, v2.y, v2.z, v2.w);
     o3 = make_uint4(v3.x, v3.y, v3.z, v3.w);
+}
+// Eight of them.
+__device__ __forceinline__ void ld_pair_l2_x8(const u64 *const (&p)[8], uint4 (&o)[8]) {
+    u32x4 v0, v1, v2, v3, v4, v5, v6, v7;
+    asm volatile(
+        "global_load_dwordx4 %0, %8, off nt\n\t"
+        "global_load_dwordx4 %1, %9, off nt\n\t"
+        "global_load_dwordx4 %2, %10, off nt\n\t"
+        "global_load_dwordx4 %3, %11, off nt\n\t"
+        "global_load_dwordx4 %4, %12, off nt\n\t"
+        "global_load_dwordx4 %5, %13, off nt\n\t"
+        "global_load_dwordx4 %6, %14, off nt\n\t"
+        "global_load_dwordx4 %7, %15, off nt\n\t"
+        "s_waitcnt vmcnt(0)"
+        : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3), "=&v"(v4), "=&v"(v5), "=&v"(v6), "=&v"(v7)
+        : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7])
+        : "memory");
+    o[0] = make_uint4(v0.x, v0.y, v0.z, v0.w);
+    o[1] = make_uint4(v1.x, v1.y, v1.z, v1.w);
+    o[2] = make_uint4(v2.x, v2.y, v2.z, v2.w);
+    o[3] = make_uint4(v3.x, v3.y, v3.z, v3.w);
+    o[4] = make_uint4(v4.x, v4.y, v4.z, v4.w);
+    o[5] = make_uint4(v5.x, v5.y, v5.z, v5.w);
+    o[6] = make_uint4(v6.x, v6.y, v6.z, v6.w);
+    o[7] = make_uint4(v7.x, v7.y, v7.z, v7.w);
 }
 // Coherent across the XCDs: four times two pairs from memory, in flight at once.
 __device__ __forceinline__ void ld_pair_mem_x4(const u64 *p0, const u64 *p1, const u64 *p2, const u64 *p3, uint4 &o0, uint4 &o1,
@@ -223,11 +262,21 @@ __device__ __forceinline__ bool spin_fail(Ctl &c, int &spins) {
 }
 
 __device__ __forceinline__ int rfl(int v) { return __builtin_amdgcn_readfirstlane(v); }
+// A pointer out of the stage table, wave-uniform.  All of them point to device memory, and the compiler is told so: a
+// pointer read from memory is otherwise taken for one that may also point into LDS, its loads become flat loads, and a
+// flat load in flight holds up every wait for LDS (the counter LDS reads use counts it too).
 template <typename P>
 __device__ __forceinline__ P *rflp(P *p) {
     const u64 v = (u64)p;
     const uint32_t lo = (uint32_t)rfl((int)(uint32_t)v), hi = (uint32_t)rfl((int)(uint32_t)(v >> 32));
-    return (P *)(((u64)hi << 32) | lo);
+    typedef __attribute__((address_space(1))) P *global_ptr;
+    return (P *)(global_ptr)(((u64)hi << 32) | lo);
+}
+
+// The tile of a layer's Linear that Linear workgroup `rank` of n_lin has (beyond n_tiles: none).
+__device__ __forceinline__ int tile_of(int rank0, int rank, int n_lin) {
+    const int t = rank - rank0;
+    return t < 0 ? t + n_lin : t;
 }
 
 // A stage's fields as wave-uniform values (the table lives in LDS).
@@ -243,7 +292,8 @@ __device__ __forceinline__ Stage load_stage(const Stage *t) {
     s.flags = rfl(t->flags);
     s.tpc = rfl(t->tpc);
     s.inv_k = __int_as_float(rfl(__float_as_int(t->inv_k)));
-    s.pad_[0] = s.pad_[1] = 0;
+    s.rank0 = rfl(t->rank0);
+    s.pad_ = 0;
     return s;
 }
 
@@ -380,27 +430,32 @@ __device__ __forceinline__ void compute_chunk(const Stage &st, const Regs &r, co
 // Lane (col, j) of wave w holds, in slot u, group (u W + w) gpw + j of column col of the workgroup's tile
 // (gpw = 4 >> tws groups per wave-wide load): a wave-wide load reads runs of 64 to 256 contiguous bytes.
 template <int MODE>
-__device__ __forceinline__ void lay_prefetch(const Stage &st, Regs &r, int rank, int wave, int lane) {
+__device__ __forceinline__ void lay_prefetch(const Stage &st, Regs &r, int tile, int wave, int lane) {
     if (MODE != 0) return;
     const int tw = 16 << st.tws, gpw = 4 >> st.tws;
     const int col = lane & (tw - 1), j = lane >> (4 + st.tws);
-    const int n = rank * tw + col;
-    const bool okc = n < st.stride;
-    const uint32_t *wp = st.packed + n;
-    const float *sp = st.scales + n;
+    const int wv = rfl(wave);
+    // a column beyond the matrix reads the last one's words: nobody looks at its sums
+    const int n = min(tile * tw + col, st.stride - 1);
+    // An address is a base that all lanes share (scalar arithmetic) plus this lane's 32-bit byte offset, the same in
+    // every round: 64-bit arithmetic per lane and load made requesting seven slots take 1.2 us.
+    const uint32_t lane_w = ((uint32_t)(4 * j) * (uint32_t)st.stride + (uint32_t)n) * 4u;
+    const uint32_t lane_s = ((uint32_t)j * (uint32_t)st.stride + (uint32_t)n) * 4u;
+    const size_t row = (size_t)st.stride * 4;  // bytes
+    const char *pw = reinterpret_cast<const char *>(st.packed), *ps = reinterpret_cast<const char *>(st.scales);
 #pragma unroll
     for (int u = 0; u < SL; ++u) {
         if (u >= st.nl) break;  // wave-uniform
-        const int g = (u * W + wave) * gpw + j;
+        const int gs = (u * W + wv) * gpw;  // the round's first group of this wave
         r.w[u][0] = r.w[u][1] = r.w[u][2] = r.w[u][3] = 0u;
         r.sc[u] = 0.0f;
-        if (okc && g < st.n_groups) {
-            const uint32_t *q = wp + (size_t)(4 * g) * st.stride;
-            r.w[u][0] = q[0];
-            r.w[u][1] = q[st.stride];
-            r.w[u][2] = q[2 * (size_t)st.stride];
-            r.w[u][3] = q[3 * (size_t)st.stride];
-            r.sc[u] = sp[(size_t)g * st.stride];
+        if (gs + j < st.n_groups) {
+            const char *bw = pw + (size_t)(4 * gs) * row;
+            r.w[u][0] = *reinterpret_cast<const uint32_t *>(bw + lane_w);
+            r.w[u][1] = *reinterpret_cast<const uint32_t *>(bw + row + lane_w);
+            r.w[u][2] = *reinterpret_cast<const uint32_t *>(bw + 2 * row + lane_w);
+            r.w[u][3] = *reinterpret_cast<const uint32_t *>(bw + 3 * row + lane_w);
+            r.sc[u] = *reinterpret_cast<const float *>(ps + (size_t)gs * row + lane_s);
         }
     }
 }
@@ -516,8 +571,36 @@ __device__ __forceinline__ void stage_input(const Params &p, const Stage &st, Ct
         }
     } else {
         const u64 *src = mirror + st.in_off;
+        static_assert(PMAX == 8, "the longest vectors are polled eight pairs of pairs at a time");
+        if (__builtin_expect(n_pairs > 4 * T, 0)) {  // workgroup-uniform
+            // more than four per thread: all eight in flight at once
+            uint4 v[8];
+            const u64 *ptr[8];
+            bool need[8];
 #pragma unroll
-        for (int b4 = 0; b4 < PMAX; b4 += 4) {
+            for (int k = 0; k < 8; ++k) {
+                const int pr = tid + k * T;
+                need[k] = pr < n_pairs;
+                ptr[k] = src + 2 * (need[k] ? pr : tid);
+                v[k] = make_uint4(0u, 0u, 0u, 0u);
+            }
+            int spins = 0;
+            while (!c.dead) {
+                uint4 t[8];
+                ld_pair_l2_x8(ptr, t);
+                bool ok = true;
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    if (need[k]) {
+                        if (pair_ok(t[k], c.epoch)) { v[k] = t[k]; need[k] = false; } else ok = false;
+                    }
+                if (ok || spin_fail(c, spins)) break;
+            }
+#pragma unroll
+            for (int k = 0; k < 8; ++k) xv[k] = make_float2(__uint_as_float(v[k].x), __uint_as_float(v[k].z));
+        } else
+#pragma unroll
+        for (int b4 = 0; b4 < 4; b4 += 4) {
             if (b4 * T >= n_pairs) break;  // workgroup-uniform
             uint4 v[4];
             const u64 *ptr[4];
@@ -535,6 +618,15 @@ __device__ __forceinline__ void stage_input(const Params &p, const Stage &st, Ct
                 while (need[0] && !c.dead) {
                     v[0] = ld_pair_l2(ptr[0]);
                     if (pair_ok(v[0], c.epoch) || spin_fail(c, spins)) break;
+                }
+            } else if (n_pairs <= (b4 + 2) * T) {
+                while (!c.dead) {
+                    uint4 t0, t1;
+                    ld_pair_l2_x2(ptr[0], ptr[1], t0, t1);
+                    bool ok = true;
+                    if (need[0]) { if (pair_ok(t0, c.epoch)) { v[0] = t0; need[0] = false; } else ok = false; }
+                    if (need[1]) { if (pair_ok(t1, c.epoch)) { v[1] = t1; need[1] = false; } else ok = false; }
+                    if (ok || spin_fail(c, spins)) break;
                 }
             } else {
                 while (!c.dead) {
@@ -622,11 +714,11 @@ __device__ __forceinline__ void stage_input(const Params &p, const Stage &st, Ct
 // store (the tile's outputs are one contiguous run), and for K and V columns the row of the cache.
 template <int MODE>
 __device__ __forceinline__ void lay_stage(const Params &p, const Stage &st, Ctl &c, const Regs &r, float *xs, float *xsum, float4 *stat,
-                                          float *red, const u64 *mirror, int pos, uint32_t tok, int rank, int tid) {
+                                          float *red, const u64 *mirror, int pos, uint32_t tok, int tile, int tid) {
     const int lane = tid & 63, wave = tid >> 6;
     const bool real = MODE == 0;
     const int tw = 16 << st.tws;
-    const int n = rank * tw + tid;
+    const int n = tile * tw + tid;
     const bool fin = tid < tw && n < st.n_valid;  // this thread finishes column n
     float bias = 0.0f, resf = 0.0f;
     u64 res = 0ull;
@@ -738,6 +830,15 @@ __device__ __forceinline__ void relay_copy(const Params &p, Ctl &c, u64 *mirror,
                 }
                 if (spin_fail(c, spins)) break;
             }
+        } else if (n_pairs <= (b4 + 2) * T) {
+            while (!c.dead) {
+                uint4 t0, t1;
+                ld_pair_mem_x2(ptr[0], ptr[1], t0, t1);
+                bool ok = true;
+                if (need[0]) { if (pair_ok(t0, c.epoch)) { *reinterpret_cast<uint4 *>(dst + 2 * (tid + (b4 + 0) * T)) = t0; need[0] = false; } else ok = false; }
+                if (need[1]) { if (pair_ok(t1, c.epoch)) { *reinterpret_cast<uint4 *>(dst + 2 * (tid + (b4 + 1) * T)) = t1; need[1] = false; } else ok = false; }
+                if (ok || spin_fail(c, spins)) break;
+            }
         } else {
             while (!c.dead) {
                 uint4 t0, t1, t2, t3;
@@ -755,12 +856,16 @@ __device__ __forceinline__ void relay_copy(const Params &p, Ctl &c, u64 *mirror,
 }
 
 // Every input vector of a Linear, in the order the step produces them, that a workgroup of this XCD reads: the tiles of
-// a layer's Linear go to the Linear workgroups XCD by XCD (`first_rank` is the first of this XCD's), the head to everybody.
-__device__ __forceinline__ void relay_role(const Params &p, const Stage *tab, Ctl &c, u64 *mirror, int tid, int phase, int first_rank) {
+// a layer's Linear go to the Linear workgroups rank by rank from the stage's first (`first_rank` is the first of this XCD's),
+// the head to everybody.
+__device__ __forceinline__ void relay_role(const Params &p, const Stage *tab, Ctl &c, u64 *mirror, int tid, int phase, int first_rank,
+                                           int lin_per_xcd) {
     for (int s = 0; s < p.n_stages; ++s) {
         c.stage = s;
         const int in_off = rfl(tab[s].in_off), K = rfl(tab[s].K);
-        const bool wanted = (rfl(tab[s].flags) & F_HEAD) || first_rank < rfl(tab[s].n_tiles);
+        // the XCD's workgroups have the tiles t0, t0 + 1, ..., and from where the ranks wrap around, 0, 1, ...
+        const int t0 = tile_of(rfl(tab[s].rank0), first_rank, 8 * lin_per_xcd);
+        const bool wanted = (rfl(tab[s].flags) & F_HEAD) || t0 < rfl(tab[s].n_tiles) || t0 + lin_per_xcd > 8 * lin_per_xcd;
         if (in_off >= 0 && wanted) relay_copy(p, c, mirror, in_off, K, tid, phase);
     }
 }
@@ -1049,9 +1154,9 @@ __device__ __forceinline__ void head_ahead_step(const Stage *th, HeadAhead &ha, 
 }
 
 // First stage from `from` on, before the head, in which workgroup `rank` has a tile; the head (n_lay) if none.
-__device__ __forceinline__ int next_active(const Stage *tab, int from, int rank, int n_lay) {
+__device__ __forceinline__ int next_active(const Stage *tab, int from, int rank, int n_lin, int n_lay) {
     int s = from;
-    while (s < n_lay && rfl(tab[s].n_tiles) <= rank) ++s;
+    while (s < n_lay && rfl(tab[s].n_tiles) <= tile_of(rfl(tab[s].rank0), rank, n_lin)) ++s;
     return s;
 }
 
@@ -1105,7 +1210,8 @@ __global__ __launch_bounds__(T) void decode_step_kernel(const Params p) {
     const int per_xcd = G >> 3;
     u64 *mirror = p.arena + (size_t)(1 + xcd) * p.arena_elems;
     if (in_xcd < NRELAY) {
-        relay_role(p, tab, c, mirror, tid, in_xcd, xcd * (per_xcd - NRELAY - p.att_per_xcd));
+        const int lpx = per_xcd - NRELAY - p.att_per_xcd;
+        relay_role(p, tab, c, mirror, tid, in_xcd, xcd * lpx, lpx);
         PK_DUMP();
         return;
     }
@@ -1128,10 +1234,10 @@ __global__ __launch_bounds__(T) void decode_step_kernel(const Params p) {
     // ---- Linears: the stages of the layers in which this workgroup has a tile (one at most), then the head ----
     Regs regs;
     const int n_lay = p.n_stages - 1;
-    int s = is_att ? n_lay : next_active(tab, 0, rank, n_lay);
+    int s = is_att ? n_lay : next_active(tab, 0, rank, n_lin, n_lay);
     int n_enter = 0;  // staging buffers are used in turn
     Stage st = load_stage(tab + s);
-    if (s < n_lay) lay_prefetch<MODE>(st, regs, rank, wave, lane);
+    if (s < n_lay) lay_prefetch<MODE>(st, regs, tile_of(st.rank0, rank, n_lin), wave, lane);
     HeadAhead ha;
     ha.n_slots = ha.s = ha.tt = ha.u = 0;
     ha.pending = -1;
@@ -1144,12 +1250,13 @@ __global__ __launch_bounds__(T) void decode_step_kernel(const Params p) {
     while (s < n_lay) {
         c.stage = s;
         lay_stage<MODE>(p, st, c, regs, L.xs + (n_enter & 1) * p.xbuf, L.xsum + (n_enter & 1) * (XMAX / 32), L.stat,
-                        L.red + (n_enter & 1) * (SL * W * 64), mirror, pos, tok, rank, tid);
+                        L.red + (n_enter & 1) * (SL * W * 64), mirror, pos, tok, tile_of(st.rank0, rank, n_lin), tid);
         // the outputs are on their way: now the next stage this workgroup takes part in, and its weights
         ++n_enter;
-        s = next_active(tab, s + 1, rank, n_lay);
+        s = next_active(tab, s + 1, rank, n_lin, n_lay);
         st = load_stage(tab + s);
-        if (s < n_lay) lay_prefetch<MODE>(st, regs, rank, wave, lane);
+        PK_STAMP(6);
+        if (s < n_lay) lay_prefetch<MODE>(st, regs, tile_of(st.rank0, rank, n_lin), wave, lane);
         if (MODE == 0) head_ahead_step(tab + n_lay, ha, L.hl, rank, wave, lane, tid);
         PK_STAMP(5);
     }
@@ -1340,6 +1447,14 @@ int32_t agpu_pk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
     st.reserve((size_t)4 * m.n_layer + 1);
     const int gelu = m.gelu_quick ? F_GELU_QUICK : F_GELU_TANH;
     int prev_h2 = -2;
+    // A stage's tiles go to the workgroups after those of the stage before it, so that two stages in a row share as few
+    // workgroups as possible: a workgroup requests the weights of its next stage when it has published the one before,
+    // and they are late when that is the stage right behind.
+    int next_rank0 = 0;
+    auto place = [&](Stage &s) {
+        s.rank0 = next_rank0;
+        next_rank0 = (next_rank0 + s.n_tiles) % r.n_lin;
+    };
     for (int L = 0; L < m.n_layer; ++L) {
         const PkLayer &y = m.layers[L];
         const int base = (int)(per_layer * L);
@@ -1348,18 +1463,22 @@ int32_t agpu_pk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
         plan_linear(s, y.qkv, r.n_lin, false);
         s.in_off = prev_h2; s.out_off = o_qkv; s.flags = F_LN | F_SCATTER; s.ln_g = y.ln1_g; s.ln_b = y.ln1_b;
         s.kc = y.kcache; s.vc = y.vcache; s.att_off = o_att; s.part_off = o_part;
+        place(s);
         st.push_back(s);
         s = Stage{};
         plan_linear(s, y.proj, r.n_lin, false);
         s.in_off = o_att; s.out_off = o_h1; s.res_off = prev_h2;
+        place(s);
         st.push_back(s);
         s = Stage{};
         plan_linear(s, y.fc, r.n_lin, false);
         s.in_off = o_h1; s.out_off = o_ffn; s.flags = F_LN | gelu; s.ln_g = y.ln2_g; s.ln_b = y.ln2_b;
+        place(s);
         st.push_back(s);
         s = Stage{};
         plan_linear(s, y.fc_proj, r.n_lin, false);
         s.in_off = o_ffn; s.out_off = o_h2; s.res_off = o_h1;
+        place(s);
         st.push_back(s);
         prev_h2 = o_h2;
     }
