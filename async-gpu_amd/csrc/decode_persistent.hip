@@ -64,7 +64,7 @@ constexpr int DH = 64;
 constexpr int NRELAY = 4;       // relay workgroups per XCD: they poll a short vector out of step (the first to see a pair copies it)
                                 // and share out a long one
 
-enum : int { F_LN = 1, F_GELU_TANH = 2, F_GELU_QUICK = 4, F_HEAD = 8, F_SCATTER = 16 };
+enum : int { F_LN = 1, F_GELU_TANH = 2, F_GELU_QUICK = 4, F_HEAD = 8, F_SCATTER = 16, F_WARM = 32 };
 
 // One Linear of the step.  The QKV entry of a layer also carries what the layer's attention needs.
 struct Stage {
@@ -708,13 +708,33 @@ __device__ __forceinline__ void stage_input(const Params &p, const Stage &st, Ct
     PK_STAMP(2);
 }
 
+// One word of every cache line of the weights that tile `tile` of stage `e` consists of (two of the packed words and one
+// of the scales per thread at most): they then wait in the XCD's L2.  For a workgroup with tiles in two stages in a
+// row: it can request the second one's weights into registers only when it has published the first, and from memory
+// they then arrive after the input.  The words are handed back so that the caller can keep them until a wait it has anyway.
+template <int MODE>
+__device__ __forceinline__ void warm_tile(const Stage *e, int tile, int tid, uint32_t (&sink)[3]) {
+    if (MODE != 0) return;
+    const uint32_t *packed = rflp(e->packed);
+    const uint32_t *scales = reinterpret_cast<const uint32_t *>(rflp(e->scales));
+    const int stride = rfl(e->stride), K = rfl(e->K), tws = rfl(e->tws);
+    const int tw = 16 << tws, sh = tws == 2 ? 1 : 0;  // a tile's row of words: 64, 128 or 256 bytes = 1, 1 or 2 lines
+    const int n_w = (K >> 3) << sh, n_s = (K >> 5) << sh;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const int i = tid + k * T;
+        if (i < n_w) sink[k] = packed[(size_t)(i >> sh) * stride + min(tile * tw + 32 * (i & sh), stride - 1)];
+    }
+    if (tid < n_s) sink[2] = scales[(size_t)(tid >> sh) * stride + min(tile * tw + 32 * (tid & sh), stride - 1)];
+}
+
 // ---- one Linear of a layer, for a workgroup that has a tile of it ----
 // Thread col of the tile requests the column's bias and residual first; then the input; then every lane its groups
 // of its column; the waves' sums meet in LDS and thread col finishes the column: bias, GELU, residual, the tagged
 // store (the tile's outputs are one contiguous run), and for K and V columns the row of the cache.
 template <int MODE>
 __device__ __forceinline__ void lay_stage(const Params &p, const Stage &st, Ctl &c, const Regs &r, float *xs, float *xsum, float4 *stat,
-                                          float *red, const u64 *mirror, int pos, uint32_t tok, int tile, int tid) {
+                                          float *red, const u64 *mirror, int pos, uint32_t tok, int tile, int tid, uint32_t (&sink)[3]) {
     const int lane = tid & 63, wave = tid >> 6;
     const bool real = MODE == 0;
     const int tw = 16 << st.tws;
@@ -728,7 +748,8 @@ __device__ __forceinline__ void lay_stage(const Params &p, const Stage &st, Ctl 
         else if (st.res_off == -2 && real) resf = p.wte[(size_t)tok * p.d + n] + p.wpe[(size_t)pos * p.d + n];
     }
     PK_STAMP(0);
-    stage_input<MODE>(p, st, c, xs, xsum, stat, mirror, pos, tok, tid, [&] { asm volatile("" ::"v"(bias), "v"(resf), "v"(res)); });
+    stage_input<MODE>(p, st, c, xs, xsum, stat, mirror, pos, tok, tid,
+                      [&] { asm volatile("" ::"v"(bias), "v"(resf), "v"(res), "v"(sink[0]), "v"(sink[1]), "v"(sink[2])); });
     if (real) {
         const float part = lay_compute(st, r, xs, xsum, wave, lane);
         if (lane < tw) red[wave * 64 + lane] = part;
@@ -1247,16 +1268,22 @@ __global__ __launch_bounds__(T) void decode_step_kernel(const Params p) {
         const int my_tiles = rank < n_tiles ? (n_tiles - rank + n_wgs - 1) / n_wgs : 0;
         ha.n_slots = min(p.head_slots, min(tpc, max(0, my_tiles - tpc)) * rfl(th->nl));
     }
+    uint32_t sink[3] = {0u, 0u, 0u};
     while (s < n_lay) {
         c.stage = s;
         lay_stage<MODE>(p, st, c, regs, L.xs + (n_enter & 1) * p.xbuf, L.xsum + (n_enter & 1) * (XMAX / 32), L.stat,
-                        L.red + (n_enter & 1) * (SL * W * 64), mirror, pos, tok, tile_of(st.rank0, rank, n_lin), tid);
+                        L.red + (n_enter & 1) * (SL * W * 64), mirror, pos, tok, tile_of(st.rank0, rank, n_lin), tid, sink);
         // the outputs are on their way: now the next stage this workgroup takes part in, and its weights
         ++n_enter;
         s = next_active(tab, s + 1, rank, n_lin, n_lay);
         st = load_stage(tab + s);
         PK_STAMP(6);
         if (s < n_lay) lay_prefetch<MODE>(st, regs, tile_of(st.rank0, rank, n_lin), wave, lane);
+        // a large tile in the stage right behind that one as well: its weights go to the L2 now
+        if (s + 1 < n_lay && (rfl(tab[s + 1].flags) & F_WARM)) {
+            const int t2 = tile_of(rfl(tab[s + 1].rank0), rank, n_lin);
+            if (t2 < rfl(tab[s + 1].n_tiles)) warm_tile<MODE>(tab + s + 1, t2, tid, sink);
+        }
         if (MODE == 0) head_ahead_step(tab + n_lay, ha, L.hl, rank, wave, lane, tid);
         PK_STAMP(5);
     }
@@ -1452,6 +1479,8 @@ int32_t agpu_pk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
     // and they are late when that is the stage right behind.
     int next_rank0 = 0;
     auto place = [&](Stage &s) {
+        // a tile of 32 KB or more: worth touching ahead of time where a workgroup comes to it straight from the stage before
+        if ((size_t)(16 << s.tws) * s.K / 2 >= (size_t)32 * 1024) s.flags |= F_WARM;
         s.rank0 = next_rank0;
         next_rank0 = (next_rank0 + s.n_tiles) % r.n_lin;
     };
