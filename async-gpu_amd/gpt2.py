@@ -191,6 +191,15 @@ class Int4Gpt2Model:
         self._call("agpu_gpt2_generate_cached", prompt, B, n, max_new_tokens, eos, out, lens, ms)
         return [out[b, :lens[b]].copy() for b in range(B)], (float(ms[0]), float(ms[1]))
 
+    def generate_text(self, tokenizer, prompt, max_new_tokens, eos=50256):
+        """Text in, text out, as the reference's callers do around the model (tokenizer.encode(prompt) -> tokens ->
+        generate -> tokenizer.decode, gpt2.rs:1619-1630, 1790-1836): greedy continuation of `prompt`, prompt included."""
+        tokens = tokenizer.encode(prompt)
+        if not tokens:
+            raise ValueError("empty prompt")
+        (out,), _ = self.generate_cached(np.asarray(tokens, np.uint32), max_new_tokens, eos=eos)
+        return tokenizer.decode(out.tolist())
+
     def generate_cached_sampling(self, prompt, max_new_tokens, top_k, temperature, rng, eos=50256):
         """Int4Gpt2Model::generate_cached_sampling (gpt2.rs:931-977); rng is an ops.SimpleRng and is advanced."""
         prompt = _np(prompt, np.uint32).ravel()

@@ -285,3 +285,28 @@ def test_decode_step_picks_the_token_itself(orc, agpu, dev, last):
         ties = np.flatnonzero(logits == logits.max())
         assert ties.size >= 2
         assert tokens[t] == (ties[-1] if last else ties[0]), (t, ties)
+
+
+def test_generate_text_through_the_tokenizer(tiny, orc):
+    """Text -> tokens -> model -> tokens -> text, as the reference's callers chain them (gpt2.rs:1619-1630): the
+    tokenizer's ids drive the same greedy run as the ids given directly, and the oracle agrees on them.  The
+    vocabulary is a byte-level one without merges (no vocabulary file is in the image) cut to the tiny model's size."""
+    from async_gpu_amd import tokenizer as T
+    cfg, w, qz, om, gm = tiny
+    tok = T.Gpt2Tokenizer({bytes([b]): i for i, b in enumerate(T.bytes_to_unicode())}, special_tokens={})
+    assert tok.vocab_size() == 256 <= cfg["vocab"]
+    prompt = "GPU "
+    ids = tok.encode(prompt)
+    ref, margins = om.generate(np.asarray(ids, np.uint32), 10, cached=True, eos=-1)
+    (got,), _ = gm.generate_cached(np.asarray(ids, np.uint32), 10, eos=-1)
+    _assert_tokens_match(got, ref, margins, len(ids), "generate_cached on tokenizer ids")
+    if all(t < 256 for t in got):
+        try:
+            text = tok.decode(got.tolist())
+        except T.TokenizerError:
+            text = None  # the random model may emit bytes that are no UTF-8: decode must say so, not guess
+        if text is not None:
+            assert gm.generate_text(tok, prompt, 10, eos=-1) == text and text.startswith(prompt)
+    else:
+        with pytest.raises(T.TokenizerError):
+            gm.generate_text(tok, prompt, 10, eos=-1)
