@@ -37,8 +37,8 @@ def dev():
 
 
 def progress(msg):
-    """A line for long GPU tests: printed, and appended to gpurun_out/test_progress.log so that a run whose output
-    pytest captures still shows signs of life on the GPU box."""
+    """A line for long GPU tests: printed, and appended to a progress log in the run's output folder, so that a run
+    whose output pytest captures still shows signs of life."""
     import time
     line = f"[{time.strftime('%H:%M:%S')}] {msg}"
     print(line, flush=True)
