@@ -56,6 +56,30 @@ def test_one_launch_equals_per_stage_and_oracle(orc, agpu, dev, options):
     assert gm.decode_floor(8) > 0.0
 
 
+@pytest.mark.parametrize("d,heads", [(1024, 16), (1280, 20), (1600, 25), (192, 3), (512, 8)])
+def test_one_launch_other_model_widths(orc, agpu, dev, d, heads):
+    """Widths between the two benchmark models (GPT-2 medium, large, XL) and below them: other tile widths, other numbers
+    of tiles per stage (so the stages start at other workgroups and share other ones), tiles above and below the size
+    from which a second stage in a row is touched ahead.  Three layers; tokens against the per-stage path and the oracle."""
+    from async_gpu_amd import gpt2, workloads
+    cfg = dict(n_layer=3, n_embd=d, n_head=heads, vocab=2003, n_positions=96)
+    w = workloads.gpt2_fp32_weights(cfg, 5, std=0.05, nonzero_bias=True, random_ln=True)
+    qz = workloads.quantize_gpt2(w, 32, lambda wt, g: orc.quantize_weight_int4(wt, g, orc.SCRIPT))
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg), qz)
+    prompt = workloads.random_prompt(cfg, 2, 9)
+    gm.set_decode_mode(gm.DECODE_PER_STAGE)
+    (a,), _ = gm.generate_cached(prompt, 24, eos=-1)
+    la = gm.last_logits()
+    gm.set_decode_mode(gm.DECODE_AUTO)
+    (b,), _ = gm.generate_cached(prompt, 24, eos=-1)
+    assert gm.decode_is_one_launch()
+    assert np.array_equal(a, b)
+    assert np.abs(la - gm.last_logits()).max() <= 2e-5
+    om = build_oracle_model(cfg, qz)
+    ref, margins = om.generate(prompt, 24, cached=True, eos=-1)
+    _match(b, ref, margins, 9, f"one-launch step, d={d}")
+
+
 @pytest.mark.parametrize("batch", [1, 3])
 def test_eager_steps_equal_graph_replays(orc, agpu, dev, batch):
     """The per-stage step launched kernel by kernel gives the bits of its graph replay."""
