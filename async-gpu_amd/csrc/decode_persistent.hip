@@ -31,7 +31,10 @@
 // reads runs of 64 to 256 contiguous bytes and a lane's 32 products need one scale and no other lane.  The input
 // vector is staged in LDS together with the sum of every group (the zero point 8 comes off per group:
 // u = sum x n - 8 sum x, acc += scale u); fp32 FMAs on the unsigned nibbles; lanes of one column are added with the
-// gfx950 row swaps, waves through LDS in wave order.
+// gfx950 row swaps, waves through LDS in wave order.  A stage's tiles are dealt to the Linear workgroups starting where
+// the stage before it ended, so that few workgroups have tiles in two stages in a row: such a workgroup can request the
+// second stage's weights only when it has published the first, and then they arrive after the input.  Where it cannot
+// be avoided and the tile is large, the workgroup touches the tile's cache lines a stage earlier (warm_tile).
 //
 // Every wait is bounded: a poll that does not succeed within kSpinLimit rounds sets the error word, all
 // workgroups then stop waiting, and the step ends with garbage that the host reports as an error.
