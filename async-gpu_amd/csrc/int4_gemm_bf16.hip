@@ -20,8 +20,10 @@
 //   A fragment: lane (i, hh) = row i, the 8 k of half hh of a 16-k step
 //   B fragment: lane (j, hh) = column j, the same 8 k: packed row 4 * chunk + 2 * step + hh
 //   D: register r of lane (j, hh) = row 8 * (r / 4) + 4 * hh + r % 4, column j
-// With fewer tiles than the chip has room for, K is sliced over gridDim.z workgroups per tile: partial sums go
-// out past the L2, the last workgroup of a tile to take a ticket adds them in slice order.
+// With fewer tiles than the chip has room for, K is sliced over several workgroups per tile: partial sums go
+// out past the L2, the last workgroup of a tile to take a ticket adds them in slice order.  With more tiles than CUs
+// but not a multiple of them, only the tiles left over after whole rounds are sliced, in the same launch (the grid is
+// one-dimensional: whole tiles first, then the slices), so that every CU gets the same share of them.
 #include "linear_common.h"
 #include <type_traits>
 
@@ -41,8 +43,11 @@ struct GemmBfParams {
     float *y;
     int M, N, K, chunk_shift;
     uint32_t flags;
-    int blocks_per_split;    // K blocks of 64 per workgroup (gridDim.z slices of K)
-    float *partial;          // [ksplit, M, N] when gridDim.z > 1
+    int blocks_per_split;    // K blocks per workgroup of a tile whose K is sliced
+    int col_tiles;           // tiles per row of tiles; tile t = (t / col_tiles, t % col_tiles)
+    int full_tiles;          // tiles 0 .. full_tiles - 1 have one workgroup each, the others tail_ks workgroups (slices of K)
+    int tail_ks, n_tail;     // ... and how many tiles those others are
+    float *partial;          // [tail_ks, n_tail tiles] partial results
     unsigned int *counters;  // one ticket per output tile, left at zero
     KvScatter kv;            // kcache == nullptr: none
     int strict;              // the context's strict_sync
@@ -82,9 +87,18 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
     __shared__ int s_last;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int j = lane & 31, hh = lane >> 5;
-    const int m0 = blockIdx.y * GB_BM, n0 = blockIdx.x * GB_BN + wave * 32 * CB;
     const int chunks = p.K / 32, kblocks = (chunks + NCH - 1) / NCH;
-    const int ksplit = gridDim.z, kb0 = blockIdx.z * p.blocks_per_split, kb1 = min(kblocks, kb0 + p.blocks_per_split);
+    // workgroup -> (tile, slice of K): whole tiles first, then the slices of the remaining tiles
+    int tile_no, split, ksplit, bps;
+    if ((int)blockIdx.x < p.full_tiles) {
+        tile_no = blockIdx.x; split = 0; ksplit = 1; bps = kblocks;
+    } else {
+        const int t = blockIdx.x - p.full_tiles, q = t / p.tail_ks;
+        tile_no = p.full_tiles + q; split = t - q * p.tail_ks; ksplit = p.tail_ks; bps = p.blocks_per_split;
+    }
+    const int tile_row = tile_no / p.col_tiles, tile_col = tile_no - tile_row * p.col_tiles;
+    const int m0 = tile_row * GB_BM, n0 = tile_col * GB_BN + wave * 32 * CB;
+    const int kb0 = split * bps, kb1 = min(kblocks, kb0 + bps);
     const bool wave_active = n0 < p.N;
     int col[CB];  // out-of-range columns read the last one and are not stored
 #pragma unroll
@@ -246,10 +260,10 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
     if (ksplit > 1) {
         // Partial sums live in the order of the registers: [slice][tile][wave][rb][cb][pair of r][lane] 8-byte
         // words, so that a wave writes and reads whole 512-byte lines with constant offsets from one address.
-        const int tile = blockIdx.y * gridDim.x + blockIdx.x, tiles = gridDim.x * gridDim.y;
+        const int tile = tile_no - p.full_tiles, tiles = p.n_tail;
         constexpr int kWaveWords = RB * CB * 8 * 64;  // 8-byte words of one wave's results
         unsigned long long *mine = reinterpret_cast<unsigned long long *>(p.partial) +
-                                   ((size_t)(blockIdx.z * tiles + tile) * GB_WAVES + wave) * kWaveWords + lane;
+                                   ((size_t)(split * tiles + tile) * GB_WAVES + wave) * kWaveWords + lane;
         if (wave_active) {
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb)
@@ -273,7 +287,7 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
         if (!s_last) return;
         if (wave_active) {
             const size_t slice_words = (size_t)tiles * GB_WAVES * kWaveWords;
-            const unsigned long long *first = mine - (size_t)blockIdx.z * slice_words;
+            const unsigned long long *first = mine - (size_t)split * slice_words;
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
@@ -384,9 +398,34 @@ int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t
     while (ksplit > 1 && (size_t)ksplit * tiles * BM * BN * sizeof(float) > ctx->ws_bytes / 2) --ksplit;
     p.blocks_per_split = ceil_div(kblocks, ksplit);
     ksplit = ceil_div(kblocks, p.blocks_per_split);
+    p.col_tiles = ceil_div(N, BN);
+    p.full_tiles = ksplit > 1 ? 0 : tiles;
+    p.tail_ks = ksplit;
+    // More tiles than CUs, not a multiple of them: every CU runs the same number of whole tiles, and the tiles left over
+    // (M = 1024, N = 2304: 64 of 576) are sliced so finely that every CU gets the same share of them too; otherwise the
+    // CUs with one tile more set the time (the 2304-column Linear took as long as the 3072-column one).
+    if (ksplit == 1 && tiles > ctx->num_cus && tiles % ctx->num_cus != 0) {
+        const int rem = tiles % ctx->num_cus;
+        int best_ks = 1;
+        float best_c = (float)kblocks * (KB / 64) + 2.2f;
+        for (int ks = 2; ks <= 8 && ks <= kblocks; ++ks) {
+            const int bps = ceil_div(kblocks, ks), ks2 = ceil_div(kblocks, bps);
+            const float c = (float)ceil_div(rem * ks2, ctx->num_cus) * (bps * (KB / 64) + 2.2f) + 0.75f + 0.18f * ks2;
+            if (c < best_c - 1.5f) {
+                best_c = c;
+                best_ks = ks2;
+            }
+        }
+        if (best_ks > 1 && rem <= ctx->n_counters && (size_t)best_ks * rem * BM * BN * sizeof(float) <= ctx->ws_bytes / 2) {
+            p.full_tiles = tiles - rem;
+            p.tail_ks = best_ks;
+            p.blocks_per_split = ceil_div(kblocks, best_ks);
+        }
+    }
+    p.n_tail = tiles - p.full_tiles;
     p.partial = reinterpret_cast<float *>(ctx->workspace);
     p.counters = ctx->counters;
-    const dim3 grid(ceil_div(N, BN), ceil_div(M, BM), ksplit);
+    const dim3 grid(p.full_tiles + p.n_tail * p.tail_ks);
     if (large) hipLaunchKernelGGL((int4_gemm_bf16_kernel<2, 2, 2, 4>), grid, dim3(256), 0, ctx->stream, p);
     else if (wide) hipLaunchKernelGGL((int4_gemm_bf16_kernel<1, 1, 2, 8>), grid, dim3(512), 0, ctx->stream, p);
     else if (long_blocks) hipLaunchKernelGGL((int4_gemm_bf16_kernel<1, 1, 4, 4>), grid, dim3(256), 0, ctx->stream, p);
