@@ -93,8 +93,10 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
     if ((int)blockIdx.x < p.full_tiles) {
         tile_no = blockIdx.x; split = 0; ksplit = 1; bps = kblocks;
     } else {
-        const int t = blockIdx.x - p.full_tiles, q = t / p.tail_ks;
-        tile_no = p.full_tiles + q; split = t - q * p.tail_ks; ksplit = p.tail_ks; bps = p.blocks_per_split;
+        // slice-major: neighbours in the grid are neighbouring tiles of one slice of K, which read the same rows of x or
+        // the same weights (tile-major order cost the 3072 -> 768 Linear 3 us of 31)
+        const int t = blockIdx.x - p.full_tiles;
+        split = t / p.n_tail; tile_no = p.full_tiles + (t - split * p.n_tail); ksplit = p.tail_ks; bps = p.blocks_per_split;
     }
     const int tile_row = tile_no / p.col_tiles, tile_col = tile_no - tile_row * p.col_tiles;
     const int m0 = tile_row * GB_BM, n0 = tile_col * GB_BN + wave * 32 * CB;
@@ -406,16 +408,21 @@ int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t
     // CUs with one tile more set the time (the 2304-column Linear took as long as the 3072-column one).
     if (ksplit == 1 && tiles > ctx->num_cus && tiles % ctx->num_cus != 0) {
         const int rem = tiles % ctx->num_cus;
+        // the leftover tiles' share of the time, in the units of the model above: unsliced, a whole tile more for some CUs
+        const float whole = (float)kblocks * (KB / 64) + 2.2f;
         int best_ks = 1;
-        float best_c = (float)kblocks * (KB / 64) + 2.2f;
+        float best_c = whole;
         for (int ks = 2; ks <= 8 && ks <= kblocks; ++ks) {
             const int bps = ceil_div(kblocks, ks), ks2 = ceil_div(kblocks, bps);
-            const float c = (float)ceil_div(rem * ks2, ctx->num_cus) * (bps * (KB / 64) + 2.2f) + 0.75f + 0.18f * ks2;
-            if (c < best_c - 1.5f) {
+            // a slice more costs more here than above: the last workgroup of a tile reads them all while its CU's
+            // other workgroups are at work (measured, 64 tiles left over of 576: 2, 3, 4, 6 slices = 23.5, 22.6, 22.1, 22.4 us)
+            const float c = (float)ceil_div(rem * ks2, ctx->num_cus) * (bps * (KB / 64) + 2.2f) + 0.75f + 0.5f * ks2;
+            if (c < best_c) {
                 best_c = c;
                 best_ks = ks2;
             }
         }
+        if (best_c > whole - 1.5f) best_ks = 1;  // not worth the partial sums
         if (best_ks > 1 && rem <= ctx->n_counters && (size_t)best_ks * rem * BM * BN * sizeof(float) <= ctx->ws_bytes / 2) {
             p.full_tiles = tiles - rem;
             p.tail_ks = best_ks;
