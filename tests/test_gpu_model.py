@@ -310,3 +310,29 @@ def test_generate_text_through_the_tokenizer(tiny, orc):
     else:
         with pytest.raises(T.TokenizerError):
             gm.generate_text(tok, prompt, 10, eos=-1)
+
+
+@pytest.mark.parametrize("prompt_len", [600, 1000])
+def test_long_prefill_small_width(orc, agpu, dev, prompt_len):
+    """GPT-2 small's width with prompts of many rows: the QKV Linear then has more tiles than the chip has CUs and the
+    tiles left over after whole rounds are sliced along K, K/V rows of those tiles included (they go into the cache from
+    the workgroup that adds the slices up).  Last-row logits and the next tokens, which read that cache, against the
+    oracle; a prefill in chunks, whose Linears have fewer tiles and no slices, must give the same tokens."""
+    from async_gpu_amd import gpt2, workloads
+    cfg = dict(n_layer=2, n_embd=768, n_head=12, vocab=1031, n_positions=1024)
+    w, qz = _quantized(orc, cfg, 17, nonzero_bias=True, random_ln=True)
+    om = build_oracle_model(cfg, qz)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg), qz)
+    prompt = workloads.random_prompt(cfg, 5, prompt_len)
+    gm.reset_cache()
+    lg = gm.forward_cached(prompt.reshape(1, -1))[0]
+    om.reset_cache()
+    lo = om.forward(prompt, all_rows=False)
+    assert np.abs(lg[-1] - lo[0]).max() <= TOL_LOGITS
+    ref, margins = om.generate(prompt, 8, cached=True, eos=-1)
+    (got,), _ = gm.generate_cached(prompt, 8, eos=-1)
+    _assert_tokens_match(got, ref, margins, prompt_len, f"prefill of {prompt_len} rows")
+    gm.reset_cache()
+    for lo_i in range(0, prompt_len, 250):
+        lc = gm.forward_cached(prompt[lo_i:lo_i + 250].reshape(1, -1))[0]
+    assert np.abs(lc[-1] - lg[-1]).max() <= 2e-5
