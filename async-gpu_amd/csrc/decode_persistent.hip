@@ -441,7 +441,8 @@ __device__ __forceinline__ void lay_prefetch(const Stage &st, Regs &r, int tile,
     // a column beyond the matrix reads the last one's words: nobody looks at its sums
     const int n = min(tile * tw + col, st.stride - 1);
     // An address is a base that all lanes share (scalar arithmetic) plus this lane's 32-bit byte offset, the same in
-    // every round: 64-bit arithmetic per lane and load made requesting seven slots take 1.2 us.
+    // every round: one vector instruction per load instead of 64-bit arithmetic per lane.  (Requesting seven slots still
+    // takes a wave 1.2 us: the loads queue behind those of the workgroup's other waves.)
     const uint32_t lane_w = ((uint32_t)(4 * j) * (uint32_t)st.stride + (uint32_t)n) * 4u;
     const uint32_t lane_s = ((uint32_t)j * (uint32_t)st.stride + (uint32_t)n) * 4u;
     const size_t row = (size_t)st.stride * 4;  // bytes
