@@ -1,8 +1,9 @@
 // Prefill GEMM of the int4 weight-only Linear (M > 16 rows) on the bf16 matrix cores of gfx950, at fp32 accuracy.
 //
 // An fp32 x is the exact sum of three bf16 numbers (8 + 8 + 8 significant bits: x = hi + mid + lo, each the leading
-// bits of what the previous ones left; below about 2^-110 the smallest piece underflows, which no error bound
-// notices), and the weights q - 8 in [-8, 7] are bf16 numbers as they are.  So
+// bits of what the previous ones left; below about 2^-106 the smallest piece's products underflow, which no error
+// bound notices), and the weights q - 8 in [-8, 7] are bf16 numbers as they are (the kernel holds them as (q - 8) / 16
+// and the scales as 16 * scale, which is what the conversion instruction gives).  So
 //     sum_k x[k] * (q[k] - 8)  =  sum over the three pieces of  sum_k piece[k] * (q[k] - 8)
 // with every product exact in fp32: three v_mfma_f32_32x32x16_bf16 per 16 k replace the multiply-adds of the fp32
 // reference, and only the additions round (fp32 accumulation inside the matrix core, smallest piece first).

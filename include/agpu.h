@@ -144,6 +144,11 @@ int32_t agpu_kernel_lookup(const agpu_ctx *ctx, const char *name, const char **e
  * alone; a row holding NaN or Inf gives NaN in every output of that row.  Results stay within
  * 4e-7 * sum_k |x_k| |w_kn| of the exact dot product, tighter than the reference's fp32 chain.
  * AGPU_EPI_FORCE_FP32_GEMV selects the plain fp32 kernels instead.
+ *
+ * Arithmetic for M > 16 (prefill): x is taken as the exact sum of three bf16 numbers and multiplied with the weights
+ * (q - 8) / 16 on the bf16 matrix cores, every product exact; a group's sum is then scaled by 16 * scale.  Only
+ * the additions round (fp32).  A caller can observe: a group scale of 2^124 or more gives Inf (16 * scale
+ * overflows), and the parts of an x below 2^-106 are lost.
  */
 int32_t agpu_int4_linear(agpu_ctx *ctx, const float *x, const uint32_t *packed, const float *scales,
                          const float *bias, const float *residual, float *y, int32_t M, int32_t N,
