@@ -28,3 +28,9 @@ struct AttnParams {
 
 // max_kv_len bounds kv_len for launches that read it from pos_dev (sizes the key split).
 int32_t agpu_attention_launch(agpu_ctx *ctx, const AttnParams &p, int max_kv_len);
+
+// Causal prefill attention of queries 0 .. q_len - 1 over keys 0 .. kv_len - 1 (kv_len >= q_len >= 256, host values; p.k and
+// p.v are not read) with K and V given as bf16 operand fragments: [batch * n_heads][tiles_cap tiles of 32 keys][768
+// fragments of 16 bytes] each, in the layout attention.hip describes; agpu_attention_fragment_bytes sizes one array.
+size_t agpu_attention_fragment_bytes(int heads, int kv_len);
+int32_t agpu_attention_fragments_launch(agpu_ctx *ctx, const AttnParams &p, const uint4 *kfrag, const uint4 *vfrag, int tiles_cap);

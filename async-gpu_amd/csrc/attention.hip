@@ -261,6 +261,211 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(const AttnParams p) {
     }  // query blocks of this workgroup
 }
 
+// ---- prefill attention on the bf16 matrix cores, at fp32 accuracy ----
+// An fp32 number is the exact sum of three bf16 numbers (hi + mid + lo, 8 significant bits each), so a product of two
+// fp32 numbers is the sum of nine exact bf16 products, of which the six with hi in them or mid * mid carry all but the
+// last bit or two of 48.  S^T = K Q^T and O^T = V^T P^T then take 6 v_mfma_f32_32x32x16_bf16 per 16 terms of the sum
+// (8 passes each) where the fp32 kernel above takes 8 v_mfma_f32_32x32x2_f32 (16 passes each).  The operands come as
+// fragments, 16 bytes per lane and instruction, pieces 0 = hi, 1 = mid, 2 = lo:
+//   K: [head][tile of 32 keys][d step ds of 16][piece][half hh][key i]     8 bf16: d = 16 ds + 8 hh + e
+//   V: [head][tile][d block of 32][piece][key step s][half hh][d i]         8 bf16: key = att_vkey(s, hh, e)
+// written once per prefill (by split_kv_kernel, or by the GEMM that produces K and V), read straight into registers
+// with one 1 KiB request per wave and instruction.  att_vkey is the order in which a 32 x 32 MFMA result holds its
+// rows: the probabilities of a key tile come out of the first product in exactly the layout the second one wants.
+typedef __bf16 att_bf16x8 __attribute__((ext_vector_type(8)));
+constexpr int ATT_FRAGS_PER_TILE = 4 * 3 * 2 * 32;  // uint4 per (head, tile), the same for K and for V
+
+__device__ __forceinline__ int att_vkey(int s, int hh, int e) { return 16 * s + 8 * (e >> 2) + 4 * hh + (e & 3); }
+__device__ __forceinline__ uint32_t att_pack_top(float a, float b) {
+    return __builtin_amdgcn_perm(__float_as_uint(b), __float_as_uint(a), 0x07060302u);
+}
+__device__ __forceinline__ float att_top(float v) { return __uint_as_float(__float_as_uint(v) & 0xffff0000u); }
+// eight floats -> their three bf16 pieces as three fragments
+__device__ __forceinline__ void att_split8(const float (&v)[8], uint4 (&out)[3]) {
+    float r1[8], r2[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        r1[e] = v[e] - att_top(v[e]);    // exact
+        r2[e] = r1[e] - att_top(r1[e]);  // exact, at most 8 significant bits
+    }
+    out[0] = make_uint4(att_pack_top(v[0], v[1]), att_pack_top(v[2], v[3]), att_pack_top(v[4], v[5]), att_pack_top(v[6], v[7]));
+    out[1] = make_uint4(att_pack_top(r1[0], r1[1]), att_pack_top(r1[2], r1[3]), att_pack_top(r1[4], r1[5]), att_pack_top(r1[6], r1[7]));
+    out[2] = make_uint4(att_pack_top(r2[0], r2[1]), att_pack_top(r2[2], r2[3]), att_pack_top(r2[4], r2[5]), att_pack_top(r2[6], r2[7]));
+}
+
+// K and V rows [head][kv_stride][64] -> fragments of the tiles 0 .. gridDim.x - 1; rows from kv_len on count as zeros.
+// grid (tiles, heads), 256 threads.
+__global__ __launch_bounds__(256) void split_kv_kernel(const float *k, const float *v, uint4 *kfrag, uint4 *vfrag, int kv_len,
+                                                       int kv_stride, int tiles_cap) {
+    const int t = threadIdx.x, tile = blockIdx.x, hb = blockIdx.y;
+    const int i = t & 31, hh = (t >> 5) & 1;
+    const size_t base = ((size_t)hb * tiles_cap + tile) * ATT_FRAGS_PER_TILE;
+    uint4 out[3];
+    float x[8];
+    {
+        const int ds = t >> 6, key = tile * 32 + i;
+        const float *src = k + ((size_t)hb * kv_stride + key) * DH + 16 * ds + 8 * hh;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = key < kv_len ? src[e] : 0.0f;
+        att_split8(x, out);
+#pragma unroll
+        for (int pc = 0; pc < 3; ++pc) kfrag[base + ((ds * 3 + pc) * 2 + hh) * 32 + i] = out[pc];
+    }
+    {
+        const int s = (t >> 6) & 1, dblk = t >> 7;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int key = tile * 32 + att_vkey(s, hh, e);
+            x[e] = key < kv_len ? v[((size_t)hb * kv_stride + key) * DH + 32 * dblk + i] : 0.0f;
+        }
+        att_split8(x, out);
+#pragma unroll
+        for (int pc = 0; pc < 3; ++pc) vfrag[base + (((dblk * 3 + pc) * 2 + s) * 2 + hh) * 32 + i] = out[pc];
+    }
+}
+
+// The six piece products that matter, smallest first: (piece of the first operand, piece of the second)
+#define ATT_SIX(F) F(2, 0) F(0, 2) F(1, 1) F(1, 0) F(0, 1) F(0, 0)
+
+// grid ((nb + 1) / 2 paired query blocks or nb, heads), 512 threads: as attn_mfma_kernel with eight waves, which split
+// the key tiles; queries start at key position 0 (q_offset = 0, kv_len >= q_len).
+__global__ __launch_bounds__(512) void attn_bf16_kernel(const AttnParams p, const uint4 *__restrict__ kfrag, const uint4 *__restrict__ vfrag,
+                                                        int tiles_cap) {
+    extern __shared__ __align__(16) float att_smem[];
+    constexpr int S = 8;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = lane & 31, h2 = lane >> 5;
+    float *Ks = att_smem + wave * ATT_TILE_FLOATS;                               // this wave's partial result for the merge
+    uint4 *qs = reinterpret_cast<uint4 *>(att_smem + S * ATT_TILE_FLOATS);  // the query block's fragments [ds][piece][lane]
+    const int hb = blockIdx.y, b = hb / p.n_heads, h = hb % p.n_heads;
+    const int kv_len = p.kv_len;
+    const int nb = (p.q_len + 31) >> 5;
+    const uint4 *kf_head = kfrag + (size_t)hb * tiles_cap * ATT_FRAGS_PER_TILE + lane;
+    const uint4 *vf_head = vfrag + (size_t)hb * tiles_cap * ATT_FRAGS_PER_TILE + lane;
+    for (int rep = 0; rep < (p.pair_blocks ? 2 : 1); ++rep) {
+    const int qb = rep == 0 ? nb - 1 - (int)blockIdx.x : (int)blockIdx.x;
+    if (rep == 1 && qb >= nb - 1 - (int)blockIdx.x) break;
+    const int i0 = qb * 32;
+    const int last_q = min(p.q_len, i0 + 32) - 1;
+    const int jmax = p.causal ? min(kv_len, last_q + 1) : kv_len;
+    const int my_limit = p.causal ? i0 + c : 0x7fffffff;
+
+    uint4 kf[4][3], vf[2][3][2];
+    auto fetch_k = [&](int tile) {
+        const uint4 *src = kf_head + (size_t)tile * ATT_FRAGS_PER_TILE;
+#pragma unroll
+        for (int ds = 0; ds < 4; ++ds)
+#pragma unroll
+            for (int pc = 0; pc < 3; ++pc) kf[ds][pc] = src[(ds * 3 + pc) * 64];
+    };
+    auto fetch_v = [&](int tile) {
+        const uint4 *src = vf_head + (size_t)tile * ATT_FRAGS_PER_TILE;
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+#pragma unroll
+            for (int pc = 0; pc < 3; ++pc)
+#pragma unroll
+                for (int s = 0; s < 2; ++s) vf[db][pc][s] = src[((db * 3 + pc) * 2 + s) * 64];
+    };
+    if (wave * 32 < jmax) fetch_k(wave);
+    // the query block, times 1/8 (exact), as fragments of the second operand: waves 0..3 build d step ds = wave
+    if (wave < 4) {
+        const int qi = i0 + c;
+        float x[8];
+        const float *src = p.q + (size_t)b * p.q_batch_stride + (size_t)h * p.q_head_stride + (size_t)min(qi, p.q_len - 1) * p.q_row_stride +
+                           16 * wave + 8 * h2;
+        const float4 lo = *reinterpret_cast<const float4 *>(src), hi = *reinterpret_cast<const float4 *>(src + 4);
+        x[0] = lo.x * 0.125f; x[1] = lo.y * 0.125f; x[2] = lo.z * 0.125f; x[3] = lo.w * 0.125f;
+        x[4] = hi.x * 0.125f; x[5] = hi.y * 0.125f; x[6] = hi.z * 0.125f; x[7] = hi.w * 0.125f;
+        uint4 out[3];
+        att_split8(x, out);
+#pragma unroll
+        for (int pc = 0; pc < 3; ++pc) qs[(wave * 3 + pc) * 64 + lane] = out[pc];
+    }
+    __syncthreads();
+    floatx16 o0 = {0}, o1 = {0};
+    float m_run = -INFINITY, l_run = 0.0f;
+
+    for (int j0 = wave * 32; j0 < jmax; j0 += 32 * S) {
+        const int tile = j0 >> 5;
+        fetch_v(tile);
+        floatx16 sacc = {0};
+#pragma unroll
+        for (int ds = 0; ds < 4; ++ds) {
+            att_bf16x8 qf[3];
+#pragma unroll
+            for (int pc = 0; pc < 3; ++pc) qf[pc] = __builtin_bit_cast(att_bf16x8, qs[(ds * 3 + pc) * 64 + lane]);
+#define ATT_S_STEP(PK, PQ) sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(att_bf16x8, kf[ds][PK]), qf[PQ], sacc, 0, 0, 0);
+            ATT_SIX(ATT_S_STEP)
+#undef ATT_S_STEP
+        }
+        if (j0 + 32 * S < jmax) fetch_k(tile + S);
+        // register r holds key j0 + 8*(r/4) + 4*h2 + r%4 for query c
+        float tmax = -INFINITY;
+        if (j0 + 32 > kv_len || (p.causal && j0 + 31 > i0)) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int j = j0 + 8 * (r >> 2) + 4 * h2 + (r & 3);
+                const bool vis = (j <= my_limit) && (j < kv_len);
+                sacc[r] = vis ? sacc[r] : -INFINITY;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, sacc[r]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+        const float m_new = fmaxf(m_run, tmax);
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = ATT_EXP(m_run - m_use);
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            sacc[r] = ATT_EXP(sacc[r] - m_use);
+            psum += sacc[r];
+        }
+        psum += __shfl_xor(psum, 32, kWave);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            o0[r] *= alpha;
+            o1[r] *= alpha;
+        }
+        // the probabilities as fragments: element e of key step s is register 8 s + e
+        uint4 pf[2][3];
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            const float x[8] = {sacc[8 * s], sacc[8 * s + 1], sacc[8 * s + 2], sacc[8 * s + 3],
+                                sacc[8 * s + 4], sacc[8 * s + 5], sacc[8 * s + 6], sacc[8 * s + 7]};
+            att_split8(x, pf[s]);
+        }
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+#define ATT_O_STEP(PV, PP)                                                                                                                   \
+    o0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(att_bf16x8, vf[0][PV][s]), __builtin_bit_cast(att_bf16x8, pf[s][PP]), o0, 0, 0, 0); \
+    o1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(att_bf16x8, vf[1][PV][s]), __builtin_bit_cast(att_bf16x8, pf[s][PP]), o1, 0, 0, 0);
+            ATT_SIX(ATT_O_STEP)
+#undef ATT_O_STEP
+        }
+    }
+    // the merge of the eight waves' partial results, as in attn_mfma_kernel
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int d = 8 * (r >> 2) + 4 * h2 + (r & 3);
+        Ks[d * OLD + c] = o0[r];
+        Ks[(d + 32) * OLD + c] = o1[r];
+    }
+    if (h2 == 0) {
+        Ks[64 * OLD + c] = m_run;
+        Ks[64 * OLD + 32 + c] = l_run;
+    }
+    __syncthreads();
+    float *obase = p.o + (size_t)b * p.o_batch_stride + (size_t)h * p.o_head_stride + lane;
+    merge_partials<8>(att_smem, lane, wave, i0, p.q_len, obase, p.o_row_stride);
+    if (p.pair_blocks) __syncthreads();  // the tiles and the query fragments are reused by the second block
+    }
+}
+#undef ATT_SIX
+
 // Merge (m, l, o) of `other` into (m, l, o); empty partials have l == 0 and m == -inf.
 __device__ __forceinline__ void merge_partial(float &m, float &l, float4 &o, float m2, float l2, float4 o2) {
     const float mn = fmaxf(m, m2);
@@ -468,6 +673,28 @@ int32_t agpu_attention_launch(agpu_ctx *ctx, const AttnParams &p, int max_kv_len
     hipLaunchKernelGGL(attn_mfma_kernel, dim3(pm.pair_blocks ? (nb + 1) / 2 : nb, hb), dim3(64 * S), sizeof(float) * ATT_TILE_FLOATS * S,
                        ctx->stream, pm);
     return AGPU_LAUNCH_CHECK(ctx, "attn_mfma_kernel");
+}
+
+size_t agpu_attention_fragment_bytes(int heads, int kv_len) {
+    return (size_t)heads * ceil_div(kv_len, 32) * ATT_FRAGS_PER_TILE * sizeof(uint4);
+}
+
+int32_t agpu_attention_fragments_launch(agpu_ctx *ctx, const AttnParams &p, const uint4 *kfrag, const uint4 *vfrag, int tiles_cap) {
+    const int hb = p.n_heads * p.batch, nb = ceil_div(p.q_len, 32);
+    if (!p.causal || p.pos_dev || p.q_offset != 0 || p.kv_len < p.q_len || p.q_len < 256 || tiles_cap < ceil_div(p.kv_len, 32))
+        return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "attention on fragments: causal, from position 0, 256 queries or more");
+    AttnParams pm = p;
+    pm.pair_blocks = (nb >= 4 && nb * hb > ctx->num_cus) ? 1 : 0;
+    const int lds = (int)(sizeof(float) * ATT_TILE_FLOATS * 8 + 12 * 64 * sizeof(uint4));
+    static std::atomic<unsigned long long> lds_raised{0};  // one bit per device
+    const unsigned long long bit = 1ull << (ctx->device & 63);
+    if (!(lds_raised.load(std::memory_order_relaxed) & bit)) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_bf16_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return agpu_hip(ctx, e, "hipFuncSetAttribute");
+        lds_raised.fetch_or(bit, std::memory_order_relaxed);
+    }
+    hipLaunchKernelGGL(attn_bf16_kernel, dim3(pm.pair_blocks ? (nb + 1) / 2 : nb, hb), dim3(512), lds, ctx->stream, pm, kfrag, vfrag, tiles_cap);
+    return AGPU_LAUNCH_CHECK(ctx, "attn_bf16_kernel");
 }
 
 AGPU_EXPORT int32_t agpu_attention(agpu_ctx *ctx, const float *q, const float *k, const float *v, float *o,

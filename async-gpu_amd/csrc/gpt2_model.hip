@@ -58,6 +58,7 @@ struct agpu_gpt2 {
     int cache_len = 0;
     // activations (grown on demand, never inside a captured region)
     DevBuf hid, qkv, att, ffn, lnb, last, logits, tok_in;
+    DevBuf kfrag, vfrag;  // K and V of one layer as bf16 operand fragments (prefill of one sequence from position 0)
     uint32_t *cur_tok = nullptr, *next_tok = nullptr, *out_tok = nullptr;
     int out_capacity = 0;  // steps recorded in out_tok
     int *pos_dev = nullptr, *step_dev = nullptr;
@@ -309,6 +310,13 @@ int32_t launch_embed(agpu_gpt2 *m, const uint32_t *tokens, int B, int new_len) {
     return AGPU_LAUNCH_CHECK(m->ctx, "embed_rows_kernel");
 }
 
+// A prompt of one sequence into an empty cache, long enough for eight key tiles: the QKV Linear also writes K and V as
+// the operand fragments of the bf16 attention kernel (where its kernel for the shape can).
+bool prefill_uses_fragments(const agpu_gpt2 *m, int B, int new_len) {
+    return B == 1 && m->cache_len == 0 && new_len >= 256 && m->cfg.group_size % 32 == 0 &&
+           agpu_int4_gemm_bf16_writes_kv_frags(m->ctx, new_len, 3 * m->d, m->d);
+}
+
 // Block L on the hidden rows in place: x += Attn(LN1 x), x += FFN(LN2 x); its K and V rows go into the cache.
 int32_t launch_block(agpu_gpt2 *m, int L, int B, int new_len, int max_kv) {
     agpu_ctx *ctx = m->ctx;
@@ -318,6 +326,7 @@ int32_t launch_block(agpu_gpt2 *m, int L, int B, int new_len, int max_kv) {
     float *hid = (float *)m->hid.p, *qkv = (float *)m->qkv.p, *att = (float *)m->att.p, *ffn = (float *)m->ffn.p;
     const uint32_t gelu_flag = m->cfg.gelu == AGPU_GELU_QUICK ? AGPU_EPI_GELU_QUICK : AGPU_EPI_GELU_TANH;
     int32_t rc;
+    bool frags = false;  // this layer's K and V also exist as bf16 fragments
     const size_t layer_stride = (size_t)m->cfg.max_batch * H * P * DH;
     const Block &b = m->blocks[L];
     const Int4Lin &wq = b.lin[AGPU_LINEAR_QKV], &wp = b.lin[AGPU_LINEAR_PROJ], &wf = b.lin[AGPU_LINEAR_FC],
@@ -347,10 +356,16 @@ int32_t launch_block(agpu_gpt2 *m, int L, int B, int new_len, int max_kv) {
         if (rc != AGPU_OK) return rc;
     } else {
         // prefill: the GEMM writes the K/V rows into the cache itself where it can
-        const KvScatter kv{kc, vc, m->pos_dev, H, P, new_len};
+        KvScatter kv{kc, vc, m->pos_dev, H, P, new_len};
+        if (prefill_uses_fragments(m, B, new_len)) {
+            kv.kfrag = (uint4 *)m->kfrag.p;
+            kv.vfrag = (uint4 *)m->vfrag.p;
+            kv.tiles_cap = ceil_div(new_len, 32);
+        }
         bool kv_done = false;
         rc = ln_linear(m, hid, b.ln1_g, b.ln1_b, wq, nullptr, qkv, R, 3 * d, 0, &kv, &kv_done);
         if (rc != AGPU_OK) return rc;
+        frags = kv_done && kv.kfrag != nullptr;
         if (!kv_done) {
             hipLaunchKernelGGL(kv_scatter_kernel, dim3((unsigned)(((size_t)R * d + 255) / 256)), dim3(256), 0, ctx->stream, qkv,
                                kc, vc, R, new_len, H, P, m->pos_dev);
@@ -363,7 +378,14 @@ int32_t launch_block(agpu_gpt2 *m, int L, int B, int new_len, int max_kv) {
     ap.q_batch_stride = (long long)new_len * 3 * d; ap.q_head_stride = DH; ap.q_row_stride = 3 * d;
     ap.o_batch_stride = (long long)new_len * d; ap.o_head_stride = DH; ap.o_row_stride = d;
     ap.pos_dev = m->pos_dev;
-    if ((rc = agpu_attention_launch(ctx, ap, max_kv)) != AGPU_OK) return rc;
+    if (frags) {
+        ap.pos_dev = nullptr;
+        ap.kv_len = new_len;
+        rc = agpu_attention_fragments_launch(ctx, ap, (const uint4 *)m->kfrag.p, (const uint4 *)m->vfrag.p, ceil_div(new_len, 32));
+    } else {
+        rc = agpu_attention_launch(ctx, ap, max_kv);
+    }
+    if (rc != AGPU_OK) return rc;
     rc = agpu_int4_linear(ctx, att, wp.packed, wp.scales, wp.bias, hid, hid, R, d, d, g, 0);
     if (rc != AGPU_OK) return rc;
     if ((rc = ln_linear(m, hid, b.ln2_g, b.ln2_b, wf, nullptr, ffn, R, ff, gelu_flag)) != AGPU_OK) return rc;
@@ -432,6 +454,11 @@ int32_t ensure_buffers(agpu_gpt2 *m, int B, int new_len, bool all_rows_logits) {
     if ((rc = ensure(m, m->lnb, (R > Rl ? R : Rl) * d * 4)) != AGPU_OK) return rc;
     if ((rc = ensure(m, m->last, (size_t)B * d * 4)) != AGPU_OK) return rc;
     if ((rc = ensure(m, m->logits, Rl * logits_stride(m) * 4)) != AGPU_OK) return rc;
+    if (prefill_uses_fragments(m, B, new_len)) {
+        const size_t bytes = agpu_attention_fragment_bytes(m->H, new_len);
+        if ((rc = ensure(m, m->kfrag, bytes)) != AGPU_OK) return rc;
+        if ((rc = ensure(m, m->vfrag, bytes)) != AGPU_OK) return rc;
+    }
     return AGPU_OK;
 }
 
@@ -786,7 +813,7 @@ AGPU_EXPORT int32_t agpu_gpt2_destroy(agpu_gpt2 *m) {
     free_lin(m->lm_head);
     for (void *p : {(void *)m->wte, (void *)m->wpe, (void *)m->lnf_g, (void *)m->lnf_b, (void *)m->wte_t, (void *)m->kcache,
                     (void *)m->vcache, (void *)m->cur_tok, (void *)m->next_tok, (void *)m->out_tok, (void *)m->pos_dev,
-                    m->hid.p, m->qkv.p, m->att.p, m->ffn.p, m->lnb.p, m->last.p, m->logits.p, m->tok_in.p})
+                    m->hid.p, m->qkv.p, m->att.p, m->ffn.p, m->lnb.p, m->last.p, m->logits.p, m->tok_in.p, m->kfrag.p, m->vfrag.p})
         if (p) (void)hipFree(p);
     for (hipEvent_t e : {m->ev0, m->ev1, m->ev2})
         if (e) (void)hipEventDestroy(e);

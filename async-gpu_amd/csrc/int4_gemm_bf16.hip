@@ -33,6 +33,7 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
+constexpr int KV_FRAGS_PER_TILE = 4 * 3 * 2 * 32;  // 16-byte fragments of one (head, 32 keys): the attention's layout
 constexpr int GB_FRAG_BYTES = 32 * 16;                                      // one half of an A operand: 32 rows x 8 bf16
 
 struct GemmBfParams {
@@ -341,14 +342,16 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
         if (n >= p.N) continue;
         const float bias = p.bias ? p.bias[n] : 0.0f;
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
+        for (int rb = 0; rb < RB; ++rb) {
+            float vals[16];
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int m = row_of(rb, r);
+                float v = acc[rb][cb][r] + bias;
+                if (p.flags & AGPU_EPI_GELU_TANH) v = gelu_tanh_dev(v);
+                else if (p.flags & AGPU_EPI_GELU_QUICK) v = gelu_quick_dev(v);
+                vals[r] = v;
                 if (m < p.M) {
-                    float v = acc[rb][cb][r] + bias;
-                    if (p.flags & AGPU_EPI_GELU_TANH) v = gelu_tanh_dev(v);
-                    else if (p.flags & AGPU_EPI_GELU_QUICK) v = gelu_quick_dev(v);
                     if (p.residual) v += p.residual[(size_t)m * p.N + n];
                     p.y[(size_t)m * p.N + n] = v;
                     if (p.kv.kcache && n >= p.N / 3) {
@@ -359,10 +362,83 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
                     }
                 }
             }
+            // The K and V columns once more as the bf16 operand fragments of the prefill attention (one sequence, rows =
+            // key positions from 0; rows past M repeat the last row and are never visible).  A wave's 32 columns are
+            // half a head.  V: a lane holds column d and the 16 keys of its registers, which is the operand as it is.
+            // K: a lane needs 8 columns of one key, so the tile goes through LDS (free after the K loop) transposed.
+            if constexpr (RB == 1 && CB == 1 && GB_WAVES == 4) {
+                if (p.kv.kfrag && n0 >= p.N / 3) {  // wave-uniform
+                    const int dm = p.N / 3, e0 = n0 - dm, in_v = e0 >= dm ? 1 : 0, c0 = e0 - in_v * dm;
+                    const int head = c0 >> 6, dblk = (c0 >> 5) & 1, tile = m0 >> 5;
+                    const size_t base = ((size_t)head * p.kv.tiles_cap + tile) * KV_FRAGS_PER_TILE;
+                    float r1[16], r2[16];
+                    if (in_v) {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            r1[r] = vals[r] - top_bits(vals[r]);
+                            r2[r] = r1[r] - top_bits(r1[r]);
+                        }
+#pragma unroll
+                        for (int s = 0; s < 2; ++s) {
+                            const float *a = vals + 8 * s, *b1 = r1 + 8 * s, *b2 = r2 + 8 * s;
+                            uint4 *dst = p.kv.vfrag + base + (size_t)(((dblk * 3 + 0) * 2 + s) * 2 + hh) * 32 + j;
+                            dst[0] = make_uint4(pack_top(a[0], a[1]), pack_top(a[2], a[3]), pack_top(a[4], a[5]), pack_top(a[6], a[7]));
+                            dst[2 * 2 * 32] = make_uint4(pack_top(b1[0], b1[1]), pack_top(b1[2], b1[3]), pack_top(b1[4], b1[5]), pack_top(b1[6], b1[7]));
+                            dst[2 * 2 * 2 * 32] = make_uint4(pack_top(b2[0], b2[1]), pack_top(b2[2], b2[3]), pack_top(b2[4], b2[5]), pack_top(b2[6], b2[7]));
+                        }
+                    } else {
+                        float *tr = reinterpret_cast<float *>(s_a[0]) + wave * (32 * 36);
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) tr[(8 * (r >> 2) + 4 * hh + (r & 3)) * 36 + j] = vals[r];
+                        // same wave: LDS operations complete in order
+#pragma unroll
+                        for (int sl = 0; sl < 2; ++sl) {
+                            const float4 lo = *reinterpret_cast<const float4 *>(tr + j * 36 + 16 * sl + 8 * hh);
+                            const float4 hi = *reinterpret_cast<const float4 *>(tr + j * 36 + 16 * sl + 8 * hh + 4);
+                            const float a[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+                            float b1[8], b2[8];
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) {
+                                b1[e] = a[e] - top_bits(a[e]);
+                                b2[e] = b1[e] - top_bits(b1[e]);
+                            }
+                            uint4 *dst = p.kv.kfrag + base + (size_t)(((2 * dblk + sl) * 3 + 0) * 2 + hh) * 32 + j;
+                            dst[0] = make_uint4(pack_top(a[0], a[1]), pack_top(a[2], a[3]), pack_top(a[4], a[5]), pack_top(a[6], a[7]));
+                            dst[2 * 32] = make_uint4(pack_top(b1[0], b1[1]), pack_top(b1[2], b1[3]), pack_top(b1[4], b1[5]), pack_top(b1[6], b1[7]));
+                            dst[2 * 2 * 32] = make_uint4(pack_top(b2[0], b2[1]), pack_top(b2[2], b2[3]), pack_top(b2[4], b2[5]), pack_top(b2[6], b2[7]));
+                        }
+                    }
+                }
+            }
+        }
     }
 }
 
+enum class GemmVariant { Small, LongBlocks, Wide, Large };
+
+GemmVariant pick_variant(const agpu_ctx *ctx, int M, int N, int K) {
+    // Workgroup tile: 32 rows x 128 columns (one 32 x 32 tile per wave), which puts the most waves on the chip for
+    // the layer sizes of GPT-2 small; 64 x 256 (every weight fragment serves two row blocks, every x fragment two
+    // column blocks) once that still leaves a workgroup per CU.  M = 1024, K = 768, N = 2304: 25.8 us with the
+    // small tile, 28.2 us with 32 x 256, 33.1 us with 64 x 256; K = 1600, N = 6400: 96.5 us with the large tile,
+    // 105.6 us with 32 x 256.
+    const bool large = ceil_div(N, 256) * ceil_div(M, 64) >= ctx->num_cus;
+    // K per block: 64; 128 for the small tile on small problems (fewer barriers and loop ends per k, but 159
+    // registers against 126, three waves per SIMD against four: M = 512, K = 768, N = 2304: 17.5 us against 18.7 us;
+    // M = 1024: 27.3 us against 25.8 us)
+    const bool long_blocks = !large && (long long)ceil_div(N, 128) * ceil_div(M, 32) * ceil_div(K, 64) <= 5000;
+    // With a long K the split of x weighs more: eight waves share one 32-row x tile over 256 columns, the first four
+    // stage it (M = 1024, K = 1600, N = 1600: 32.8 us against 38.1 us; K = 768, N = 2304: 27.3 us against 25.2 us)
+    const bool wide = !large && !long_blocks && K >= 1536;
+    return large ? GemmVariant::Large : long_blocks ? GemmVariant::LongBlocks : wide ? GemmVariant::Wide : GemmVariant::Small;
+}
+
 }  // namespace
+
+bool agpu_int4_gemm_bf16_writes_kv_frags(const agpu_ctx *ctx, int M, int N, int K) {
+    const GemmVariant v = pick_variant(ctx, M, N, K);
+    return (v == GemmVariant::Small || v == GemmVariant::LongBlocks) && N % 3 == 0 && (N / 3) % 64 == 0;
+}
 
 bool agpu_int4_gemm_bf16_supported(const void *x, int M, int N, int K, int group) {
     (void)N;
@@ -377,19 +453,9 @@ int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t
     p.strict = ctx->strict_sync;
     p.x = x; p.packed = packed; p.scales = scales; p.bias = bias; p.residual = residual; p.y = y;
     p.M = M; p.N = N; p.K = K; p.chunk_shift = __builtin_ctz((unsigned)(group / 32)); p.flags = flags;
-    // Workgroup tile: 32 rows x 128 columns (one 32 x 32 tile per wave), which puts the most waves on the chip for
-    // the layer sizes of GPT-2 small; 64 x 256 (every weight fragment serves two row blocks, every x fragment two
-    // column blocks) once that still leaves a workgroup per CU.  M = 1024, K = 768, N = 2304: 25.8 us with the
-    // small tile, 28.2 us with 32 x 256, 33.1 us with 64 x 256; K = 1600, N = 6400: 96.5 us with the large tile,
-    // 105.6 us with 32 x 256.
-    const bool large = ceil_div(N, 256) * ceil_div(M, 64) >= ctx->num_cus;
-    // K per block: 64; 128 for the small tile on small problems (fewer barriers and loop ends per k, but 159
-    // registers against 126, three waves per SIMD against four: M = 512, K = 768, N = 2304: 17.5 us against 18.7 us;
-    // M = 1024: 27.3 us against 25.8 us)
-    const bool long_blocks = !large && (long long)ceil_div(N, 128) * ceil_div(M, 32) * ceil_div(K, 64) <= 5000;
-    // With a long K the split of x weighs more: eight waves share one 32-row x tile over 256 columns, the first four
-    // stage it (M = 1024, K = 1600, N = 1600: 32.8 us against 38.1 us; K = 768, N = 2304: 27.3 us against 25.2 us)
-    const bool wide = !large && !long_blocks && K >= 1536;
+    const GemmVariant var = pick_variant(ctx, M, N, K);
+    const bool large = var == GemmVariant::Large, long_blocks = var == GemmVariant::LongBlocks, wide = var == GemmVariant::Wide;
+    if (large || wide) p.kv.kfrag = p.kv.vfrag = nullptr;  // only the four-wave 32 x 128 kernels write the attention's fragments
     const int BM = large ? 64 : 32, BN = large || wide ? 256 : 128;
     const int tiles = ceil_div(N, BN) * ceil_div(M, BM);
     const int KB = long_blocks ? 128 : 64;
