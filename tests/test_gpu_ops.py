@@ -526,6 +526,21 @@ def test_attention_chunked_prefill(agpu, orc, dev, q_len, q_offset):
     assert np.abs(o.cpu().numpy() - ref).max() <= 1e-5
 
 
+@pytest.mark.parametrize("H,q_len,extra", [(12, 1000, 0), (5, 800, 24), (25, 777, 0), (3, 768, 1)])
+def test_attention_prefill_bf16_pieces(agpu, orc, dev, H, q_len, extra):
+    """From 768 queries at position 0 the prefill runs on the bf16 matrix cores: K and V are first split into their
+    three bf16 pieces (fragments in the workspace), and six piece products per term keep fp32 accuracy.  Ragged
+    lengths, a cache longer than the queries (kv_len > q_len: the extra keys are behind the mask), odd head counts."""
+    from async_gpu_amd import ops, workloads
+    kv_len = q_len + extra
+    w = workloads.config3_attention(seed=22, H=H, seq=kv_len + 5)
+    q = w["q"][:, :q_len].copy()
+    o = ops.attention(to_dev(q, dev), to_dev(w["k"], dev), to_dev(w["v"], dev), kv_len=kv_len, q_offset=0).cpu().numpy()
+    ref = orc.attention_kv(q, w["k"], w["v"], kv_len=kv_len, q_offset=0)
+    assert np.abs(o - ref).max() <= 1e-5
+    assert np.abs(o[:, 0] - w["v"][:, 0]).max() <= 1e-6  # row 0 sees only key 0
+
+
 def test_attention_rejects_other_head_dims(agpu, dev):
     from async_gpu_amd import ops
     t = torch.zeros((2, 4, 32), device=dev)
