@@ -41,7 +41,8 @@ constexpr int ATT_TILE_FLOATS = 32 * KLD;  // per wave: the K tile (padded rows)
 // w, w + S, ...  Lane x first works out the weight exp(m_v - m) / l of partial v = x % S for the wave's query number
 // x / S; the sums then take the weights from those lanes.  S is a constant here so that no read waits for another.
 template <int S>
-__device__ __noinline__ void merge_partials(const float *att_smem, int lane, int wave, int i0, int q_len, float *obase, long long o_row_stride) {
+__device__ __forceinline__ void merge_partials_inline(const float *att_smem, int lane, int wave, int i0, int q_len, float *obase,
+                                                      long long o_row_stride) {
     constexpr int NQ = (32 + S - 1) / S;
     float wgt;
     {
@@ -72,6 +73,11 @@ __device__ __noinline__ void merge_partials(const float *att_smem, int lane, int
                    __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wgt), i * S + w));
         if (qc < 32 && i0 + qc < q_len) obase[(size_t)(i0 + qc) * o_row_stride] = acc;
     }
+}
+
+template <int S>
+__device__ __noinline__ void merge_partials(const float *att_smem, int lane, int wave, int i0, int q_len, float *obase, long long o_row_stride) {
+    merge_partials_inline<S>(att_smem, lane, wave, i0, q_len, obase, o_row_stride);
 }
 
 __global__ __launch_bounds__(512) void attn_mfma_kernel(const AttnParams p) {
@@ -330,7 +336,8 @@ __global__ __launch_bounds__(256) void split_kv_kernel(const float *k, const flo
 // The six piece products that matter, smallest first: (piece of the first operand, piece of the second)
 #define ATT_SIX(F) F(2, 0) F(0, 2) F(1, 1) F(1, 0) F(0, 1) F(0, 0)
 
-// grid ((nb + 1) / 2 paired query blocks or nb, heads), 512 threads: as attn_mfma_kernel with eight waves, which split
+// grid: (nb + 1) / 2 paired query blocks or nb, times heads, rounded up to a multiple of 8 (one dimension), 512 threads:
+// as attn_mfma_kernel with eight waves, which split
 // the key tiles; queries start at key position 0 (q_offset = 0, kv_len >= q_len).
 __global__ __launch_bounds__(512) void attn_bf16_kernel(const AttnParams p, const uint4 *__restrict__ kfrag, const uint4 *__restrict__ vfrag,
                                                         int tiles_cap) {
@@ -340,19 +347,17 @@ __global__ __launch_bounds__(512) void attn_bf16_kernel(const AttnParams p, cons
     const int c = lane & 31, h2 = lane >> 5;
     float *Ks = att_smem + wave * ATT_TILE_FLOATS;                               // this wave's partial result for the merge
     uint4 *qs = reinterpret_cast<uint4 *>(att_smem + S * ATT_TILE_FLOATS);  // the query block's fragments [ds][piece][lane]
-    const int hb = blockIdx.y, b = hb / p.n_heads, h = hb % p.n_heads;
+    // Workgroup -> (head, block pair), head-major within an XCD: consecutive workgroup numbers go round the eight XCDs,
+    // so number n is entry n / 8 of XCD n % 8, and an XCD takes a run of consecutive (head, pair) entries: the
+    // fragments of one or two heads stay in its L2.
+    const int nb = (p.q_len + 31) >> 5, gx = p.pair_blocks ? (nb + 1) >> 1 : nb;
+    const int total = gx * p.n_heads * p.batch, per_xcd = (total + 7) >> 3;
+    const int entry = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+    if (entry >= total) return;
+    const int hb = entry / gx, bx = entry - hb * gx, b = hb / p.n_heads, h = hb % p.n_heads;
     const int kv_len = p.kv_len;
-    const int nb = (p.q_len + 31) >> 5;
     const uint4 *kf_head = kfrag + (size_t)hb * tiles_cap * ATT_FRAGS_PER_TILE + lane;
     const uint4 *vf_head = vfrag + (size_t)hb * tiles_cap * ATT_FRAGS_PER_TILE + lane;
-    for (int rep = 0; rep < (p.pair_blocks ? 2 : 1); ++rep) {
-    const int qb = rep == 0 ? nb - 1 - (int)blockIdx.x : (int)blockIdx.x;
-    if (rep == 1 && qb >= nb - 1 - (int)blockIdx.x) break;
-    const int i0 = qb * 32;
-    const int last_q = min(p.q_len, i0 + 32) - 1;
-    const int jmax = p.causal ? min(kv_len, last_q + 1) : kv_len;
-    const int my_limit = p.causal ? i0 + c : 0x7fffffff;
-
     uint4 kf[4][3], vf[2][3][2];
     auto fetch_k = [&](int tile) {
         const uint4 *src = kf_head + (size_t)tile * ATT_FRAGS_PER_TILE;
@@ -370,16 +375,31 @@ __global__ __launch_bounds__(512) void attn_bf16_kernel(const AttnParams p, cons
 #pragma unroll
                 for (int s = 0; s < 2; ++s) vf[db][pc][s] = src[((db * 3 + pc) * 2 + s) * 64];
     };
-    if (wave * 32 < jmax) fetch_k(wave);
-    // the query block, times 1/8 (exact), as fragments of the second operand: waves 0..3 build d step ds = wave
+    auto jmax_of = [&](int qb_) { return p.causal ? min(kv_len, min(p.q_len, qb_ * 32 + 32)) : kv_len; };
+    // A block's queries (waves 0..3: d step ds = wave of query c, 8 floats) and its first key tile are requested ahead:
+    // for the first block here, for the second one before the first one's partial results are merged.
+    float4 qlo = make_float4(0.f, 0.f, 0.f, 0.f), qhi = qlo;
+    auto request_block = [&](int qb_) {
+        if (wave < 4) {
+            const float *src = p.q + (size_t)b * p.q_batch_stride + (size_t)h * p.q_head_stride +
+                               (size_t)min(qb_ * 32 + c, p.q_len - 1) * p.q_row_stride + 16 * wave + 8 * h2;
+            qlo = *reinterpret_cast<const float4 *>(src);
+            qhi = *reinterpret_cast<const float4 *>(src + 4);
+        }
+        if (wave * 32 < jmax_of(qb_)) fetch_k(wave);
+    };
+    request_block(nb - 1 - bx);
+    for (int rep = 0; rep < (p.pair_blocks ? 2 : 1); ++rep) {
+    const int qb = rep == 0 ? nb - 1 - bx : bx;
+    if (rep == 1 && qb >= nb - 1 - bx) break;
+    const bool more = p.pair_blocks && rep == 0 && bx < nb - 1 - bx;  // a second block follows
+    const int i0 = qb * 32;
+    const int jmax = jmax_of(qb);
+    const int my_limit = p.causal ? i0 + c : 0x7fffffff;
+    // the query block, times 1/8 (exact), as fragments of the second operand
     if (wave < 4) {
-        const int qi = i0 + c;
-        float x[8];
-        const float *src = p.q + (size_t)b * p.q_batch_stride + (size_t)h * p.q_head_stride + (size_t)min(qi, p.q_len - 1) * p.q_row_stride +
-                           16 * wave + 8 * h2;
-        const float4 lo = *reinterpret_cast<const float4 *>(src), hi = *reinterpret_cast<const float4 *>(src + 4);
-        x[0] = lo.x * 0.125f; x[1] = lo.y * 0.125f; x[2] = lo.z * 0.125f; x[3] = lo.w * 0.125f;
-        x[4] = hi.x * 0.125f; x[5] = hi.y * 0.125f; x[6] = hi.z * 0.125f; x[7] = hi.w * 0.125f;
+        const float x[8] = {qlo.x * 0.125f, qlo.y * 0.125f, qlo.z * 0.125f, qlo.w * 0.125f,
+                            qhi.x * 0.125f, qhi.y * 0.125f, qhi.z * 0.125f, qhi.w * 0.125f};
         uint4 out[3];
         att_split8(x, out);
 #pragma unroll
@@ -461,9 +481,10 @@ __global__ __launch_bounds__(512) void attn_bf16_kernel(const AttnParams p, cons
         Ks[64 * OLD + c] = m_run;
         Ks[64 * OLD + 32 + c] = l_run;
     }
+    if (more) request_block(bx);
     __syncthreads();
     float *obase = p.o + (size_t)b * p.o_batch_stride + (size_t)h * p.o_head_stride + lane;
-    merge_partials<8>(att_smem, lane, wave, i0, p.q_len, obase, p.o_row_stride);
+    merge_partials_inline<8>(att_smem, lane, wave, i0, p.q_len, obase, p.o_row_stride);
     if (p.pair_blocks) __syncthreads();  // the tiles and the query fragments are reused by the second block
     }
 }
@@ -709,7 +730,8 @@ int32_t agpu_attention_fragments_launch(agpu_ctx *ctx, const AttnParams &p, cons
         if (e != hipSuccess) return agpu_hip(ctx, e, "hipFuncSetAttribute");
         lds_raised.fetch_or(bit, std::memory_order_relaxed);
     }
-    hipLaunchKernelGGL(attn_bf16_kernel, dim3(pm.pair_blocks ? (nb + 1) / 2 : nb, hb), dim3(512), lds, ctx->stream, pm, kfrag, vfrag, tiles_cap);
+    const int total = (pm.pair_blocks ? (nb + 1) / 2 : nb) * hb;
+    hipLaunchKernelGGL(attn_bf16_kernel, dim3(ceil_div(total, 8) * 8), dim3(512), lds, ctx->stream, pm, kfrag, vfrag, tiles_cap);
     return AGPU_LAUNCH_CHECK(ctx, "attn_bf16_kernel");
 }
 
