@@ -336,3 +336,22 @@ def test_long_prefill_small_width(orc, agpu, dev, prompt_len):
     for lo_i in range(0, prompt_len, 250):
         lc = gm.forward_cached(prompt[lo_i:lo_i + 250].reshape(1, -1))[0]
     assert np.abs(lc[-1] - lg[-1]).max() <= 2e-5
+
+
+def test_long_early_exit_forward_after_a_generation(orc, agpu, dev):
+    """forward_early_exit sizes its buffers while the cache still holds an earlier generation and empties it afterwards;
+    with 256 rows or more its attention then takes the bf16 path, whose K/V fragment buffers must exist by then.  All rows
+    of the logits against the oracle, and again after a longer call has grown the buffers."""
+    from async_gpu_amd import gpt2, workloads
+    cfg = dict(n_layer=2, n_embd=768, n_head=12, vocab=1031, n_positions=1024)
+    w, qz = _quantized(orc, cfg, 18, nonzero_bias=True, random_ln=True)
+    om = build_oracle_model(cfg, qz)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg), qz)
+    gm.generate_cached(workloads.random_prompt(cfg, 6, 40), 4, eos=-1)  # leaves 43 positions in the cache
+    for n in (300, 420):
+        tokens = workloads.random_prompt(cfg, 7, n)
+        want, wu, _ = om.forward_early_exit(tokens, 2.0)
+        got, gu = gm.forward_early_exit(tokens, 2.0)
+        assert gu == wu == 2
+        assert np.abs(got - want).max() <= TOL_LOGITS * max(1.0, np.abs(want).max())
+
