@@ -13,6 +13,7 @@
 #define AGPU_EXPORT extern "C" __attribute__((visibility("default")))
 
 constexpr int kWave = 64;                                  // CDNA4 wavefront width
+constexpr int kKvFragsPerTile = 4 * 3 * 2 * 32;              // 16-byte bf16 operand fragments of one (head, 32 keys) of K, and of V
 constexpr size_t kWorkspaceBytes = size_t(96) << 20;       // default scratch of a context: split-K / attention partials, LayerNorm rows
 constexpr size_t kMinWorkspaceBytes = size_t(1) << 20;     // smallest scratch a caller may bring
 constexpr int kNumCounters = 1 << 16;                      // arrival tickets of a context (always left at zero)

@@ -282,7 +282,7 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(const AttnParams p) {
 // with one 1 KiB request per wave and instruction.  att_vkey is the order in which a 32 x 32 MFMA result holds its
 // rows: the probabilities of a key tile come out of the first product in exactly the layout the second one wants.
 typedef __bf16 att_bf16x8 __attribute__((ext_vector_type(8)));
-constexpr int ATT_FRAGS_PER_TILE = 4 * 3 * 2 * 32;  // uint4 per (head, tile), the same for K and for V
+constexpr int ATT_FRAGS_PER_TILE = kKvFragsPerTile;  // uint4 per (head, tile), the same for K and for V
 
 __device__ __forceinline__ int att_vkey(int s, int hh, int e) { return 16 * s + 8 * (e >> 2) + 4 * hh + (e & 3); }
 __device__ __forceinline__ uint32_t att_pack_top(float a, float b) {

@@ -33,7 +33,7 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int KV_FRAGS_PER_TILE = 4 * 3 * 2 * 32;  // 16-byte fragments of one (head, 32 keys): the attention's layout
+constexpr int KV_FRAGS_PER_TILE = kKvFragsPerTile;  // 16-byte fragments of one (head, 32 keys): the attention's layout
 constexpr int GB_FRAG_BYTES = 32 * 16;                                      // one half of an A operand: 32 rows x 8 bf16
 
 struct GemmBfParams {
