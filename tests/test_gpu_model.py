@@ -312,12 +312,14 @@ def test_generate_text_through_the_tokenizer(tiny, orc):
             gm.generate_text(tok, prompt, 10, eos=-1)
 
 
-@pytest.mark.parametrize("prompt_len", [600, 1000])
+@pytest.mark.parametrize("prompt_len", [255, 256, 257, 600, 1000])
 def test_long_prefill_small_width(orc, agpu, dev, prompt_len):
     """GPT-2 small's width with prompts of many rows: the QKV Linear then has more tiles than the chip has CUs and the
     tiles left over after whole rounds are sliced along K, K/V rows of those tiles included (they go into the cache from
     the workgroup that adds the slices up).  Last-row logits and the next tokens, which read that cache, against the
-    oracle; a prefill in chunks, whose Linears have fewer tiles and no slices, must give the same tokens."""
+    oracle; a prefill in chunks, whose Linears have fewer tiles and no slices, must give the same tokens.  From 256 rows on
+    the attention of an unchunked prompt runs on the bf16 matrix cores from fragments the QKV Linear writes (255: the
+    fp32 kernel; 256 and 257: the first lengths on the other path, whole and ragged last tile)."""
     from async_gpu_amd import gpt2, workloads
     cfg = dict(n_layer=2, n_embd=768, n_head=12, vocab=1031, n_positions=1024)
     w, qz = _quantized(orc, cfg, 17, nonzero_bias=True, random_ln=True)
@@ -335,7 +337,8 @@ def test_long_prefill_small_width(orc, agpu, dev, prompt_len):
     gm.reset_cache()
     for lo_i in range(0, prompt_len, 250):
         lc = gm.forward_cached(prompt[lo_i:lo_i + 250].reshape(1, -1))[0]
-    assert np.abs(lc[-1] - lg[-1]).max() <= 2e-5
+    # the chunks take other kernels (a last chunk of 5 to 7 rows: the batched decode Linear), so other orders of summation
+    assert np.abs(lc[-1] - lg[-1]).max() <= 5e-5
 
 
 def test_long_early_exit_forward_after_a_generation(orc, agpu, dev):
