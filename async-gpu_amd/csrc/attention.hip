@@ -1,7 +1,7 @@
 // Causal attention for gfx950, d_head = 64, fp32.
 //   * attn_mfma_kernel: prefill / chunked prefill.  One wave per 32 query rows; S^T = K Q^T and
 //     O^T = V^T P^T on v_mfma_f32_32x32x2_f32 with online softmax; K/V tiles of 32 keys in LDS.
-//   * attn_bf16_kernel: the same for a prompt of 256 queries or more at position 0, on v_mfma_f32_32x32x16_bf16 with every
+//   * attn_bf16_kernel: the same for prompts of 256 queries or more at position 0, on v_mfma_f32_32x32x16_bf16 with every
 //     operand as three exact bf16 pieces; K and V come as operand fragments (written by split_kv_kernel here or by
 //     the Linear that produces them).
 //   * attn_decode_kernel: decode (few query rows).  One workgroup per (head, query row); its waves

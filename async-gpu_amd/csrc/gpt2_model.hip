@@ -310,15 +310,16 @@ int32_t launch_embed(agpu_gpt2 *m, const uint32_t *tokens, int B, int new_len) {
     return AGPU_LAUNCH_CHECK(m->ctx, "embed_rows_kernel");
 }
 
-// A prompt of one sequence, long enough for eight key tiles, into an empty cache: the QKV Linear also writes K and V as
+// Prompts long enough for eight key tiles (whole numbers of key tiles when there are several) into an empty cache: the QKV Linear also writes K and V as
 // the operand fragments of the bf16 attention kernel (where its kernel for the shape can).  The buffers are sized
 // whatever the cache holds at the time; a launch uses them only if they are large enough.
 bool fragments_possible(const agpu_gpt2 *m, int B, int new_len) {
-    return B == 1 && new_len >= 256 && m->cfg.group_size % 32 == 0 && agpu_int4_gemm_bf16_writes_kv_frags(m->ctx, new_len, 3 * m->d, m->d);
+    return (B == 1 || new_len % 32 == 0) && new_len >= 256 && m->cfg.group_size % 32 == 0 &&
+           agpu_int4_gemm_bf16_writes_kv_frags(m->ctx, B * new_len, 3 * m->d, m->d);
 }
 bool prefill_uses_fragments(const agpu_gpt2 *m, int B, int new_len) {
     if (!fragments_possible(m, B, new_len) || m->cache_len != 0) return false;
-    const size_t need = agpu_attention_fragment_bytes(m->H, new_len);
+    const size_t need = agpu_attention_fragment_bytes(B * m->H, new_len);
     return m->kfrag.p && m->vfrag.p && m->kfrag.bytes >= need && m->vfrag.bytes >= need;
 }
 
@@ -460,7 +461,7 @@ int32_t ensure_buffers(agpu_gpt2 *m, int B, int new_len, bool all_rows_logits) {
     if ((rc = ensure(m, m->last, (size_t)B * d * 4)) != AGPU_OK) return rc;
     if ((rc = ensure(m, m->logits, Rl * logits_stride(m) * 4)) != AGPU_OK) return rc;
     if (fragments_possible(m, B, new_len)) {
-        const size_t bytes = agpu_attention_fragment_bytes(m->H, new_len);
+        const size_t bytes = agpu_attention_fragment_bytes(B * m->H, new_len);
         if ((rc = ensure(m, m->kfrag, bytes)) != AGPU_OK) return rc;
         if ((rc = ensure(m, m->vfrag, bytes)) != AGPU_OK) return rc;
     }

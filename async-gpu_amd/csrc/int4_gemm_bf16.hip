@@ -99,7 +99,9 @@ template <int RB, int CB, int NCH, int GB_WAVES>
 __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const GemmBfParams p) {
     static_assert(NCH % 2 == 0, "staging works on 64-k halves");
     constexpr int GB_BM = 32 * RB, GB_BN = 32 * CB * GB_WAVES, GB_KB = 32 * NCH, NP = RB * NCH / 2;
-    __shared__ __align__(16) unsigned char s_a[2][NCH * RB * 3 * 2 * 2 * GB_FRAG_BYTES];  // 6 KiB per (chunk, row block)
+    constexpr int STAGE_BYTES = NCH * RB * 3 * 2 * 2 * GB_FRAG_BYTES;  // 6 KiB per (chunk, row block)
+    constexpr int TRANSPOSE_BYTES = GB_WAVES * 32 * 36 * 4;            // the epilogue's K tiles, one per wave
+    __shared__ __align__(16) unsigned char s_a[2][STAGE_BYTES > TRANSPOSE_BYTES / 2 ? STAGE_BYTES : TRANSPOSE_BYTES / 2];
     __shared__ int s_last;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int j = lane & 31, hh = lane >> 5;
@@ -366,10 +368,12 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
             // key positions from 0; rows past M repeat the last row and are never visible).  A wave's 32 columns are
             // half a head.  V: a lane holds column d and the 16 keys of its registers, which is the operand as it is.
             // K: a lane needs 8 columns of one key, so the tile goes through LDS (free after the K loop) transposed.
-            if constexpr (RB == 1 && CB == 1 && GB_WAVES == 4) {
-                if (p.kv.kfrag && n0 >= p.N / 3) {  // wave-uniform
-                    const int dm = p.N / 3, e0 = n0 - dm, in_v = e0 >= dm ? 1 : 0, c0 = e0 - in_v * dm;
-                    const int head = c0 >> 6, dblk = (c0 >> 5) & 1, tile = m0 >> 5;
+            {
+                if (p.kv.kfrag && n0 + 32 * cb >= p.N / 3) {  // wave-uniform
+                    const int dm = p.N / 3, e0 = n0 + 32 * cb - dm, in_v = e0 >= dm ? 1 : 0, c0 = e0 - in_v * dm;
+                    // the 32 rows are keys 32 tile .. of sequence seq (sequences are whole numbers of 32-row blocks)
+                    const int row0 = m0 + 32 * rb, seq = row0 / p.kv.new_len, tile = (row0 - seq * p.kv.new_len) >> 5;
+                    const int head = seq * p.kv.n_heads + (c0 >> 6), dblk = (c0 >> 5) & 1;
                     const size_t base = ((size_t)head * p.kv.tiles_cap + tile) * KV_FRAGS_PER_TILE;
                     float r1[16], r2[16];
                     if (in_v) {
@@ -436,8 +440,8 @@ GemmVariant pick_variant(const agpu_ctx *ctx, int M, int N, int K) {
 }  // namespace
 
 bool agpu_int4_gemm_bf16_writes_kv_frags(const agpu_ctx *ctx, int M, int N, int K) {
-    const GemmVariant v = pick_variant(ctx, M, N, K);
-    return (v == GemmVariant::Small || v == GemmVariant::LongBlocks) && N % 3 == 0 && (N / 3) % 64 == 0;
+    (void)ctx; (void)M; (void)K;
+    return N % 3 == 0 && (N / 3) % 64 == 0;
 }
 
 bool agpu_int4_gemm_bf16_supported(const void *x, int M, int N, int K, int group) {
@@ -455,7 +459,6 @@ int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t
     p.M = M; p.N = N; p.K = K; p.chunk_shift = __builtin_ctz((unsigned)(group / 32)); p.flags = flags;
     const GemmVariant var = pick_variant(ctx, M, N, K);
     const bool large = var == GemmVariant::Large, long_blocks = var == GemmVariant::LongBlocks, wide = var == GemmVariant::Wide;
-    if (large || wide) p.kv.kfrag = p.kv.vfrag = nullptr;  // only the four-wave 32 x 128 kernels write the attention's fragments
     const int BM = large ? 64 : 32, BN = large || wide ? 256 : 128;
     const int tiles = ceil_div(N, BN) * ceil_div(M, BM);
     const int KB = long_blocks ? 128 : 64;

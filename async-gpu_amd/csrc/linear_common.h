@@ -86,16 +86,16 @@ struct KvScatter {
     float *vcache;
     const int *pos_dev;
     int n_heads, n_positions, new_len;
-    // Optional (one sequence written from position 0): K and V also as the bf16 operand fragments of the prefill
-    // attention, [head][tiles_cap tiles of 32 keys][768 fragments of 16 bytes] each.  The launcher clears the pointers
-    // when the kernel variant it picks cannot write them.
+    // Optional (sequences written from position 0; with more than one sequence new_len % 32 == 0): K and V also as the
+    // bf16 operand fragments of the prefill attention, [sequence * n_heads + head][tiles_cap tiles of 32 keys][768
+    // fragments of 16 bytes] each.
     uint4 *kfrag = nullptr, *vfrag = nullptr;
     int tiles_cap = 0;
 };
 // bf16-MFMA GEMM for M > 16 with x split into three bf16 pieces (needs group / 32 a power of two, K % 32 == 0,
 // 16-byte aligned x).  kv (optional): the K/V scatter above, done by the same launch.
 bool agpu_int4_gemm_bf16_supported(const void *x, int M, int N, int K, int group);
-// Whether the launch for this shape can also write kv->kfrag / kv->vfrag (else it leaves them alone).
+// Whether the launch for this shape also writes kv->kfrag / kv->vfrag.
 bool agpu_int4_gemm_bf16_writes_kv_frags(const agpu_ctx *ctx, int M, int N, int K);
 int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t *packed, const float *scales, const float *bias,
                                    const float *residual, float *y, int M, int N, int K, int group, uint32_t flags,

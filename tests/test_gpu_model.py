@@ -358,3 +358,28 @@ def test_long_early_exit_forward_after_a_generation(orc, agpu, dev):
         assert gu == wu == 2
         assert np.abs(got - want).max() <= TOL_LOGITS * max(1.0, np.abs(want).max())
 
+
+@pytest.mark.parametrize("batch,prompt_len", [(2, 288), (4, 512), (3, 300)])
+def test_long_prompts_in_a_batch(orc, agpu, dev, batch, prompt_len):
+    """Several long prompts at once.  Where a prompt is a whole number of 32-row blocks, the QKV Linear (2048 rows: its
+    64 x 256 tiles; 576 rows: 32 x 128) writes every sequence's K and V fragments and the attention runs on the bf16
+    matrix cores; 300 rows per prompt stay on the fp32 kernel.  Last-row logits of every sequence against the oracle,
+    the next tokens against the same prompt run alone."""
+    from async_gpu_amd import gpt2, workloads
+    cfg = dict(n_layer=2, n_embd=768, n_head=12, vocab=1031, n_positions=640)
+    w, qz = _quantized(orc, cfg, 19, nonzero_bias=True, random_ln=True)
+    om = build_oracle_model(cfg, qz)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg, max_batch=batch), qz)
+    prompts = workloads.random_prompt(cfg, 8, prompt_len, batch=batch)
+    gm.reset_cache()
+    lg = gm.forward_cached(prompts, all_rows=False)
+    for b in range(batch):
+        om.reset_cache()
+        lo = om.forward(prompts[b], all_rows=False)
+        assert np.abs(lg[b] - lo[0]).max() <= TOL_LOGITS, b
+    outs, _ = gm.generate_cached(prompts, 6, eos=-1)
+    one = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg), qz)
+    for b in (0, batch - 1):
+        (alone,), _ = one.generate_cached(prompts[b], 6, eos=-1)
+        assert np.array_equal(outs[b], alone), b
+
