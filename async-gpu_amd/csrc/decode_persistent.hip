@@ -367,6 +367,31 @@ __device__ __forceinline__ float slot_dot(const uint32_t (&w)[4], const float *x
     return ((dq[0] + dq[1]) + (dq[2] + dq[3])) - 8.0f * sx;
 }
 
+// The same with the nibbles of the four words already converted (done while the stage's input was awaited).
+__device__ __forceinline__ float slot_dot_pre(const float (&nf)[32], const float *xs, const float *xsum, int g) {
+    const float4 *xg = reinterpret_cast<const float4 *>(xs + GS * g);
+    float4 xr[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) xr[i] = xg[i];
+    const float sx = xsum[g];
+    __builtin_amdgcn_sched_barrier(0);
+    float dq[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const float4 xa = xr[2 * q], xb = xr[2 * q + 1];
+        float dot = xa.x * nf[8 * q];
+        dot = fmaf(xa.y, nf[8 * q + 1], dot);
+        dot = fmaf(xa.z, nf[8 * q + 2], dot);
+        dot = fmaf(xa.w, nf[8 * q + 3], dot);
+        dot = fmaf(xb.x, nf[8 * q + 4], dot);
+        dot = fmaf(xb.y, nf[8 * q + 5], dot);
+        dot = fmaf(xb.z, nf[8 * q + 6], dot);
+        dot = fmaf(xb.w, nf[8 * q + 7], dot);
+        dq[q] = dot;
+    }
+    return ((dq[0] + dq[1]) + (dq[2] + dq[3])) - 8.0f * sx;
+}
+
 // ---- what a wave requests ahead of a Linear stage ----
 // Slot s of a chunk = (tile tt, round u), tile-major.  Round u of wave w covers groups (u W + w) gpw + j,
 // gpw = 4 >> tws groups per wave-wide load; lane (col, j) takes group j of the round for column col of the tile.
@@ -465,7 +490,8 @@ __device__ __forceinline__ void lay_prefetch(const Stage &st, Regs &r, int tile,
 }
 
 // This lane's column over its groups, then over the lanes of the wave that hold the same column.
-__device__ __forceinline__ float lay_compute(const Stage &st, const Regs &r, const float *xs, const float *xsum, int wave, int lane) {
+__device__ __forceinline__ float lay_compute(const Stage &st, const Regs &r, const float (&pre)[32], const float *xs, const float *xsum, int wave,
+                                             int lane) {
     const int gpw = 4 >> st.tws;
     const int j = lane >> (4 + st.tws);
     float acc = 0.0f;
@@ -474,7 +500,7 @@ __device__ __forceinline__ float lay_compute(const Stage &st, const Regs &r, con
         if (u >= st.nl) break;  // wave-uniform
         int g = (u * W + wave) * gpw + j;
         g = g < st.n_groups ? g : st.n_groups - 1;  // beyond the last group the words and the scale are zero
-        acc = fmaf(r.sc[u], slot_dot(r.w[u], xs, xsum, g), acc);
+        acc = fmaf(r.sc[u], u == 0 ? slot_dot_pre(pre, xs, xsum, g) : slot_dot(r.w[u], xs, xsum, g), acc);
     }
     return reduce_groups(acc, st.tws);
 }
@@ -752,10 +778,22 @@ __device__ __forceinline__ void lay_stage(const Params &p, const Stage &st, Ctl 
         else if (st.res_off == -2 && real) resf = p.wte[(size_t)tok * p.d + n] + p.wpe[(size_t)pos * p.d + n];
     }
     PK_STAMP(0);
+    // the first slot's nibbles become floats before the input is awaited: the weights have been there for a stage, and
+    // the conversions (two thirds of a slot's vector time) then cost nothing once the input has arrived
+    float pre[32];
+    if (real) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            float nf[8];
+            unpack_bytes(r.w[0][q], nf);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pre[8 * q + e] = nf[e];
+        }
+    }
     stage_input<MODE>(p, st, c, xs, xsum, stat, mirror, pos, tok, tid,
                       [&] { asm volatile("" ::"v"(bias), "v"(resf), "v"(res), "v"(sink[0]), "v"(sink[1]), "v"(sink[2])); });
     if (real) {
-        const float part = lay_compute(st, r, xs, xsum, wave, lane);
+        const float part = lay_compute(st, r, pre, xs, xsum, wave, lane);
         if (lane < tw) red[wave * 64 + lane] = part;
     }
     PK_STAMP(4);
