@@ -367,8 +367,9 @@ __device__ __forceinline__ float slot_dot(const uint32_t (&w)[4], const float *x
     return ((dq[0] + dq[1]) + (dq[2] + dq[3])) - 8.0f * sx;
 }
 
+constexpr int NPRE = 2;  // slots whose nibbles are converted ahead of the input
 // The same with the nibbles of the four words already converted (done while the stage's input was awaited).
-__device__ __forceinline__ float slot_dot_pre(const float (&nf)[32], const float *xs, const float *xsum, int g) {
+__device__ __forceinline__ float slot_dot_pre(const float *nf, const float *xs, const float *xsum, int g) {
     const float4 *xg = reinterpret_cast<const float4 *>(xs + GS * g);
     float4 xr[8];
 #pragma unroll
@@ -490,8 +491,8 @@ __device__ __forceinline__ void lay_prefetch(const Stage &st, Regs &r, int tile,
 }
 
 // This lane's column over its groups, then over the lanes of the wave that hold the same column.
-__device__ __forceinline__ float lay_compute(const Stage &st, const Regs &r, const float (&pre)[32], const float *xs, const float *xsum, int wave,
-                                             int lane) {
+__device__ __forceinline__ float lay_compute(const Stage &st, const Regs &r, const float (&pre)[NPRE * 32], const float *xs, const float *xsum,
+                                             int wave, int lane) {
     const int gpw = 4 >> st.tws;
     const int j = lane >> (4 + st.tws);
     float acc = 0.0f;
@@ -500,7 +501,7 @@ __device__ __forceinline__ float lay_compute(const Stage &st, const Regs &r, con
         if (u >= st.nl) break;  // wave-uniform
         int g = (u * W + wave) * gpw + j;
         g = g < st.n_groups ? g : st.n_groups - 1;  // beyond the last group the words and the scale are zero
-        acc = fmaf(r.sc[u], u == 0 ? slot_dot_pre(pre, xs, xsum, g) : slot_dot(r.w[u], xs, xsum, g), acc);
+        acc = fmaf(r.sc[u], u < NPRE ? slot_dot_pre(pre + 32 * (u < NPRE ? u : 0), xs, xsum, g) : slot_dot(r.w[u], xs, xsum, g), acc);
     }
     return reduce_groups(acc, st.tws);
 }
@@ -780,14 +781,18 @@ __device__ __forceinline__ void lay_stage(const Params &p, const Stage &st, Ctl 
     PK_STAMP(0);
     // the first slot's nibbles become floats before the input is awaited: the weights have been there for a stage, and
     // the conversions (two thirds of a slot's vector time) then cost nothing once the input has arrived
-    float pre[32];
+    float pre[NPRE * 32];
     if (real) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            float nf[8];
-            unpack_bytes(r.w[0][q], nf);
+        for (int u = 0; u < NPRE; ++u) {
+            if (u >= st.nl) break;  // wave-uniform
 #pragma unroll
-            for (int e = 0; e < 8; ++e) pre[8 * q + e] = nf[e];
+            for (int q = 0; q < 4; ++q) {
+                float nf[8];
+                unpack_bytes(r.w[u][q], nf);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pre[32 * u + 8 * q + e] = nf[e];
+            }
         }
     }
     stage_input<MODE>(p, st, c, xs, xsum, stat, mirror, pos, tok, tid,
