@@ -367,7 +367,7 @@ __device__ __forceinline__ float slot_dot(const uint32_t (&w)[4], const float *x
     return ((dq[0] + dq[1]) + (dq[2] + dq[3])) - 8.0f * sx;
 }
 
-constexpr int NPRE = 2;  // slots whose nibbles are converted ahead of the input
+constexpr int NPRE = 3;  // slots whose nibbles are converted ahead of the input
 // The same with the nibbles of the four words already converted (done while the stage's input was awaited).
 __device__ __forceinline__ float slot_dot_pre(const float *nf, const float *xs, const float *xsum, int g) {
     const float4 *xg = reinterpret_cast<const float4 *>(xs + GS * g);
