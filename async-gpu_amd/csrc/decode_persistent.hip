@@ -35,6 +35,9 @@
 // the stage before it ended, so that few workgroups have tiles in two stages in a row: such a workgroup can request the
 // second stage's weights only when it has published the first, and then they arrive after the input.  Where it cannot
 // be avoided and the tile is large, the workgroup touches the tile's cache lines a stage earlier (warm_tile).
+// What does not depend on a stage's input is done before the workgroup starts to wait for it: besides the requests
+// above, the nibbles of the first NPRE slots are turned into floats then (a byte convert takes twice the issue time of
+// the multiply-add that follows it), so that after the wait those slots cost their multiply-adds only.
 //
 // Every wait is bounded: a poll that does not succeed within kSpinLimit rounds sets the error word, all
 // workgroups then stop waiting, and the step ends with garbage that the host reports as an error.
