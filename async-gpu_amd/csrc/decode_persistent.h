@@ -46,6 +46,9 @@ struct PkPlan {
     int kmax = 0;         // longest input vector of a Linear: sizes the staging buffers
     int head_slots = 0;   // slots of the head's second chunk that wait in LDS (0: fetched when their turn comes)
     int spin_limit = 0;   // poll rounds a wait inside the kernel may take; 0 = the default
+    int kind = 0;         // 0: every Linear spread over the device (decode_persistent.hip); 1: one tensor-parallel rank per XCD (decode_xcd.hip)
+    int lin_per_xcd = 0;  // kind 1: Linear workgroups per XCD
+    int touch_dist = 0;   // kind 1: how many exchanges ahead the relays touch the weights (0: not at all)
 };
 
 // Whether the persistent step can run this model (int4 head, head_dim 64, group 32, size limits).
@@ -55,5 +58,13 @@ void agpu_pk_plan_free(PkPlan *plan);
 // One decode step on the context's stream.  mode 0: the real step; mode 1: the same stage chain with empty bodies
 // (every wait and every tagged store, no weights, no arithmetic): the latency floor of the chain.
 int32_t agpu_pk_launch(agpu_ctx *ctx, const PkModel &m, const PkPlan &plan, int mode, unsigned long long *trace = nullptr);
+// The same step with the XCDs as tensor-parallel ranks (decode_xcd.hip): plan (freed by agpu_pk_plan_free) and launch.
+bool agpu_xk_supported(const agpu_ctx *ctx, const PkModel &m);
+int32_t agpu_xk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan);
+int32_t agpu_xk_launch(agpu_ctx *ctx, const PkModel &m, const PkPlan &plan, int mode, unsigned long long *trace = nullptr);
+// Launches a plan of either kind.
+inline int32_t agpu_step_launch(agpu_ctx *ctx, const PkModel &m, const PkPlan &plan, int mode, unsigned long long *trace = nullptr) {
+    return plan.kind == 1 ? agpu_xk_launch(ctx, m, plan, mode, trace) : agpu_pk_launch(ctx, m, plan, mode, trace);
+}
 // Reads and clears the error word (synchronises the stream).  0 = no error.
 int32_t agpu_pk_take_error(agpu_ctx *ctx, const PkPlan &plan, unsigned int *err_out);

@@ -1,0 +1,1692 @@
+// One launch per decoded token for a single sequence, with the eight XCDs of the device as eight tensor-parallel
+// ranks: the step of generate_cached's loop (nn/models/gpt2.rs:760-780 over Int4TransformerBlock::forward,
+// gpt2.rs:1307-1338) inside one kernel whose workgroups stay resident, one per CU.
+//
+// An XCD's CUs share one L2; a word that another XCD must see has to travel through memory (about 0.55 us one way,
+// against 0.2 us for a round trip through the L2).  A layer is therefore cut so that as little as possible crosses
+// XCDs, Megatron style:
+//
+//   XCD x owns the heads h0_x .. h0_x + nh_x - 1 and the columns f0_x .. f0_x + nf_x - 1 of the MLP's hidden vector.
+//     LN1 + QKV Linear, columns q, k, v of its heads only (+ K/V rows into the cache)      -> stays in the XCD's L2
+//     attention of its heads                                                              -> stays in the L2
+//     proj Linear over the rows of its heads: a partial sum of all d outputs              -> memory      (exchange 1)
+//     LN2 + fc Linear + GELU, its columns only                                            -> stays in the L2
+//     fc-proj Linear over the rows f0_x ..: a partial sum of all d outputs                -> memory      (exchange 2)
+//   then final LayerNorm + LM head + arg-max + token feed on everybody.
+//
+// An exchange: a few relay workgroups per XCD poll the partial sums of all XCDs in memory, add them in a fixed order
+// with the bias and the residual (which they keep in registers from the exchange before), and put the new hidden
+// vector into their own XCD's mirror; every XCD so holds the same bits.  Per layer two hand-offs go through memory and
+// three through an L2, where the step with all Linears spread over the whole device needs five through memory.
+//
+// Everything that travels is a (value, tag) pair, tag = number of the step: a consumer polls the very words it needs
+// and takes a value once its tag is the current step's.  The data is its own flag: no counters, no fences; a stale read
+// can only delay a tag.  Every vector of a step has its own place, so nothing is overwritten while the step runs.
+//
+// Roles per XCD: NR relays, a few attention workgroups ((head, key range) each, the cached K and V rows of the next
+// layer requested into registers as soon as this layer's are used up), the rest Linear workgroups.  A Linear stage of
+// an XCD is cut into units of 16, 32 or 64 adjacent columns; `wpt` waves share a unit (they split its scale groups),
+// a workgroup has up to 8 / wpt units.  A lane holds, per slot, the four packed words of one scale group (32 k) of one
+// column and that group's scale.  The input vector is staged in LDS together with the sum of every group
+// (u = sum x n - 8 sum x, acc += scale u); fp32 FMAs on the unsigned nibbles; the lanes of a column meet by row swaps,
+// the waves of a unit through LDS.  The weights of the next stage are requested into registers as soon as a stage is
+// published; the relays touch the XCD's share of the weights a half layer or more ahead, so that these requests are
+// served from the L2.  Every wait is bounded: a poll that does not succeed within the limit sets the error word, all
+// workgroups then stop waiting, and the step ends with garbage that the host reports as an error.
+#include "decode_persistent.h"
+
+#include <algorithm>
+#include <vector>
+
+#include "linear_common.h"
+
+namespace {
+
+using u64 = unsigned long long;
+constexpr int T = 512, W = T / 64;
+constexpr int SL = 8;           // (group, column) items a lane holds per register set: 4 words + 1 scale each
+constexpr int KVP = 8;          // attention: rounds of KR keys (K and V, 16 bytes per lane each) held in registers
+constexpr int KR = 4 * W;       // keys per round: four per wave
+constexpr int XMAX = 2048;      // longest input vector of a stage (staged in LDS): d, or an XCD's share of the MLP's hidden vector
+constexpr int GS = 36;          // floats between the groups of 32 in LDS (bank spread for 16-byte reads)
+constexpr int PMAX = XMAX / (2 * T);  // pairs of input elements a thread polls at most
+constexpr int LNP = 2048 / (2 * T);   // ... of a stage with LayerNorm (K <= 2048)
+constexpr int SMAX = 4;         // key ranges per head at most
+constexpr int PSTRIDE = 68;     // floats per partial attention result: o[64], m, l
+constexpr int kSpinLimit = 1 << 16;
+constexpr int DH = 64;
+#ifndef AGPU_XK_NR
+#define AGPU_XK_NR 2
+#endif
+constexpr int NR = AGPU_XK_NR;  // relay workgroups per XCD
+constexpr int XI = 8;           // column pairs a relay thread owns at most (d <= 2048)
+constexpr int NPRE = 3;         // slots whose nibbles are converted ahead of the input
+
+enum : int { F_LN = 1, F_GELU_TANH = 2, F_GELU_QUICK = 4, F_HEAD = 8, F_SCATTER = 16, F_PARTIAL = 32 };
+
+// One Linear of the step as one XCD sees it (every XCD has its own table).  The QKV entry of a layer also carries what
+// the layer's attention needs, the two partial-sum entries what the exchange behind them needs.
+struct Stage {
+    const uint32_t *packed;                // first packed row of the XCD's k range
+    const float *scales;                   // first scale row of it
+    const float *bias, *ln_g, *ln_b;       // bias: null for partial sums (the exchange adds it)
+    const float *xbias;                    // exchange: bias of the whole Linear
+    float *kc, *vc;                        // this layer's cache, sequence 0: [H, n_positions, 64]
+    int K, n_groups, stride, tws;          // the XCD's k range; tws = log2(unit width / 16)
+    int wps, nl, n_units, upp;             // log2(waves per unit), slots per lane, units, units per column part
+    int col0, part_stride, pcols, n_cparts;  // unit u: part = u / upp, columns col0 + part * part_stride + (u % upp) * tw ..; pcols valid per part
+    int in_off, out_off, att_off, part_off;  // mirror offsets; in_off -2: embedding row; out_off of a partial sum: in the arena
+    int xout_off, xn_parts, n_valid, n_tiles;  // exchange: where the sum goes, how many XCDs contribute; head: columns, tiles
+    int n_wgs, tpc, flags;                 // head: workgroups sharing the tiles, tiles per chunk of SL slots
+    float inv_k;
+    int li0, ngrp;                         // the Linear workgroups li0 .. li0 + ngrp - 1 of the XCD share the stage's units
+    int pad_[2];
+};
+static_assert(sizeof(Stage) % 16 == 0, "stage table is copied in 16-byte pieces");
+
+struct Params {
+    const Stage *stages;  // [8][n_stages]
+    int n_stages, n_layer;
+    u64 *arena;           // [8][mirror_elems] mirrors, then the partial sums, then the arg-max candidates
+    size_t mirror_elems;
+    size_t cand_off;
+    unsigned *state;      // [0] epoch, [1] error, [2] workgroups started so far
+    const float *wte, *wpe;
+    float *logits;
+    uint32_t *cur_tok, *out_tok, *next_tok;
+    int *pos_dev, *step_dev;
+    int out_capacity;
+    int d, H, P, V;
+    float eps;
+    int argmax_last;
+    int att_per_xcd, smax, nlin;
+    int spin_limit;
+    int xbuf;             // floats of one staging buffer
+    int head_slots;       // slots of the head's second chunk kept in LDS ahead of the head stage (0: none)
+    int touch_dist;       // exchanges between a relay's touch of a half layer's weights and their use (0: no touching)
+    unsigned long long *trace;
+};
+
+struct Ctl {
+    uint32_t epoch;
+    unsigned *err;
+    int stage;
+    bool dead;
+    int spin_limit;
+    u64 *tr;
+};
+
+// Coherent across the XCDs: to and from memory.
+__device__ __forceinline__ u64 ld_tag(const u64 *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void st_tag(u64 *p, float v, uint32_t tag) {
+    __hip_atomic_store(p, ((u64)tag << 32) | (u64)__float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Within an XCD: an ordinary store lands in the L2 the XCD's CUs share (the CU's own cache writes through) ...
+__device__ __forceinline__ void st_loc(u64 *p, float v, uint32_t tag) {
+    const u64 w = ((u64)tag << 32) | (u64)__float_as_uint(v);
+    asm volatile("global_store_dwordx2 %0, %1, off" ::"v"(p), "v"(w) : "memory");
+}
+__device__ __forceinline__ void st_loc2(u64 *p, float a, float b, uint32_t tag) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 w;
+    w.x = __float_as_uint(a); w.y = tag; w.z = __float_as_uint(b); w.w = tag;
+    asm volatile("global_store_dwordx4 %0, %1, off" ::"v"(p), "v"(w) : "memory");
+}
+// ... and a load past the CU's own cache finds it there.
+__device__ __forceinline__ u64 ld_loc(const u64 *p) {
+    u64 v;
+    asm volatile("global_load_dwordx2 %0, %1, off nt\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(p) : "memory");
+    return v;
+}
+__device__ __forceinline__ float tag_val(u64 w) { return __uint_as_float((uint32_t)w); }
+__device__ __forceinline__ bool tag_ok(u64 w, uint32_t epoch) { return (uint32_t)(w >> 32) == epoch; }
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 as_u4(const u32x4 &v) { return make_uint4(v.x, v.y, v.z, v.w); }
+
+// N 16-byte loads (two pairs each) in flight at once; L2: past the CU's cache, from the XCD's L2; else from memory.
+#define AGPU_LD1(POL) "global_load_dwordx4 %0, %1, off " POL "\n\ts_waitcnt vmcnt(0)"
+template <bool L2>
+__device__ __forceinline__ void ld_pairs(const u64 *const (&p)[1], uint4 (&o)[1]) {
+    u32x4 v0;
+    if (L2) asm volatile(AGPU_LD1("nt") : "=&v"(v0) : "v"(p[0]) : "memory");
+    else asm volatile(AGPU_LD1("sc1") : "=&v"(v0) : "v"(p[0]) : "memory");
+    o[0] = as_u4(v0);
+}
+#define AGPU_LD2(POL) "global_load_dwordx4 %0, %2, off " POL "\n\tglobal_load_dwordx4 %1, %3, off " POL "\n\ts_waitcnt vmcnt(0)"
+template <bool L2>
+__device__ __forceinline__ void ld_pairs(const u64 *const (&p)[2], uint4 (&o)[2]) {
+    u32x4 v0, v1;
+    if (L2) asm volatile(AGPU_LD2("nt") : "=&v"(v0), "=&v"(v1) : "v"(p[0]), "v"(p[1]) : "memory");
+    else asm volatile(AGPU_LD2("sc1") : "=&v"(v0), "=&v"(v1) : "v"(p[0]), "v"(p[1]) : "memory");
+    o[0] = as_u4(v0); o[1] = as_u4(v1);
+}
+#define AGPU_LD4(POL)                                                                                              \
+    "global_load_dwordx4 %0, %4, off " POL "\n\tglobal_load_dwordx4 %1, %5, off " POL "\n\t"                        \
+    "global_load_dwordx4 %2, %6, off " POL "\n\tglobal_load_dwordx4 %3, %7, off " POL "\n\ts_waitcnt vmcnt(0)"
+template <bool L2>
+__device__ __forceinline__ void ld_pairs(const u64 *const (&p)[4], uint4 (&o)[4]) {
+    u32x4 v0, v1, v2, v3;
+    if (L2) asm volatile(AGPU_LD4("nt") : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3) : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]) : "memory");
+    else asm volatile(AGPU_LD4("sc1") : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3) : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]) : "memory");
+    o[0] = as_u4(v0); o[1] = as_u4(v1); o[2] = as_u4(v2); o[3] = as_u4(v3);
+}
+#define AGPU_LD6(POL)                                                                                              \
+    "global_load_dwordx4 %0, %6, off " POL "\n\tglobal_load_dwordx4 %1, %7, off " POL "\n\t"                        \
+    "global_load_dwordx4 %2, %8, off " POL "\n\tglobal_load_dwordx4 %3, %9, off " POL "\n\t"                        \
+    "global_load_dwordx4 %4, %10, off " POL "\n\tglobal_load_dwordx4 %5, %11, off " POL "\n\ts_waitcnt vmcnt(0)"
+template <bool L2>
+__device__ __forceinline__ void ld_pairs(const u64 *const (&p)[6], uint4 (&o)[6]) {
+    u32x4 v0, v1, v2, v3, v4, v5;
+    if (L2)
+        asm volatile(AGPU_LD6("nt") : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3), "=&v"(v4), "=&v"(v5)
+                     : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]) : "memory");
+    else
+        asm volatile(AGPU_LD6("sc1") : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3), "=&v"(v4), "=&v"(v5)
+                     : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]) : "memory");
+    o[0] = as_u4(v0); o[1] = as_u4(v1); o[2] = as_u4(v2); o[3] = as_u4(v3); o[4] = as_u4(v4); o[5] = as_u4(v5);
+}
+#define AGPU_LD8(POL)                                                                                              \
+    "global_load_dwordx4 %0, %8, off " POL "\n\tglobal_load_dwordx4 %1, %9, off " POL "\n\t"                        \
+    "global_load_dwordx4 %2, %10, off " POL "\n\tglobal_load_dwordx4 %3, %11, off " POL "\n\t"                      \
+    "global_load_dwordx4 %4, %12, off " POL "\n\tglobal_load_dwordx4 %5, %13, off " POL "\n\t"                      \
+    "global_load_dwordx4 %6, %14, off " POL "\n\tglobal_load_dwordx4 %7, %15, off " POL "\n\ts_waitcnt vmcnt(0)"
+template <bool L2>
+__device__ __forceinline__ void ld_pairs(const u64 *const (&p)[8], uint4 (&o)[8]) {
+    u32x4 v0, v1, v2, v3, v4, v5, v6, v7;
+    if (L2)
+        asm volatile(AGPU_LD8("nt") : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3), "=&v"(v4), "=&v"(v5), "=&v"(v6), "=&v"(v7)
+                     : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]) : "memory");
+    else
+        asm volatile(AGPU_LD8("sc1") : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3), "=&v"(v4), "=&v"(v5), "=&v"(v6), "=&v"(v7)
+                     : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]) : "memory");
+    o[0] = as_u4(v0); o[1] = as_u4(v1); o[2] = as_u4(v2); o[3] = as_u4(v3);
+    o[4] = as_u4(v4); o[5] = as_u4(v5); o[6] = as_u4(v6); o[7] = as_u4(v7);
+}
+__device__ __forceinline__ bool pair_ok(const uint4 &v, uint32_t epoch) { return v.y == epoch && v.w == epoch; }
+
+// After an unsuccessful poll round: true when the caller must give up.
+__device__ __forceinline__ bool spin_fail(Ctl &c, int &spins) {
+    ++spins;
+    if (spins > c.spin_limit) {
+        atomicCAS(c.err, 0u, 0x1000u + (unsigned)c.stage);
+        c.dead = true;
+        return true;
+    }
+    if ((spins & 255) == 0 && __hip_atomic_load(c.err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
+        c.dead = true;
+        return true;
+    }
+    return false;
+}
+
+// Polls N pairs of pairs (those with need[k]) until every one carries the step's tags; the values stay in v.
+template <bool L2, int N>
+__device__ __forceinline__ void poll_pairs(Ctl &c, const u64 *const (&ptr)[N], bool (&need)[N], uint4 (&v)[N]) {
+    int spins = 0;
+    while (!c.dead) {
+        uint4 t[N];
+        ld_pairs<L2>(ptr, t);
+        bool ok = true;
+#pragma unroll
+        for (int k = 0; k < N; ++k)
+            if (need[k]) {
+                if (pair_ok(t[k], c.epoch)) { v[k] = t[k]; need[k] = false; } else ok = false;
+            }
+        if (ok || spin_fail(c, spins)) break;
+    }
+}
+
+__device__ __forceinline__ int rfl(int v) { return __builtin_amdgcn_readfirstlane(v); }
+// The stage tables are read with scalar loads (the constant address space says so to the compiler): a stage's 44 words
+// come in three instructions, straight into scalar registers, and can be requested long before they are looked at.
+typedef const __attribute__((address_space(4))) Stage *CStage;
+__device__ __forceinline__ CStage cstage(const Stage *g) { return (CStage)(u64)g; }
+// A pointer out of the stage table, known to point to device memory (a pointer read from memory is otherwise taken
+// for one that may point into LDS, and its loads become flat loads, which every LDS wait waits for).
+template <typename P>
+__device__ __forceinline__ P *glob(P *p) {
+    typedef __attribute__((address_space(1))) P *global_ptr;
+    return (P *)(global_ptr)(u64)p;
+}
+
+__device__ __forceinline__ Stage load_stage(CStage t) {
+    Stage s;
+    s.packed = glob(t->packed); s.scales = glob(t->scales); s.bias = glob(t->bias); s.ln_g = glob(t->ln_g); s.ln_b = glob(t->ln_b);
+    s.xbias = glob(t->xbias); s.kc = glob(t->kc); s.vc = glob(t->vc);
+    s.K = t->K; s.n_groups = t->n_groups; s.stride = t->stride; s.tws = t->tws;
+    s.wps = t->wps; s.nl = t->nl; s.n_units = t->n_units; s.upp = t->upp;
+    s.col0 = t->col0; s.part_stride = t->part_stride; s.pcols = t->pcols; s.n_cparts = t->n_cparts;
+    s.in_off = t->in_off; s.out_off = t->out_off; s.att_off = t->att_off; s.part_off = t->part_off;
+    s.xout_off = t->xout_off; s.xn_parts = t->xn_parts; s.n_valid = t->n_valid; s.n_tiles = t->n_tiles;
+    s.n_wgs = t->n_wgs; s.tpc = t->tpc; s.flags = t->flags;
+    s.inv_k = t->inv_k;
+    s.li0 = t->li0; s.ngrp = t->ngrp;
+    return s;
+}
+
+__device__ __forceinline__ float4 as_f4(const uint4 &v) {
+    return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+}
+
+// Sum over the lanes that hold the same column of a unit of 16 << tws columns, result in every lane.
+__device__ __forceinline__ float reduce_groups(float v, int tws) {
+    if (tws == 0) {
+        const unsigned u = __float_as_uint(v);
+        const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+        v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    }
+    if (tws <= 1) {
+        const unsigned u = __float_as_uint(v);
+        const auto b = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+        v = __uint_as_float(b[0]) + __uint_as_float(b[1]);
+    }
+    return v;
+}
+
+// Sum over each run of eight lanes, the same bits in every lane of the run: ((a0 + a1) + (a2 + a3)) + ((a4 + a5) + (a6 + a7)).
+__device__ __forceinline__ float oct_sum(float v) {
+    v += dpp_move<0xb1, 0xf>(0.0f, v);   // quad_perm [1,0,3,2]
+    v += dpp_move<0x4e, 0xf>(0.0f, v);   // quad_perm [2,3,0,1]
+    v += dpp_move<0x141, 0xf>(0.0f, v);  // row_half_mirror: lane i of the eight <-> lane 7 - i
+    return v;
+}
+
+struct Regs {
+    uint32_t w[SL][4];
+    float sc[SL];
+};
+
+// The eight nibbles of a word as floats (two masks, then the byte converts).
+__device__ __forceinline__ void unpack_bytes(uint32_t w, float (&nf)[8]) {
+    const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+    asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(nf[0]) : "v"(lo));
+    asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(nf[1]) : "v"(hi));
+    asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(nf[2]) : "v"(lo));
+    asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(nf[3]) : "v"(hi));
+    asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(nf[4]) : "v"(lo));
+    asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(nf[5]) : "v"(hi));
+    asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(nf[6]) : "v"(lo));
+    asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(nf[7]) : "v"(hi));
+}
+
+// One slot: the lane's group of 32 inputs against its four packed words; all eight LDS reads are issued before the
+// first product.
+__device__ __forceinline__ float slot_dot(const uint32_t (&w)[4], const float *xs, const float *xsum, int g) {
+    const float4 *xg = reinterpret_cast<const float4 *>(xs + GS * g);
+    float4 xr[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) xr[i] = xg[i];
+    const float sx = xsum[g];
+    __builtin_amdgcn_sched_barrier(0);
+    float dq[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        float nf[8];
+        unpack_bytes(w[q], nf);
+        const float4 xa = xr[2 * q], xb = xr[2 * q + 1];
+        float dot = xa.x * nf[0];
+        dot = fmaf(xa.y, nf[1], dot);
+        dot = fmaf(xa.z, nf[2], dot);
+        dot = fmaf(xa.w, nf[3], dot);
+        dot = fmaf(xb.x, nf[4], dot);
+        dot = fmaf(xb.y, nf[5], dot);
+        dot = fmaf(xb.z, nf[6], dot);
+        dot = fmaf(xb.w, nf[7], dot);
+        dq[q] = dot;
+    }
+    return ((dq[0] + dq[1]) + (dq[2] + dq[3])) - 8.0f * sx;
+}
+
+// The same with the nibbles of the four words already converted (done while the stage's input was awaited).
+__device__ __forceinline__ float slot_dot_pre(const float *nf, const float *xs, const float *xsum, int g) {
+    const float4 *xg = reinterpret_cast<const float4 *>(xs + GS * g);
+    float4 xr[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) xr[i] = xg[i];
+    const float sx = xsum[g];
+    __builtin_amdgcn_sched_barrier(0);
+    float dq[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const float4 xa = xr[2 * q], xb = xr[2 * q + 1];
+        float dot = xa.x * nf[8 * q];
+        dot = fmaf(xa.y, nf[8 * q + 1], dot);
+        dot = fmaf(xa.z, nf[8 * q + 2], dot);
+        dot = fmaf(xa.w, nf[8 * q + 3], dot);
+        dot = fmaf(xb.x, nf[8 * q + 4], dot);
+        dot = fmaf(xb.y, nf[8 * q + 5], dot);
+        dot = fmaf(xb.z, nf[8 * q + 6], dot);
+        dot = fmaf(xb.w, nf[8 * q + 7], dot);
+        dq[q] = dot;
+    }
+    return ((dq[0] + dq[1]) + (dq[2] + dq[3])) - 8.0f * sx;
+}
+
+// ---- the head: what a wave requests ahead of a chunk, and the chunk's dot products ----
+// Slot s of a chunk = (tile tt, round u), tile-major.  Round u of wave w covers groups (u W + w) gpw + j,
+// gpw = 4 >> tws groups per wave-wide load; lane (col, j) takes group j of the round for column col of the tile.
+template <int MODE>
+__device__ __forceinline__ void prefetch_lin(const Stage &st, Regs &r, int chunk, int rank, int wave, int lane) {
+    if (MODE != 0) return;
+    const int tw = 16 << st.tws, gpw = 4 >> st.tws;
+    const int col = lane & (tw - 1), j = lane >> (4 + st.tws);
+    int tt = 0, u = 0;
+#pragma unroll
+    for (int s = 0; s < SL; ++s) {
+        const int tile = rank + (chunk * st.tpc + tt) * st.n_wgs;
+        if (tt >= st.tpc || tile >= st.n_tiles) break;  // wave-uniform
+        r.w[s][0] = r.w[s][1] = r.w[s][2] = r.w[s][3] = 0u;
+        r.sc[s] = 0.0f;
+        {
+            const int g = (u * W + wave) * gpw + j;
+            const int n = tile * tw + col;
+            if (g < st.n_groups && n < st.stride) {
+                const uint32_t *wp = st.packed + (size_t)(4 * g) * st.stride + n;
+                r.w[s][0] = wp[0];
+                r.w[s][1] = wp[st.stride];
+                r.w[s][2] = wp[2 * (size_t)st.stride];
+                r.w[s][3] = wp[3 * (size_t)st.stride];
+                r.sc[s] = st.scales[(size_t)g * st.stride + n];
+            }
+        }
+        if (++u == st.nl) {
+            u = 0;
+            ++tt;
+        }
+    }
+}
+
+__device__ __forceinline__ void compute_chunk(const Stage &st, const Regs &r, const float *xs, const float *xsum, float *red, int tiles,
+                                              int wave, int lane) {
+    const int tw = 16 << st.tws, gpw = 4 >> st.tws;
+    const int col = lane & (tw - 1), j = lane >> (4 + st.tws);
+    float acc = 0.0f;
+    int tt = 0, u = 0;
+#pragma unroll
+    for (int s = 0; s < SL; ++s) {
+        if (tt >= tiles) break;  // wave-uniform
+        {
+            int g = (u * W + wave) * gpw + j;
+            g = g < st.n_groups ? g : st.n_groups - 1;  // beyond the last group the words and the scale are zero
+            acc = fmaf(r.sc[s], slot_dot(r.w[s], xs, xsum, g), acc);
+            if (u == st.nl - 1) {  // wave-uniform: the tile is complete
+                const float tot = reduce_groups(acc, st.tws);
+                if (lane < tw) red[(tt * W + wave) * 64 + col] = tot;
+                acc = 0.0f;
+            }
+        }
+        if (++u == st.nl) {
+            u = 0;
+            ++tt;
+        }
+    }
+}
+
+// ---- the Linears of the layers ----
+// Wave w of Linear workgroup li works on the workgroup's unit k = w >> wps (unit li + k nlin of the stage) as wave
+// ws = w & (wpt - 1) of that unit (li counted from the first workgroup of the stage's group, nlin = size of the group): lane (col, j) holds, in slot u, group (u wpt + ws) gpw + j of column col.
+struct Unit {
+    int unit;   // -1: this wave has none
+    int n0;     // first column
+    int ws, wpt;
+};
+__device__ __forceinline__ Unit wave_unit(const Stage &st, int li, int wave) {
+    Unit q;
+    q.wpt = 1 << st.wps;
+    q.ws = wave & (q.wpt - 1);
+    const int unit = li - st.li0 + (wave >> st.wps) * st.ngrp;
+    q.unit = unit < st.n_units ? unit : -1;
+    const int part = st.n_cparts == 1 ? 0 : (unit >= st.upp) + (unit >= 2 * st.upp);
+    q.n0 = st.col0 + part * st.part_stride + ((unit - part * st.upp) << (4 + st.tws));
+    return q;
+}
+
+template <int MODE>
+__device__ __forceinline__ void lay_prefetch(const Stage &st, Regs &r, int li, int wave, int lane) {
+    if (MODE != 0) return;
+    const int tw = 16 << st.tws, gpw = 4 >> st.tws;
+    const int col = lane & (tw - 1), j = lane >> (4 + st.tws);
+    const Unit q = wave_unit(st, li, rfl(wave));
+    // a column beyond the matrix reads the last one's words: nobody looks at its sums
+    const int n = min(q.n0 + col, st.stride - 1);
+    const uint32_t lane_w = ((uint32_t)(4 * j) * (uint32_t)st.stride + (uint32_t)n) * 4u;
+    const uint32_t lane_s = ((uint32_t)j * (uint32_t)st.stride + (uint32_t)n) * 4u;
+    const size_t row = (size_t)st.stride * 4;  // bytes
+    const char *pw = reinterpret_cast<const char *>(st.packed), *ps = reinterpret_cast<const char *>(st.scales);
+#pragma unroll
+    for (int u = 0; u < SL; ++u) {
+        if (u >= st.nl) break;  // wave-uniform
+        const int gs = (u * q.wpt + q.ws) * gpw;  // the round's first group of this wave
+        r.w[u][0] = r.w[u][1] = r.w[u][2] = r.w[u][3] = 0u;
+        r.sc[u] = 0.0f;
+        if (q.unit >= 0 && gs + j < st.n_groups) {
+            const char *bw = pw + (size_t)(4 * gs) * row;
+            r.w[u][0] = *reinterpret_cast<const uint32_t *>(bw + lane_w);
+            r.w[u][1] = *reinterpret_cast<const uint32_t *>(bw + row + lane_w);
+            r.w[u][2] = *reinterpret_cast<const uint32_t *>(bw + 2 * row + lane_w);
+            r.w[u][3] = *reinterpret_cast<const uint32_t *>(bw + 3 * row + lane_w);
+            r.sc[u] = *reinterpret_cast<const float *>(ps + (size_t)gs * row + lane_s);
+        }
+    }
+}
+
+__device__ __forceinline__ float lay_compute(const Stage &st, const Regs &r, const float (&pre)[NPRE * 32], const float *xs, const float *xsum,
+                                             int wave, int lane) {
+    const int gpw = 4 >> st.tws;
+    const int j = lane >> (4 + st.tws);
+    const int wpt = 1 << st.wps, ws = wave & (wpt - 1);
+    float acc = 0.0f;
+#pragma unroll
+    for (int u = 0; u < SL; ++u) {
+        if (u >= st.nl) break;  // wave-uniform
+        int g = (u * wpt + ws) * gpw + j;
+        g = g < st.n_groups ? g : st.n_groups - 1;  // beyond the last group the words and the scale are zero
+        acc = fmaf(r.sc[u], u < NPRE ? slot_dot_pre(pre + 32 * (u < NPRE ? u : 0), xs, xsum, g) : slot_dot(r.w[u], xs, xsum, g), acc);
+    }
+    return reduce_groups(acc, st.tws);
+}
+
+// Order-preserving key of a float (NaN lowest, both zeros equal).
+__device__ __forceinline__ uint32_t order_key(float v) {
+    if (v != v) return 0u;
+    const uint32_t u = v == 0.0f ? 0u : __float_as_uint(v);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// Largest 48-bit word over the workgroup (scratch: 2 * W uint32); valid in every thread.
+__device__ __forceinline__ u64 block_max48(u64 w, uint32_t *scratch, int lane, int wave) {
+    const uint32_t hi = (uint32_t)(w >> 32), lo = (uint32_t)w;
+    const uint32_t mh = wave_minmax_u32<true>(hi);
+    const uint32_t ml = wave_minmax_u32<true>(hi == mh ? lo : 0u);
+    __syncthreads();  // scratch free
+    if (lane == 0) {
+        scratch[wave] = mh;
+        scratch[W + wave] = ml;
+    }
+    __syncthreads();
+    u64 best = 0ull;
+#pragma unroll
+    for (int i = 0; i < W; ++i) {
+        const u64 c = ((u64)scratch[i] << 32) | scratch[W + i];
+        best = c > best ? c : best;
+    }
+    return best;
+}
+
+struct Lds {
+    float *xs;       // [2][xbuf]: the staged input, stages in turn
+    float *xsum;     // [2][XMAX / 32]: sum of every group of 32 inputs
+    float *red;      // [2][SL][W][64]: per-wave sums, chunks in turn; attention: per-wave partial results
+    float4 *stat;    // [W]: LayerNorm statistics per wave
+    float *fin;      // attention: [PSTRIDE] + [SMAX][PSTRIDE]
+    uint32_t *scr;   // [2 W]
+    uint32_t *hl;    // [head_slots][5][T]: the head's second chunk as the registers will hold it
+};
+
+#ifdef AGPU_PK_TRACE
+#define PK_STAMP(slot)                                                                                     \
+    do {                                                                                                   \
+        if (p.trace && tid == 0 && c.stage < p.n_stages) c.tr[c.stage * 8 + (slot)] = wall_clock64();      \
+    } while (0)
+#define PK_DUMP()                                                                                          \
+    do {                                                                                                   \
+        __syncthreads();                                                                                   \
+        if (p.trace)                                                                                       \
+            for (int i_ = tid; i_ < p.n_stages * 8; i_ += T) p.trace[(size_t)blockIdx.x * p.n_stages * 8 + i_] = c.tr[i_]; \
+    } while (0)
+#else
+#define PK_DUMP() \
+    do {          \
+    } while (0)
+#define PK_STAMP(slot) \
+    do {               \
+    } while (0)
+#endif
+
+// ---- input of a Linear stage ----
+// The input vector is awaited in the XCD's mirror (thread t owns the element pairs t, t + T, ...), normalised where
+// the stage has a LayerNorm, and staged in LDS with the sums of its groups.  `settle` is called right after the
+// poll: whatever its caller requested before has arrived with the polled data (a wave's loads return in order).
+template <int MODE, typename Settle>
+__device__ __forceinline__ void stage_input(const Params &p, const Stage &st, Ctl &c, float *xs, float *xsum, float4 *stat, const u64 *mirror,
+                                            int pos, uint32_t tok, int tid, Settle settle) {
+    const int lane = tid & 63, wave = tid >> 6;
+    const bool real = MODE == 0;
+    const int n_pairs = st.K >> 1;
+    float2 lg[LNP], lb[LNP];
+#pragma unroll
+    for (int i = 0; i < LNP; ++i) {
+        const int pr = tid + i * T;
+        lg[i] = make_float2(1.0f, 1.0f);
+        lb[i] = make_float2(0.0f, 0.0f);
+        if ((st.flags & F_LN) && real && pr < n_pairs) {
+            lg[i] = *reinterpret_cast<const float2 *>(st.ln_g + 2 * pr);
+            lb[i] = *reinterpret_cast<const float2 *>(st.ln_b + 2 * pr);
+        }
+    }
+    float2 xv[PMAX];
+#pragma unroll
+    for (int i = 0; i < PMAX; ++i) xv[i] = make_float2(0.0f, 0.0f);
+    if (st.in_off == -2) {
+#pragma unroll
+        for (int i = 0; i < LNP; ++i) {
+            const int pr = tid + i * T;
+            if (pr < n_pairs && real) {
+                const float2 a = *reinterpret_cast<const float2 *>(p.wte + (size_t)tok * p.d + 2 * pr);
+                const float2 b = *reinterpret_cast<const float2 *>(p.wpe + (size_t)pos * p.d + 2 * pr);
+                xv[i] = make_float2(a.x + b.x, a.y + b.y);
+            }
+        }
+    } else {
+        const u64 *src = mirror + st.in_off;
+        if (n_pairs <= T) {  // workgroup-uniform; one pair of pairs per thread at most: the common case
+            const u64 *ptr[1] = {src + 2 * (tid < n_pairs ? tid : 0)};
+            bool need[1] = {tid < n_pairs};
+            uint4 v[1] = {make_uint4(0u, 0u, 0u, 0u)};
+            poll_pairs<true, 1>(c, ptr, need, v);
+            xv[0] = make_float2(__uint_as_float(v[0].x), __uint_as_float(v[0].z));
+        } else {
+            static_assert(PMAX == 2, "a thread polls two pairs of pairs at most");
+            const u64 *ptr[2];
+            bool need[2];
+            uint4 v[2];
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                need[k] = tid + k * T < n_pairs;
+                ptr[k] = src + 2 * (need[k] ? tid + k * T : tid);
+                v[k] = make_uint4(0u, 0u, 0u, 0u);
+            }
+            poll_pairs<true, 2>(c, ptr, need, v);
+#pragma unroll
+            for (int k = 0; k < 2; ++k) xv[k] = make_float2(__uint_as_float(v[k].x), __uint_as_float(v[k].z));
+        }
+    }
+    settle();
+#pragma unroll
+    for (int i = 0; i < LNP; ++i) asm volatile("" ::"v"(lg[i].x), "v"(lg[i].y), "v"(lb[i].x), "v"(lb[i].y));
+    PK_STAMP(1);
+    if (st.flags & F_LN) {  // workgroup-uniform; K <= 2048
+        // Every wave takes the mean of its own elements and their squared distances from it (two passes over the
+        // registers, nn/cpu_ref.rs:38-47); the waves' (count, sum, mean, M2) are put together after one barrier.
+        int cnt = 0;
+#pragma unroll
+        for (int i = 0; i < LNP; ++i) cnt += 2 * max(0, min(64, n_pairs - (wave * 64 + i * T)));  // wave-uniform
+        float sm = 0.0f;
+#pragma unroll
+        for (int i = 0; i < LNP; ++i) sm += xv[i].x + xv[i].y;  // absent pairs are zero
+        sm = wave_sum(sm);
+        const float mw = cnt > 0 ? sm * __builtin_amdgcn_rcpf((float)cnt) : 0.0f;
+        float m2 = 0.0f;
+#pragma unroll
+        for (int i = 0; i < LNP; ++i)
+            if (tid + i * T < n_pairs) {
+                const float d0 = xv[i].x - mw, d1 = xv[i].y - mw;
+                m2 = fmaf(d0, d0, m2);
+                m2 = fmaf(d1, d1, m2);
+            }
+        m2 = wave_sum(m2);
+        if (lane == 0) stat[wave] = make_float4((float)cnt, sm, mw, m2);
+        __syncthreads();
+        float4 sw[W];
+#pragma unroll
+        for (int w8 = 0; w8 < W; ++w8) sw[w8] = stat[w8];
+        float tot = 0.0f;
+#pragma unroll
+        for (int w8 = 0; w8 < W; ++w8) tot += sw[w8].y;
+        const float mean = tot * st.inv_k;
+        float M2 = 0.0f;
+#pragma unroll
+        for (int w8 = 0; w8 < W; ++w8) {
+            const float dl = sw[w8].z - mean;
+            M2 += fmaf(sw[w8].x * dl, dl, sw[w8].w);
+        }
+        const float var = M2 * st.inv_k + p.eps;
+        float rstd = __builtin_amdgcn_rsqf(var);
+        rstd = rstd * fmaf(-0.5f * var * rstd, rstd, 1.5f);  // one Newton step: the hardware estimate is good to 1 ulp
+#pragma unroll
+        for (int i = 0; i < LNP; ++i) {
+            xv[i].x = (xv[i].x - mean) * rstd * lg[i].x + lb[i].x;
+            xv[i].y = (xv[i].y - mean) * rstd * lg[i].y + lb[i].y;
+        }
+    }
+    // the vector and the sums of its groups (16 pairs = 16 adjacent lanes) into LDS
+#pragma unroll
+    for (int i = 0; i < PMAX; ++i) {
+        if (i * T >= n_pairs) break;  // workgroup-uniform
+        const int pr = tid + i * T;
+        const bool have = pr < n_pairs;
+        const float gs = row16_sum(have ? xv[i].x + xv[i].y : 0.0f);
+        if (have) {
+            *reinterpret_cast<float2 *>(xs + (pr >> 4) * GS + 2 * (pr & 15)) = xv[i];
+            if ((lane & 15) == 0) xsum[pr >> 4] = gs;
+        }
+    }
+    __syncthreads();
+    PK_STAMP(2);
+}
+
+// ---- one Linear of a layer, for a workgroup that has a unit of it ----
+// The finishing threads (one per column of the workgroup's units) request bias first; then the input; then every lane
+// its groups of its column; the waves of a unit meet in LDS and the finishing thread completes the column: bias, GELU,
+// the tagged store (into the XCD's mirror, or as a partial sum into memory), and for K and V columns the row of the cache.
+template <int MODE>
+__device__ __forceinline__ void lay_stage(const Params &p, const Stage &st, Ctl &c, const Regs &r, float *xs, float *xsum, float4 *stat,
+                                          float *red, u64 *mirror, int pos, uint32_t tok, int li, int tid) {
+    const int lane = tid & 63, wave = tid >> 6;
+    const bool real = MODE == 0;
+    const int tsh = 4 + st.tws, tw = 1 << tsh;
+    const int wpt = 1 << st.wps;
+    // finishing thread (kf, colf): column colf of the workgroup's unit kf
+    const int kf = tid >> tsh, colf = tid & (tw - 1);
+    const int unit_f = li - st.li0 + kf * st.ngrp;
+    const int part_f = st.n_cparts == 1 ? 0 : (unit_f >= st.upp) + (unit_f >= 2 * st.upp);
+    const int lc = ((unit_f - part_f * st.upp) << tsh) + colf;
+    const int n = st.col0 + part_f * st.part_stride + lc;
+    const bool fin = kf < (W >> st.wps) && unit_f < st.n_units && lc < st.pcols;
+    float bias = 0.0f;
+    if (fin && st.bias && real) bias = st.bias[n];
+    PK_STAMP(0);
+    // the first slots' nibbles become floats before the input is awaited
+    float pre[NPRE * 32];
+    if (real) {
+#pragma unroll
+        for (int u = 0; u < NPRE; ++u) {
+            if (u >= st.nl) break;  // wave-uniform
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float nf[8];
+                unpack_bytes(r.w[u][q], nf);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pre[32 * u + 8 * q + e] = nf[e];
+            }
+        }
+    }
+    stage_input<MODE>(p, st, c, xs, xsum, stat, mirror, pos, tok, tid, [&] { asm volatile("" ::"v"(bias)); });
+    if (real) {
+        const float part = lay_compute(st, r, pre, xs, xsum, wave, lane);
+        if (lane < tw) red[wave * 64 + lane] = part;
+    }
+    PK_STAMP(4);
+    __syncthreads();
+    if (fin) {
+        float v = 0.0f;
+        if (real) {
+            // all eight reads are issued at once; those beyond the unit's waves read its last wave again and count as zero
+            float rv[W];
+#pragma unroll
+            for (int w8 = 0; w8 < W; ++w8) rv[w8] = red[((kf << st.wps) + min(w8, wpt - 1)) * 64 + colf];
+#pragma unroll
+            for (int w8 = 0; w8 < W; ++w8) v += w8 < wpt ? rv[w8] : 0.0f;
+            v += bias;
+            if (st.flags & F_GELU_TANH) v = gelu_tanh_dev(v);
+            else if (st.flags & F_GELU_QUICK) v = gelu_quick_dev(v);
+        }
+        if (st.flags & F_PARTIAL) st_tag(p.arena + st.out_off + n, v, c.epoch);
+        else st_loc(mirror + st.out_off + n, v, c.epoch);
+        if ((st.flags & F_SCATTER) && real && n >= p.d) {
+            const int jn = n - p.d;
+            const bool is_v = jn >= p.d;
+            const int jj = is_v ? jn - p.d : jn;
+            (is_v ? st.vc : st.kc)[((size_t)(jj >> 6) * p.P + pos) * DH + (jj & 63)] = v;
+        }
+    }
+    PK_STAMP(3);
+}
+
+// ---- the head ----
+template <int MODE>
+__device__ __forceinline__ void head_finish(const Params &p, const Stage &st, const float *red, int rank, int ch, int tiles, int tid, u64 &best) {
+    if (MODE != 0) return;
+    const int tw_shift = st.tws + 4;
+    for (int o = tid; o < (tiles << tw_shift); o += T) {
+        const int tt = o >> tw_shift, col = o & ((1 << tw_shift) - 1);
+        const int n = ((rank + (ch * st.tpc + tt) * st.n_wgs) << tw_shift) + col;
+        if (n >= st.n_valid) continue;
+        float v = 0.0f;
+#pragma unroll
+        for (int w8 = 0; w8 < W; ++w8) v += red[(tt * W + w8) * 64 + col];
+        if (st.bias) v += st.bias[n];
+        p.logits[n] = v;
+        const uint32_t code = p.argmax_last ? (uint32_t)n : 0xFFFFu - (uint32_t)n;
+        const u64 cand = ((u64)order_key(v) << 16) | code;
+        if (order_key(v) != 0u) best = cand > best ? cand : best;
+    }
+}
+
+// ---- relay ----
+constexpr int TK = 6;  // cache lines of one stage's weights a relay thread touches at most
+// One word of every 128 bytes of the XCD's share of a stage's weights, so that they wait in the XCD's L2 when the Linear
+// workgroups request them: thread tid of relay r takes the lines tid + r T + s NR T.  The loaded words are handed back;
+// the caller keeps them until after its next poll, so nothing but that poll waits for them.
+__device__ __forceinline__ void touch_stage(CStage e, int tid, int r, uint32_t (&tk)[TK]) {
+    const int n_units = e->n_units;
+    if (n_units <= 0) return;  // workgroup-uniform
+    const int n_cparts = e->n_cparts, stride = e->stride, K = e->K;
+    const int col0 = e->col0, part_stride = e->part_stride, pcols = e->pcols;
+    const char *pw = reinterpret_cast<const char *>(glob(e->packed));
+    const char *ps = reinterpret_cast<const char *>(glob(e->scales));
+    const int rows_w = K >> 3, rows = rows_w + (K >> 5);
+    const int lpr = ((((col0 * 4) & 127) + pcols * 4) + 127) >> 7;  // lines per row and column part
+    const int per_part = rows * lpr, n_all = n_cparts * per_part;
+    const size_t row_b = (size_t)stride * 4;
+#pragma unroll
+    for (int s = 0; s < TK; ++s) {
+        const int i = tid + r * T + s * NR * T;
+        if (i < n_all) {
+            const int part = i / per_part, q = i - part * per_part;
+            const int row = q / lpr, line = q - row * lpr;
+            const int b = min((((col0 + part * part_stride) * 4) & ~127) + line * 128, stride * 4 - 4);
+            const char *a = row < rows_w ? pw + (size_t)row * row_b + b : ps + (size_t)(row - rows_w) * row_b + b;
+            tk[s] = *reinterpret_cast<const uint32_t *>(a);
+        }
+    }
+}
+
+// The exchanges of the step, for relay r of the XCD: thread (cp_local, part) = (tid >> 3, tid & 7) polls the partial
+// sum of XCD `part` for the column pairs r cps + cp_local + 64 k; the eight lanes of a column pair add up what they
+// got, and lane 0 of them adds bias and residual, keeps the result as the next residual and stores it into the mirror.
+template <int MODE>
+__device__ __forceinline__ void relay_role(const Params &p, CStage tab, Ctl &c, u64 *mirror, int pos, uint32_t tok, int tid, int r) {
+    const bool real = MODE == 0;
+    const int part = tid & 7, cpl = tid >> 3;
+    const int half = p.d >> 1;
+    const int cps = (half + NR - 1) / NR;
+    const int n_it = (cps + 63) >> 6;  // <= XI
+    float2 res[XI];
+    bool valid[XI];
+    int cp[XI];
+#pragma unroll
+    for (int k = 0; k < XI; ++k) {
+        const int l = cpl + 64 * k;
+        cp[k] = r * cps + l;
+        valid[k] = k < n_it && l < cps && cp[k] < half;
+        res[k] = make_float2(0.0f, 0.0f);
+        if (valid[k] && part == 0 && real) {
+            const float2 a = *reinterpret_cast<const float2 *>(p.wte + (size_t)tok * p.d + 2 * cp[k]);
+            const float2 b = *reinterpret_cast<const float2 *>(p.wpe + (size_t)pos * p.d + 2 * cp[k]);
+            res[k] = make_float2(a.x + b.x, a.y + b.y);
+        }
+    }
+    uint32_t tk0[TK], tk1[TK];
+#pragma unroll
+    for (int s = 0; s < TK; ++s) tk0[s] = tk1[s] = 0u;
+    const int n_half = 2 * p.n_layer;  // half layers = exchanges; half layer x is in use from exchange x - 1 on
+    // the weights of the first half layers, as far ahead as the later ones will be touched
+    if (real && p.touch_dist > 0)
+        for (int hh = 0; hh < min(p.touch_dist + 1, n_half); ++hh) {
+            touch_stage(tab + 2 * hh, tid, r, tk0);
+            touch_stage(tab + 2 * hh + 1, tid, r, tk1);
+        }
+    for (int x = 0; x < n_half; ++x) {
+        CStage e = tab + 2 * x + 1;  // the partial-sum stage in front of this exchange
+        c.stage = 2 * x + 1;
+        const int n_parts = e->xn_parts, src_off = e->part_off, dst_off = e->xout_off;
+        const float *xbias = glob(e->xbias);
+        float2 bias[XI];
+#pragma unroll
+        for (int k = 0; k < XI; ++k) {
+            bias[k] = make_float2(0.0f, 0.0f);
+            if (valid[k] && part == 0 && real && xbias) bias[k] = *reinterpret_cast<const float2 *>(xbias + 2 * cp[k]);
+        }
+        const u64 *src = p.arena + src_off + (size_t)part * p.d;
+        uint4 v[XI];
+        bool need[XI];
+#pragma unroll
+        for (int k = 0; k < XI; ++k) {
+            v[k] = make_uint4(0u, 0u, 0u, 0u);
+            need[k] = valid[k] && part < n_parts;
+        }
+        PK_STAMP(5);
+        if (n_it <= 1) {
+            const u64 *ptr[1] = {src + 2 * (need[0] ? cp[0] : 0)};
+            bool nd[1] = {need[0]};
+            uint4 vv[1] = {v[0]};
+            poll_pairs<false, 1>(c, ptr, nd, vv);
+            v[0] = vv[0];
+        } else if (n_it <= 2) {
+            const u64 *ptr[2];
+            bool nd[2];
+            uint4 vv[2];
+#pragma unroll
+            for (int k = 0; k < 2; ++k) { ptr[k] = src + 2 * (need[k] ? cp[k] : 0); nd[k] = need[k]; vv[k] = v[k]; }
+            poll_pairs<false, 2>(c, ptr, nd, vv);
+#pragma unroll
+            for (int k = 0; k < 2; ++k) v[k] = vv[k];
+        } else if (n_it <= 4) {
+            const u64 *ptr[4];
+            bool nd[4];
+            uint4 vv[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) { ptr[k] = src + 2 * (need[k] ? cp[k] : 0); nd[k] = need[k]; vv[k] = v[k]; }
+            poll_pairs<false, 4>(c, ptr, nd, vv);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v[k] = vv[k];
+        } else {
+            const u64 *ptr[8];
+            bool nd[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) { ptr[k] = src + 2 * (need[k] ? cp[k] : 0); nd[k] = need[k]; }
+            poll_pairs<false, 8>(c, ptr, nd, v);
+        }
+#pragma unroll
+        for (int s = 0; s < TK; ++s) asm volatile("" ::"v"(tk0[s]), "v"(tk1[s]));
+        PK_STAMP(6);
+#pragma unroll
+        for (int k = 0; k < XI; ++k) {
+            if (k >= n_it) break;  // workgroup-uniform
+            const float sx = oct_sum(__uint_as_float(v[k].x)), sy = oct_sum(__uint_as_float(v[k].z));
+            if (valid[k] && part == 0) {
+                const float hx = real ? (sx + bias[k].x) + res[k].x : 0.0f, hy = real ? (sy + bias[k].y) + res[k].y : 0.0f;
+                res[k] = make_float2(hx, hy);
+                st_loc2(mirror + dst_off + 2 * cp[k], hx, hy, c.epoch);
+            }
+        }
+        PK_STAMP(7);
+        // half layer x + 1 begins now: the weights of the one touch_dist further on
+        if (real && p.touch_dist > 0 && x + 1 + p.touch_dist < n_half) {
+            touch_stage(tab + 2 * (x + 1 + p.touch_dist), tid, r, tk0);
+            touch_stage(tab + 2 * (x + 1 + p.touch_dist) + 1, tid, r, tk1);
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < TK; ++s) asm volatile("" ::"v"(tk0[s]), "v"(tk1[s]));
+}
+
+// Lane-wise sum over the four rows of 16 lanes (gfx950 row swaps), result in every lane.
+__device__ __forceinline__ float rows_sum(float v) { return reduce_groups(v, 0); }
+
+// ---- attention ----
+// Key range ks of S of head h: cached keys r0 .. r1 - 1; round t covers keys r0 + KR t + 4 wave + kq, 16 lanes x 16 bytes per key.
+__device__ __forceinline__ void attn_range(int pos, int S, int ks, int &r0, int &r1) {
+    const int per = (((pos + S - 1) / S) + 31) & ~31;
+    r0 = min(pos, ks * per);
+    r1 = min(pos, r0 + per);
+}
+
+__device__ __forceinline__ void prefetch_attn(const float *kc, const float *vc, int P, uint4 (&kv)[2 * KVP], int h, int r0, int r1, int first,
+                                              int wave, int lane) {
+    const int e4 = lane & 15, kq = lane >> 4;
+#pragma unroll
+    for (int t = 0; t < KVP; ++t) {
+        const int j = r0 + (first + t) * KR + wave * 4 + kq;
+        kv[2 * t] = make_uint4(0u, 0u, 0u, 0u);
+        kv[2 * t + 1] = make_uint4(0u, 0u, 0u, 0u);
+        if (j < r1) {
+            const size_t at = ((size_t)h * P + j) * DH + 4 * e4;
+            kv[2 * t] = *reinterpret_cast<const uint4 *>(kc + at);
+            kv[2 * t + 1] = *reinterpret_cast<const uint4 *>(vc + at);
+        }
+    }
+}
+
+// All layers' attention for (head h, key range ks of S): a flat loop over (layer, batch of KVP rounds) whose
+// next batch, of this layer or the next, is requested before anything else is waited for.  q, the new k and v, the
+// partial results of the key ranges and the output all stay in the XCD's mirror.
+template <int MODE>
+__device__ __forceinline__ void attn_role(const Params &p, CStage tab, Ctl &c, const Lds &L, u64 *mirror, int pos, int h, int S, int ks, int tid) {
+    const int lane = tid & 63, wave = tid >> 6;
+    const int e4 = lane & 15, kq = lane >> 4;
+    const bool real = MODE == 0;
+    const float ninf = -__builtin_inff();
+    const float scale = 0.125f;  // 1 / sqrt(64)
+    float *part = L.red;               // [W][64]
+    float *wm = L.red + W * 4 * DH;    // [W]
+    float *wl = wm + W;                // [W]
+    float *own = L.fin;                // [PSTRIDE]: o[64], m, l of this workgroup
+    float *oth = L.fin + PSTRIDE;      // [S - 1][PSTRIDE]
+    const bool with_new = ks == 0 && wave == 0;  // this wave also takes the new position's key and value
+    int r0, r1;
+    attn_range(pos, S, ks, r0, r1);
+    const int n_rounds = (r1 - r0 + KR - 1) / KR;
+
+    uint4 kv[2 * KVP];
+#pragma unroll
+    for (int i = 0; i < 2 * KVP; ++i) kv[i] = make_uint4(0u, 0u, 0u, 0u);
+    int Ly = 0, first = 0;
+    Stage st = load_stage(tab);
+    if (real) prefetch_attn(st.kc, st.vc, p.P, kv, h, r0, r1, 0, wave, lane);
+    float4 q = make_float4(0.f, 0.f, 0.f, 0.f), o = q;
+    float m = ninf, l = 0.0f;
+    float kn[4], vn[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) kn[k] = vn[k] = 0.0f;
+
+    while (Ly < p.n_layer) {
+        c.stage = 4 * Ly;
+        if (first == 0) {
+            PK_STAMP(0);
+            // q of this head, and for one wave the new key and value, from the QKV vector in the mirror
+            const u64 *qsrc = mirror + st.out_off + h * DH + 4 * e4;
+            uint4 w6[6];
+#pragma unroll
+            for (int k = 0; k < 6; ++k) w6[k] = make_uint4(0u, 0u, 0u, 0u);
+            if (with_new) {
+                const u64 *ptr[6] = {qsrc, qsrc + 2, qsrc + p.d, qsrc + p.d + 2, qsrc + 2 * p.d, qsrc + 2 * p.d + 2};
+                bool need[6] = {true, true, true, true, true, true};
+                poll_pairs<true, 6>(c, ptr, need, w6);
+            } else {
+                const u64 *ptr[2] = {qsrc, qsrc + 2};
+                bool need[2] = {true, true};
+                uint4 w2[2] = {w6[0], w6[1]};
+                poll_pairs<true, 2>(c, ptr, need, w2);
+                w6[0] = w2[0];
+                w6[1] = w2[1];
+            }
+            q = make_float4(__uint_as_float(w6[0].x), __uint_as_float(w6[0].z), __uint_as_float(w6[1].x), __uint_as_float(w6[1].z));
+            kn[0] = __uint_as_float(w6[2].x); kn[1] = __uint_as_float(w6[2].z); kn[2] = __uint_as_float(w6[3].x); kn[3] = __uint_as_float(w6[3].z);
+            vn[0] = __uint_as_float(w6[4].x); vn[1] = __uint_as_float(w6[4].z); vn[2] = __uint_as_float(w6[5].x); vn[3] = __uint_as_float(w6[5].z);
+            m = ninf;
+            l = 0.0f;
+            o = make_float4(0.f, 0.f, 0.f, 0.f);
+            PK_STAMP(1);
+        }
+        if (real) {
+            float s[KVP];
+            float bm = ninf;
+#pragma unroll
+            for (int t = 0; t < KVP; ++t) {
+                s[t] = ninf;
+                if (first + t >= n_rounds) continue;  // wave-uniform: no key of the range in this round
+                const float4 kk = as_f4(kv[2 * t]);
+                float dot = q.x * kk.x;
+                dot = fmaf(q.y, kk.y, dot);
+                dot = fmaf(q.z, kk.z, dot);
+                dot = fmaf(q.w, kk.w, dot);
+                dot = row16_sum(dot) * scale;
+                const int j = r0 + (first + t) * KR + wave * 4 + kq;
+                s[t] = j < r1 ? dot : ninf;
+                bm = fmaxf(bm, s[t]);
+            }
+            float s_new = ninf;
+            if (with_new && first == 0) {
+                float dot = q.x * kn[0];
+                dot = fmaf(q.y, kn[1], dot);
+                dot = fmaf(q.z, kn[2], dot);
+                dot = fmaf(q.w, kn[3], dot);
+                dot = row16_sum(dot) * scale;
+                s_new = kq == 0 ? dot : ninf;
+                bm = fmaxf(bm, s_new);
+            }
+            const float m2 = fmaxf(m, wave_max(bm));
+            if (m2 > ninf) {  // wave-uniform: the wave has seen at least one key
+                const float f = m > ninf ? __expf(m - m2) : 0.0f;
+                l *= f;
+                o.x *= f; o.y *= f; o.z *= f; o.w *= f;
+#pragma unroll
+                for (int t = 0; t < KVP; ++t) {
+                    if (first + t >= n_rounds) continue;  // wave-uniform
+                    const float pr = s[t] > ninf ? __expf(s[t] - m2) : 0.0f;
+                    const float4 vv = as_f4(kv[2 * t + 1]);
+                    l += pr;
+                    o.x = fmaf(pr, vv.x, o.x);
+                    o.y = fmaf(pr, vv.y, o.y);
+                    o.z = fmaf(pr, vv.z, o.z);
+                    o.w = fmaf(pr, vv.w, o.w);
+                }
+                if (s_new > ninf) {
+                    const float pr = __expf(s_new - m2);
+                    l += pr;
+                    o.x = fmaf(pr, vn[0], o.x);
+                    o.y = fmaf(pr, vn[1], o.y);
+                    o.z = fmaf(pr, vn[2], o.z);
+                    o.w = fmaf(pr, vn[3], o.w);
+                }
+                m = m2;
+            }
+        }
+        PK_STAMP(4);
+        const bool last_batch = first + KVP >= n_rounds;
+        const Stage cur = st;
+        const int nLy = last_batch ? Ly + 1 : Ly, nfirst = last_batch ? 0 : first + KVP;
+        if (!last_batch && real) prefetch_attn(st.kc, st.vc, p.P, kv, h, r0, r1, nfirst, wave, lane);
+        if (last_batch) {
+            if (real) {
+                // every lane of a 16-lane row holds the same l: the wave sum counts it 16 times (exactly)
+                const float lw = wave_sum(l) * 0.0625f;
+                o.x = rows_sum(o.x);
+                o.y = rows_sum(o.y);
+                o.z = rows_sum(o.z);
+                o.w = rows_sum(o.w);
+                if (kq == 0) *reinterpret_cast<float4 *>(part + wave * DH + 4 * e4) = o;
+                if (lane == 0) {
+                    wm[wave] = m;
+                    wl[wave] = lw;
+                }
+            }
+            __syncthreads();
+            PK_STAMP(5);
+            float res = 0.0f;  // thread e < 64: o[e]; 64: m; 65: l of this workgroup
+            if (real && wave <= 1) {  // whole waves: the weights travel between lanes
+                float mm = ninf;
+#pragma unroll
+                for (int w8 = 0; w8 < W; ++w8) mm = fmaxf(mm, wm[w8]);
+                const float mine = wm[lane & (W - 1)];
+                const float a_mine = mine > ninf ? __expf(mine - mm) : 0.0f;
+                float den = 0.0f, num = 0.0f;
+#pragma unroll
+                for (int w8 = 0; w8 < W; ++w8) {
+                    const float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, a_mine), w8));
+                    den = fmaf(a, wl[w8], den);
+                    num = fmaf(a, part[w8 * DH + lane], num);
+                }
+                res = tid < DH ? num : (tid == DH ? mm : den);
+                if (S == 1 && tid < DH) res = num / den;
+            }
+            PK_STAMP(2);
+            if (S == 1) {
+                if (tid < DH) st_loc(mirror + cur.att_off + h * DH + tid, res, c.epoch);
+            } else if (ks != 0) {
+                if (tid < DH + 2) st_loc(mirror + cur.part_off + (h * SMAX + ks) * PSTRIDE + tid, res, c.epoch);
+            } else {
+                // key range 0 merges the ranges of its head
+                if (tid < DH + 2) own[tid] = res;
+                const int other = tid / PSTRIDE + 1, i = tid % PSTRIDE;  // T >= (SMAX - 1) * PSTRIDE
+                if (other < S && i < DH + 2) {
+                    const u64 *src = mirror + cur.part_off + (h * SMAX + other) * PSTRIDE + i;
+                    u64 w = ld_loc(src);
+                    int spins = 0;
+                    while (!tag_ok(w, c.epoch) && !c.dead) {
+                        if (spin_fail(c, spins)) break;
+                        w = ld_loc(src);
+                    }
+                    oth[(other - 1) * PSTRIDE + i] = tag_val(w);
+                }
+                __syncthreads();
+                if (tid < DH) {
+                    float v = 0.0f;
+                    if (real) {
+                        float mm = own[DH];
+                        for (int rr = 0; rr < S - 1; ++rr) mm = fmaxf(mm, oth[rr * PSTRIDE + DH]);
+                        const float a0 = own[DH] > ninf ? __expf(own[DH] - mm) : 0.0f;
+                        float num = a0 * own[tid], den = a0 * own[DH + 1];
+                        for (int rr = 0; rr < S - 1; ++rr) {
+                            const float mr = oth[rr * PSTRIDE + DH];
+                            const float a = mr > ninf ? __expf(mr - mm) : 0.0f;
+                            num = fmaf(a, oth[rr * PSTRIDE + tid], num);
+                            den = fmaf(a, oth[rr * PSTRIDE + DH + 1], den);
+                        }
+                        v = num / den;
+                    }
+                    st_loc(mirror + cur.att_off + h * DH + tid, v, c.epoch);
+                }
+            }
+            PK_STAMP(3);
+            if (nLy < p.n_layer) {
+                st = load_stage(tab + 4 * nLy);
+                if (real) prefetch_attn(st.kc, st.vc, p.P, kv, h, r0, r1, 0, wave, lane);
+            }
+            __syncthreads();  // the per-wave results and the merge area are free again
+        }
+        Ly = nLy;
+        first = nfirst;
+    }
+}
+
+// ---- the head's second chunk, fetched into LDS while the layers run ----
+struct HeadAhead {
+    int n_slots;  // slots of chunk 1 this workgroup has (0: nothing to do)
+    int s, tt, u; // next slot to request, as (tile of the chunk, round)
+    int pending;  // slot whose words are in v, -1: none
+    uint32_t v[5];
+};
+__device__ __forceinline__ void head_ahead_step(CStage th, HeadAhead &ha, uint32_t *hl, int rank, int wave, int lane, int tid) {
+    if (ha.pending >= 0) {
+#pragma unroll
+        for (int q = 0; q < 5; ++q) hl[(size_t)(ha.pending * 5 + q) * T + tid] = ha.v[q];
+        ha.pending = -1;
+    }
+    if (ha.s >= ha.n_slots) return;  // workgroup-uniform
+    const int tws = th->tws, nl = th->nl, tpc = th->tpc, n_wgs = th->n_wgs;
+    const int n_groups = th->n_groups, stride = th->stride;
+    const uint32_t *packed = glob(th->packed);
+    const float *scales = glob(th->scales);
+    const int tw = 16 << tws, gpw = 4 >> tws;
+    const int col = lane & (tw - 1), j = lane >> (4 + tws);
+    const int tile = rank + (tpc + ha.tt) * n_wgs;  // chunk 1
+    const int g = (ha.u * W + wave) * gpw + j, n = tile * tw + col;
+#pragma unroll
+    for (int q = 0; q < 5; ++q) ha.v[q] = 0u;
+    if (g < n_groups && n < stride) {
+        const uint32_t *wp = packed + (size_t)(4 * g) * stride + n;
+        ha.v[0] = wp[0];
+        ha.v[1] = wp[stride];
+        ha.v[2] = wp[2 * (size_t)stride];
+        ha.v[3] = wp[3 * (size_t)stride];
+        ha.v[4] = __float_as_uint(scales[(size_t)g * stride + n]);
+    }
+    ha.pending = ha.s;
+    ++ha.s;
+    if (++ha.u == nl) {
+        ha.u = 0;
+        ++ha.tt;
+    }
+}
+
+// First stage from `from` on, before the head, in which Linear workgroup li of its XCD has a unit; the head (n_lay) if none.
+__device__ __forceinline__ int next_active(CStage tab, int from, int li, int n_lay) {
+    int t = from;
+    while (t < n_lay) {
+        const int l = li - tab[t].li0;
+        if (l >= 0 && l < min(tab[t].ngrp, tab[t].n_units)) break;
+        ++t;
+    }
+    return t;
+}
+
+__device__ __forceinline__ void head_share(const Stage &st, int rank, int &my_tiles, int &n_chunks) {
+    my_tiles = rank < st.n_tiles ? (st.n_tiles - rank + st.n_wgs - 1) / st.n_wgs : 0;
+    n_chunks = (my_tiles + st.tpc - 1) / st.tpc;
+}
+
+// The XCD this wave runs on (XCC_ID, bits 3:0 of hardware register 20).
+__device__ __forceinline__ unsigned xcc_id() { return (unsigned)__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 0xfu; }
+
+// Where the workgroups of a launch shaped like the step's land: out[b] = XCD of workgroup b.
+__global__ __launch_bounds__(T) void xcc_probe_kernel(unsigned *out) {
+    if (threadIdx.x == 0) out[blockIdx.x] = xcc_id();
+}
+
+template <int MODE>
+__global__ __launch_bounds__(T) void decode_xcd_kernel(const Params p) {
+    extern __shared__ __align__(16) float smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int G = gridDim.x;
+    // workgroups b, b + 8, ... share an XCD (and its L2)
+    const int xcd = blockIdx.x & 7, in_xcd = blockIdx.x >> 3;
+    const int per_xcd = G >> 3;
+    const CStage tab = cstage(p.stages + (size_t)xcd * p.n_stages);  // this XCD's stage table
+    Lds L;
+    L.xs = smem;
+    L.xsum = L.xs + 2 * p.xbuf;
+    L.red = L.xsum + 2 * (XMAX / 32);
+    L.stat = reinterpret_cast<float4 *>(L.red + 2 * SL * W * 64);
+    L.fin = L.red + 2 * SL * W * 64 + 4 * W;
+    L.scr = reinterpret_cast<uint32_t *>(L.fin + (SMAX + 1) * PSTRIDE);
+    L.hl = L.scr + 2 * W;
+    u64 *tr_lds = reinterpret_cast<u64 *>(L.hl + (size_t)p.head_slots * 5 * T);
+#ifdef AGPU_PK_TRACE
+    for (int i = tid; i < p.n_stages * 8; i += T) tr_lds[i] = 0ull;
+#endif
+
+    Ctl c;
+    c.epoch = p.state[0] + 1u;
+    c.err = p.state + 1;
+    c.stage = 0;
+    c.dead = p.state[1] != 0u;
+    c.spin_limit = p.spin_limit;
+    c.tr = tr_lds;
+    // The step's number has been read: workgroup 0 advances it only once every workgroup of this launch has said so.
+    if (tid == 0) (void)__hip_atomic_fetch_add(p.state + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // The hand-offs through an L2 need the workgroups b, b + 8, ... on one XCD, the one the plan's probe found them on:
+    // checked in every launch, not assumed.
+    if (tid == 0 && xcc_id() != p.state[8 + xcd]) atomicCAS(c.err, 0u, 0x2000u + (unsigned)xcd);
+    int pos = *p.pos_dev;
+    pos = pos < 0 ? 0 : (pos > p.P - 1 ? p.P - 1 : pos);
+    uint32_t tok = p.cur_tok[0];
+    tok = tok < (uint32_t)p.V ? tok : (uint32_t)(p.V - 1);
+    __syncthreads();
+
+    u64 *mirror = p.arena + (size_t)xcd * p.mirror_elems;
+    if (in_xcd < NR) {
+        relay_role<MODE>(p, tab, c, mirror, pos, tok, tid, in_xcd);
+        PK_DUMP();
+        return;
+    }
+    const bool is_att = in_xcd < NR + p.att_per_xcd;
+    const int nlin = p.nlin;
+    const int li = in_xcd - NR - p.att_per_xcd;  // Linear workgroup of its XCD
+    // in the head, Linear workgroups are numbered XCD by XCD (neighbouring tiles, which read neighbouring pieces of the
+    // same weight rows, meet in one L2); attention workgroups follow them
+    const int att_a = in_xcd - NR;
+    const int rank = is_att ? 8 * nlin + att_a * 8 + xcd : xcd * nlin + li;
+    const int n_head_wgs = G - 8 * NR;
+    (void)per_xcd;
+
+    if (is_att) {
+        // this XCD's heads: H / 8 each, one more for the first H % 8 XCDs
+        const int hq = p.H >> 3, hr = p.H & 7;
+        const int nh = hq + (xcd < hr ? 1 : 0), h0 = xcd * hq + min(xcd, hr);
+        // key ranges per head in this step: about 256 keys each, within what the roles allow
+        const int S = min(p.smax, max(1, (pos + 255) >> 8));
+        const int hl = att_a / p.smax, ks = att_a % p.smax;
+        if (hl < nh && ks < S) attn_role<MODE>(p, tab, c, L, mirror, pos, h0 + hl, S, ks, tid);
+    }
+
+    // ---- Linears: the stages of the layers in which this workgroup has a unit, then the head ----
+    // The Linear workgroups of an XCD form groups that take the stages of a layer in turn, so that a workgroup has a
+    // stage's time to find its next stage, request its weights and convert their nibbles before that stage's input comes.
+    Regs regs;
+    const int n_lay = p.n_stages - 1;
+    int s = is_att ? n_lay : next_active(tab, 0, li, n_lay);
+    int n_enter = 0;  // staging buffers are used in turn
+    Stage st = load_stage(tab + s);
+    if (s < n_lay) lay_prefetch<MODE>(st, regs, li, wave, lane);
+    HeadAhead ha;
+    ha.n_slots = ha.s = ha.tt = ha.u = 0;
+    ha.pending = -1;
+    if (MODE == 0 && p.head_slots > 0 && !is_att) {
+        CStage th = tab + n_lay;
+        const int n_tiles = th->n_tiles, n_wgs = th->n_wgs, tpc = th->tpc;
+        const int my_tiles = rank < n_tiles ? (n_tiles - rank + n_wgs - 1) / n_wgs : 0;
+        ha.n_slots = min(p.head_slots, min(tpc, max(0, my_tiles - tpc)) * th->nl);
+    }
+    while (s < n_lay) {
+        c.stage = s;
+        lay_stage<MODE>(p, st, c, regs, L.xs + (n_enter & 1) * p.xbuf, L.xsum + (n_enter & 1) * (XMAX / 32), L.stat,
+                        L.red + (n_enter & 1) * (SL * W * 64), mirror, pos, tok, li, tid);
+        // the outputs are on their way: now the next stage this workgroup takes part in, and its weights
+        ++n_enter;
+        s = next_active(tab, s + 1, li, n_lay);
+        st = load_stage(tab + s);
+        PK_STAMP(6);
+        if (s < n_lay) lay_prefetch<MODE>(st, regs, li, wave, lane);
+        if (MODE == 0) head_ahead_step(tab + n_lay, ha, L.hl, rank, wave, lane, tid);
+        PK_STAMP(5);
+    }
+    // the head: tiles dealt round robin, in chunks of SL slots
+    u64 best = 0ull;
+    c.stage = n_lay;
+    {
+        int my_tiles, n_chunks;
+        head_share(st, rank, my_tiles, n_chunks);
+        prefetch_lin<MODE>(st, regs, 0, rank, wave, lane);
+        if (MODE == 0)
+            while (ha.pending >= 0 || ha.s < ha.n_slots) head_ahead_step(tab + n_lay, ha, L.hl, rank, wave, lane, tid);
+        float *xs = L.xs + (n_enter & 1) * p.xbuf, *xsum = L.xsum + (n_enter & 1) * (XMAX / 32);
+        if (my_tiles > 0) {  // workgroup-uniform
+            PK_STAMP(0);
+            stage_input<MODE>(p, st, c, xs, xsum, L.stat, mirror, pos, tok, tid, [] {});
+            for (int ch = 0; ch < n_chunks; ++ch) {
+                const int tiles = min(st.tpc, my_tiles - ch * st.tpc);
+                float *red = L.red + (ch & 1) * (SL * W * 64);
+                if (MODE == 0) compute_chunk(st, regs, xs, xsum, red, tiles, wave, lane);
+                if (ch == 0) PK_STAMP(4);
+                if (ch == 1) PK_STAMP(6);
+                if (ch + 1 < n_chunks) {
+                    if (ch == 0 && ha.n_slots > 0 && MODE == 0) {
+#pragma unroll
+                        for (int sl = 0; sl < SL; ++sl) {
+                            if (sl >= ha.n_slots) break;  // workgroup-uniform
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) regs.w[sl][q] = L.hl[(size_t)(sl * 5 + q) * T + tid];
+                            regs.sc[sl] = __uint_as_float(L.hl[(size_t)(sl * 5 + 4) * T + tid]);
+                        }
+                    } else {
+                        prefetch_lin<MODE>(st, regs, ch + 1, rank, wave, lane);
+                    }
+                }
+                __syncthreads();
+                head_finish<MODE>(p, st, L.red + (ch & 1) * (SL * W * 64), rank, ch, tiles, tid, best);
+                if (ch == 0) PK_STAMP(5);
+                if (ch == 1) PK_STAMP(7);
+            }
+            PK_STAMP(3);
+        }
+    }
+
+    // ---- arg-max over the workgroups' candidates, token feed ----
+    c.stage = p.n_stages;
+    u64 *cand = p.arena + p.cand_off;
+    best = block_max48(best, L.scr, lane, wave);
+    if (tid == 0) {
+        // key (32) | index code (16) | low 16 bits of the epoch: the tag of a candidate
+        __hip_atomic_store(cand + rank, (best << 16) | (u64)(c.epoch & 0xFFFFu), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (rank == 0) {
+        u64 w = 0ull;
+        if (tid < n_head_wgs) {
+            int spins = 0;
+            while (true) {
+                w = __hip_atomic_load(cand + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if ((uint32_t)(w & 0xFFFFu) == (c.epoch & 0xFFFFu) || c.dead) break;
+                if (spin_fail(c, spins)) break;
+            }
+            w >>= 16;
+        }
+        const u64 win = block_max48(w, L.scr, lane, wave);
+        if (tid == 0) {
+            if (MODE == 0) {
+                const uint32_t code = (uint32_t)(win & 0xFFFFu);
+                const uint32_t idx = (win >> 16) == 0ull ? 0u : (p.argmax_last ? code : 0xFFFFu - code);
+                p.next_tok[0] = idx;
+                p.cur_tok[0] = idx;
+                const int stp = *p.step_dev;
+                if (stp < p.out_capacity) p.out_tok[stp] = idx;
+                *p.pos_dev = pos + 1;
+                *p.step_dev = stp + 1;
+            }
+            // every workgroup of this launch has read the step's number (a relay may start late): only then the next one
+            {
+                int spins = 0;
+                const unsigned want = c.epoch * (unsigned)G;
+                while (!c.dead && (int)(__hip_atomic_load(p.state + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - want) < 0)
+                    if (spin_fail(c, spins)) break;
+            }
+            p.state[0] = c.epoch;
+        }
+    }
+    PK_DUMP();
+}
+
+int ilog2(int v) {
+    int s = 0;
+    while ((1 << s) < v) ++s;
+    return s;
+}
+
+bool aligned16(const void *q) { return ((uintptr_t)q & 15u) == 0; }
+
+bool linear_ok(const PkLinear &l) {
+    if (!l.packed || !l.scales) return false;
+    if (l.K % 32 != 0 || l.K < 32 || l.N > l.stride || l.N < 1) return false;
+    return true;
+}
+
+struct Roles {
+    int G, att_per_xcd, smax, nlin;
+};
+
+Roles plan_roles(const agpu_ctx *ctx, int H) {
+    Roles r{};
+    r.G = (ctx->num_cus / 8) * 8;
+    const int hx = ceil_div(H, 8);  // heads of an XCD at most
+    r.smax = NR <= 2 ? (hx <= 2 ? 3 : (hx <= 4 ? 2 : 1)) : (NR <= 4 && hx <= 2 ? 2 : 1);
+    r.att_per_xcd = hx * r.smax;
+    r.nlin = r.G / 8 - NR - r.att_per_xcd;
+    return r;
+}
+
+// Unit width, waves per unit and slots per lane for `ncols` columns (in n_cparts equal parts) over a k range of
+// n_groups scale groups, shared by nlin workgroups: the fewest slots per lane, then the fewest waves per unit, then
+// the narrowest unit.  False when nothing fits.
+bool plan_units(Stage &s, int pcols, int n_cparts, int n_groups, int li0, int nlin) {
+    s.li0 = li0;
+    s.ngrp = nlin;
+    int best_nl = SL + 1;
+    for (int tws = 0; tws <= 2; ++tws) {
+        const int tw = 16 << tws, gpw = 4 >> tws;
+        if (n_cparts > 1 && pcols % tw != 0) continue;  // parts are whole units
+        const int upp = ceil_div(pcols, tw), n_units = upp * n_cparts;
+        for (int wps = 0; wps <= 3; ++wps) {
+            const int wpt = 1 << wps, upw = W / wpt;
+            if (ceil_div(n_units, nlin) > upw) continue;
+            const int nl = ceil_div(n_groups, wpt * gpw);
+            if (nl < best_nl) {
+                best_nl = nl;
+                s.tws = tws; s.wps = wps; s.nl = nl; s.n_units = n_units; s.upp = upp;
+            }
+        }
+    }
+    return best_nl <= SL;
+}
+
+// The head: tiles of 64 columns dealt round robin.
+bool plan_head(Stage &s, const PkLinear &l, int n_wgs) {
+    s = Stage{};
+    s.K = l.K; s.n_valid = l.N; s.stride = l.stride; s.n_groups = l.K / 32; s.n_wgs = n_wgs;
+    s.packed = l.packed; s.scales = l.scales; s.bias = l.bias;
+    s.tws = 2;
+    s.n_tiles = ceil_div(l.N, 64);
+    s.nl = ceil_div(s.n_groups, W);
+    if (s.nl > SL) return false;
+    s.tpc = SL / s.nl;
+    s.inv_k = 1.0f / (float)l.K;
+    s.n_cparts = 1;
+    return true;
+}
+
+int xbuf_floats(int kmax) { return kmax / 32 * GS; }
+
+size_t lds_bytes_for(int n_stages, int kmax, int head_slots) {
+    (void)n_stages;
+    size_t b = (size_t)(2 * xbuf_floats(kmax) + 2 * (XMAX / 32) + 2 * SL * W * 64 + 4 * W + (SMAX + 1) * PSTRIDE + 2 * W) * 4 +
+               (size_t)head_slots * 5 * T * 4;
+#ifdef AGPU_PK_TRACE
+    b += (size_t)n_stages * 8 * sizeof(u64);
+#endif
+    return b;
+}
+
+// Heads and groups of 32 MLP columns of XCD x.
+void xcd_share(int total, int x, int &first, int &count) {
+    const int q = total / 8, r = total % 8;
+    count = q + (x < r ? 1 : 0);
+    first = x * q + std::min(x, r);
+}
+
+// The stage table of all eight XCDs, [8][4 n_layer + 1]; false when a stage does not fit.
+bool build_tables(const PkModel &m, const Roles &r, int lin_groups, size_t part_base, std::vector<Stage> &out, int *kmax_out) {
+    // Linear workgroups of an XCD in lin_groups groups (1, 2 or 4); stage kind k of a layer goes to group k % lin_groups
+    int g_first[4], g_size[4];
+    for (int k = 0; k < 4; ++k) {
+        const int g = k % lin_groups;
+        g_first[k] = g * r.nlin / lin_groups;
+        g_size[k] = (g + 1) * r.nlin / lin_groups - g_first[k];
+    }
+    const int d = m.d, ff = m.ff, n_st = 4 * m.n_layer + 1;
+    const size_t per_layer = (size_t)3 * d + d + d + ff + d + (size_t)m.H * SMAX * PSTRIDE;
+    const int gelu = m.gelu_quick ? F_GELU_QUICK : F_GELU_TANH;
+    out.assign((size_t)8 * n_st, Stage{});
+    int kmax = d;
+    for (int x = 0; x < 8; ++x) {
+        int h0, nh, g0, ng;
+        xcd_share(m.H, x, h0, nh);
+        xcd_share(ff / 32, x, g0, ng);
+        int prev_h2 = -2;
+        for (int L = 0; L < m.n_layer; ++L) {
+            const PkLayer &y = m.layers[L];
+            const int base = (int)(per_layer * L);
+            const int o_qkv = base, o_att = base + 3 * d, o_h1 = o_att + d, o_ffn = o_h1 + d, o_h2 = o_ffn + ff, o_part = o_h2 + d;
+            Stage *t = &out[(size_t)x * n_st + 4 * L];
+            // LN1 + QKV, the columns of this XCD's heads
+            {
+                Stage s{};
+                s.packed = y.qkv.packed; s.scales = y.qkv.scales; s.bias = y.qkv.bias; s.ln_g = y.ln1_g; s.ln_b = y.ln1_b;
+                s.kc = y.kcache; s.vc = y.vcache;
+                s.K = d; s.n_groups = d / 32; s.stride = y.qkv.stride; s.inv_k = 1.0f / (float)d;
+                s.col0 = h0 * DH; s.part_stride = d; s.pcols = nh * DH; s.n_cparts = 3;
+                s.in_off = prev_h2; s.out_off = o_qkv; s.att_off = o_att; s.part_off = o_part;
+                s.flags = F_LN | F_SCATTER;
+                if (nh > 0 && !plan_units(s, s.pcols, 3, s.n_groups, g_first[0], g_size[0])) return false;
+                t[0] = s;
+            }
+            // proj over the rows of this XCD's heads: a partial sum of all d outputs
+            {
+                Stage s{};
+                s.K = nh * DH; s.n_groups = s.K / 32; s.stride = y.proj.stride; s.inv_k = 1.0f;
+                s.packed = y.proj.packed + (size_t)(h0 * DH / 8) * y.proj.stride;
+                s.scales = y.proj.scales + (size_t)(h0 * DH / 32) * y.proj.stride;
+                s.col0 = 0; s.part_stride = 0; s.pcols = d; s.n_cparts = 1;
+                s.in_off = o_att + h0 * DH;
+                s.part_off = (int)(part_base + (size_t)(2 * L) * 8 * d);  // slot of XCD 0; this XCD's: x vectors on
+                s.out_off = s.part_off + x * d;
+                s.xbias = y.proj.bias; s.xout_off = o_h1; s.xn_parts = std::min(m.H, 8);
+                s.flags = F_PARTIAL;
+                if (nh > 0 && !plan_units(s, d, 1, s.n_groups, g_first[1], g_size[1])) return false;
+                kmax = std::max(kmax, s.K);
+                t[1] = s;
+            }
+            // LN2 + fc + GELU, this XCD's columns
+            {
+                Stage s{};
+                s.packed = y.fc.packed; s.scales = y.fc.scales; s.bias = y.fc.bias; s.ln_g = y.ln2_g; s.ln_b = y.ln2_b;
+                s.K = d; s.n_groups = d / 32; s.stride = y.fc.stride; s.inv_k = 1.0f / (float)d;
+                s.col0 = g0 * 32; s.part_stride = 0; s.pcols = ng * 32; s.n_cparts = 1;
+                s.in_off = o_h1; s.out_off = o_ffn;
+                s.flags = F_LN | gelu;
+                if (ng > 0 && !plan_units(s, s.pcols, 1, s.n_groups, g_first[2], g_size[2])) return false;
+                t[2] = s;
+            }
+            // fc-proj over the rows of those columns: a partial sum of all d outputs
+            {
+                Stage s{};
+                s.K = ng * 32; s.n_groups = ng; s.stride = y.fc_proj.stride; s.inv_k = 1.0f;
+                s.packed = y.fc_proj.packed + (size_t)(g0 * 4) * y.fc_proj.stride;
+                s.scales = y.fc_proj.scales + (size_t)g0 * y.fc_proj.stride;
+                s.col0 = 0; s.part_stride = 0; s.pcols = d; s.n_cparts = 1;
+                s.in_off = o_ffn + g0 * 32;
+                s.part_off = (int)(part_base + (size_t)(2 * L + 1) * 8 * d);
+                s.out_off = s.part_off + x * d;
+                s.xbias = y.fc_proj.bias; s.xout_off = o_h2; s.xn_parts = std::min(ff / 32, 8);
+                s.flags = F_PARTIAL;
+                if (ng > 0 && !plan_units(s, d, 1, s.n_groups, g_first[3], g_size[3])) return false;
+                kmax = std::max(kmax, s.K);
+                t[3] = s;
+            }
+            prev_h2 = o_h2;
+        }
+        Stage hs;
+        if (!plan_head(hs, m.head, r.G - 8 * NR)) return false;
+        hs.in_off = prev_h2; hs.flags = F_LN | F_HEAD; hs.ln_g = m.lnf_g; hs.ln_b = m.lnf_b;
+        out[(size_t)x * n_st + 4 * m.n_layer] = hs;
+    }
+    if (kmax_out) *kmax_out = kmax;
+    return kmax <= XMAX;
+}
+
+}  // namespace
+
+bool agpu_xk_supported(const agpu_ctx *ctx, const PkModel &m) {
+    const Roles r = plan_roles(ctx, m.H);
+    // eight XCDs of 32 CUs: the roles and the hand-offs through an L2 are laid out for this part
+    if (ctx->num_cus != 256 || r.nlin < 8 || m.H < 1 || r.G - 8 * NR > T) return false;
+    if (m.d != m.H * DH || m.d % 32 != 0 || m.d > 2 * T * LNP || m.d / 2 > NR * 64 * XI) return false;
+    if (m.ff % 32 != 0 || m.ff < 32 || m.V > 65535 || m.V < 1 || m.n_layer < 1 || m.group != 32) return false;
+    if (!linear_ok(m.head) || m.head.K != m.d) return false;
+    for (int L = 0; L < m.n_layer; ++L) {
+        const PkLayer &y = m.layers[L];
+        if (!linear_ok(y.qkv) || !linear_ok(y.proj) || !linear_ok(y.fc) || !linear_ok(y.fc_proj)) return false;
+        if (y.qkv.K != m.d || y.proj.K != m.d || y.fc.K != m.d) return false;
+        if (y.qkv.N != 3 * m.d || y.proj.N != m.d || y.fc.N != m.ff || y.fc_proj.N != m.d || y.fc_proj.K != m.ff) return false;
+        if (!y.ln1_g || !y.ln1_b || !y.ln2_g || !y.ln2_b || !y.kcache || !y.vcache) return false;
+        if (!aligned16(y.kcache) || !aligned16(y.vcache)) return false;
+    }
+    if (!m.lnf_g || !m.lnf_b || !m.wte || !m.wpe) return false;
+    std::vector<Stage> tab;
+    int kmax = 0;
+    if (!build_tables(m, r, 1, 0, tab, &kmax)) return false;
+    if (lds_bytes_for(4 * m.n_layer + 1, kmax, 0) > (size_t)160 * 1024) return false;
+    return true;
+}
+
+int32_t agpu_xk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
+    agpu_pk_plan_free(plan);
+    if (!agpu_xk_supported(ctx, m)) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "decode step: model shape not supported by the one-launch step");
+    const Roles r = plan_roles(ctx, m.H);
+    const int d = m.d, ff = m.ff;
+    const size_t per_layer = (size_t)3 * d + d + d + ff + d + (size_t)m.H * SMAX * PSTRIDE;
+    const size_t mirror_elems = (per_layer * m.n_layer + 15) & ~(size_t)15;
+    const size_t part_base = 8 * mirror_elems;
+    const size_t n_parts_elems = (size_t)m.n_layer * 2 * 8 * d;
+    const size_t cand_off = part_base + n_parts_elems;
+    const size_t total = (cand_off + (size_t)r.G + 1) & ~(size_t)1;
+    if (total > (size_t)0x7fffffff) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "decode step: activation arena too large");
+    std::vector<Stage> st;
+    int kmax = d;
+    // two groups of Linear workgroups taking the stages in turn where every stage then still fits, else one
+    int lin_groups = 2;
+    if (const char *env = getenv("AGPU_XK_GROUPS")) lin_groups = atoi(env) == 4 ? 4 : (atoi(env) == 1 ? 1 : 2);
+    while (lin_groups > 1 && !build_tables(m, r, lin_groups, part_base, st, &kmax)) lin_groups /= 2;
+    if (lin_groups == 1 && !build_tables(m, r, 1, part_base, st, &kmax))
+        return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "decode step: a stage does not fit");
+    plan->kind = 1;
+    plan->n_stages = 4 * m.n_layer + 1;
+    plan->grid = r.G;
+    plan->att_per_xcd = r.att_per_xcd;
+    plan->smax = r.smax;
+    plan->lin_per_xcd = r.nlin;
+    plan->cand_off = cand_off;
+    plan->arena_elems = mirror_elems;
+    const size_t arena_bytes = total * sizeof(u64);
+    hipError_t e = hipMalloc(&plan->stages_dev, st.size() * sizeof(Stage));
+    if (e == hipSuccess) e = hipMalloc((void **)&plan->arena, arena_bytes);
+    if (e == hipSuccess) e = hipMalloc((void **)&plan->state, 64);
+    if (e == hipSuccess) e = hipMemcpy(plan->stages_dev, st.data(), st.size() * sizeof(Stage), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemset(plan->arena, 0, arena_bytes);
+    if (e == hipSuccess) e = hipMemset(plan->state, 0, 64);
+    {
+        const Stage &hs = st.back();
+        const int tiles_max = ceil_div(hs.n_tiles, hs.n_wgs);
+        const int want = std::min(SL, std::min(hs.tpc, std::max(0, tiles_max - hs.tpc)) * hs.nl);
+        plan->head_slots = want > 0 && lds_bytes_for(plan->n_stages, kmax, want) <= (size_t)160 * 1024 ? want : 0;
+    }
+    plan->kmax = kmax;
+    // one workgroup per CU: the request is sized so that two never share a CU
+    plan->lds_bytes = std::max(lds_bytes_for(plan->n_stages, plan->kmax, plan->head_slots), (size_t)96 * 1024);
+    // An XCD's share of a layer's weights is touched two exchanges (one layer) before its use where two layers' shares
+    // leave room in the 4 MiB L2, else one exchange ahead.
+    {
+        const double share = ((double)3 * d * d + (double)d * d + 2.0 * d * ff) * 0.625 / 8.0;
+        plan->touch_dist = share <= 1.0e6 ? 2 : 1;
+        if (const char *env = getenv("AGPU_XK_TOUCH")) plan->touch_dist = atoi(env);
+    }
+    // the largest request any plan can make, once per device: the attribute belongs to the kernel, not to a plan
+    static bool attr_set[64] = {false};
+    if (e == hipSuccess && !attr_set[ctx->device & 63]) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(decode_xcd_kernel<0>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(decode_xcd_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e == hipSuccess) attr_set[ctx->device & 63] = true;
+    }
+    // Where the workgroups land: b, b + 8, ... must share an XCD, and the eight classes must sit on eight different ones.
+    // state[8 + x] keeps the XCD of class x; every launch of the step checks itself against it.
+    if (e == hipSuccess) {
+        unsigned *probe = nullptr;
+        std::vector<unsigned> where((size_t)r.G, 0u);
+        e = hipMalloc((void **)&probe, (size_t)r.G * sizeof(unsigned));
+        if (e == hipSuccess) {
+            hipLaunchKernelGGL(xcc_probe_kernel, dim3(r.G), dim3(T), 0, ctx->stream, probe);
+            e = hipGetLastError();
+            if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+            if (e == hipSuccess) e = hipMemcpy(where.data(), probe, where.size() * sizeof(unsigned), hipMemcpyDeviceToHost);
+            (void)hipFree(probe);
+        }
+        if (e == hipSuccess) {
+            unsigned cls[8], seen = 0u;
+            bool ok = true;
+            for (int x = 0; x < 8; ++x) {
+                cls[x] = where[(size_t)x];
+                ok = ok && cls[x] < 16u && !((seen >> cls[x]) & 1u);
+                seen |= 1u << (cls[x] & 15u);
+            }
+            for (int b = 0; b < r.G && ok; ++b) ok = where[(size_t)b] == cls[b & 7];
+            if (!ok) {
+                agpu_pk_plan_free(plan);
+                return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "decode step: workgroups b, b + 8, ... do not share an XCD on this device");
+            }
+            e = hipMemcpy(plan->state + 8, cls, sizeof(cls), hipMemcpyHostToDevice);
+        }
+    }
+    if (e != hipSuccess) {
+        agpu_pk_plan_free(plan);
+        return agpu_hip(ctx, e, "decode step: plan");
+    }
+    return AGPU_OK;
+}
+
+int32_t agpu_xk_launch(agpu_ctx *ctx, const PkModel &m, const PkPlan &plan, int mode, unsigned long long *trace) {
+    Params p{};
+    p.stages = reinterpret_cast<const Stage *>(plan.stages_dev);
+    p.n_stages = plan.n_stages;
+    p.n_layer = m.n_layer;
+    p.arena = plan.arena;
+    p.mirror_elems = plan.arena_elems;
+    p.cand_off = plan.cand_off;
+    p.state = plan.state;
+    p.wte = m.wte; p.wpe = m.wpe; p.logits = m.logits;
+    p.cur_tok = m.cur_tok; p.out_tok = m.out_tok; p.next_tok = m.next_tok;
+    p.pos_dev = m.pos_dev; p.step_dev = m.step_dev; p.out_capacity = m.out_capacity;
+    p.d = m.d; p.H = m.H; p.P = m.P; p.V = m.V; p.eps = m.eps; p.argmax_last = m.argmax_last;
+    p.att_per_xcd = plan.att_per_xcd;
+    p.smax = plan.smax;
+    p.nlin = plan.lin_per_xcd;
+    p.spin_limit = plan.spin_limit > 0 ? plan.spin_limit : kSpinLimit;
+    p.xbuf = xbuf_floats(plan.kmax);
+    p.head_slots = plan.head_slots;
+    p.touch_dist = plan.touch_dist;
+    p.trace = trace;
+    if (mode == 0) hipLaunchKernelGGL(decode_xcd_kernel<0>, dim3(plan.grid), dim3(T), plan.lds_bytes, ctx->stream, p);
+    else hipLaunchKernelGGL(decode_xcd_kernel<1>, dim3(plan.grid), dim3(T), plan.lds_bytes, ctx->stream, p);
+    return AGPU_LAUNCH_CHECK(ctx, "decode_xcd_kernel");
+}

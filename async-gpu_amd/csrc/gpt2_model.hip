@@ -545,8 +545,15 @@ bool pk_ready(agpu_gpt2 *m) {
     m->pk_tried = true;
     if (!m->logits.p || !m->out_tok) return false;
     const PkModel v = pk_view(m);
-    if (!agpu_pk_supported(m->ctx, v)) return false;
-    if (agpu_pk_plan_build(m->ctx, v, &m->pk) != AGPU_OK) return false;
+    // the XCD-sharded step where the shape allows, else the one with every Linear spread over the device
+    const char *pick = getenv("AGPU_DECODE_STEP");
+    const bool want_xk = !(pick && pick[0] == 'l');
+    if (want_xk && agpu_xk_supported(m->ctx, v)) {
+        if (agpu_xk_plan_build(m->ctx, v, &m->pk) != AGPU_OK) return false;
+    } else {
+        if (!agpu_pk_supported(m->ctx, v)) return false;
+        if (agpu_pk_plan_build(m->ctx, v, &m->pk) != AGPU_OK) return false;
+    }
     m->pk.spin_limit = m->pk_spin_limit;
     return true;
 }
@@ -585,7 +592,7 @@ int32_t decode_graph(agpu_gpt2 *m, int B, int bucket, hipGraphExec_t *out, int r
         // one sequence: the whole step, arg-max and token feed included, is one launch
         const PkModel view = pk_view(m);
         rc = AGPU_OK;
-        for (int r = 0; r < reps && rc == AGPU_OK; ++r) rc = agpu_pk_launch(ctx, view, m->pk, 0);
+        for (int r = 0; r < reps && rc == AGPU_OK; ++r) rc = agpu_step_launch(ctx, view, m->pk, 0);
     } else if (reps > 1) {
         rc = agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "gpt2: several steps per graph need the one-launch step");
     } else {
@@ -665,9 +672,9 @@ int32_t pk_check(agpu_gpt2 *m) {
         m->pk_failed = true;
         drop_graphs(m);
         return agpu_fail(m->ctx, AGPU_ERR_DEVICE_WAIT,
-                         "gpt2: a wait of the one-launch decode step gave up (stage %u); the steps since the last check are invalid, "
-                         "decode steps run per stage from now on",
-                         err & 0xfffu);
+                         "gpt2: a wait of the one-launch decode step gave up (code 0x%x, stage %u); the steps since the last check are "
+                         "invalid, decode steps run per stage from now on",
+                         err, err & 0xfffu);
     }
     return AGPU_OK;
 }
@@ -1029,7 +1036,7 @@ AGPU_EXPORT int32_t agpu_gpt2_decode_trace(agpu_gpt2 *m, int32_t mode, unsigned 
     unsigned long long *dev = nullptr;
     if (hipMalloc((void **)&dev, n * 8) != hipSuccess) return AGPU_ERR_WORKSPACE;
     (void)hipMemset(dev, 0, n * 8);
-    int32_t rc = agpu_pk_launch(m->ctx, pk_view(m), m->pk, mode, dev);
+    int32_t rc = agpu_step_launch(m->ctx, pk_view(m), m->pk, mode, dev);
     (void)hipStreamSynchronize(m->ctx->stream);
     (void)hipMemcpy(out_host, dev, n * 8, hipMemcpyDeviceToHost);
     (void)hipFree(dev);
@@ -1066,7 +1073,7 @@ AGPU_EXPORT int32_t agpu_gpt2_decode_floor(agpu_gpt2 *m, int32_t steps, float *m
     const PkModel v = pk_view(m);
     if ((rc = agpu_hip(ctx, hipEventRecord(m->ev0, ctx->stream), "hipEventRecord")) != AGPU_OK) return rc;
     for (int s = 0; s < steps; ++s)
-        if ((rc = agpu_pk_launch(ctx, v, m->pk, 1)) != AGPU_OK) return rc;
+        if ((rc = agpu_step_launch(ctx, v, m->pk, 1)) != AGPU_OK) return rc;
     if ((rc = agpu_hip(ctx, hipEventRecord(m->ev1, ctx->stream), "hipEventRecord")) != AGPU_OK) return rc;
     if ((rc = agpu_hip(ctx, hipEventSynchronize(m->ev1), "hipEventSynchronize")) != AGPU_OK) return rc;
     if (ms_total_out_host) (void)hipEventElapsedTime(ms_total_out_host, m->ev0, m->ev1);
