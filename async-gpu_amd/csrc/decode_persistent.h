@@ -49,6 +49,7 @@ struct PkPlan {
     int kind = 0;         // 0: every Linear spread over the device (decode_persistent.hip); 1: one tensor-parallel rank per XCD (decode_xcd.hip)
     int lin_per_xcd = 0;  // kind 1: Linear workgroups per XCD
     int touch_dist = 0;   // kind 1: how many exchanges ahead the relays touch the weights (0: not at all)
+    size_t parts_elems = 0;  // kind 1: floats of one set of partial sums
 };
 
 // Whether the persistent step can run this model (int4 head, head_dim 64, group 32, size limits).

@@ -19,9 +19,12 @@
 // vector into their own XCD's mirror; every XCD so holds the same bits.  Per layer two hand-offs go through memory and
 // three through an L2, where the step with all Linears spread over the whole device needs five through memory.
 //
-// Everything that travels is a (value, tag) pair, tag = number of the step: a consumer polls the very words it needs
-// and takes a value once its tag is the current step's.  The data is its own flag: no counters, no fences; a stale read
-// can only delay a tag.  Every vector of a step has its own place, so nothing is overwritten while the step runs.
+// The data is its own flag: every place that carries an activation holds an all-ones word (a NaN no arithmetic here
+// produces; a result with those bits is stored as another NaN) until its value is written, and a consumer polls the
+// very words it needs, 16 bytes = four values a load, until none of them is all-ones.  No counters, no fences; a
+// stale read can only delay a value.  Every vector of a step has its own place, and there are two sets of places that
+// the steps use in turn: whoever writes a place in one set resets the same place of the other set, which the step
+// before has finished with and the next step will poll.
 //
 // Roles per XCD: NR relays, a few attention workgroups ((head, key range) each, the cached K and V rows of the next
 // layer requested into registers as soon as this layer's are used up), the rest Linear workgroups.  A Linear stage of
@@ -49,17 +52,17 @@ constexpr int KVP = 8;          // attention: rounds of KR keys (K and V, 16 byt
 constexpr int KR = 4 * W;       // keys per round: four per wave
 constexpr int XMAX = 2048;      // longest input vector of a stage (staged in LDS): d, or an XCD's share of the MLP's hidden vector
 constexpr int GS = 36;          // floats between the groups of 32 in LDS (bank spread for 16-byte reads)
-constexpr int PMAX = XMAX / (2 * T);  // pairs of input elements a thread polls at most
-constexpr int LNP = 2048 / (2 * T);   // ... of a stage with LayerNorm (K <= 2048)
+static_assert(XMAX == 4 * T, "a thread owns one group of four input elements at most");
 constexpr int SMAX = 4;         // key ranges per head at most
 constexpr int PSTRIDE = 68;     // floats per partial attention result: o[64], m, l
 constexpr int kSpinLimit = 1 << 16;
 constexpr int DH = 64;
 #ifndef AGPU_XK_NR
-#define AGPU_XK_NR 2
+#define AGPU_XK_NR 4
 #endif
 constexpr int NR = AGPU_XK_NR;  // relay workgroups per XCD
-constexpr int XI = 8;           // column pairs a relay thread owns at most (d <= 2048)
+constexpr int XI = 4;           // groups of four columns a relay thread owns at most
+constexpr uint32_t SENT = 0xFFFFFFFFu;  // "not written yet"
 constexpr int NPRE = 3;         // slots whose nibbles are converted ahead of the input
 
 enum : int { F_LN = 1, F_GELU_TANH = 2, F_GELU_QUICK = 4, F_HEAD = 8, F_SCATTER = 16, F_PARTIAL = 32 };
@@ -87,8 +90,8 @@ static_assert(sizeof(Stage) % 16 == 0, "stage table is copied in 16-byte pieces"
 struct Params {
     const Stage *stages;  // [8][n_stages]
     int n_stages, n_layer;
-    u64 *arena;           // [8][mirror_elems] mirrors, then the partial sums, then the arg-max candidates
-    size_t mirror_elems;
+    float *arena;         // [2][8][mirror_elems] mirrors (two sets, one per XCD each), [2][parts_elems] partial sums, the arg-max candidates
+    size_t mirror_elems, parts_elems;
     size_t cand_off;
     unsigned *state;      // [0] epoch, [1] error, [2] workgroups started so far
     const float *wte, *wpe;
@@ -108,6 +111,9 @@ struct Params {
 };
 
 struct Ctl {
+    long oth;        // from a place in this step's set of mirrors to the same place in the other set (floats)
+    float *parts;    // arena + this step's set of partial sums (stage offsets count from the arena's start)
+    long poth;       // the same distance for the partial sums
     uint32_t epoch;
     unsigned *err;
     int stage;
@@ -116,38 +122,44 @@ struct Ctl {
     u64 *tr;
 };
 
-// Coherent across the XCDs: to and from memory.
-__device__ __forceinline__ u64 ld_tag(const u64 *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ void st_tag(u64 *p, float v, uint32_t tag) {
-    __hip_atomic_store(p, ((u64)tag << 32) | (u64)__float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// Coherent across the XCDs: write-through stores to memory.  The value, and the reset of the same place in the other set.
+__device__ __forceinline__ uint32_t canon(float v) {
+    const uint32_t b = __float_as_uint(v);
+    return b == SENT ? 0x7FFFFFFFu : b;
+}
+__device__ __forceinline__ void st_mem(float *p, long oth, float v) {
+    __hip_atomic_store(reinterpret_cast<uint32_t *>(p), canon(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(reinterpret_cast<uint32_t *>(p + oth), SENT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 // Within an XCD: an ordinary store lands in the L2 the XCD's CUs share (the CU's own cache writes through) ...
-__device__ __forceinline__ void st_loc(u64 *p, float v, uint32_t tag) {
-    const u64 w = ((u64)tag << 32) | (u64)__float_as_uint(v);
-    asm volatile("global_store_dwordx2 %0, %1, off" ::"v"(p), "v"(w) : "memory");
+__device__ __forceinline__ void st_raw(float *p, uint32_t w) { asm volatile("global_store_dword %0, %1, off" ::"v"(p), "v"(w) : "memory"); }
+__device__ __forceinline__ void st_loc(float *p, long oth, float v) {
+    st_raw(p, canon(v));
+    st_raw(p + oth, SENT);
 }
-__device__ __forceinline__ void st_loc2(u64 *p, float a, float b, uint32_t tag) {
-    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    u32x4 w;
-    w.x = __float_as_uint(a); w.y = tag; w.z = __float_as_uint(b); w.w = tag;
-    asm volatile("global_store_dwordx4 %0, %1, off" ::"v"(p), "v"(w) : "memory");
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void st_loc4(float *p, long oth, const float4 &v) {
+    u32x4 w, e;
+    w.x = canon(v.x); w.y = canon(v.y); w.z = canon(v.z); w.w = canon(v.w);
+    e.x = e.y = e.z = e.w = SENT;
+    // A store of more than 8 bytes reads its data registers after it has been issued; the compiler keeps the next
+    // instructions off them for its own stores, not for one written here: hence the s_nop.
+    asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 2" ::"v"(p), "v"(w) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 2" ::"v"(p + oth), "v"(e) : "memory");
 }
 // ... and a load past the CU's own cache finds it there.
-__device__ __forceinline__ u64 ld_loc(const u64 *p) {
-    u64 v;
-    asm volatile("global_load_dwordx2 %0, %1, off nt\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(p) : "memory");
+__device__ __forceinline__ uint32_t ld_loc(const float *p) {
+    uint32_t v;
+    asm volatile("global_load_dword %0, %1, off nt\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(p) : "memory");
     return v;
 }
-__device__ __forceinline__ float tag_val(u64 w) { return __uint_as_float((uint32_t)w); }
-__device__ __forceinline__ bool tag_ok(u64 w, uint32_t epoch) { return (uint32_t)(w >> 32) == epoch; }
 
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint4 as_u4(const u32x4 &v) { return make_uint4(v.x, v.y, v.z, v.w); }
 
-// N 16-byte loads (two pairs each) in flight at once; L2: past the CU's cache, from the XCD's L2; else from memory.
+// N 16-byte loads (four values each) in flight at once; L2: past the CU's cache, from the XCD's L2; else from memory.
 #define AGPU_LD1(POL) "global_load_dwordx4 %0, %1, off " POL "\n\ts_waitcnt vmcnt(0)"
 template <bool L2>
-__device__ __forceinline__ void ld_pairs(const u64 *const (&p)[1], uint4 (&o)[1]) {
+__device__ __forceinline__ void ld_pairs(const float *const (&p)[1], uint4 (&o)[1]) {
     u32x4 v0;
     if (L2) asm volatile(AGPU_LD1("nt") : "=&v"(v0) : "v"(p[0]) : "memory");
     else asm volatile(AGPU_LD1("sc1") : "=&v"(v0) : "v"(p[0]) : "memory");
@@ -155,7 +167,7 @@ __device__ __forceinline__ void ld_pairs(const u64 *const (&p)[1], uint4 (&o)[1]
 }
 #define AGPU_LD2(POL) "global_load_dwordx4 %0, %2, off " POL "\n\tglobal_load_dwordx4 %1, %3, off " POL "\n\ts_waitcnt vmcnt(0)"
 template <bool L2>
-__device__ __forceinline__ void ld_pairs(const u64 *const (&p)[2], uint4 (&o)[2]) {
+__device__ __forceinline__ void ld_pairs(const float *const (&p)[2], uint4 (&o)[2]) {
     u32x4 v0, v1;
     if (L2) asm volatile(AGPU_LD2("nt") : "=&v"(v0), "=&v"(v1) : "v"(p[0]), "v"(p[1]) : "memory");
     else asm volatile(AGPU_LD2("sc1") : "=&v"(v0), "=&v"(v1) : "v"(p[0]), "v"(p[1]) : "memory");
@@ -165,45 +177,23 @@ __device__ __forceinline__ void ld_pairs(const u64 *const (&p)[2], uint4 (&o)[2]
     "global_load_dwordx4 %0, %4, off " POL "\n\tglobal_load_dwordx4 %1, %5, off " POL "\n\t"                        \
     "global_load_dwordx4 %2, %6, off " POL "\n\tglobal_load_dwordx4 %3, %7, off " POL "\n\ts_waitcnt vmcnt(0)"
 template <bool L2>
-__device__ __forceinline__ void ld_pairs(const u64 *const (&p)[4], uint4 (&o)[4]) {
+__device__ __forceinline__ void ld_pairs(const float *const (&p)[4], uint4 (&o)[4]) {
     u32x4 v0, v1, v2, v3;
     if (L2) asm volatile(AGPU_LD4("nt") : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3) : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]) : "memory");
     else asm volatile(AGPU_LD4("sc1") : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3) : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]) : "memory");
     o[0] = as_u4(v0); o[1] = as_u4(v1); o[2] = as_u4(v2); o[3] = as_u4(v3);
 }
-#define AGPU_LD6(POL)                                                                                              \
-    "global_load_dwordx4 %0, %6, off " POL "\n\tglobal_load_dwordx4 %1, %7, off " POL "\n\t"                        \
-    "global_load_dwordx4 %2, %8, off " POL "\n\tglobal_load_dwordx4 %3, %9, off " POL "\n\t"                        \
-    "global_load_dwordx4 %4, %10, off " POL "\n\tglobal_load_dwordx4 %5, %11, off " POL "\n\ts_waitcnt vmcnt(0)"
+#define AGPU_LD3(POL)                                                                                              \
+    "global_load_dwordx4 %0, %3, off " POL "\n\tglobal_load_dwordx4 %1, %4, off " POL "\n\t"                        \
+    "global_load_dwordx4 %2, %5, off " POL "\n\ts_waitcnt vmcnt(0)"
 template <bool L2>
-__device__ __forceinline__ void ld_pairs(const u64 *const (&p)[6], uint4 (&o)[6]) {
-    u32x4 v0, v1, v2, v3, v4, v5;
-    if (L2)
-        asm volatile(AGPU_LD6("nt") : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3), "=&v"(v4), "=&v"(v5)
-                     : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]) : "memory");
-    else
-        asm volatile(AGPU_LD6("sc1") : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3), "=&v"(v4), "=&v"(v5)
-                     : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]) : "memory");
-    o[0] = as_u4(v0); o[1] = as_u4(v1); o[2] = as_u4(v2); o[3] = as_u4(v3); o[4] = as_u4(v4); o[5] = as_u4(v5);
+__device__ __forceinline__ void ld_pairs(const float *const (&p)[3], uint4 (&o)[3]) {
+    u32x4 v0, v1, v2;
+    if (L2) asm volatile(AGPU_LD3("nt") : "=&v"(v0), "=&v"(v1), "=&v"(v2) : "v"(p[0]), "v"(p[1]), "v"(p[2]) : "memory");
+    else asm volatile(AGPU_LD3("sc1") : "=&v"(v0), "=&v"(v1), "=&v"(v2) : "v"(p[0]), "v"(p[1]), "v"(p[2]) : "memory");
+    o[0] = as_u4(v0); o[1] = as_u4(v1); o[2] = as_u4(v2);
 }
-#define AGPU_LD8(POL)                                                                                              \
-    "global_load_dwordx4 %0, %8, off " POL "\n\tglobal_load_dwordx4 %1, %9, off " POL "\n\t"                        \
-    "global_load_dwordx4 %2, %10, off " POL "\n\tglobal_load_dwordx4 %3, %11, off " POL "\n\t"                      \
-    "global_load_dwordx4 %4, %12, off " POL "\n\tglobal_load_dwordx4 %5, %13, off " POL "\n\t"                      \
-    "global_load_dwordx4 %6, %14, off " POL "\n\tglobal_load_dwordx4 %7, %15, off " POL "\n\ts_waitcnt vmcnt(0)"
-template <bool L2>
-__device__ __forceinline__ void ld_pairs(const u64 *const (&p)[8], uint4 (&o)[8]) {
-    u32x4 v0, v1, v2, v3, v4, v5, v6, v7;
-    if (L2)
-        asm volatile(AGPU_LD8("nt") : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3), "=&v"(v4), "=&v"(v5), "=&v"(v6), "=&v"(v7)
-                     : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]) : "memory");
-    else
-        asm volatile(AGPU_LD8("sc1") : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3), "=&v"(v4), "=&v"(v5), "=&v"(v6), "=&v"(v7)
-                     : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]) : "memory");
-    o[0] = as_u4(v0); o[1] = as_u4(v1); o[2] = as_u4(v2); o[3] = as_u4(v3);
-    o[4] = as_u4(v4); o[5] = as_u4(v5); o[6] = as_u4(v6); o[7] = as_u4(v7);
-}
-__device__ __forceinline__ bool pair_ok(const uint4 &v, uint32_t epoch) { return v.y == epoch && v.w == epoch; }
+__device__ __forceinline__ bool quad_ok(const uint4 &v) { return v.x != SENT && v.y != SENT && v.z != SENT && v.w != SENT; }
 
 // After an unsuccessful poll round: true when the caller must give up.
 __device__ __forceinline__ bool spin_fail(Ctl &c, int &spins) {
@@ -220,9 +210,9 @@ __device__ __forceinline__ bool spin_fail(Ctl &c, int &spins) {
     return false;
 }
 
-// Polls N pairs of pairs (those with need[k]) until every one carries the step's tags; the values stay in v.
+// Polls N groups of four values (those with need[k]) until every one has been written; the values stay in v.
 template <bool L2, int N>
-__device__ __forceinline__ void poll_pairs(Ctl &c, const u64 *const (&ptr)[N], bool (&need)[N], uint4 (&v)[N]) {
+__device__ __forceinline__ void poll_quads(Ctl &c, const float *const (&ptr)[N], bool (&need)[N], uint4 (&v)[N]) {
     int spins = 0;
     while (!c.dead) {
         uint4 t[N];
@@ -231,7 +221,7 @@ __device__ __forceinline__ void poll_pairs(Ctl &c, const u64 *const (&ptr)[N], b
 #pragma unroll
         for (int k = 0; k < N; ++k)
             if (need[k]) {
-                if (pair_ok(t[k], c.epoch)) { v[k] = t[k]; need[k] = false; } else ok = false;
+                if (quad_ok(t[k])) { v[k] = t[k]; need[k] = false; } else ok = false;
             }
         if (ok || spin_fail(c, spins)) break;
     }
@@ -545,86 +535,52 @@ struct Lds {
 #endif
 
 // ---- input of a Linear stage ----
-// The input vector is awaited in the XCD's mirror (thread t owns the element pairs t, t + T, ...), normalised where
-// the stage has a LayerNorm, and staged in LDS with the sums of its groups.  `settle` is called right after the
-// poll: whatever its caller requested before has arrived with the polled data (a wave's loads return in order).
+// The input vector is awaited in the XCD's mirror (thread t owns the elements 4 t .. 4 t + 3), normalised where the
+// stage has a LayerNorm, and staged in LDS with the sums of its groups.  `settle` is called right after the poll:
+// whatever its caller requested before has arrived with the polled data (a wave's loads return in order).
 template <int MODE, typename Settle>
-__device__ __forceinline__ void stage_input(const Params &p, const Stage &st, Ctl &c, float *xs, float *xsum, float4 *stat, const u64 *mirror,
+__device__ __forceinline__ void stage_input(const Params &p, const Stage &st, Ctl &c, float *xs, float *xsum, float4 *stat, const float *mirror,
                                             int pos, uint32_t tok, int tid, Settle settle) {
     const int lane = tid & 63, wave = tid >> 6;
     const bool real = MODE == 0;
-    const int n_pairs = st.K >> 1;
-    float2 lg[LNP], lb[LNP];
-#pragma unroll
-    for (int i = 0; i < LNP; ++i) {
-        const int pr = tid + i * T;
-        lg[i] = make_float2(1.0f, 1.0f);
-        lb[i] = make_float2(0.0f, 0.0f);
-        if ((st.flags & F_LN) && real && pr < n_pairs) {
-            lg[i] = *reinterpret_cast<const float2 *>(st.ln_g + 2 * pr);
-            lb[i] = *reinterpret_cast<const float2 *>(st.ln_b + 2 * pr);
-        }
+    const int n_quads = st.K >> 2;
+    const bool have = tid < n_quads;
+    float4 lg = make_float4(1.0f, 1.0f, 1.0f, 1.0f), lb = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if ((st.flags & F_LN) && real && have) {
+        lg = *reinterpret_cast<const float4 *>(st.ln_g + 4 * tid);
+        lb = *reinterpret_cast<const float4 *>(st.ln_b + 4 * tid);
     }
-    float2 xv[PMAX];
-#pragma unroll
-    for (int i = 0; i < PMAX; ++i) xv[i] = make_float2(0.0f, 0.0f);
+    float4 x = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     if (st.in_off == -2) {
-#pragma unroll
-        for (int i = 0; i < LNP; ++i) {
-            const int pr = tid + i * T;
-            if (pr < n_pairs && real) {
-                const float2 a = *reinterpret_cast<const float2 *>(p.wte + (size_t)tok * p.d + 2 * pr);
-                const float2 b = *reinterpret_cast<const float2 *>(p.wpe + (size_t)pos * p.d + 2 * pr);
-                xv[i] = make_float2(a.x + b.x, a.y + b.y);
-            }
+        if (have && real) {
+            const float4 a = *reinterpret_cast<const float4 *>(p.wte + (size_t)tok * p.d + 4 * tid);
+            const float4 b = *reinterpret_cast<const float4 *>(p.wpe + (size_t)pos * p.d + 4 * tid);
+            x = make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
         }
     } else {
-        const u64 *src = mirror + st.in_off;
-        if (n_pairs <= T) {  // workgroup-uniform; one pair of pairs per thread at most: the common case
-            const u64 *ptr[1] = {src + 2 * (tid < n_pairs ? tid : 0)};
-            bool need[1] = {tid < n_pairs};
-            uint4 v[1] = {make_uint4(0u, 0u, 0u, 0u)};
-            poll_pairs<true, 1>(c, ptr, need, v);
-            xv[0] = make_float2(__uint_as_float(v[0].x), __uint_as_float(v[0].z));
-        } else {
-            static_assert(PMAX == 2, "a thread polls two pairs of pairs at most");
-            const u64 *ptr[2];
-            bool need[2];
-            uint4 v[2];
-#pragma unroll
-            for (int k = 0; k < 2; ++k) {
-                need[k] = tid + k * T < n_pairs;
-                ptr[k] = src + 2 * (need[k] ? tid + k * T : tid);
-                v[k] = make_uint4(0u, 0u, 0u, 0u);
-            }
-            poll_pairs<true, 2>(c, ptr, need, v);
-#pragma unroll
-            for (int k = 0; k < 2; ++k) xv[k] = make_float2(__uint_as_float(v[k].x), __uint_as_float(v[k].z));
-        }
+        const float *ptr[1] = {mirror + st.in_off + 4 * (have ? tid : 0)};
+        bool need[1] = {have};
+        uint4 v[1] = {make_uint4(0u, 0u, 0u, 0u)};
+        poll_quads<true, 1>(c, ptr, need, v);
+        x = as_f4(v[0]);
     }
     settle();
-#pragma unroll
-    for (int i = 0; i < LNP; ++i) asm volatile("" ::"v"(lg[i].x), "v"(lg[i].y), "v"(lb[i].x), "v"(lb[i].y));
+    asm volatile("" ::"v"(lg.x), "v"(lg.y), "v"(lg.z), "v"(lg.w), "v"(lb.x), "v"(lb.y), "v"(lb.z), "v"(lb.w));
     PK_STAMP(1);
-    if (st.flags & F_LN) {  // workgroup-uniform; K <= 2048
+    if (st.flags & F_LN) {  // workgroup-uniform
         // Every wave takes the mean of its own elements and their squared distances from it (two passes over the
         // registers, nn/cpu_ref.rs:38-47); the waves' (count, sum, mean, M2) are put together after one barrier.
-        int cnt = 0;
-#pragma unroll
-        for (int i = 0; i < LNP; ++i) cnt += 2 * max(0, min(64, n_pairs - (wave * 64 + i * T)));  // wave-uniform
-        float sm = 0.0f;
-#pragma unroll
-        for (int i = 0; i < LNP; ++i) sm += xv[i].x + xv[i].y;  // absent pairs are zero
-        sm = wave_sum(sm);
+        const int cnt = 4 * max(0, min(64, n_quads - wave * 64));  // wave-uniform
+        const float sm = wave_sum((x.x + x.y) + (x.z + x.w));  // absent elements are zero
         const float mw = cnt > 0 ? sm * __builtin_amdgcn_rcpf((float)cnt) : 0.0f;
         float m2 = 0.0f;
-#pragma unroll
-        for (int i = 0; i < LNP; ++i)
-            if (tid + i * T < n_pairs) {
-                const float d0 = xv[i].x - mw, d1 = xv[i].y - mw;
-                m2 = fmaf(d0, d0, m2);
-                m2 = fmaf(d1, d1, m2);
-            }
+        if (have) {
+            const float d0 = x.x - mw, d1 = x.y - mw, d2 = x.z - mw, d3 = x.w - mw;
+            m2 = fmaf(d0, d0, m2);
+            m2 = fmaf(d1, d1, m2);
+            m2 = fmaf(d2, d2, m2);
+            m2 = fmaf(d3, d3, m2);
+        }
         m2 = wave_sum(m2);
         if (lane == 0) stat[wave] = make_float4((float)cnt, sm, mw, m2);
         __syncthreads();
@@ -644,23 +600,16 @@ __device__ __forceinline__ void stage_input(const Params &p, const Stage &st, Ct
         const float var = M2 * st.inv_k + p.eps;
         float rstd = __builtin_amdgcn_rsqf(var);
         rstd = rstd * fmaf(-0.5f * var * rstd, rstd, 1.5f);  // one Newton step: the hardware estimate is good to 1 ulp
-#pragma unroll
-        for (int i = 0; i < LNP; ++i) {
-            xv[i].x = (xv[i].x - mean) * rstd * lg[i].x + lb[i].x;
-            xv[i].y = (xv[i].y - mean) * rstd * lg[i].y + lb[i].y;
-        }
+        x.x = (x.x - mean) * rstd * lg.x + lb.x;
+        x.y = (x.y - mean) * rstd * lg.y + lb.y;
+        x.z = (x.z - mean) * rstd * lg.z + lb.z;
+        x.w = (x.w - mean) * rstd * lg.w + lb.w;
     }
-    // the vector and the sums of its groups (16 pairs = 16 adjacent lanes) into LDS
-#pragma unroll
-    for (int i = 0; i < PMAX; ++i) {
-        if (i * T >= n_pairs) break;  // workgroup-uniform
-        const int pr = tid + i * T;
-        const bool have = pr < n_pairs;
-        const float gs = row16_sum(have ? xv[i].x + xv[i].y : 0.0f);
-        if (have) {
-            *reinterpret_cast<float2 *>(xs + (pr >> 4) * GS + 2 * (pr & 15)) = xv[i];
-            if ((lane & 15) == 0) xsum[pr >> 4] = gs;
-        }
+    // the vector and the sums of its groups (32 elements = 8 adjacent lanes) into LDS
+    const float gs = oct_sum(have ? (x.x + x.y) + (x.z + x.w) : 0.0f);
+    if (have) {
+        *reinterpret_cast<float4 *>(xs + (tid >> 3) * GS + 4 * (tid & 7)) = x;
+        if ((lane & 7) == 0) xsum[tid >> 3] = gs;
     }
     __syncthreads();
     PK_STAMP(2);
@@ -672,7 +621,7 @@ __device__ __forceinline__ void stage_input(const Params &p, const Stage &st, Ct
 // the tagged store (into the XCD's mirror, or as a partial sum into memory), and for K and V columns the row of the cache.
 template <int MODE>
 __device__ __forceinline__ void lay_stage(const Params &p, const Stage &st, Ctl &c, const Regs &r, float *xs, float *xsum, float4 *stat,
-                                          float *red, u64 *mirror, int pos, uint32_t tok, int li, int tid) {
+                                          float *red, float *mirror, int pos, uint32_t tok, int li, int tid) {
     const int lane = tid & 63, wave = tid >> 6;
     const bool real = MODE == 0;
     const int tsh = 4 + st.tws, tw = 1 << tsh;
@@ -722,8 +671,8 @@ __device__ __forceinline__ void lay_stage(const Params &p, const Stage &st, Ctl 
             if (st.flags & F_GELU_TANH) v = gelu_tanh_dev(v);
             else if (st.flags & F_GELU_QUICK) v = gelu_quick_dev(v);
         }
-        if (st.flags & F_PARTIAL) st_tag(p.arena + st.out_off + n, v, c.epoch);
-        else st_loc(mirror + st.out_off + n, v, c.epoch);
+        if (st.flags & F_PARTIAL) st_mem(c.parts + st.out_off + n, c.poth, v);
+        else st_loc(mirror + st.out_off + n, c.oth, v);
         if ((st.flags & F_SCATTER) && real && n >= p.d) {
             const int jn = n - p.d;
             const bool is_v = jn >= p.d;
@@ -783,29 +732,29 @@ __device__ __forceinline__ void touch_stage(CStage e, int tid, int r, uint32_t (
     }
 }
 
-// The exchanges of the step, for relay r of the XCD: thread (cp_local, part) = (tid >> 3, tid & 7) polls the partial
-// sum of XCD `part` for the column pairs r cps + cp_local + 64 k; the eight lanes of a column pair add up what they
-// got, and lane 0 of them adds bias and residual, keeps the result as the next residual and stores it into the mirror.
+// The exchanges of the step, for relay r of the XCD: thread (cq_local, part) = (tid >> 3, tid & 7) polls the partial
+// sum of XCD `part` for the groups of four columns r cqs + cq_local + 64 k; the eight lanes of such a group add up what
+// they got, and lane 0 of them adds bias and residual, keeps the result as the next residual and stores it into the mirror.
 template <int MODE>
-__device__ __forceinline__ void relay_role(const Params &p, CStage tab, Ctl &c, u64 *mirror, int pos, uint32_t tok, int tid, int r) {
+__device__ __forceinline__ void relay_role(const Params &p, CStage tab, Ctl &c, float *mirror, int pos, uint32_t tok, int tid, int r) {
     const bool real = MODE == 0;
-    const int part = tid & 7, cpl = tid >> 3;
-    const int half = p.d >> 1;
-    const int cps = (half + NR - 1) / NR;
-    const int n_it = (cps + 63) >> 6;  // <= XI
-    float2 res[XI];
+    const int part = tid & 7, cql = tid >> 3;
+    const int quads = p.d >> 2;
+    const int cqs = (quads + NR - 1) / NR;
+    const int n_it = (cqs + 63) >> 6;  // <= XI
+    float4 res[XI];
     bool valid[XI];
-    int cp[XI];
+    int cq[XI];
 #pragma unroll
     for (int k = 0; k < XI; ++k) {
-        const int l = cpl + 64 * k;
-        cp[k] = r * cps + l;
-        valid[k] = k < n_it && l < cps && cp[k] < half;
-        res[k] = make_float2(0.0f, 0.0f);
+        const int l = cql + 64 * k;
+        cq[k] = r * cqs + l;
+        valid[k] = k < n_it && l < cqs && cq[k] < quads;
+        res[k] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         if (valid[k] && part == 0 && real) {
-            const float2 a = *reinterpret_cast<const float2 *>(p.wte + (size_t)tok * p.d + 2 * cp[k]);
-            const float2 b = *reinterpret_cast<const float2 *>(p.wpe + (size_t)pos * p.d + 2 * cp[k]);
-            res[k] = make_float2(a.x + b.x, a.y + b.y);
+            const float4 a = *reinterpret_cast<const float4 *>(p.wte + (size_t)tok * p.d + 4 * cq[k]);
+            const float4 b = *reinterpret_cast<const float4 *>(p.wpe + (size_t)pos * p.d + 4 * cq[k]);
+            res[k] = make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
         }
     }
     uint32_t tk0[TK], tk1[TK];
@@ -823,13 +772,13 @@ __device__ __forceinline__ void relay_role(const Params &p, CStage tab, Ctl &c, 
         c.stage = 2 * x + 1;
         const int n_parts = e->xn_parts, src_off = e->part_off, dst_off = e->xout_off;
         const float *xbias = glob(e->xbias);
-        float2 bias[XI];
+        float4 bias[XI];
 #pragma unroll
         for (int k = 0; k < XI; ++k) {
-            bias[k] = make_float2(0.0f, 0.0f);
-            if (valid[k] && part == 0 && real && xbias) bias[k] = *reinterpret_cast<const float2 *>(xbias + 2 * cp[k]);
+            bias[k] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (valid[k] && part == 0 && real && xbias) bias[k] = *reinterpret_cast<const float4 *>(xbias + 4 * cq[k]);
         }
-        const u64 *src = p.arena + src_off + (size_t)part * p.d;
+        const float *src = c.parts + src_off + (size_t)part * p.d;
         uint4 v[XI];
         bool need[XI];
 #pragma unroll
@@ -839,35 +788,27 @@ __device__ __forceinline__ void relay_role(const Params &p, CStage tab, Ctl &c, 
         }
         PK_STAMP(5);
         if (n_it <= 1) {
-            const u64 *ptr[1] = {src + 2 * (need[0] ? cp[0] : 0)};
+            const float *ptr[1] = {src + 4 * (need[0] ? cq[0] : 0)};
             bool nd[1] = {need[0]};
             uint4 vv[1] = {v[0]};
-            poll_pairs<false, 1>(c, ptr, nd, vv);
+            poll_quads<false, 1>(c, ptr, nd, vv);
             v[0] = vv[0];
         } else if (n_it <= 2) {
-            const u64 *ptr[2];
+            const float *ptr[2];
             bool nd[2];
             uint4 vv[2];
 #pragma unroll
-            for (int k = 0; k < 2; ++k) { ptr[k] = src + 2 * (need[k] ? cp[k] : 0); nd[k] = need[k]; vv[k] = v[k]; }
-            poll_pairs<false, 2>(c, ptr, nd, vv);
+            for (int k = 0; k < 2; ++k) { ptr[k] = src + 4 * (need[k] ? cq[k] : 0); nd[k] = need[k]; vv[k] = v[k]; }
+            poll_quads<false, 2>(c, ptr, nd, vv);
 #pragma unroll
             for (int k = 0; k < 2; ++k) v[k] = vv[k];
-        } else if (n_it <= 4) {
-            const u64 *ptr[4];
-            bool nd[4];
-            uint4 vv[4];
-#pragma unroll
-            for (int k = 0; k < 4; ++k) { ptr[k] = src + 2 * (need[k] ? cp[k] : 0); nd[k] = need[k]; vv[k] = v[k]; }
-            poll_pairs<false, 4>(c, ptr, nd, vv);
-#pragma unroll
-            for (int k = 0; k < 4; ++k) v[k] = vv[k];
         } else {
-            const u64 *ptr[8];
-            bool nd[8];
+            static_assert(XI == 4, "a relay thread polls four groups at most");
+            const float *ptr[4];
+            bool nd[4];
 #pragma unroll
-            for (int k = 0; k < 8; ++k) { ptr[k] = src + 2 * (need[k] ? cp[k] : 0); nd[k] = need[k]; }
-            poll_pairs<false, 8>(c, ptr, nd, v);
+            for (int k = 0; k < 4; ++k) { ptr[k] = src + 4 * (need[k] ? cq[k] : 0); nd[k] = need[k]; }
+            poll_quads<false, 4>(c, ptr, nd, v);
         }
 #pragma unroll
         for (int s = 0; s < TK; ++s) asm volatile("" ::"v"(tk0[s]), "v"(tk1[s]));
@@ -875,11 +816,13 @@ __device__ __forceinline__ void relay_role(const Params &p, CStage tab, Ctl &c, 
 #pragma unroll
         for (int k = 0; k < XI; ++k) {
             if (k >= n_it) break;  // workgroup-uniform
-            const float sx = oct_sum(__uint_as_float(v[k].x)), sy = oct_sum(__uint_as_float(v[k].z));
+            const float4 t = as_f4(v[k]);  // zeros where nothing was polled
+            const float sx = oct_sum(t.x), sy = oct_sum(t.y), sz = oct_sum(t.z), sw = oct_sum(t.w);
             if (valid[k] && part == 0) {
-                const float hx = real ? (sx + bias[k].x) + res[k].x : 0.0f, hy = real ? (sy + bias[k].y) + res[k].y : 0.0f;
-                res[k] = make_float2(hx, hy);
-                st_loc2(mirror + dst_off + 2 * cp[k], hx, hy, c.epoch);
+                float4 h = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                if (real) h = make_float4((sx + bias[k].x) + res[k].x, (sy + bias[k].y) + res[k].y, (sz + bias[k].z) + res[k].z, (sw + bias[k].w) + res[k].w);
+                res[k] = h;
+                st_loc4(mirror + dst_off + 4 * cq[k], c.oth, h);
             }
         }
         PK_STAMP(7);
@@ -924,7 +867,7 @@ __device__ __forceinline__ void prefetch_attn(const float *kc, const float *vc, 
 // next batch, of this layer or the next, is requested before anything else is waited for.  q, the new k and v, the
 // partial results of the key ranges and the output all stay in the XCD's mirror.
 template <int MODE>
-__device__ __forceinline__ void attn_role(const Params &p, CStage tab, Ctl &c, const Lds &L, u64 *mirror, int pos, int h, int S, int ks, int tid) {
+__device__ __forceinline__ void attn_role(const Params &p, CStage tab, Ctl &c, const Lds &L, float *mirror, int pos, int h, int S, int ks, int tid) {
     const int lane = tid & 63, wave = tid >> 6;
     const int e4 = lane & 15, kq = lane >> 4;
     const bool real = MODE == 0;
@@ -957,25 +900,24 @@ __device__ __forceinline__ void attn_role(const Params &p, CStage tab, Ctl &c, c
         if (first == 0) {
             PK_STAMP(0);
             // q of this head, and for one wave the new key and value, from the QKV vector in the mirror
-            const u64 *qsrc = mirror + st.out_off + h * DH + 4 * e4;
-            uint4 w6[6];
+            const float *qsrc = mirror + st.out_off + h * DH + 4 * e4;
+            uint4 w3[3];
 #pragma unroll
-            for (int k = 0; k < 6; ++k) w6[k] = make_uint4(0u, 0u, 0u, 0u);
+            for (int k = 0; k < 3; ++k) w3[k] = make_uint4(0u, 0u, 0u, 0u);
             if (with_new) {
-                const u64 *ptr[6] = {qsrc, qsrc + 2, qsrc + p.d, qsrc + p.d + 2, qsrc + 2 * p.d, qsrc + 2 * p.d + 2};
-                bool need[6] = {true, true, true, true, true, true};
-                poll_pairs<true, 6>(c, ptr, need, w6);
+                const float *ptr[3] = {qsrc, qsrc + p.d, qsrc + 2 * p.d};
+                bool need[3] = {true, true, true};
+                poll_quads<true, 3>(c, ptr, need, w3);
             } else {
-                const u64 *ptr[2] = {qsrc, qsrc + 2};
-                bool need[2] = {true, true};
-                uint4 w2[2] = {w6[0], w6[1]};
-                poll_pairs<true, 2>(c, ptr, need, w2);
-                w6[0] = w2[0];
-                w6[1] = w2[1];
+                const float *ptr[1] = {qsrc};
+                bool need[1] = {true};
+                uint4 w1[1] = {w3[0]};
+                poll_quads<true, 1>(c, ptr, need, w1);
+                w3[0] = w1[0];
             }
-            q = make_float4(__uint_as_float(w6[0].x), __uint_as_float(w6[0].z), __uint_as_float(w6[1].x), __uint_as_float(w6[1].z));
-            kn[0] = __uint_as_float(w6[2].x); kn[1] = __uint_as_float(w6[2].z); kn[2] = __uint_as_float(w6[3].x); kn[3] = __uint_as_float(w6[3].z);
-            vn[0] = __uint_as_float(w6[4].x); vn[1] = __uint_as_float(w6[4].z); vn[2] = __uint_as_float(w6[5].x); vn[3] = __uint_as_float(w6[5].z);
+            q = as_f4(w3[0]);
+            kn[0] = __uint_as_float(w3[1].x); kn[1] = __uint_as_float(w3[1].y); kn[2] = __uint_as_float(w3[1].z); kn[3] = __uint_as_float(w3[1].w);
+            vn[0] = __uint_as_float(w3[2].x); vn[1] = __uint_as_float(w3[2].y); vn[2] = __uint_as_float(w3[2].z); vn[3] = __uint_as_float(w3[2].w);
             m = ninf;
             l = 0.0f;
             o = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -1075,22 +1017,23 @@ __device__ __forceinline__ void attn_role(const Params &p, CStage tab, Ctl &c, c
             }
             PK_STAMP(2);
             if (S == 1) {
-                if (tid < DH) st_loc(mirror + cur.att_off + h * DH + tid, res, c.epoch);
+                if (tid < DH) st_loc(mirror + cur.att_off + h * DH + tid, c.oth, res);
             } else if (ks != 0) {
-                if (tid < DH + 2) st_loc(mirror + cur.part_off + (h * SMAX + ks) * PSTRIDE + tid, res, c.epoch);
+                if (tid < DH + 2) st_raw(mirror + cur.part_off + (h * SMAX + ks) * PSTRIDE + tid, canon(res));  // reset by its reader
             } else {
                 // key range 0 merges the ranges of its head
                 if (tid < DH + 2) own[tid] = res;
                 const int other = tid / PSTRIDE + 1, i = tid % PSTRIDE;  // T >= (SMAX - 1) * PSTRIDE
                 if (other < S && i < DH + 2) {
-                    const u64 *src = mirror + cur.part_off + (h * SMAX + other) * PSTRIDE + i;
-                    u64 w = ld_loc(src);
+                    float *src = mirror + cur.part_off + (h * SMAX + other) * PSTRIDE + i;
+                    uint32_t w = ld_loc(src);
                     int spins = 0;
-                    while (!tag_ok(w, c.epoch) && !c.dead) {
+                    while (w == SENT && !c.dead) {
                         if (spin_fail(c, spins)) break;
                         w = ld_loc(src);
                     }
-                    oth[(other - 1) * PSTRIDE + i] = tag_val(w);
+                    st_raw(src, SENT);  // read: free for the step after the next
+                    oth[(other - 1) * PSTRIDE + i] = __uint_as_float(w);
                 }
                 __syncthreads();
                 if (tid < DH) {
@@ -1108,7 +1051,7 @@ __device__ __forceinline__ void attn_role(const Params &p, CStage tab, Ctl &c, c
                         }
                         v = num / den;
                     }
-                    st_loc(mirror + cur.att_off + h * DH + tid, v, c.epoch);
+                    st_loc(mirror + cur.att_off + h * DH + tid, c.oth, v);
                 }
             }
             PK_STAMP(3);
@@ -1227,7 +1170,12 @@ __global__ __launch_bounds__(T) void decode_xcd_kernel(const Params p) {
     tok = tok < (uint32_t)p.V ? tok : (uint32_t)(p.V - 1);
     __syncthreads();
 
-    u64 *mirror = p.arena + (size_t)xcd * p.mirror_elems;
+    // the two sets of places are used in turn
+    const int par = (int)(c.epoch & 1u);
+    float *mirror = p.arena + ((size_t)par * 8 + xcd) * p.mirror_elems;
+    c.oth = (par ? -1L : 1L) * (long)(8 * p.mirror_elems);
+    c.parts = p.arena + (size_t)par * p.parts_elems;
+    c.poth = (par ? -1L : 1L) * (long)p.parts_elems;
     if (in_xcd < NR) {
         relay_role<MODE>(p, tab, c, mirror, pos, tok, tid, in_xcd);
         PK_DUMP();
@@ -1327,7 +1275,7 @@ __global__ __launch_bounds__(T) void decode_xcd_kernel(const Params p) {
 
     // ---- arg-max over the workgroups' candidates, token feed ----
     c.stage = p.n_stages;
-    u64 *cand = p.arena + p.cand_off;
+    u64 *cand = reinterpret_cast<u64 *>(p.arena + p.cand_off);
     best = block_max48(best, L.scr, lane, wave);
     if (tid == 0) {
         // key (32) | index code (16) | low 16 bits of the epoch: the tag of a candidate
@@ -1551,7 +1499,7 @@ bool agpu_xk_supported(const agpu_ctx *ctx, const PkModel &m) {
     const Roles r = plan_roles(ctx, m.H);
     // eight XCDs of 32 CUs: the roles and the hand-offs through an L2 are laid out for this part
     if (ctx->num_cus != 256 || r.nlin < 8 || m.H < 1 || r.G - 8 * NR > T) return false;
-    if (m.d != m.H * DH || m.d % 32 != 0 || m.d > 2 * T * LNP || m.d / 2 > NR * 64 * XI) return false;
+    if (m.d != m.H * DH || m.d % 32 != 0 || m.d > XMAX || m.d / 4 > NR * 64 * XI) return false;
     if (m.ff % 32 != 0 || m.ff < 32 || m.V > 65535 || m.V < 1 || m.n_layer < 1 || m.group != 32) return false;
     if (!linear_ok(m.head) || m.head.K != m.d) return false;
     for (int L = 0; L < m.n_layer; ++L) {
@@ -1576,11 +1524,12 @@ int32_t agpu_xk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
     const Roles r = plan_roles(ctx, m.H);
     const int d = m.d, ff = m.ff;
     const size_t per_layer = (size_t)3 * d + d + d + ff + d + (size_t)m.H * SMAX * PSTRIDE;
-    const size_t mirror_elems = (per_layer * m.n_layer + 15) & ~(size_t)15;
-    const size_t part_base = 8 * mirror_elems;
-    const size_t n_parts_elems = (size_t)m.n_layer * 2 * 8 * d;
-    const size_t cand_off = part_base + n_parts_elems;
-    const size_t total = (cand_off + (size_t)r.G + 1) & ~(size_t)1;
+    // in floats: two sets of eight mirrors, two sets of partial sums, then the arg-max candidates (8 bytes each)
+    const size_t mirror_elems = (per_layer * m.n_layer + 31) & ~(size_t)31;
+    const size_t part_base = 16 * mirror_elems;
+    const size_t parts_elems = (size_t)m.n_layer * 2 * 8 * d;
+    const size_t cand_off = part_base + 2 * parts_elems;
+    const size_t total = cand_off + 2 * (size_t)r.G + 2;
     if (total > (size_t)0x7fffffff) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "decode step: activation arena too large");
     std::vector<Stage> st;
     int kmax = d;
@@ -1598,13 +1547,20 @@ int32_t agpu_xk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
     plan->lin_per_xcd = r.nlin;
     plan->cand_off = cand_off;
     plan->arena_elems = mirror_elems;
-    const size_t arena_bytes = total * sizeof(u64);
+    plan->parts_elems = parts_elems;
+    const size_t arena_bytes = total * sizeof(float);
     hipError_t e = hipMalloc(&plan->stages_dev, st.size() * sizeof(Stage));
     if (e == hipSuccess) e = hipMalloc((void **)&plan->arena, arena_bytes);
     if (e == hipSuccess) e = hipMalloc((void **)&plan->state, 64);
     if (e == hipSuccess) e = hipMemcpy(plan->stages_dev, st.data(), st.size() * sizeof(Stage), hipMemcpyHostToDevice);
-    if (e == hipSuccess) e = hipMemset(plan->arena, 0, arena_bytes);
-    if (e == hipSuccess) e = hipMemset(plan->state, 0, 64);
+    // every place "not written yet" (all-ones words); the candidates zero
+    // (on the stream the step runs on, and waited for: a fill still under way when the first step starts would leave
+    // words that are neither all-ones nor a value of the step)
+    if (e == hipSuccess) e = hipMemsetAsync(plan->arena, 0xFF, cand_off * sizeof(float), ctx->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(reinterpret_cast<float *>(plan->arena) + cand_off, 0, (total - cand_off) * sizeof(float), ctx->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(plan->state, 0, 64, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e == hipSuccess) e = hipDeviceSynchronize();
     {
         const Stage &hs = st.back();
         const int tiles_max = ceil_div(hs.n_tiles, hs.n_wgs);
@@ -1670,8 +1626,9 @@ int32_t agpu_xk_launch(agpu_ctx *ctx, const PkModel &m, const PkPlan &plan, int 
     p.stages = reinterpret_cast<const Stage *>(plan.stages_dev);
     p.n_stages = plan.n_stages;
     p.n_layer = m.n_layer;
-    p.arena = plan.arena;
+    p.arena = reinterpret_cast<float *>(plan.arena);
     p.mirror_elems = plan.arena_elems;
+    p.parts_elems = plan.parts_elems;
     p.cand_off = plan.cand_off;
     p.state = plan.state;
     p.wte = m.wte; p.wpe = m.wpe; p.logits = m.logits;

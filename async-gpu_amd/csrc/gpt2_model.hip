@@ -1029,6 +1029,14 @@ AGPU_EXPORT int32_t agpu_gpt2_decode_steps(agpu_gpt2 *m, int32_t batch, int32_t 
 }
 
 #ifdef AGPU_PK_TRACE
+// Debug builds only: the one-launch step's arena (device pointer, bytes of one mirror, of one set of partial sums).
+AGPU_EXPORT int32_t agpu_gpt2_debug_arena(agpu_gpt2 *m, void **arena_out, unsigned long long *mirror_elems, unsigned long long *parts_elems) {
+    if (!m || !m->pk.arena) return AGPU_ERR_UNSUPPORTED;
+    *arena_out = m->pk.arena;
+    *mirror_elems = m->pk.arena_elems;
+    *parts_elems = m->pk.parts_elems;
+    return AGPU_OK;
+}
 // Debug builds only: one step of the one-launch decode with time stamps, [grid][n_stages][4] ticks of 10 ns.
 AGPU_EXPORT int32_t agpu_gpt2_decode_trace(agpu_gpt2 *m, int32_t mode, unsigned long long *out_host, int32_t *grid_out, int32_t *stages_out) {
     if (!pk_ready(m)) return AGPU_ERR_UNSUPPORTED;
