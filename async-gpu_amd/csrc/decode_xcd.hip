@@ -1130,6 +1130,18 @@ __global__ __launch_bounds__(T) void xcc_probe_kernel(unsigned *out) {
     if (threadIdx.x == 0) out[blockIdx.x] = xcc_id();
 }
 
+// Before a workgroup leaves: is it on the XCD the first workgroup of its class reported for this step?
+__device__ __forceinline__ void check_xcd(const Params &p, Ctl &c, int xcd, int tid) {
+    if (tid != 0 || c.dead) return;
+    int spins = 0;
+    unsigned w = __hip_atomic_load(p.state + 8 + xcd, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    while ((w >> 4) != (c.epoch & 0x0fffffffu)) {
+        if (spin_fail(c, spins)) return;
+        w = __hip_atomic_load(p.state + 8 + xcd, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if ((w & 15u) != xcc_id()) atomicCAS(c.err, 0u, 0x2000u + (unsigned)xcd);
+}
+
 template <int MODE>
 __global__ __launch_bounds__(T) void decode_xcd_kernel(const Params p) {
     extern __shared__ __align__(16) float smem[];
@@ -1161,9 +1173,10 @@ __global__ __launch_bounds__(T) void decode_xcd_kernel(const Params p) {
     c.tr = tr_lds;
     // The step's number has been read: workgroup 0 advances it only once every workgroup of this launch has said so.
     if (tid == 0) (void)__hip_atomic_fetch_add(p.state + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    // The hand-offs through an L2 need the workgroups b, b + 8, ... on one XCD, the one the plan's probe found them on:
-    // checked in every launch, not assumed.
-    if (tid == 0 && xcc_id() != p.state[8 + xcd]) atomicCAS(c.err, 0u, 0x2000u + (unsigned)xcd);
+    // The hand-offs through an L2 need the workgroups b, b + 8, ... of this launch on one XCD (which one may change from
+    // launch to launch): the first of them says where it runs, the others compare when they are done.
+    if (tid == 0 && in_xcd == 0)
+        __hip_atomic_store(p.state + 8 + xcd, ((c.epoch & 0x0fffffffu) << 4) | xcc_id(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     int pos = *p.pos_dev;
     pos = pos < 0 ? 0 : (pos > p.P - 1 ? p.P - 1 : pos);
     uint32_t tok = p.cur_tok[0];
@@ -1178,6 +1191,7 @@ __global__ __launch_bounds__(T) void decode_xcd_kernel(const Params p) {
     c.poth = (par ? -1L : 1L) * (long)p.parts_elems;
     if (in_xcd < NR) {
         relay_role<MODE>(p, tab, c, mirror, pos, tok, tid, in_xcd);
+        check_xcd(p, c, xcd, tid);
         PK_DUMP();
         return;
     }
@@ -1275,6 +1289,7 @@ __global__ __launch_bounds__(T) void decode_xcd_kernel(const Params p) {
 
     // ---- arg-max over the workgroups' candidates, token feed ----
     c.stage = p.n_stages;
+    check_xcd(p, c, xcd, tid);
     u64 *cand = reinterpret_cast<u64 *>(p.arena + p.cand_off);
     best = block_max48(best, L.scr, lane, wave);
     if (tid == 0) {
@@ -1585,8 +1600,8 @@ int32_t agpu_xk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
             e = hipFuncSetAttribute(reinterpret_cast<const void *>(decode_xcd_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e == hipSuccess) attr_set[ctx->device & 63] = true;
     }
-    // Where the workgroups land: b, b + 8, ... must share an XCD, and the eight classes must sit on eight different ones.
-    // state[8 + x] keeps the XCD of class x; every launch of the step checks itself against it.
+    // Where the workgroups land: b, b + 8, ... must share an XCD.  A launch shaped like the step's is looked at here;
+    // every launch of the step checks itself again (state[8 + x]: step number and XCD of class x).
     if (e == hipSuccess) {
         unsigned *probe = nullptr;
         std::vector<unsigned> where((size_t)r.G, 0u);
@@ -1599,19 +1614,12 @@ int32_t agpu_xk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
             (void)hipFree(probe);
         }
         if (e == hipSuccess) {
-            unsigned cls[8], seen = 0u;
             bool ok = true;
-            for (int x = 0; x < 8; ++x) {
-                cls[x] = where[(size_t)x];
-                ok = ok && cls[x] < 16u && !((seen >> cls[x]) & 1u);
-                seen |= 1u << (cls[x] & 15u);
-            }
-            for (int b = 0; b < r.G && ok; ++b) ok = where[(size_t)b] == cls[b & 7];
+            for (int b = 0; b < r.G && ok; ++b) ok = where[(size_t)b] == where[(size_t)(b & 7)];
             if (!ok) {
                 agpu_pk_plan_free(plan);
                 return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "decode step: workgroups b, b + 8, ... do not share an XCD on this device");
             }
-            e = hipMemcpy(plan->state + 8, cls, sizeof(cls), hipMemcpyHostToDevice);
         }
     }
     if (e != hipSuccess) {
