@@ -50,6 +50,8 @@ struct PkPlan {
     int lin_per_xcd = 0;  // kind 1: Linear workgroups per XCD
     int touch_dist = 0;   // kind 1: how many exchanges ahead the relays touch the weights (0: not at all)
     size_t parts_elems = 0;  // kind 1: floats of one set of partial sums
+    int head_tpc = 0;        // kind 1: tiles per chunk of the head stage
+    float *ln_fold = nullptr;  // kind 1: the LayerNorms folded into the Linears behind them (A_n, B_n per column)
 };
 
 // Whether the persistent step can run this model (int4 head, head_dim 64, group 32, size limits).

@@ -1608,6 +1608,7 @@ void agpu_pk_plan_free(PkPlan *plan) {
     if (plan->stages_dev) (void)hipFree(plan->stages_dev);
     if (plan->arena) (void)hipFree(plan->arena);
     if (plan->state) (void)hipFree(plan->state);
+    if (plan->ln_fold) (void)hipFree(plan->ln_fold);
     *plan = PkPlan{};
 }
 

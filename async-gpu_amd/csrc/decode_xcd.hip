@@ -105,7 +105,8 @@ struct Params {
     int att_per_xcd, smax, nlin;
     int spin_limit;
     int xbuf;             // floats of one staging buffer
-    int head_slots;       // slots of the head's second chunk kept in LDS ahead of the head stage (0: none)
+    int head_slots;       // how many of a workgroup's head slots (from its first) wait in LDS when the head stage begins
+    int red_floats;       // floats of one buffer of per-wave sums
     int touch_dist;       // exchanges between a relay's touch of a half layer's weights and their use (0: no touching)
     unsigned long long *trace;
 };
@@ -357,18 +358,25 @@ __device__ __forceinline__ float slot_dot_pre(const float *nf, const float *xs, 
 // Slot s of a chunk = (tile tt, round u), tile-major.  Round u of wave w covers groups (u W + w) gpw + j,
 // gpw = 4 >> tws groups per wave-wide load; lane (col, j) takes group j of the round for column col of the tile.
 template <int MODE>
-__device__ __forceinline__ void prefetch_lin(const Stage &st, Regs &r, int chunk, int rank, int wave, int lane) {
+__device__ __forceinline__ void prefetch_lin(const Stage &st, Regs &r, int chunk, int rank, int wave, int lane, const uint32_t *hl, int n_lds,
+                                             int tid) {
     if (MODE != 0) return;
     const int tw = 16 << st.tws, gpw = 4 >> st.tws;
     const int col = lane & (tw - 1), j = lane >> (4 + st.tws);
     int tt = 0, u = 0;
 #pragma unroll
     for (int s = 0; s < SL; ++s) {
-        const int tile = rank + (chunk * st.tpc + tt) * st.n_wgs;
+        const int ti = chunk * st.tpc + tt;  // which of the workgroup's tiles
+        const int tile = rank + ti * st.n_wgs;
         if (tt >= st.tpc || tile >= st.n_tiles) break;  // wave-uniform
-        r.w[s][0] = r.w[s][1] = r.w[s][2] = r.w[s][3] = 0u;
-        r.sc[s] = 0.0f;
-        {
+        const int gslot = ti * st.nl + u;  // which of the workgroup's head slots
+        if (gslot < n_lds) {  // workgroup-uniform: fetched into LDS while the layers ran
+#pragma unroll
+            for (int q = 0; q < 4; ++q) r.w[s][q] = hl[(size_t)(gslot * 5 + q) * T + tid];
+            r.sc[s] = __uint_as_float(hl[(size_t)(gslot * 5 + 4) * T + tid]);
+        } else {
+            r.w[s][0] = r.w[s][1] = r.w[s][2] = r.w[s][3] = 0u;
+            r.sc[s] = 0.0f;
             const int g = (u * W + wave) * gpw + j;
             const int n = tile * tw + col;
             if (g < st.n_groups && n < st.stride) {
@@ -507,11 +515,11 @@ __device__ __forceinline__ u64 block_max48(u64 w, uint32_t *scratch, int lane, i
 struct Lds {
     float *xs;       // [2][xbuf]: the staged input, stages in turn
     float *xsum;     // [2][XMAX / 32]: sum of every group of 32 inputs
-    float *red;      // [2][SL][W][64]: per-wave sums, chunks in turn; attention: per-wave partial results
-    float4 *stat;    // [W]: LayerNorm statistics per wave
+    float *red;      // [2][red_floats]: per-wave sums [tile][W][64], stages and chunks in turn; attention: per-wave partial results
+    float4 *stat;    // [2][W]: LayerNorm statistics per wave, stages in turn
     float *fin;      // attention: [PSTRIDE] + [SMAX][PSTRIDE]
     uint32_t *scr;   // [2 W]
-    uint32_t *hl;    // [head_slots][5][T]: the head's second chunk as the registers will hold it
+    uint32_t *hl;    // [head_slots][5][T]: the workgroup's first head slots as the registers will hold them
 };
 
 #ifdef AGPU_PK_TRACE
@@ -545,11 +553,8 @@ __device__ __forceinline__ void stage_input(const Params &p, const Stage &st, Ct
     const bool real = MODE == 0;
     const int n_quads = st.K >> 2;
     const bool have = tid < n_quads;
-    float4 lg = make_float4(1.0f, 1.0f, 1.0f, 1.0f), lb = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    if ((st.flags & F_LN) && real && have) {
-        lg = *reinterpret_cast<const float4 *>(st.ln_g + 4 * tid);
-        lb = *reinterpret_cast<const float4 *>(st.ln_b + 4 * tid);
-    }
+    float4 lg = make_float4(1.0f, 1.0f, 1.0f, 1.0f);
+    if ((st.flags & F_LN) && real && have) lg = *reinterpret_cast<const float4 *>(st.ln_g + 4 * tid);
     float4 x = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     if (st.in_off == -2) {
         if (have && real) {
@@ -565,11 +570,13 @@ __device__ __forceinline__ void stage_input(const Params &p, const Stage &st, Ct
         x = as_f4(v[0]);
     }
     settle();
-    asm volatile("" ::"v"(lg.x), "v"(lg.y), "v"(lg.z), "v"(lg.w), "v"(lb.x), "v"(lb.y), "v"(lb.z), "v"(lb.w));
+    asm volatile("" ::"v"(lg.x), "v"(lg.y), "v"(lg.z), "v"(lg.w));
     PK_STAMP(1);
     if (st.flags & F_LN) {  // workgroup-uniform
-        // Every wave takes the mean of its own elements and their squared distances from it (two passes over the
-        // registers, nn/cpu_ref.rs:38-47); the waves' (count, sum, mean, M2) are put together after one barrier.
+        // LayerNorm folded into the Linear: y = rstd (sum_k x_k g_k W_kn - mean A_n) + B_n with A_n = sum_k g_k W_kn and
+        // B_n = sum_k b_k W_kn + bias_n worked out when the plan was built.  So the input is staged as x g, and mean and
+        // rstd are only needed by the threads that finish a column: every wave leaves the (count, sum, mean, M2) of its
+        // own elements (two passes over the registers, nn/cpu_ref.rs:38-47) and nobody waits for them here.
         const int cnt = 4 * max(0, min(64, n_quads - wave * 64));  // wave-uniform
         const float sm = wave_sum((x.x + x.y) + (x.z + x.w));  // absent elements are zero
         const float mw = cnt > 0 ? sm * __builtin_amdgcn_rcpf((float)cnt) : 0.0f;
@@ -583,27 +590,10 @@ __device__ __forceinline__ void stage_input(const Params &p, const Stage &st, Ct
         }
         m2 = wave_sum(m2);
         if (lane == 0) stat[wave] = make_float4((float)cnt, sm, mw, m2);
-        __syncthreads();
-        float4 sw[W];
-#pragma unroll
-        for (int w8 = 0; w8 < W; ++w8) sw[w8] = stat[w8];
-        float tot = 0.0f;
-#pragma unroll
-        for (int w8 = 0; w8 < W; ++w8) tot += sw[w8].y;
-        const float mean = tot * st.inv_k;
-        float M2 = 0.0f;
-#pragma unroll
-        for (int w8 = 0; w8 < W; ++w8) {
-            const float dl = sw[w8].z - mean;
-            M2 += fmaf(sw[w8].x * dl, dl, sw[w8].w);
-        }
-        const float var = M2 * st.inv_k + p.eps;
-        float rstd = __builtin_amdgcn_rsqf(var);
-        rstd = rstd * fmaf(-0.5f * var * rstd, rstd, 1.5f);  // one Newton step: the hardware estimate is good to 1 ulp
-        x.x = (x.x - mean) * rstd * lg.x + lb.x;
-        x.y = (x.y - mean) * rstd * lg.y + lb.y;
-        x.z = (x.z - mean) * rstd * lg.z + lb.z;
-        x.w = (x.w - mean) * rstd * lg.w + lb.w;
+        x.x *= lg.x;
+        x.y *= lg.y;
+        x.z *= lg.z;
+        x.w *= lg.w;
     }
     // the vector and the sums of its groups (32 elements = 8 adjacent lanes) into LDS
     const float gs = oct_sum(have ? (x.x + x.y) + (x.z + x.w) : 0.0f);
@@ -613,6 +603,26 @@ __device__ __forceinline__ void stage_input(const Params &p, const Stage &st, Ct
     }
     __syncthreads();
     PK_STAMP(2);
+}
+
+// Mean and 1 / sqrt(variance + eps) of the staged vector out of the waves' statistics (after the staging barrier).
+__device__ __forceinline__ void ln_stats(const float4 *stat, float inv_k, float eps, float &mean, float &rstd) {
+    float4 sw[W];
+#pragma unroll
+    for (int w8 = 0; w8 < W; ++w8) sw[w8] = stat[w8];
+    float tot = 0.0f;
+#pragma unroll
+    for (int w8 = 0; w8 < W; ++w8) tot += sw[w8].y;
+    mean = tot * inv_k;
+    float M2 = 0.0f;
+#pragma unroll
+    for (int w8 = 0; w8 < W; ++w8) {
+        const float dl = sw[w8].z - mean;
+        M2 += fmaf(sw[w8].x * dl, dl, sw[w8].w);
+    }
+    const float var = M2 * inv_k + eps;
+    rstd = __builtin_amdgcn_rsqf(var);
+    rstd = rstd * fmaf(-0.5f * var * rstd, rstd, 1.5f);  // one Newton step: the hardware estimate is good to 1 ulp
 }
 
 // ---- one Linear of a layer, for a workgroup that has a unit of it ----
@@ -633,8 +643,9 @@ __device__ __forceinline__ void lay_stage(const Params &p, const Stage &st, Ctl 
     const int lc = ((unit_f - part_f * st.upp) << tsh) + colf;
     const int n = st.col0 + part_f * st.part_stride + lc;
     const bool fin = kf < (W >> st.wps) && unit_f < st.n_units && lc < st.pcols;
-    float bias = 0.0f;
+    float bias = 0.0f, fold_a = 0.0f;  // with a LayerNorm: B_n (the bias is in it) and A_n
     if (fin && st.bias && real) bias = st.bias[n];
+    if (fin && (st.flags & F_LN) && real) fold_a = st.xbias[n];
     PK_STAMP(0);
     // the first slots' nibbles become floats before the input is awaited
     float pre[NPRE * 32];
@@ -651,7 +662,7 @@ __device__ __forceinline__ void lay_stage(const Params &p, const Stage &st, Ctl 
             }
         }
     }
-    stage_input<MODE>(p, st, c, xs, xsum, stat, mirror, pos, tok, tid, [&] { asm volatile("" ::"v"(bias)); });
+    stage_input<MODE>(p, st, c, xs, xsum, stat, mirror, pos, tok, tid, [&] { asm volatile("" ::"v"(bias), "v"(fold_a)); });
     if (real) {
         const float part = lay_compute(st, r, pre, xs, xsum, wave, lane);
         if (lane < tw) red[wave * 64 + lane] = part;
@@ -667,6 +678,11 @@ __device__ __forceinline__ void lay_stage(const Params &p, const Stage &st, Ctl 
             for (int w8 = 0; w8 < W; ++w8) rv[w8] = red[((kf << st.wps) + min(w8, wpt - 1)) * 64 + colf];
 #pragma unroll
             for (int w8 = 0; w8 < W; ++w8) v += w8 < wpt ? rv[w8] : 0.0f;
+            if (st.flags & F_LN) {
+                float mean, rstd;
+                ln_stats(stat, st.inv_k, p.eps, mean, rstd);
+                v = rstd * fmaf(-mean, fold_a, v);
+            }
             v += bias;
             if (st.flags & F_GELU_TANH) v = gelu_tanh_dev(v);
             else if (st.flags & F_GELU_QUICK) v = gelu_quick_dev(v);
@@ -684,23 +700,30 @@ __device__ __forceinline__ void lay_stage(const Params &p, const Stage &st, Ctl 
 }
 
 // ---- the head ----
-template <int MODE>
-__device__ __forceinline__ void head_finish(const Params &p, const Stage &st, const float *red, int rank, int ch, int tiles, int tid, u64 &best) {
-    if (MODE != 0) return;
+// A workgroup's head columns of chunk ch: thread o < 64 tiles has column col of tile tt (a chunk has 8 tiles at most).
+__device__ __forceinline__ int head_column(const Stage &st, int rank, int ch, int tiles, int tid) {
     const int tw_shift = st.tws + 4;
-    for (int o = tid; o < (tiles << tw_shift); o += T) {
-        const int tt = o >> tw_shift, col = o & ((1 << tw_shift) - 1);
-        const int n = ((rank + (ch * st.tpc + tt) * st.n_wgs) << tw_shift) + col;
-        if (n >= st.n_valid) continue;
-        float v = 0.0f;
+    if (tid >= (tiles << tw_shift)) return -1;
+    const int tt = tid >> tw_shift, col = tid & ((1 << tw_shift) - 1);
+    const int n = ((rank + (ch * st.tpc + tt) * st.n_wgs) << tw_shift) + col;
+    return n < st.n_valid ? n : -1;
+}
+// Outputs of chunk ch: waves summed in order, the LayerNorm fold (fold_a = A_n, fold_b = B_n of column n, requested
+// ahead), the logit and the arg-max candidate.
+template <int MODE>
+__device__ __forceinline__ void head_finish(const Params &p, const Stage &st, const float *red, int n, float mean, float rstd, float fold_a,
+                                            float fold_b, int tid, u64 &best) {
+    if (MODE != 0 || n < 0) return;
+    const int tw_shift = st.tws + 4;
+    const int tt = tid >> tw_shift, col = tid & ((1 << tw_shift) - 1);
+    float v = 0.0f;
 #pragma unroll
-        for (int w8 = 0; w8 < W; ++w8) v += red[(tt * W + w8) * 64 + col];
-        if (st.bias) v += st.bias[n];
-        p.logits[n] = v;
-        const uint32_t code = p.argmax_last ? (uint32_t)n : 0xFFFFu - (uint32_t)n;
-        const u64 cand = ((u64)order_key(v) << 16) | code;
-        if (order_key(v) != 0u) best = cand > best ? cand : best;
-    }
+    for (int w8 = 0; w8 < W; ++w8) v += red[(tt * W + w8) * 64 + col];
+    v = rstd * fmaf(-mean, fold_a, v) + fold_b;
+    p.logits[n] = v;
+    const uint32_t code = p.argmax_last ? (uint32_t)n : 0xFFFFu - (uint32_t)n;
+    const u64 cand = ((u64)order_key(v) << 16) | code;
+    if (order_key(v) != 0u) best = cand > best ? cand : best;
 }
 
 // ---- relay ----
@@ -874,7 +897,7 @@ __device__ __forceinline__ void attn_role(const Params &p, CStage tab, Ctl &c, c
     const float ninf = -__builtin_inff();
     const float scale = 0.125f;  // 1 / sqrt(64)
     float *part = L.red;               // [W][64]
-    float *wm = L.red + W * 4 * DH;    // [W]
+    float *wm = L.red + W * DH;        // [W]
     float *wl = wm + W;                // [W]
     float *own = L.fin;                // [PSTRIDE]: o[64], m, l of this workgroup
     float *oth = L.fin + PSTRIDE;      // [S - 1][PSTRIDE]
@@ -1066,10 +1089,13 @@ __device__ __forceinline__ void attn_role(const Params &p, CStage tab, Ctl &c, c
     }
 }
 
-// ---- the head's second chunk, fetched into LDS while the layers run ----
+// ---- the head's weights, fetched into LDS while the layers run ----
+// The head's weights depend on nothing and memory idles during the layers, so a workgroup's head slots, as many as LDS
+// has room for (all of them for the smaller models), are fetched one per stage the workgroup has just published: a slot's
+// five words are requested, the slot before it is written to LDS.  Every thread writes and later reads its own words.
 struct HeadAhead {
-    int n_slots;  // slots of chunk 1 this workgroup has (0: nothing to do)
-    int s, tt, u; // next slot to request, as (tile of the chunk, round)
+    int n_slots;  // slots to fetch (0: nothing to do)
+    int s;        // next slot to request
     int pending;  // slot whose words are in v, -1: none
     uint32_t v[5];
 };
@@ -1080,14 +1106,15 @@ __device__ __forceinline__ void head_ahead_step(CStage th, HeadAhead &ha, uint32
         ha.pending = -1;
     }
     if (ha.s >= ha.n_slots) return;  // workgroup-uniform
-    const int tws = th->tws, nl = th->nl, tpc = th->tpc, n_wgs = th->n_wgs;
+    const int tws = th->tws, nl = th->nl, n_wgs = th->n_wgs;
     const int n_groups = th->n_groups, stride = th->stride;
     const uint32_t *packed = glob(th->packed);
     const float *scales = glob(th->scales);
     const int tw = 16 << tws, gpw = 4 >> tws;
     const int col = lane & (tw - 1), j = lane >> (4 + tws);
-    const int tile = rank + (tpc + ha.tt) * n_wgs;  // chunk 1
-    const int g = (ha.u * W + wave) * gpw + j, n = tile * tw + col;
+    const int ti = ha.s / nl, u = ha.s - ti * nl;
+    const int tile = rank + ti * n_wgs;
+    const int g = (u * W + wave) * gpw + j, n = tile * tw + col;
 #pragma unroll
     for (int q = 0; q < 5; ++q) ha.v[q] = 0u;
     if (g < n_groups && n < stride) {
@@ -1100,10 +1127,6 @@ __device__ __forceinline__ void head_ahead_step(CStage th, HeadAhead &ha, uint32
     }
     ha.pending = ha.s;
     ++ha.s;
-    if (++ha.u == nl) {
-        ha.u = 0;
-        ++ha.tt;
-    }
 }
 
 // First stage from `from` on, before the head, in which Linear workgroup li of its XCD has a unit; the head (n_lay) if none.
@@ -1120,6 +1143,26 @@ __device__ __forceinline__ int next_active(CStage tab, int from, int li, int n_l
 __device__ __forceinline__ void head_share(const Stage &st, int rank, int &my_tiles, int &n_chunks) {
     my_tiles = rank < st.n_tiles ? (st.n_tiles - rank + st.n_wgs - 1) / st.n_wgs : 0;
     n_chunks = (my_tiles + st.tpc - 1) / st.tpc;
+}
+
+// When the plan is built: A_n = sum_k g_k W_kn and B_n = sum_k b_k W_kn + bias_n for the columns of an int4 Linear that
+// follows a LayerNorm with gains g and offsets b (W_kn = (nibble - 8) scale, nn/ops/quantize.rs:158-162), in double.
+__global__ void ln_fold_kernel(const uint32_t *packed, const float *scales, int stride, int K, int N, const float *g, const float *b,
+                               const float *bias, float *A, float *B) {
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= N) return;
+    double a = 0.0, o = 0.0;
+    for (int kp = 0; kp < K / 8; ++kp) {
+        const uint32_t w = packed[(size_t)kp * stride + n];
+        const double sc = (double)scales[(size_t)(kp >> 2) * stride + n];
+        for (int i = 0; i < 8; ++i) {
+            const double q = (double)((int)((w >> (4 * i)) & 15u) - 8) * sc;
+            a += (double)g[8 * kp + i] * q;
+            o += (double)b[8 * kp + i] * q;
+        }
+    }
+    A[n] = (float)a;
+    B[n] = (float)(o + (bias ? (double)bias[n] : 0.0));
 }
 
 // The XCD this wave runs on (XCC_ID, bits 3:0 of hardware register 20).
@@ -1155,8 +1198,8 @@ __global__ __launch_bounds__(T) void decode_xcd_kernel(const Params p) {
     L.xs = smem;
     L.xsum = L.xs + 2 * p.xbuf;
     L.red = L.xsum + 2 * (XMAX / 32);
-    L.stat = reinterpret_cast<float4 *>(L.red + 2 * SL * W * 64);
-    L.fin = L.red + 2 * SL * W * 64 + 4 * W;
+    L.stat = reinterpret_cast<float4 *>(L.red + 2 * p.red_floats);
+    L.fin = L.red + 2 * p.red_floats + 8 * W;
     L.scr = reinterpret_cast<uint32_t *>(L.fin + (SMAX + 1) * PSTRIDE);
     L.hl = L.scr + 2 * W;
     u64 *tr_lds = reinterpret_cast<u64 *>(L.hl + (size_t)p.head_slots * 5 * T);
@@ -1225,18 +1268,18 @@ __global__ __launch_bounds__(T) void decode_xcd_kernel(const Params p) {
     Stage st = load_stage(tab + s);
     if (s < n_lay) lay_prefetch<MODE>(st, regs, li, wave, lane);
     HeadAhead ha;
-    ha.n_slots = ha.s = ha.tt = ha.u = 0;
+    ha.n_slots = ha.s = 0;
     ha.pending = -1;
     if (MODE == 0 && p.head_slots > 0 && !is_att) {
         CStage th = tab + n_lay;
-        const int n_tiles = th->n_tiles, n_wgs = th->n_wgs, tpc = th->tpc;
+        const int n_tiles = th->n_tiles, n_wgs = th->n_wgs;
         const int my_tiles = rank < n_tiles ? (n_tiles - rank + n_wgs - 1) / n_wgs : 0;
-        ha.n_slots = min(p.head_slots, min(tpc, max(0, my_tiles - tpc)) * th->nl);
+        ha.n_slots = min(p.head_slots, my_tiles * th->nl);
     }
     while (s < n_lay) {
         c.stage = s;
-        lay_stage<MODE>(p, st, c, regs, L.xs + (n_enter & 1) * p.xbuf, L.xsum + (n_enter & 1) * (XMAX / 32), L.stat,
-                        L.red + (n_enter & 1) * (SL * W * 64), mirror, pos, tok, li, tid);
+        lay_stage<MODE>(p, st, c, regs, L.xs + (n_enter & 1) * p.xbuf, L.xsum + (n_enter & 1) * (XMAX / 32), L.stat + (n_enter & 1) * W,
+                        L.red + (n_enter & 1) * p.red_floats, mirror, pos, tok, li, tid);
         // the outputs are on their way: now the next stage this workgroup takes part in, and its weights
         ++n_enter;
         s = next_active(tab, s + 1, li, n_lay);
@@ -1252,34 +1295,45 @@ __global__ __launch_bounds__(T) void decode_xcd_kernel(const Params p) {
     {
         int my_tiles, n_chunks;
         head_share(st, rank, my_tiles, n_chunks);
-        prefetch_lin<MODE>(st, regs, 0, rank, wave, lane);
+        // what the layers left no occasion to fetch goes to LDS now; then the first chunk into the registers
         if (MODE == 0)
             while (ha.pending >= 0 || ha.s < ha.n_slots) head_ahead_step(tab + n_lay, ha, L.hl, rank, wave, lane, tid);
+        prefetch_lin<MODE>(st, regs, 0, rank, wave, lane, L.hl, ha.n_slots, tid);
         float *xs = L.xs + (n_enter & 1) * p.xbuf, *xsum = L.xsum + (n_enter & 1) * (XMAX / 32);
         if (my_tiles > 0) {  // workgroup-uniform
             PK_STAMP(0);
-            stage_input<MODE>(p, st, c, xs, xsum, L.stat, mirror, pos, tok, tid, [] {});
+            float4 *stat = L.stat + (n_enter & 1) * W;
+            // this thread's column of the first chunk, and its LayerNorm fold
+            int n_col = head_column(st, rank, 0, min(st.tpc, my_tiles), tid);
+            float fold_a = 0.0f, fold_b = 0.0f;
+            if (MODE == 0 && n_col >= 0) {
+                fold_a = st.xbias[n_col];
+                fold_b = st.bias[n_col];
+            }
+            stage_input<MODE>(p, st, c, xs, xsum, stat, mirror, pos, tok, tid, [&] { asm volatile("" ::"v"(fold_a), "v"(fold_b)); });
+            float mean, rstd;
+            ln_stats(stat, st.inv_k, p.eps, mean, rstd);
             for (int ch = 0; ch < n_chunks; ++ch) {
                 const int tiles = min(st.tpc, my_tiles - ch * st.tpc);
-                float *red = L.red + (ch & 1) * (SL * W * 64);
+                float *red = L.red + (ch & 1) * p.red_floats;
                 if (MODE == 0) compute_chunk(st, regs, xs, xsum, red, tiles, wave, lane);
                 if (ch == 0) PK_STAMP(4);
                 if (ch == 1) PK_STAMP(6);
+                int n_next = -1;
+                float a_next = 0.0f, b_next = 0.0f;
                 if (ch + 1 < n_chunks) {
-                    if (ch == 0 && ha.n_slots > 0 && MODE == 0) {
-#pragma unroll
-                        for (int sl = 0; sl < SL; ++sl) {
-                            if (sl >= ha.n_slots) break;  // workgroup-uniform
-#pragma unroll
-                            for (int q = 0; q < 4; ++q) regs.w[sl][q] = L.hl[(size_t)(sl * 5 + q) * T + tid];
-                            regs.sc[sl] = __uint_as_float(L.hl[(size_t)(sl * 5 + 4) * T + tid]);
-                        }
-                    } else {
-                        prefetch_lin<MODE>(st, regs, ch + 1, rank, wave, lane);
+                    prefetch_lin<MODE>(st, regs, ch + 1, rank, wave, lane, L.hl, ha.n_slots, tid);
+                    n_next = head_column(st, rank, ch + 1, min(st.tpc, my_tiles - (ch + 1) * st.tpc), tid);
+                    if (MODE == 0 && n_next >= 0) {
+                        a_next = st.xbias[n_next];
+                        b_next = st.bias[n_next];
                     }
                 }
                 __syncthreads();
-                head_finish<MODE>(p, st, L.red + (ch & 1) * (SL * W * 64), rank, ch, tiles, tid, best);
+                head_finish<MODE>(p, st, L.red + (ch & 1) * p.red_floats, n_col, mean, rstd, fold_a, fold_b, tid, best);
+                n_col = n_next;
+                fold_a = a_next;
+                fold_b = b_next;
                 if (ch == 0) PK_STAMP(5);
                 if (ch == 1) PK_STAMP(7);
             }
@@ -1401,9 +1455,14 @@ bool plan_head(Stage &s, const PkLinear &l, int n_wgs) {
 
 int xbuf_floats(int kmax) { return kmax / 32 * GS; }
 
-size_t lds_bytes_for(int n_stages, int kmax, int head_slots) {
+size_t fold_floats(const PkModel &m) { return 2 * ((size_t)3 * m.d + m.ff) * m.n_layer + 2 * (size_t)m.head.N; }
+
+// floats of one buffer of per-wave sums: a layer stage needs [W][64], a chunk of the head [tiles per chunk][W][64]
+int red_floats_for(int head_tpc) { return std::max(1, head_tpc) * W * 64; }
+
+size_t lds_bytes_for(int n_stages, int kmax, int head_slots, int head_tpc) {
     (void)n_stages;
-    size_t b = (size_t)(2 * xbuf_floats(kmax) + 2 * (XMAX / 32) + 2 * SL * W * 64 + 4 * W + (SMAX + 1) * PSTRIDE + 2 * W) * 4 +
+    size_t b = (size_t)(2 * xbuf_floats(kmax) + 2 * (XMAX / 32) + 2 * red_floats_for(head_tpc) + 8 * W + (SMAX + 1) * PSTRIDE + 2 * W) * 4 +
                (size_t)head_slots * 5 * T * 4;
 #ifdef AGPU_PK_TRACE
     b += (size_t)n_stages * 8 * sizeof(u64);
@@ -1419,7 +1478,9 @@ void xcd_share(int total, int x, int &first, int &count) {
 }
 
 // The stage table of all eight XCDs, [8][4 n_layer + 1]; false when a stage does not fit.
-bool build_tables(const PkModel &m, const Roles &r, int lin_groups, size_t part_base, std::vector<Stage> &out, int *kmax_out) {
+bool build_tables(const PkModel &m, const Roles &r, int lin_groups, size_t part_base, float *fold, std::vector<Stage> &out, int *kmax_out) {
+    // fold: A and B of every Linear behind a LayerNorm (fold_floats(m) floats), per layer [A qkv][B qkv][A fc][B fc], then the head's
+    const size_t fold_layer = 2 * ((size_t)3 * m.d + m.ff);
     // Linear workgroups of an XCD in lin_groups groups (1, 2 or 4); stage kind k of a layer goes to group k % lin_groups
     int g_first[4], g_size[4];
     for (int k = 0; k < 4; ++k) {
@@ -1445,7 +1506,8 @@ bool build_tables(const PkModel &m, const Roles &r, int lin_groups, size_t part_
             // LN1 + QKV, the columns of this XCD's heads
             {
                 Stage s{};
-                s.packed = y.qkv.packed; s.scales = y.qkv.scales; s.bias = y.qkv.bias; s.ln_g = y.ln1_g; s.ln_b = y.ln1_b;
+                s.packed = y.qkv.packed; s.scales = y.qkv.scales; s.ln_g = y.ln1_g; s.ln_b = y.ln1_b;
+                s.xbias = fold + fold_layer * L; s.bias = s.xbias + 3 * d;  // A and B
                 s.kc = y.kcache; s.vc = y.vcache;
                 s.K = d; s.n_groups = d / 32; s.stride = y.qkv.stride; s.inv_k = 1.0f / (float)d;
                 s.col0 = h0 * DH; s.part_stride = d; s.pcols = nh * DH; s.n_cparts = 3;
@@ -1473,7 +1535,8 @@ bool build_tables(const PkModel &m, const Roles &r, int lin_groups, size_t part_
             // LN2 + fc + GELU, this XCD's columns
             {
                 Stage s{};
-                s.packed = y.fc.packed; s.scales = y.fc.scales; s.bias = y.fc.bias; s.ln_g = y.ln2_g; s.ln_b = y.ln2_b;
+                s.packed = y.fc.packed; s.scales = y.fc.scales; s.ln_g = y.ln2_g; s.ln_b = y.ln2_b;
+                s.xbias = fold + fold_layer * L + 6 * d; s.bias = s.xbias + ff;  // A and B
                 s.K = d; s.n_groups = d / 32; s.stride = y.fc.stride; s.inv_k = 1.0f / (float)d;
                 s.col0 = g0 * 32; s.part_stride = 0; s.pcols = ng * 32; s.n_cparts = 1;
                 s.in_off = o_h1; s.out_off = o_ffn;
@@ -1502,6 +1565,7 @@ bool build_tables(const PkModel &m, const Roles &r, int lin_groups, size_t part_
         Stage hs;
         if (!plan_head(hs, m.head, r.G - 8 * NR)) return false;
         hs.in_off = prev_h2; hs.flags = F_LN | F_HEAD; hs.ln_g = m.lnf_g; hs.ln_b = m.lnf_b;
+        hs.xbias = fold + fold_layer * m.n_layer; hs.bias = hs.xbias + m.head.N;  // A and B
         out[(size_t)x * n_st + 4 * m.n_layer] = hs;
     }
     if (kmax_out) *kmax_out = kmax;
@@ -1528,8 +1592,8 @@ bool agpu_xk_supported(const agpu_ctx *ctx, const PkModel &m) {
     if (!m.lnf_g || !m.lnf_b || !m.wte || !m.wpe) return false;
     std::vector<Stage> tab;
     int kmax = 0;
-    if (!build_tables(m, r, 1, 0, tab, &kmax)) return false;
-    if (lds_bytes_for(4 * m.n_layer + 1, kmax, 0) > (size_t)160 * 1024) return false;
+    if (!build_tables(m, r, 1, 0, nullptr, tab, &kmax)) return false;
+    if (lds_bytes_for(4 * m.n_layer + 1, kmax, 0, SL) > (size_t)160 * 1024) return false;
     return true;
 }
 
@@ -1546,14 +1610,35 @@ int32_t agpu_xk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
     const size_t cand_off = part_base + 2 * parts_elems;
     const size_t total = cand_off + 2 * (size_t)r.G + 2;
     if (total > (size_t)0x7fffffff) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "decode step: activation arena too large");
+    // LayerNorm folded into the Linears behind it: their A and B
+    hipError_t e = hipMalloc((void **)&plan->ln_fold, fold_floats(m) * sizeof(float));
+    if (e != hipSuccess) return agpu_hip(ctx, e, "decode step: plan");
     std::vector<Stage> st;
     int kmax = d;
     // two groups of Linear workgroups taking the stages in turn where every stage then still fits, else one
     int lin_groups = 2;
     if (const char *env = getenv("AGPU_XK_GROUPS")) lin_groups = atoi(env) == 4 ? 4 : (atoi(env) == 1 ? 1 : 2);
-    while (lin_groups > 1 && !build_tables(m, r, lin_groups, part_base, st, &kmax)) lin_groups /= 2;
-    if (lin_groups == 1 && !build_tables(m, r, 1, part_base, st, &kmax))
+    while (lin_groups > 1 && !build_tables(m, r, lin_groups, part_base, plan->ln_fold, st, &kmax)) lin_groups /= 2;
+    if (lin_groups == 1 && !build_tables(m, r, 1, part_base, plan->ln_fold, st, &kmax)) {
+        agpu_pk_plan_free(plan);
         return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "decode step: a stage does not fit");
+    }
+    {
+        const size_t fold_layer = 2 * ((size_t)3 * d + ff);
+        auto fold = [&](const PkLinear &l, const float *g, const float *b, float *A, float *B) {
+            hipLaunchKernelGGL(ln_fold_kernel, dim3(ceil_div(l.N, 256)), dim3(256), 0, ctx->stream, l.packed, l.scales, l.stride, l.K, l.N, g, b,
+                               l.bias, A, B);
+        };
+        for (int L = 0; L < m.n_layer; ++L) {
+            const PkLayer &y = m.layers[L];
+            float *base = plan->ln_fold + fold_layer * L;
+            fold(y.qkv, y.ln1_g, y.ln1_b, base, base + 3 * d);
+            fold(y.fc, y.ln2_g, y.ln2_b, base + 6 * d, base + 6 * d + ff);
+        }
+        float *hb = plan->ln_fold + fold_layer * m.n_layer;
+        fold(m.head, m.lnf_g, m.lnf_b, hb, hb + m.head.N);
+        e = hipGetLastError();
+    }
     plan->kind = 1;
     plan->n_stages = 4 * m.n_layer + 1;
     plan->grid = r.G;
@@ -1564,7 +1649,7 @@ int32_t agpu_xk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
     plan->arena_elems = mirror_elems;
     plan->parts_elems = parts_elems;
     const size_t arena_bytes = total * sizeof(float);
-    hipError_t e = hipMalloc(&plan->stages_dev, st.size() * sizeof(Stage));
+    if (e == hipSuccess) e = hipMalloc(&plan->stages_dev, st.size() * sizeof(Stage));
     if (e == hipSuccess) e = hipMalloc((void **)&plan->arena, arena_bytes);
     if (e == hipSuccess) e = hipMalloc((void **)&plan->state, 64);
     if (e == hipSuccess) e = hipMemcpy(plan->stages_dev, st.data(), st.size() * sizeof(Stage), hipMemcpyHostToDevice);
@@ -1576,20 +1661,25 @@ int32_t agpu_xk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
     if (e == hipSuccess) e = hipMemsetAsync(plan->state, 0, 64, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e == hipSuccess) e = hipDeviceSynchronize();
-    {
-        const Stage &hs = st.back();
-        const int tiles_max = ceil_div(hs.n_tiles, hs.n_wgs);
-        const int want = std::min(SL, std::min(hs.tpc, std::max(0, tiles_max - hs.tpc)) * hs.nl);
-        plan->head_slots = want > 0 && lds_bytes_for(plan->n_stages, kmax, want) <= (size_t)160 * 1024 ? want : 0;
-    }
     plan->kmax = kmax;
-    // one workgroup per CU: the request is sized so that two never share a CU
-    plan->lds_bytes = std::max(lds_bytes_for(plan->n_stages, plan->kmax, plan->head_slots), (size_t)96 * 1024);
-    // An XCD's share of a layer's weights is touched two exchanges (one layer) before its use where two layers' shares
-    // leave room in the 4 MiB L2, else one exchange ahead.
     {
-        const double share = ((double)3 * d * d + (double)d * d + 2.0 * d * ff) * 0.625 / 8.0;
-        plan->touch_dist = share <= 1.0e6 ? 2 : 1;
+        // as many of a workgroup's head slots in LDS as there is room for
+        const Stage &hs = st.back();
+        const int slots_max = ceil_div(hs.n_tiles, hs.n_wgs) * hs.nl;
+        plan->head_tpc = hs.tpc;
+        int fit = slots_max;
+        while (fit > 0 && lds_bytes_for(plan->n_stages, kmax, fit, hs.tpc) > (size_t)160 * 1024) --fit;
+        if (const char *env = getenv("AGPU_XK_HEAD_SLOTS")) fit = std::min(fit, atoi(env));
+        plan->head_slots = fit;
+    }
+    // one workgroup per CU: the request is sized so that two never share a CU
+    plan->lds_bytes = std::max(lds_bytes_for(plan->n_stages, plan->kmax, plan->head_slots, plan->head_tpc), (size_t)96 * 1024);
+    // The relays touch an XCD's share of a half layer's weights one exchange before its use, so that the Linear
+    // workgroups' requests are served from the L2, where the model does not stay in the 256 MiB Infinity Cache between
+    // steps anyway; a smaller model is only slowed down by it.
+    {
+        const double bytes = (((double)3 * d * d + (double)d * d + 2.0 * d * ff) * m.n_layer + (double)d * m.head.N) * 0.625;
+        plan->touch_dist = bytes > 200.0e6 ? 1 : 0;
         if (const char *env = getenv("AGPU_XK_TOUCH")) plan->touch_dist = atoi(env);
     }
     // the largest request any plan can make, once per device: the attribute belongs to the kernel, not to a plan
@@ -1649,6 +1739,7 @@ int32_t agpu_xk_launch(agpu_ctx *ctx, const PkModel &m, const PkPlan &plan, int 
     p.spin_limit = plan.spin_limit > 0 ? plan.spin_limit : kSpinLimit;
     p.xbuf = xbuf_floats(plan.kmax);
     p.head_slots = plan.head_slots;
+    p.red_floats = red_floats_for(plan.head_tpc);
     p.touch_dist = plan.touch_dist;
     p.trace = trace;
     if (mode == 0) hipLaunchKernelGGL(decode_xcd_kernel<0>, dim3(plan.grid), dim3(T), plan.lds_bytes, ctx->stream, p);

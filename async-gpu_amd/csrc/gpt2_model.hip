@@ -844,6 +844,9 @@ AGPU_EXPORT int32_t agpu_gpt2_set_embeddings(agpu_gpt2 *m, const float *wte, con
     if (!m) return AGPU_ERR_NULL_POINTER;
     agpu_ctx *ctx = m->ctx;
     AGPU_REQUIRE_CTX(ctx);
+    // the plan of the one-launch step holds sums over the final LayerNorm's gains and offsets
+    (void)hipStreamSynchronize(ctx->stream);
+    drop_graphs(m);
     int32_t rc = set_vec(ctx, &m->wte, wte, (size_t)m->V * m->d, on_device);
     if (rc == AGPU_OK) rc = set_vec(ctx, &m->wpe, wpe, (size_t)m->P * m->d, on_device);
     if (rc == AGPU_OK) rc = set_vec(ctx, &m->lnf_g, lnf_g, m->d, on_device);
@@ -866,6 +869,9 @@ AGPU_EXPORT int32_t agpu_gpt2_set_layer_norms(agpu_gpt2 *m, int32_t layer, const
     if (layer < 0 || layer >= m->cfg.n_layer)
         return agpu_fail(m->ctx, AGPU_ERR_DIM_OUT_OF_RANGE, "gpt2: layer %d out of range for %d layers", layer, m->cfg.n_layer);
     Block &b = m->blocks[layer];
+    // the plan of the one-launch step holds sums over the gains and offsets
+    (void)hipStreamSynchronize(m->ctx->stream);
+    drop_graphs(m);
     int32_t rc = set_vec(m->ctx, &b.ln1_g, ln1_g, m->d, on_device);
     if (rc == AGPU_OK) rc = set_vec(m->ctx, &b.ln1_b, ln1_b, m->d, on_device);
     if (rc == AGPU_OK) rc = set_vec(m->ctx, &b.ln2_g, ln2_g, m->d, on_device);
