@@ -109,6 +109,7 @@ SIGNATURES = {
     "agpu_gpt2_decode_steps": (_i32, [_vp, _i32, _i32, _vp]),
     "agpu_gpt2_set_decode_mode": (_i32, [_vp, _i32]),
     "agpu_gpt2_decode_is_one_launch": (_i32, [_vp]),
+    "agpu_gpt2_decode_stats": (_i32, [_vp, _vp]),
     "agpu_gpt2_set_decode_wait_limit": (_i32, [_vp, _i32]),
     "agpu_gpt2_decode_floor": (_i32, [_vp, _i32, _vp]),
     "agpu_gpt2_last_logits": (_i32, [_vp, _i32, _vp]),

@@ -36,7 +36,7 @@
 // published; the relays touch the XCD's share of the weights a half layer or more ahead, so that these requests are
 // served from the L2.  Every wait is bounded: a poll that does not succeed within the limit sets the error word, all
 // workgroups then stop waiting, and the step ends with garbage that the host reports as an error.
-#include "decode_persistent.h"
+#include "decode_step.h"
 
 #include <algorithm>
 #include <vector>
@@ -1574,7 +1574,7 @@ bool build_tables(const PkModel &m, const Roles &r, int lin_groups, size_t part_
 
 }  // namespace
 
-bool agpu_xk_supported(const agpu_ctx *ctx, const PkModel &m) {
+bool agpu_step_supported(const agpu_ctx *ctx, const PkModel &m) {
     const Roles r = plan_roles(ctx, m.H);
     // eight XCDs of 32 CUs: the roles and the hand-offs through an L2 are laid out for this part
     if (ctx->num_cus != 256 || r.nlin < 8 || m.H < 1 || r.G - 8 * NR > T) return false;
@@ -1597,9 +1597,9 @@ bool agpu_xk_supported(const agpu_ctx *ctx, const PkModel &m) {
     return true;
 }
 
-int32_t agpu_xk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
-    agpu_pk_plan_free(plan);
-    if (!agpu_xk_supported(ctx, m)) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "decode step: model shape not supported by the one-launch step");
+int32_t agpu_step_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
+    agpu_step_plan_free(plan);
+    if (!agpu_step_supported(ctx, m)) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "decode step: model shape not supported by the one-launch step");
     const Roles r = plan_roles(ctx, m.H);
     const int d = m.d, ff = m.ff;
     const size_t per_layer = (size_t)3 * d + d + d + ff + d + (size_t)m.H * SMAX * PSTRIDE;
@@ -1620,7 +1620,7 @@ int32_t agpu_xk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
     if (const char *env = getenv("AGPU_XK_GROUPS")) lin_groups = atoi(env) == 4 ? 4 : (atoi(env) == 1 ? 1 : 2);
     while (lin_groups > 1 && !build_tables(m, r, lin_groups, part_base, plan->ln_fold, st, &kmax)) lin_groups /= 2;
     if (lin_groups == 1 && !build_tables(m, r, 1, part_base, plan->ln_fold, st, &kmax)) {
-        agpu_pk_plan_free(plan);
+        agpu_step_plan_free(plan);
         return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "decode step: a stage does not fit");
     }
     {
@@ -1639,7 +1639,6 @@ int32_t agpu_xk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
         fold(m.head, m.lnf_g, m.lnf_b, hb, hb + m.head.N);
         e = hipGetLastError();
     }
-    plan->kind = 1;
     plan->n_stages = 4 * m.n_layer + 1;
     plan->grid = r.G;
     plan->att_per_xcd = r.att_per_xcd;
@@ -1653,14 +1652,8 @@ int32_t agpu_xk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
     if (e == hipSuccess) e = hipMalloc((void **)&plan->arena, arena_bytes);
     if (e == hipSuccess) e = hipMalloc((void **)&plan->state, 64);
     if (e == hipSuccess) e = hipMemcpy(plan->stages_dev, st.data(), st.size() * sizeof(Stage), hipMemcpyHostToDevice);
-    // every place "not written yet" (all-ones words); the candidates zero
-    // (on the stream the step runs on, and waited for: a fill still under way when the first step starts would leave
-    // words that are neither all-ones nor a value of the step)
-    if (e == hipSuccess) e = hipMemsetAsync(plan->arena, 0xFF, cand_off * sizeof(float), ctx->stream);
-    if (e == hipSuccess) e = hipMemsetAsync(reinterpret_cast<float *>(plan->arena) + cand_off, 0, (total - cand_off) * sizeof(float), ctx->stream);
     if (e == hipSuccess) e = hipMemsetAsync(plan->state, 0, 64, ctx->stream);
-    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
-    if (e == hipSuccess) e = hipDeviceSynchronize();
+    if (e == hipSuccess && agpu_step_reset(ctx, *plan) != AGPU_OK) e = hipErrorUnknown;
     plan->kmax = kmax;
     {
         // as many of a workgroup's head slots in LDS as there is room for
@@ -1707,19 +1700,52 @@ int32_t agpu_xk_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
             bool ok = true;
             for (int b = 0; b < r.G && ok; ++b) ok = where[(size_t)b] == where[(size_t)(b & 7)];
             if (!ok) {
-                agpu_pk_plan_free(plan);
+                agpu_step_plan_free(plan);
                 return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "decode step: workgroups b, b + 8, ... do not share an XCD on this device");
             }
         }
     }
     if (e != hipSuccess) {
-        agpu_pk_plan_free(plan);
+        agpu_step_plan_free(plan);
         return agpu_hip(ctx, e, "decode step: plan");
     }
     return AGPU_OK;
 }
 
-int32_t agpu_xk_launch(agpu_ctx *ctx, const PkModel &m, const PkPlan &plan, int mode, unsigned long long *trace) {
+void agpu_step_plan_free(PkPlan *plan) {
+    if (plan->stages_dev) (void)hipFree(plan->stages_dev);
+    if (plan->arena) (void)hipFree(plan->arena);
+    if (plan->state) (void)hipFree(plan->state);
+    if (plan->ln_fold) (void)hipFree(plan->ln_fold);
+    *plan = PkPlan{};
+}
+
+// Every place "not written yet" (all-ones words), the candidates zero: on the stream the step runs on, and waited for
+// (a fill still under way when a step starts would leave words that are neither all-ones nor a value of the step).
+int32_t agpu_step_reset(agpu_ctx *ctx, const PkPlan &plan) {
+    const size_t total = plan.cand_off + 2 * (size_t)plan.grid + 2;
+    float *a = reinterpret_cast<float *>(plan.arena);
+    hipError_t e = hipMemsetAsync(a, 0xFF, plan.cand_off * sizeof(float), ctx->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(a + plan.cand_off, 0, (total - plan.cand_off) * sizeof(float), ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    return agpu_hip(ctx, e, "decode step: arena");
+}
+
+int32_t agpu_step_take_error(agpu_ctx *ctx, const PkPlan &plan, unsigned int *err_out) {
+    unsigned int st[2] = {0u, 0u};
+    hipError_t e = hipMemcpyAsync(st, plan.state, sizeof(st), hipMemcpyDeviceToHost, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "decode step: state");
+    *err_out = st[1];
+    if (st[1] != 0u) {
+        e = hipMemsetAsync(plan.state + 1, 0, sizeof(unsigned int), ctx->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess) return agpu_hip(ctx, e, "decode step: state");
+    }
+    return AGPU_OK;
+}
+
+int32_t agpu_step_launch(agpu_ctx *ctx, const PkModel &m, const PkPlan &plan, int mode, unsigned long long *trace) {
     Params p{};
     p.stages = reinterpret_cast<const Stage *>(plan.stages_dev);
     p.n_stages = plan.n_stages;

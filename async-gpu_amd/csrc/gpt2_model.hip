@@ -20,7 +20,7 @@
 #include "../../include/agpu_gpt2.h"
 #include "agpu_internal.h"
 #include "attention.h"
-#include "decode_persistent.h"
+#include "decode_step.h"
 #include "elementwise.h"
 #include "linear_common.h"
 
@@ -73,7 +73,9 @@ struct agpu_gpt2 {
     PkPlan pk;
     std::vector<PkLayer> pk_layers;
     bool pk_tried = false;
-    bool pk_failed = false;   // a wait of the one-launch step gave up once: this model keeps to the per-stage path
+    bool pk_failed = false;   // a wait of the one-launch step gave up: per stage until the step is planned anew
+    int pk_failed_looks = 0;  // looks at the decode path since then
+    long long n_one_launch = 0, n_per_stage = 0, n_wait_failures = 0;  // agpu_gpt2_decode_stats
     int pk_spin_limit = 0;    // test hook: poll rounds a wait may take (0 = default)
     int decode_mode = AGPU_DECODE_AUTO;
 };
@@ -196,7 +198,7 @@ void drop_graphs(agpu_gpt2 *m) {
     for (auto &kv : m->graphs) (void)hipGraphExecDestroy(kv.second);
     m->graphs.clear();
     // the plan of the one-launch step holds the same addresses
-    agpu_pk_plan_free(&m->pk);
+    agpu_step_plan_free(&m->pk);
     m->pk_tried = false;
 }
 
@@ -539,21 +541,22 @@ PkModel pk_view(agpu_gpt2 *m) {
 
 // Whether single-sequence decode steps run as one launch; builds the plan on first use (never inside a capture).
 bool pk_ready(agpu_gpt2 *m) {
-    if (m->decode_mode != AGPU_DECODE_AUTO || m->pk_failed || m->cfg.lm_head != AGPU_LM_HEAD_INT4) return false;
+    if (m->decode_mode != AGPU_DECODE_AUTO || m->cfg.lm_head != AGPU_LM_HEAD_INT4) return false;
+    if (m->pk_failed) {
+        // whatever kept the step's workgroups from running together may be gone: another try after a while
+        constexpr int kLooksBeforeRetry = 64;
+        if (++m->pk_failed_looks < kLooksBeforeRetry) return false;
+        m->pk_failed = false;
+        m->pk_failed_looks = 0;
+        m->pk_tried = false;
+    }
     if (m->pk.stages_dev) return true;
     if (m->pk_tried) return false;
     m->pk_tried = true;
     if (!m->logits.p || !m->out_tok) return false;
     const PkModel v = pk_view(m);
-    // the XCD-sharded step where the shape allows, else the one with every Linear spread over the device
-    const char *pick = getenv("AGPU_DECODE_STEP");
-    const bool want_xk = !(pick && pick[0] == 'l');
-    if (want_xk && agpu_xk_supported(m->ctx, v)) {
-        if (agpu_xk_plan_build(m->ctx, v, &m->pk) != AGPU_OK) return false;
-    } else {
-        if (!agpu_pk_supported(m->ctx, v)) return false;
-        if (agpu_pk_plan_build(m->ctx, v, &m->pk) != AGPU_OK) return false;
-    }
+    if (!agpu_step_supported(m->ctx, v)) return false;
+    if (agpu_step_plan_build(m->ctx, v, &m->pk) != AGPU_OK) return false;
     m->pk.spin_limit = m->pk_spin_limit;
     return true;
 }
@@ -640,10 +643,13 @@ int32_t run_decode_steps(agpu_gpt2 *m, int B, int steps) {
             const hipError_t e = hipGraphLaunch(exec, m->ctx->stream);
             if (e != hipSuccess) return agpu_hip(m->ctx, e, "hipGraphLaunch");
             m->cache_len += kStepsPerGraph;
+            m->n_one_launch += kStepsPerGraph;
         }
     }
     for (; s < steps; ++s) {
         const int bucket = kv_bucket(m, m->cache_len + 1);
+        if (B == 1 && pk_ready(m)) ++m->n_one_launch;
+        else ++m->n_per_stage;
         if (m->decode_mode == AGPU_DECODE_EAGER) {
             const int32_t rc = launch_step_per_stage(m, B, bucket);
             if (rc != AGPU_OK) return rc;
@@ -663,17 +669,19 @@ int32_t run_decode_steps(agpu_gpt2 *m, int B, int steps) {
 int32_t pk_check(agpu_gpt2 *m) {
     if (!m->pk.stages_dev) return AGPU_OK;
     unsigned int err = 0u;
-    int32_t rc = agpu_pk_take_error(m->ctx, m->pk, &err);
+    int32_t rc = agpu_step_take_error(m->ctx, m->pk, &err);
     if (rc != AGPU_OK) return rc;
     if (err != 0u) {
         // The steps since the last check are void.  Nothing is known about why the wait gave up (the workgroups of the
         // step must all be resident at once: another process on the device can prevent that), so this model keeps to
         // the per-stage path from now on; the caller resets the cache and runs again.
         m->pk_failed = true;
+        m->pk_failed_looks = 0;
+        ++m->n_wait_failures;
         drop_graphs(m);
         return agpu_fail(m->ctx, AGPU_ERR_DEVICE_WAIT,
                          "gpt2: a wait of the one-launch decode step gave up (code 0x%x, stage %u); the steps since the last check are "
-                         "invalid, decode steps run per stage from now on",
+                         "invalid, decode steps run per stage for a while",
                          err, err & 0xfffu);
     }
     return AGPU_OK;
@@ -952,6 +960,23 @@ AGPU_EXPORT int32_t agpu_gpt2_set_decode_mode(agpu_gpt2 *m, int32_t mode) {
         drop_graphs(m);
         m->decode_mode = mode;
     }
+    if (mode == AGPU_DECODE_AUTO) {  // asked for again: the one-launch step gets another try
+        m->pk_failed = false;
+        m->pk_failed_looks = 0;
+    }
+    return AGPU_OK;
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_decode_stats(agpu_gpt2 *m, int64_t *stats_out_host) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    if (!stats_out_host) return agpu_fail(m->ctx, AGPU_ERR_NULL_POINTER, "gpt2_decode_stats: null pointer");
+    stats_out_host[0] = m->n_one_launch;
+    stats_out_host[1] = m->n_per_stage;
+    stats_out_host[2] = m->n_wait_failures;
+    stats_out_host[3] = (m->pk.stages_dev || (m->decode_mode == AGPU_DECODE_AUTO && !m->pk_failed && !m->pk_tried &&
+                                              m->cfg.lm_head == AGPU_LM_HEAD_INT4))
+                            ? 1
+                            : 0;
     return AGPU_OK;
 }
 

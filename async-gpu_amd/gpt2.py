@@ -261,6 +261,12 @@ class Int4Gpt2Model:
     def decode_is_one_launch(self):
         return bool(self._lib.agpu_gpt2_decode_is_one_launch(self.handle))
 
+    def decode_stats(self):
+        """(steps run as one launch, steps run per stage, calls that ended with ERR_DEVICE_WAIT, would a step now be one launch)."""
+        out = np.zeros(4, np.int64)
+        self._call("agpu_gpt2_decode_stats", out)
+        return int(out[0]), int(out[1]), int(out[2]), bool(out[3])
+
     def set_decode_wait_limit(self, poll_rounds):
         """Test hook: poll rounds a wait inside the one-launch step may take (0 = default)."""
         self._call("agpu_gpt2_set_decode_wait_limit", poll_rounds)

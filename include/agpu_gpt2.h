@@ -141,8 +141,11 @@ int32_t agpu_gpt2_generate_cached_early_exit(agpu_gpt2 *m, const uint32_t *promp
 /*
  * How single-sequence decode steps run.  No counterpart in the reference, whose host loop launches every kernel
  * of every step (gpt2.rs:760-780).
- *   AGPU_DECODE_AUTO       one launch per token where the model's shape allows it (int4 head, head_dim 64, group a
- *                          power of two >= 8, vocab < 65536, K <= 8192), else as below
+ *   AGPU_DECODE_AUTO       one launch per token where the model and the device allow it, else as below.  The one-launch
+ *                          step takes: one sequence, an int4 LM head, group size 32, head_dim 64 (n_embd = 64 n_head),
+ *                          n_embd <= 2048, an MLP width that is a multiple of 32 and at most 16384, a vocabulary below
+ *                          65536, and a device of 8 XCDs with 32 CUs each (256 CUs) whose workgroups b, b + 8, ... share
+ *                          an XCD: probed when the step is planned and checked again by every launch
  *   AGPU_DECODE_PER_STAGE  one launch per stage (5 per block + 1), replayed as a HIP graph
  *   AGPU_DECODE_EAGER      the same launches issued one by one, without a graph (for profilers that cannot follow
  *                          graph replays, and for callers whose stream is under a capture of their own)
@@ -150,7 +153,9 @@ int32_t agpu_gpt2_generate_cached_early_exit(agpu_gpt2 *m, const uint32_t *promp
  * summation order only (both within 2e-4 of the f64 forward).  The one-launch step keeps one workgroup resident on
  * every CU for the duration of the step: nothing else should run on the device meanwhile.  Its waits are bounded;
  * a wait that gives up makes the call that ran the step return AGPU_ERR_DEVICE_WAIT: the tokens of that call are
- * void, the model then keeps to the per-stage path, and the caller may simply run the call again.
+ * void and the caller may simply run the call again.  The model then runs its steps per stage; it plans the one-launch
+ * step anew after 64 further looks at the decode path (a few generations), or at once when AGPU_DECODE_AUTO is set
+ * again.  agpu_gpt2_decode_stats says which path the steps have taken.
  */
 #define AGPU_DECODE_AUTO 0
 #define AGPU_DECODE_PER_STAGE 1
@@ -158,13 +163,20 @@ int32_t agpu_gpt2_generate_cached_early_exit(agpu_gpt2 *m, const uint32_t *promp
 int32_t agpu_gpt2_set_decode_mode(agpu_gpt2 *m, int32_t mode);
 /* 1 once a single-sequence decode step has been planned as one launch, else 0. */
 int32_t agpu_gpt2_decode_is_one_launch(agpu_gpt2 *m);
+/*
+ * Which way the decode steps of this model have gone so far.  No counterpart in the reference.
+ *   stats_out (HOST, 4 x int64): [0] steps run as one launch, [1] steps run per stage (graph replay or eager),
+ *   [2] calls that ended with AGPU_ERR_DEVICE_WAIT, [3] 1 if a single-sequence step would now run as one launch
+ *   (planned, or not yet tried), else 0.
+ */
+int32_t agpu_gpt2_decode_stats(agpu_gpt2 *m, int64_t *stats_out_host);
 /* Test hook: the number of poll rounds a wait inside the one-launch step may take before it gives up (0 = the
  * default, tens of milliseconds).  With a limit of a few rounds every wait gives up, the kernel still runs to its end,
  * and the call that ran the step returns AGPU_ERR_DEVICE_WAIT: the error path without a hung device. */
 int32_t agpu_gpt2_set_decode_wait_limit(agpu_gpt2 *m, int32_t poll_rounds);
 /*
  * Benchmark hook: the latency floor of the one-launch decode step.  Runs `steps` launches of the same stage chain
- * with empty bodies (every tagged store and every wait, no weights, no arithmetic; cache, tokens and counters are
+ * with empty bodies (every store and every wait, no weights, no arithmetic; cache, tokens and counters are
  * left alone) and reports the total time.  AGPU_ERR_UNSUPPORTED when the model does not take the one-launch step.
  */
 int32_t agpu_gpt2_decode_floor(agpu_gpt2 *m, int32_t steps, float *ms_total_out_host);

@@ -138,6 +138,7 @@ extern "C" {
     pub fn agpu_gpt2_generate_cached_early_exit(m: *mut agpu_gpt2, prompt_host: *const u32, prompt_len: i32, max_new_tokens: i32, threshold: f32, eos: i32, tokens_out_host: *mut u32, length_out_host: *mut i32, layers_out_host: *mut i32, steps_out_host: *mut i32) -> i32;
     pub fn agpu_gpt2_set_decode_mode(m: *mut agpu_gpt2, mode: i32) -> i32;
     pub fn agpu_gpt2_decode_is_one_launch(m: *mut agpu_gpt2) -> i32;
+    pub fn agpu_gpt2_decode_stats(m: *mut agpu_gpt2, stats_out_host: *mut i64) -> i32;
     pub fn agpu_gpt2_set_decode_wait_limit(m: *mut agpu_gpt2, poll_rounds: i32) -> i32;
     pub fn agpu_gpt2_decode_floor(m: *mut agpu_gpt2, steps: i32, ms_total_out_host: *mut f32) -> i32;
     pub fn agpu_gpt2_last_logits(m: *mut agpu_gpt2, batch: i32, logits_out_host: *mut f32) -> i32;

@@ -74,12 +74,18 @@ def test_config5_prefill_logits_and_first_tokens_against_the_oracle(xl, orc):
     # 8 greedy tokens: the oracle continues from its cache, one KV-cached step per token
     ref_tokens, margins = [], []
     lg = ref_logits
-    for _ in range(8):
+    for i in range(8):
         t = int(np.argmax(lg))
         ref_tokens.append(t)
         margins.append(_top2_gap(lg))
-        lg = om.forward(np.array([t], np.uint32), all_rows=False)[0]
+        if i < 7:
+            lg = om.forward(np.array([t], np.uint32), all_rows=False)[0]
     (got,), _ = gm.generate_cached(prompt, 8, eos=-1)
+    # the logits of the seventh decode step (one launch per token) against the oracle's, which chose the eighth token
+    assert gm.decode_is_one_launch()
+    err = float(np.abs(gm.last_logits()[0] - lg).max())
+    progress(f"config 5: logits of the last decode step differ from the oracle's by {err:.3e}")
+    assert err <= TOL_LOGITS, f"XL decode-step logits differ by {err}"
     progress(f"config 5: oracle tokens {ref_tokens}, smallest top-1/top-2 gap {min(margins):.3e}, {time.time() - t0:.0f} s")
     assert list(got[PROMPT:]) == ref_tokens, (list(got[PROMPT:]), ref_tokens, margins)
 

@@ -136,6 +136,79 @@ def test_wait_that_gives_up_is_reported_and_the_model_recovers(orc, agpu, dev):
     (again,), _ = gm.generate_cached(prompt, 12, eos=-1)
     assert not gm.decode_is_one_launch()
     assert np.array_equal(again, good)
+    one, per, gave_up, would = gm.decode_stats()
+    assert gave_up == 1 and per >= 11 and one >= 11 and not would
+    # asked for again (and allowed to wait again), the model plans the one-launch step anew
+    gm.set_decode_wait_limit(0)
+    gm.set_decode_mode(gm.DECODE_AUTO)
+    assert gm.decode_stats()[3]
+    (third,), _ = gm.generate_cached(prompt, 12, eos=-1)
+    assert gm.decode_is_one_launch()
+    assert np.array_equal(third, good)
+    assert gm.decode_stats()[2] == 1
+
+
+def test_a_model_that_fell_back_tries_the_one_launch_step_again_after_a_while(orc, agpu, dev):
+    """Without being asked, the model looks at the one-launch step again after 64 looks at the decode path."""
+    from async_gpu_amd import _lib, gpt2, workloads
+    cfg = workloads.GPT2_TINY
+    qz = _quantized(orc, cfg, 35)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg), qz)
+    prompt = workloads.random_prompt(cfg, 11, 5)
+    (good,), _ = gm.generate_cached(prompt, 20, eos=-1)
+    gm.set_decode_wait_limit(2)
+    with pytest.raises(_lib.AgpuError):
+        gm.generate_cached(prompt, 20, eos=-1)
+    gm.set_decode_wait_limit(0)  # whatever was in the way is gone
+    came_back = False
+    for _ in range(40):
+        (got,), _ = gm.generate_cached(prompt, 20, eos=-1)
+        assert np.array_equal(got, good)
+        if gm.decode_is_one_launch():
+            came_back = True
+            break
+    assert came_back
+    assert gm.decode_stats()[2] == 1
+
+
+def test_one_launch_step_on_raw_nibbles_over_the_whole_range(orc, agpu, dev):
+    """The Linear inside the one-launch step, pinned on its own: one block of GPT-2 small's width whose packed words are
+    drawn directly (nibbles uniform over all sixteen values, so the value -8 that the quantizer never emits is there;
+    scales U(0.002, 0.02): BASELINE config 1's distribution, compute_gemm.rs:2882-2895), non-zero biases, random LayerNorm
+    gains and offsets, and embedding rows whose magnitudes span four decades.  The logits of every decode step against
+    the f64 oracle on the same token sequence (2e-4 of the largest logit magnitude), and against the per-stage path."""
+    from async_gpu_amd import gpt2, workloads
+    cfg = dict(n_layer=1, n_embd=768, n_head=12, vocab=2003, n_positions=32)
+    d, ff, V, P = 768, 3072, cfg["vocab"], cfg["n_positions"]
+    rng = np.random.default_rng(77)
+    layer = dict(ln1_g=(1.0 + 0.1 * rng.standard_normal(d)).astype(np.float32), ln1_b=(0.1 * rng.standard_normal(d)).astype(np.float32),
+                 ln2_g=(1.0 + 0.1 * rng.standard_normal(d)).astype(np.float32), ln2_b=(0.1 * rng.standard_normal(d)).astype(np.float32))
+    for name, (k, n) in zip(workloads.LINEAR_NAMES, ((d, 3 * d), (d, d), (d, ff), (ff, d))):
+        layer[name] = workloads.random_int4_linear(rng, k, n, 32, bias=True)
+    head_packed, head_scales, _ = workloads.random_int4_linear(rng, d, V, 32)
+    wte = (rng.standard_normal((V, d)) * 10.0 ** rng.uniform(-2, 2, size=(V, 1))).astype(np.float32)
+    wpe = (0.01 * rng.standard_normal((P, d))).astype(np.float32)
+    qz = dict(group=32, wte=wte, wpe=wpe, lnf_g=(1.0 + 0.1 * rng.standard_normal(d)).astype(np.float32),
+              lnf_b=(0.1 * rng.standard_normal(d)).astype(np.float32), layers=[layer], lm_head=(head_packed, head_scales))
+    assert any((layer[n][0] & 0xF == 0).any() for n in workloads.LINEAR_NAMES)  # the nibble of -8 is among the weights
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg), qz)
+    om = build_oracle_model(cfg, qz)
+    prompt = workloads.random_prompt(cfg, 12, 6)
+    for steps in (2, 3, 9):
+        gm.set_decode_mode(gm.DECODE_AUTO)
+        (got,), _ = gm.generate_cached(prompt, steps, eos=-1)
+        assert gm.decode_is_one_launch()
+        lg = gm.last_logits()[0]
+        om.reset_cache()
+        lo = om.forward(got[:-1], all_rows=False)[0]
+        scale = max(1.0, float(np.abs(lo).max()))
+        err = float(np.abs(lg - lo).max())
+        assert err <= TOL_LOGITS * scale, f"{steps - 1} decode steps: logits differ from the oracle's by {err:.3e} (largest logit {scale:.3e})"
+        gm.set_decode_mode(gm.DECODE_PER_STAGE)
+        (per,), _ = gm.generate_cached(prompt, steps, eos=-1)
+        lp = gm.last_logits()[0]
+        if np.array_equal(per, got):  # the same sequence (a near tie may part them): the two paths' logits side by side
+            assert float(np.abs(lp - lg).max()) <= TOL_LOGITS * scale
 
 
 def test_sampling_runs_on_the_one_launch_step(orc, agpu, dev):

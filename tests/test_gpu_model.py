@@ -221,6 +221,12 @@ def test_config4_gpt2_small_generation(orc, agpu, dev):
     (got,), (ms_prefill, ms_decode) = gm.generate_cached(prompt, 128, eos=-1)
     _assert_tokens_match(got, ref, margins, 64, "config 4")
     assert len(got) == 192
+    # the logits of the last decode step (one launch per token) against the oracle's for the same position
+    assert gm.decode_is_one_launch()
+    om.reset_cache()
+    last_ref = om.forward(ref[:-1], all_rows=False)[0]
+    err = float(np.abs(gm.last_logits()[0] - last_ref).max())
+    assert err <= TOL_LOGITS, f"logits of the last decode step differ from the oracle's by {err}"
     print(f"config4: prefill {ms_prefill:.3f} ms, decode {ms_decode / 127:.4f} ms/token, min oracle margin {margins.min():.3e}")
 
 
