@@ -69,9 +69,10 @@ AGPU_EXPORT int32_t agpu_int4_linear_static(int32_t device, void *hip_stream, co
                                             const float *scales, const float *bias, const float *residual, float *y, int32_t M,
                                             int32_t N, int32_t K, int32_t group, uint32_t flags, char *err_out, int32_t err_cap) {
     if (device < 0 || device >= kMaxDevices) return say(AGPU_ERR_DIM_OUT_OF_RANGE, err_out, err_cap, "int4_linear_static: device out of range");
-    if (M > 0 && N > 0 && ((size_t)M * (size_t)N * sizeof(float) > kStaticWorkspaceBytes / 2 || (N + 63) / 64 > kStaticCounters - 1))
-        return say(AGPU_ERR_WORKSPACE, err_out, err_cap,
-                   "int4_linear_static: M*N*4 bytes must fit the 4 MiB of partial sums and N must not exceed 262080");
+    // The tickets bound N; whether the partial sums of a shape fit the scratch depends on how its kernel splits K (many
+    // shapes need none): the launchers know, and refuse with AGPU_ERR_WORKSPACE when 4 MiB do not do.
+    if (N > 0 && (N + 63) / 64 > kStaticCounters - 1)
+        return say(AGPU_ERR_WORKSPACE, err_out, err_cap, "int4_linear_static: N must not exceed 262080 (one ticket per 64 columns)");
     std::lock_guard<std::mutex> lock(g_mu);  // host state only: calls that overlap on the GPU still share the scratch
     int prev = -1;
     hipError_t e = hipGetDevice(&prev);

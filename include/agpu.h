@@ -162,8 +162,10 @@ int32_t agpu_int4_linear(agpu_ctx *ctx, const float *x, const uint32_t *packed, 
  * until the process ends); the kernels and results are those of agpu_int4_linear (bit-identical for M <= 16; the
  * prefill GEMM may split K less deeply, which only reorders its additions).
  *   device      GPU the pointers belong to; hip_stream a hipStream_t of that GPU (NULL = the default stream).
- *   Limits      M * N * 4 bytes <= 4 MiB and N <= 262080, else AGPU_ERR_WORKSPACE; a K split that does not fit the
- *               4 MiB is made shallower, and the call returns AGPU_ERR_WORKSPACE where the kernel cannot do that.
+ *   Limits      N <= 262080 (one ticket per 64 columns), and the partial sums of the shape's K split within 4 MiB,
+ *               else AGPU_ERR_WORKSPACE.  A shape whose kernel splits K needs splits * M * N * 4 bytes; a split that
+ *               does not fit is made shallower where the kernel can do that, and many shapes need none at all (a
+ *               Linear with K up to 2048 at M <= 2, a prefill GEMM whose tiles already fill the device).
  *   err_out     optional buffer of err_cap bytes for the message of a failed call.
  * Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams, two threads) race.
  * The first call on a GPU looks up the array's address (hipGetSymbolAddress) and the CU count; make it outside

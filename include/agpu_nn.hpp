@@ -220,11 +220,26 @@ public:
         return host_;
     }
     const T &operator[](size_t i) const { return read()[i]; }
-    // DerefMut (gpu_array.rs:372-385): as read(), then the host copy is the newer one.
-    std::vector<T> &write() {
+    // The elements as DerefMut hands them out (gpu_array.rs:372-385): &mut [T], a view of fixed length.  The array's
+    // size and its device allocation belong together, so the host data cannot be resized through it.
+    class Slice {
+      public:
+        Slice(T *p, size_t n) : p_(p), n_(n) {}
+        T &operator[](size_t i) const { return p_[i]; }
+        T *data() const { return p_; }
+        size_t size() const { return n_; }
+        T *begin() const { return p_; }
+        T *end() const { return p_ + n_; }
+
+      private:
+        T *p_;
+        size_t n_;
+    };
+    // DerefMut: as read(), then the host copy is the newer one.
+    Slice write() {
         if (residency_ == Residency::DeviceOnly) sync_to_host();
         residency_ = Residency::HostDirty;
-        return host_;
+        return Slice(host_.data(), host_.size());
     }
 
     // mark_device_dirty (gpu_array.rs:227-240): a kernel wrote the device copy.
