@@ -106,6 +106,8 @@ SIGNATURES = {
     "agpu_gpt2_generate_cached_sampling": (_i32, [_vp, _vp, _i32, _i32, _i32, _f, _vp, _i32, _vp, _vp]),
     "agpu_gpt2_forward_early_exit": (_i32, [_vp, _vp, _i32, _f, _vp, _vp]),
     "agpu_gpt2_generate_cached_early_exit": (_i32, [_vp, _vp, _i32, _i32, _f, _i32, _vp, _vp, _vp, _vp]),
+    "agpu_gpt2_forward_profiled": (_i32, [_vp, _vp, _i32, _vp, _vp, _i32, _vp]),
+    "agpu_gpt2_forward_diagnostic": (_i32, [_vp, _vp, _i32, _vp, _vp, _i32, _vp, _vp, _vp]),
     "agpu_gpt2_decode_steps": (_i32, [_vp, _i32, _i32, _vp]),
     "agpu_gpt2_set_decode_mode": (_i32, [_vp, _i32]),
     "agpu_gpt2_decode_is_one_launch": (_i32, [_vp]),
@@ -114,6 +116,12 @@ SIGNATURES = {
     "agpu_gpt2_decode_floor": (_i32, [_vp, _i32, _vp]),
     "agpu_gpt2_last_logits": (_i32, [_vp, _i32, _vp]),
 }
+
+
+class StageReport(C.Structure):
+    """agpu_gpt2_stage_report of include/agpu_gpt2.h."""
+    _fields_ = [("name", C.c_char * 24), ("ms", C.c_float), ("pos0_first4", C.c_float * 4), ("last_first4", C.c_float * 4),
+                ("non_finite", C.c_int32)]
 
 
 class Gpt2ConfigStruct(C.Structure):

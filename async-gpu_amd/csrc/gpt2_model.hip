@@ -13,6 +13,7 @@
 //   LN2 + fc Linear + bias + GELU      (layer_norm_v3, int4_gemm_w4a16, bias_add, gelu_forward)
 //   fc-proj Linear + bias + residual   (int4_gemm_w4a16, bias_add, elementwise_add_v3)
 #include <cstring>
+#include <cmath>
 #include <map>
 #include <new>
 #include <vector>
@@ -63,6 +64,7 @@ struct agpu_gpt2 {
     int out_capacity = 0;  // steps recorded in out_tok
     int *pos_dev = nullptr, *step_dev = nullptr;
     std::map<long long, hipGraphExec_t> graphs;  // key: batch << 32 | kv bucket
+    std::map<long long, unsigned long long> graph_addr;  // per graph: fingerprint of the device addresses it was captured with
     unsigned long long ws_epoch = 0;             // the context's scratch the graphs were captured with
     hipEvent_t ev0 = nullptr, ev1 = nullptr, ev2 = nullptr;
     // early exit: per block one (confidence, arg-max) pair in host-visible memory and one event
@@ -194,9 +196,37 @@ void free_lin(Int4Lin &l) {
     l = Int4Lin{};
 }
 
+// Every device address a decode step refers to, folded into one word.  A captured graph holds these addresses; a
+// replay is only right while they are still the model's.  Every path that frees or moves one of them drops the graphs
+// (ensure, ensure_out_tokens, the weight setters, a new scratch); this is the check behind that rule.
+unsigned long long step_addresses(const agpu_gpt2 *m, bool one_launch) {
+    unsigned long long h = 1469598103934665603ull;
+    auto mix = [&](const void *p) { h = (h ^ (unsigned long long)(uintptr_t)p) * 1099511628211ull; };
+    for (const void *p : {(const void *)m->wte, (const void *)m->wpe, (const void *)m->lnf_g, (const void *)m->lnf_b, (const void *)m->wte_t,
+                          (const void *)m->kcache, (const void *)m->vcache, (const void *)m->cur_tok, (const void *)m->next_tok,
+                          (const void *)m->out_tok, (const void *)m->pos_dev, (const void *)m->step_dev, (const void *)m->lm_head.packed,
+                          (const void *)m->lm_head.scales, (const void *)m->ctx->workspace, (const void *)m->ctx->counters})
+        mix(p);
+    if (one_launch)  // the step's plan; a graph of per-stage launches does not refer to it
+        for (const void *p : {(const void *)m->pk.arena, (const void *)m->pk.stages_dev, (const void *)m->pk.state, (const void *)m->pk.ln_fold}) mix(p);
+    for (const DevBuf *b : {&m->hid, &m->qkv, &m->att, &m->ffn, &m->lnb, &m->last, &m->logits, &m->tok_in}) mix(b->p);
+    for (const Block &b : m->blocks) {
+        for (const void *p : {(const void *)b.ln1_g, (const void *)b.ln1_b, (const void *)b.ln2_g, (const void *)b.ln2_b}) mix(p);
+        for (const Int4Lin &l : b.lin) {
+            mix(l.packed);
+            mix(l.scales);
+            mix(l.bias);
+        }
+    }
+    return h;
+}
+
 void drop_graphs(agpu_gpt2 *m) {
+    // a replay still on the stream must not lose its graph, nor the plan its arena
+    if (m->ctx && !m->graphs.empty()) (void)hipStreamSynchronize(m->ctx->stream);
     for (auto &kv : m->graphs) (void)hipGraphExecDestroy(kv.second);
     m->graphs.clear();
+    m->graph_addr.clear();
     // the plan of the one-launch step holds the same addresses
     agpu_step_plan_free(&m->pk);
     m->pk_tried = false;
@@ -581,8 +611,12 @@ int32_t decode_graph(agpu_gpt2 *m, int B, int bucket, hipGraphExec_t *out, int r
     }
     auto it = m->graphs.find(key);
     if (it != m->graphs.end()) {
-        *out = it->second;
-        return AGPU_OK;
+        if (m->graph_addr[key] == step_addresses(m, reps > 1 || (B == 1 && m->pk.stages_dev != nullptr))) {
+            *out = it->second;
+            return AGPU_OK;
+        }
+        // an address changed under a cached graph: never replay it; every graph goes and this one is captured anew
+        drop_graphs(m);
     }
     agpu_ctx *ctx = m->ctx;
     if (ctx->stream == nullptr)
@@ -613,6 +647,7 @@ int32_t decode_graph(agpu_gpt2 *m, int B, int bucket, hipGraphExec_t *out, int r
     (void)hipGraphDestroy(graph);
     if (e != hipSuccess) return agpu_hip(ctx, e, "hipGraphInstantiate");
     m->graphs[key] = exec;
+    m->graph_addr[key] = step_addresses(m, one_launch);
     *out = exec;
     return AGPU_OK;
 }
@@ -1032,6 +1067,119 @@ AGPU_EXPORT int32_t agpu_gpt2_forward_cached(agpu_gpt2 *m, const uint32_t *token
         if (e != hipSuccess) return agpu_hip(ctx, e, "hipMemcpy2DAsync(logits)");
     }
     return AGPU_OK;
+}
+
+namespace {
+
+// The forward of one sequence from an empty cache, one stage at a time: timed (profile) or looked at (diagnostic).
+int32_t forward_staged(agpu_gpt2 *m, const uint32_t *tokens, int seq_len, float *logits_out, agpu_gpt2_stage_report *rep, int capacity,
+                       int32_t *n_out, bool diagnostic, uint32_t *top5_tok, float *top5_val, const char *who) {
+    agpu_ctx *ctx = m->ctx;
+    if (!tokens || !rep || !n_out) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "%s: null pointer", who);
+    if (diagnostic && (!top5_tok || !top5_val)) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "%s: null pointer", who);
+    if (seq_len <= 0 || seq_len > m->P) return agpu_fail(ctx, AGPU_ERR_DIM_OUT_OF_RANGE, "%s: seq_len %d not in 1..%d", who, seq_len, m->P);
+    const int n_rep = m->cfg.n_layer + 3;
+    if (capacity < n_rep) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "%s: %d reports do not fit %d entries", who, n_rep, capacity);
+    int32_t rc = check_ready(m);
+    if (rc != AGPU_OK) return rc;
+    if ((rc = ensure_buffers(m, 1, seq_len, false)) != AGPU_OK) return rc;
+    if ((rc = ensure_out_tokens(m, m->P, 1)) != AGPU_OK) return rc;
+    m->cache_len = 0;
+    if ((rc = set_counters(m, 0, -1)) != AGPU_OK) return rc;
+    const int d = m->d;
+    std::vector<float> host;
+    int r = 0;
+    // one stage: launch, timed between two synchronisations; then what the diagnostic wants of its output [rows, width]
+    auto stage = [&](const char *name, auto &&launch, const float *out, int rows, int width) -> int32_t {
+        agpu_gpt2_stage_report &e = rep[r++];
+        std::memset(&e, 0, sizeof(e));
+        std::snprintf(e.name, sizeof(e.name), "%s", name);
+        hipError_t he = hipStreamSynchronize(ctx->stream);
+        if (he == hipSuccess) he = hipEventRecord(m->ev0, ctx->stream);
+        if (he != hipSuccess) return agpu_hip(ctx, he, who);
+        const int32_t lrc = launch();
+        if (lrc != AGPU_OK) return lrc;
+        he = hipEventRecord(m->ev1, ctx->stream);
+        if (he == hipSuccess) he = hipEventSynchronize(m->ev1);
+        if (he == hipSuccess) he = hipEventElapsedTime(&e.ms, m->ev0, m->ev1);
+        if (he != hipSuccess) return agpu_hip(ctx, he, who);
+        if (!diagnostic) return AGPU_OK;
+        host.resize((size_t)rows * width);
+        he = hipMemcpy2DAsync(host.data(), (size_t)width * 4, out, (size_t)width * 4, (size_t)width * 4, (size_t)rows, hipMemcpyDeviceToHost,
+                              ctx->stream);
+        if (he == hipSuccess) he = hipStreamSynchronize(ctx->stream);
+        if (he != hipSuccess) return agpu_hip(ctx, he, who);
+        for (int i = 0; i < 4 && i < width; ++i) {
+            e.pos0_first4[i] = host[(size_t)i];
+            e.last_first4[i] = host[(size_t)(rows - 1) * width + i];
+        }
+        int bad = 0;
+        for (float v : host) bad += std::isfinite(v) ? 0 : 1;
+        e.non_finite = bad;
+        return AGPU_OK;
+    };
+    float *hid = (float *)m->hid.p;
+    if ((rc = stage("embedding", [&] { return launch_embed(m, tokens, 1, seq_len); }, hid, seq_len, d)) != AGPU_OK) return rc;
+    for (int L = 0; L < m->cfg.n_layer; ++L) {
+        char name[24];
+        std::snprintf(name, sizeof(name), "block_%d", L);
+        if ((rc = stage(name, [&] { return launch_block(m, L, 1, seq_len, seq_len); }, hid, seq_len, d)) != AGPU_OK) return rc;
+    }
+    float *lnb = (float *)m->lnb.p;
+    if ((rc = stage("ln_f", [&] { return agpu_layer_norm(ctx, hid, m->lnf_g, m->lnf_b, lnb, seq_len, d, m->cfg.layer_norm_epsilon); }, lnb,
+                    seq_len, d)) != AGPU_OK)
+        return rc;
+    if ((rc = stage("lm_head",
+                    [&] {
+                        int32_t h = launch_gather_last(m, 1, seq_len);
+                        return h == AGPU_OK ? launch_head(m, (float *)m->last.p, 1) : h;
+                    },
+                    (float *)m->logits.p, 1, m->V)) != AGPU_OK)
+        return rc;
+    *n_out = r;
+    if (diagnostic) {
+        // the five largest logits of the last position (`host` holds the logits row of the last stage)
+        std::vector<int> idx((size_t)m->V);
+        for (int i = 0; i < m->V; ++i) idx[(size_t)i] = i;
+        const int k = m->V < 5 ? m->V : 5;
+        std::partial_sort(idx.begin(), idx.begin() + k, idx.end(), [&](int a, int b) {
+            const float x = host[(size_t)a], y = host[(size_t)b];
+            const bool xn = x != x, yn = y != y;
+            if (xn != yn) return yn;  // NaN last
+            return x > y || (x == y && a < b);
+        });
+        for (int i = 0; i < 5; ++i) {
+            top5_tok[i] = i < k ? (uint32_t)idx[(size_t)i] : 0u;
+            top5_val[i] = i < k ? host[(size_t)idx[(size_t)i]] : 0.0f;
+        }
+    }
+    // the generation state as after forward_cached: the next token is the arg-max of the last row
+    if ((rc = launch_argmax_advance(m, 1, seq_len)) != AGPU_OK) return rc;
+    m->cache_len = seq_len;
+    if (logits_out) {
+        hipError_t he = hipMemcpyAsync(logits_out, m->logits.p, (size_t)m->V * 4, hipMemcpyDeviceToDevice, ctx->stream);
+        if (he != hipSuccess) return agpu_hip(ctx, he, who);
+    }
+    return AGPU_OK;
+}
+
+}  // namespace
+
+AGPU_EXPORT int32_t agpu_gpt2_forward_profiled(agpu_gpt2 *m, const uint32_t *tokens, int32_t seq_len, float *logits_out,
+                                               agpu_gpt2_stage_report *reports_out_host, int32_t capacity, int32_t *n_reports_out_host) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    AGPU_REQUIRE_CTX(m->ctx);
+    return forward_staged(m, tokens, seq_len, logits_out, reports_out_host, capacity, n_reports_out_host, false, nullptr, nullptr,
+                          "gpt2_forward_profiled");
+}
+
+AGPU_EXPORT int32_t agpu_gpt2_forward_diagnostic(agpu_gpt2 *m, const uint32_t *tokens, int32_t seq_len, float *logits_out,
+                                                 agpu_gpt2_stage_report *reports_out_host, int32_t capacity, int32_t *n_reports_out_host,
+                                                 uint32_t *top5_tokens_out_host, float *top5_logits_out_host) {
+    if (!m) return AGPU_ERR_NULL_POINTER;
+    AGPU_REQUIRE_CTX(m->ctx);
+    return forward_staged(m, tokens, seq_len, logits_out, reports_out_host, capacity, n_reports_out_host, true, top5_tokens_out_host,
+                          top5_logits_out_host, "gpt2_forward_diagnostic");
 }
 
 AGPU_EXPORT int32_t agpu_gpt2_decode_steps(agpu_gpt2 *m, int32_t batch, int32_t steps, float *ms_total_out_host) {

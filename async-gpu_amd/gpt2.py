@@ -181,6 +181,63 @@ class Int4Gpt2Model:
         self.reset_cache()
         return self.forward_cached(np.asarray(tokens).reshape(1, -1), all_rows=True)[0]
 
+    def _forward_staged(self, tokens, diagnostic):
+        tokens = _np(tokens, np.uint32).reshape(-1)
+        n_rep = self.config.n_layer + 3
+        reports = (_lib.StageReport * n_rep)()
+        n = C.c_int32(0)
+        p = C.c_void_p()
+        self.ctx.call("agpu_malloc", tokens.nbytes, C.byref(p))
+        lg = C.c_void_p()
+        self.ctx.call("agpu_malloc", self.config.vocab_size * 4, C.byref(lg))
+        top_tok, top_val = np.zeros(5, np.uint32), np.zeros(5, np.float32)
+        try:
+            self.ctx.call("agpu_memcpy_h2d", p.value, tokens, tokens.nbytes)
+            if diagnostic:
+                self._call("agpu_gpt2_forward_diagnostic", p.value, tokens.size, lg.value, C.addressof(reports), n_rep, C.addressof(n),
+                           top_tok, top_val)
+            else:
+                self._call("agpu_gpt2_forward_profiled", p.value, tokens.size, lg.value, C.addressof(reports), n_rep, C.addressof(n))
+            logits = np.empty(self.config.vocab_size, np.float32)
+            self.ctx.call("agpu_memcpy_d2h", logits, lg.value, logits.nbytes)
+        finally:
+            self.ctx.call("agpu_free", p.value)
+            self.ctx.call("agpu_free", lg.value)
+        return logits, [reports[i] for i in range(n.value)], top_tok, top_val
+
+    def forward_profiled(self, tokens):
+        """forward_profiled (gpt2.rs:529-568): (logits of the last position, [(stage name, milliseconds)]) of a forward from
+        an empty cache, every stage between two synchronisations."""
+        logits, reports, _, _ = self._forward_staged(tokens, False)
+        return logits, [(r.name.decode(), float(r.ms)) for r in reports]
+
+    def forward_diagnostic(self, tokens, out=None):
+        """forward_diagnostic (gpt2.rs:595-667): the forward with the reference's `[diag]` lines written to `out` (stderr by
+        default): first four values of position 0 and of the last position after the embedding, of the last position after
+        the first and the last block and after the final LayerNorm, NaN/Inf warnings, and the five best tokens.  Returns
+        (logits of the last position, reports, top-5 tokens, top-5 logits)."""
+        import sys
+        out = out or sys.stderr
+        logits, reports, top_tok, top_val = self._forward_staged(tokens, True)
+        last = np.asarray(tokens).size - 1
+        fmt = lambda a: "[" + ", ".join(f"{float(x):.6f}" for x in a) + "]"
+        for r in reports:
+            name = r.name.decode()
+            if name == "embedding":
+                print(f"[diag] Embedding pos0 first4: {fmt(r.pos0_first4)}", file=out)
+                print(f"[diag] Embedding pos{last} first4: {fmt(r.last_first4)}", file=out)
+            elif name in ("block_0", f"block_{self.config.n_layer - 1}"):
+                i = int(name.split("_")[1])
+                print(f"[diag] Layer {i} pos{last} first4: {fmt(r.last_first4)}", file=out)
+                if r.non_finite:
+                    print(f"[diag] WARNING: Layer {i} has {r.non_finite} NaN/Inf values!", file=out)
+            elif name == "ln_f":
+                print(f"[diag] Final LN pos{last} first4: {fmt(r.last_first4)}", file=out)
+        print(f"[diag] Top-5 tokens at pos{last}:", file=out)
+        for t, s in zip(top_tok, top_val):
+            print(f"  token {int(t)}: {float(s):.4f}", file=out)
+        return logits, reports, top_tok, top_val
+
     def generate_cached(self, prompt, max_new_tokens, eos=50256):
         """Returns (list of token arrays per sequence, (prefill_ms, decode_ms))."""
         prompt = np.atleast_2d(_np(prompt, np.uint32))

@@ -179,6 +179,20 @@ def quantize_gpt2_file(src, dst, group=32, quantize_fn=None, lm_head_int4=True):
     return cfg, qz
 
 
+def count_params(path):
+    """(values, bytes) of every tensor in a safetensors file: what the reference's loader reports as total_params and
+    memory_bytes (model.rs:380-396); packed int4 words count eight values each."""
+    n = b = 0
+    with _open(path) as f:
+        for k in f.keys():
+            sl = f.get_slice(k)
+            size = int(np.prod(sl.get_shape())) if sl.get_shape() else 1
+            width = {"F32": 4, "F16": 2, "BF16": 2, "I32": 4, "U32": 4, "I64": 8, "U8": 1, "I8": 1}.get(str(sl.get_dtype()), 4)
+            n += size * (8 if k.endswith(".int4_packed") else 1)
+            b += size * width
+    return n, b
+
+
 def describe(path):
     """Keys, dtypes and shapes of a safetensors file, as JSON text (a debugging aid like load_tensors_generic,
     model_generic.rs:127-213)."""

@@ -111,6 +111,38 @@ int32_t agpu_gpt2_generate_cached_sampling(agpu_gpt2 *m, const uint32_t *prompt_
                                            int32_t eos, uint32_t *tokens_out_host, int32_t *length_out_host);
 
 /*
+ * One stage of forward_profiled / forward_diagnostic: "embedding", "block_<i>", "ln_f", "lm_head", in the order the
+ * forward runs them (gpt2.rs:540-565, 611-664).
+ */
+typedef struct agpu_gpt2_stage_report {
+    char name[24];
+    float ms;              /* forward_profiled: duration of the stage, synchronised on both sides as the reference times it */
+    float pos0_first4[4];  /* forward_diagnostic: the first four values of position 0 after the stage */
+    float last_first4[4];  /* ... and of the last position */
+    int32_t non_finite;    /* ... and how many values of the stage's output are NaN or Inf */
+} agpu_gpt2_stage_report;
+
+/*
+ * forward_profiled (gpt2.rs:529-568): the forward of one sequence from an empty cache over seq_len tokens (DEVICE
+ * pointer), stage by stage with a synchronisation and a clock around each: n_layer + 3 reports (HOST array of
+ * `capacity` entries; AGPU_ERR_SHAPE_MISMATCH when it is too short).  logits_out: DEVICE pointer, [vocab_size] of the
+ * last position, may be NULL.  "ln_f" is the final LayerNorm on its own (its output is what the diagnostic shows);
+ * "lm_head" is the head as the model runs it, which normalises the row itself once more.  The cache afterwards
+ * holds the seq_len positions, as after forward_cached.
+ */
+int32_t agpu_gpt2_forward_profiled(agpu_gpt2 *m, const uint32_t *tokens, int32_t seq_len, float *logits_out,
+                                   agpu_gpt2_stage_report *reports_out_host, int32_t capacity, int32_t *n_reports_out_host);
+/*
+ * forward_diagnostic (gpt2.rs:595-667): the same forward, with the values the reference prints after each stage (first
+ * four of position 0 and of the last position, NaN/Inf count; the reference prints them for the embedding, the first
+ * and the last block and the final LayerNorm: here every stage has them) and the five largest logits of the last
+ * position (top5_*: HOST arrays of 5, largest first, ties to the lower id).
+ */
+int32_t agpu_gpt2_forward_diagnostic(agpu_gpt2 *m, const uint32_t *tokens, int32_t seq_len, float *logits_out,
+                                     agpu_gpt2_stage_report *reports_out_host, int32_t capacity, int32_t *n_reports_out_host,
+                                     uint32_t *top5_tokens_out_host, float *top5_logits_out_host);
+
+/*
  * Gpt2Model::forward_early_exit (gpt2.rs:797-830): uncached forward over seq_len tokens (device ids) that stops
  * after the first block whose confidence (agpu_softmax_max_prob of the last row's logits behind the final
  * LayerNorm and the LM head) reaches `threshold`; the last block is never probed.  logits_out (device,

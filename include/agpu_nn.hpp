@@ -655,6 +655,48 @@ public:
         reg_->check(agpu_gpt2_forward_cached(h_, token_ids.data(), 1, (int32_t)new_len, logits.data(), 1));
         return logits;
     }
+    // forward_profiled (gpt2.rs:529-568): logits [1, vocab_size] of the last position and (stage, milliseconds) per stage
+    std::pair<GpuTensor, std::vector<std::pair<std::string, double>>> forward_profiled(const GpuBufferU32 &token_ids, size_t seq_len) const {
+        GpuTensor logits = GpuTensor::zeros({1, config_.vocab_size}, reg_);
+        std::vector<agpu_gpt2_stage_report> rep(config_.n_layer + 3);
+        int32_t n = 0;
+        reg_->check(agpu_gpt2_forward_profiled(h_, token_ids.data(), (int32_t)seq_len, logits.data(), rep.data(), (int32_t)rep.size(), &n));
+        std::vector<std::pair<std::string, double>> timings;
+        for (int32_t i = 0; i < n; ++i) timings.emplace_back(rep[(size_t)i].name, (double)rep[(size_t)i].ms);
+        return {std::move(logits), std::move(timings)};
+    }
+    // forward_diagnostic (gpt2.rs:595-667): the forward with the reference's [diag] lines on stderr; logits [1, vocab_size]
+    GpuTensor forward_diagnostic(const GpuBufferU32 &token_ids, size_t seq_len) const {
+        GpuTensor logits = GpuTensor::zeros({1, config_.vocab_size}, reg_);
+        std::vector<agpu_gpt2_stage_report> rep(config_.n_layer + 3);
+        int32_t n = 0;
+        uint32_t top_tok[5];
+        float top_val[5];
+        reg_->check(agpu_gpt2_forward_diagnostic(h_, token_ids.data(), (int32_t)seq_len, logits.data(), rep.data(), (int32_t)rep.size(), &n,
+                                                 top_tok, top_val));
+        const size_t last = seq_len - 1;
+        auto four = [](const float *a) {
+            char b[96];
+            std::snprintf(b, sizeof(b), "[%.6f, %.6f, %.6f, %.6f]", a[0], a[1], a[2], a[3]);
+            return std::string(b);
+        };
+        for (int32_t i = 0; i < n; ++i) {
+            const agpu_gpt2_stage_report &r = rep[(size_t)i];
+            const std::string name = r.name;
+            if (name == "embedding") {
+                std::fprintf(stderr, "[diag] Embedding pos0 first4: %s\n", four(r.pos0_first4).c_str());
+                std::fprintf(stderr, "[diag] Embedding pos%zu first4: %s\n", last, four(r.last_first4).c_str());
+            } else if (name == "block_0" || name == "block_" + std::to_string(config_.n_layer - 1)) {
+                std::fprintf(stderr, "[diag] Layer %s pos%zu first4: %s\n", name.c_str() + 6, last, four(r.last_first4).c_str());
+                if (r.non_finite) std::fprintf(stderr, "[diag] WARNING: Layer %s has %d NaN/Inf values!\n", name.c_str() + 6, r.non_finite);
+            } else if (name == "ln_f") {
+                std::fprintf(stderr, "[diag] Final LN pos%zu first4: %s\n", last, four(r.last_first4).c_str());
+            }
+        }
+        std::fprintf(stderr, "[diag] Top-5 tokens at pos%zu:\n", last);
+        for (int i = 0; i < 5; ++i) std::fprintf(stderr, "  token %u: %.4f\n", top_tok[i], top_val[i]);
+        return logits;
+    }
     size_t cache_len() const { return (size_t)agpu_gpt2_cache_len(h_); }
     void reset_cache() const { reg_->check(agpu_gpt2_reset_cache(h_)); }
     // generate (gpt2.rs:1536-1560)

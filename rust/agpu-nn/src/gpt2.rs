@@ -147,6 +147,73 @@ impl Int4Gpt2Model {
         rc.map(|_| out)
     }
 
+    /// forward_profiled (gpt2.rs:529-568): logits of the last position and (stage, milliseconds) per stage, every stage
+    /// between two synchronisations.
+    pub fn forward_profiled(&self, tokens: &[u32]) -> Result<(Vec<f32>, Vec<(String, f64)>)> {
+        let (logits, reports, _, _) = self.forward_staged(tokens, false)?;
+        Ok((logits, reports.iter().map(|r| (stage_name(r), r.ms as f64)).collect()))
+    }
+
+    /// forward_diagnostic (gpt2.rs:595-667): the forward with the reference's `[diag]` lines on stderr.
+    pub fn forward_diagnostic(&self, tokens: &[u32]) -> Result<Vec<f32>> {
+        let (logits, reports, top_tok, top_val) = self.forward_staged(tokens, true)?;
+        let last = tokens.len() - 1;
+        let four = |a: &[f32; 4]| format!("[{:.6}, {:.6}, {:.6}, {:.6}]", a[0], a[1], a[2], a[3]);
+        for r in &reports {
+            let name = stage_name(r);
+            if name == "embedding" {
+                eprintln!("[diag] Embedding pos0 first4: {}", four(&r.pos0_first4));
+                eprintln!("[diag] Embedding pos{last} first4: {}", four(&r.last_first4));
+            } else if name == "block_0" || name == format!("block_{}", self.config.n_layer - 1) {
+                let i = &name[6..];
+                eprintln!("[diag] Layer {i} pos{last} first4: {}", four(&r.last_first4));
+                if r.non_finite > 0 {
+                    eprintln!("[diag] WARNING: Layer {i} has {} NaN/Inf values!", r.non_finite);
+                }
+            } else if name == "ln_f" {
+                eprintln!("[diag] Final LN pos{last} first4: {}", four(&r.last_first4));
+            }
+        }
+        eprintln!("[diag] Top-5 tokens at pos{last}:");
+        for (tok, score) in top_tok.iter().zip(top_val.iter()) {
+            eprintln!("  token {tok}: {score:.4}");
+        }
+        Ok(logits)
+    }
+
+    fn forward_staged(&self, tokens: &[u32], diagnostic: bool) -> Result<(Vec<f32>, Vec<sys::agpu_gpt2_stage_report>, [u32; 5], [f32; 5])> {
+        if tokens.is_empty() {
+            return Err(NnError::ShapeMismatch { expected: "a non-empty sequence".to_string(), actual: "0 tokens".to_string() });
+        }
+        let reg = &self.registry;
+        let v = self.config.vocab_size;
+        let mut reports = vec![sys::agpu_gpt2_stage_report::default(); self.config.n_layer + 3];
+        let (mut n, mut top_tok, mut top_val) = (0i32, [0u32; 5], [0f32; 5]);
+        let (mut dtok, mut dlog): (*mut c_void, *mut c_void) = (std::ptr::null_mut(), std::ptr::null_mut());
+        reg.check(unsafe { sys::agpu_malloc(reg.raw(), tokens.len() * 4, &mut dtok) })?;
+        reg.check(unsafe { sys::agpu_malloc(reg.raw(), v * 4, &mut dlog) })?;
+        let mut logits = vec![0f32; v];
+        let rc = (|| -> Result<()> {
+            reg.check(unsafe { sys::agpu_memcpy_h2d(reg.raw(), dtok, tokens.as_ptr() as *const c_void, tokens.len() * 4) })?;
+            reg.check(unsafe {
+                if diagnostic {
+                    sys::agpu_gpt2_forward_diagnostic(self.handle, dtok as *const u32, tokens.len() as i32, dlog as *mut f32, reports.as_mut_ptr(),
+                                                      reports.len() as i32, &mut n, top_tok.as_mut_ptr(), top_val.as_mut_ptr())
+                } else {
+                    sys::agpu_gpt2_forward_profiled(self.handle, dtok as *const u32, tokens.len() as i32, dlog as *mut f32, reports.as_mut_ptr(),
+                                                    reports.len() as i32, &mut n)
+                }
+            })?;
+            reg.check(unsafe { sys::agpu_memcpy_d2h(reg.raw(), logits.as_mut_ptr() as *mut c_void, dlog, v * 4) })
+        })();
+        unsafe {
+            sys::agpu_free(reg.raw(), dtok);
+            sys::agpu_free(reg.raw(), dlog);
+        }
+        reports.truncate(n as usize);
+        rc.map(|_| (logits, reports, top_tok, top_val))
+    }
+
     /// Int4Gpt2Model::generate (gpt2.rs:1535-1560): greedy, the whole sequence recomputed per token, stops before
     /// appending the end-of-text token 50256.
     pub fn generate(&self, prompt: &[u32], max_new_tokens: usize) -> Result<Vec<u32>> {
@@ -173,6 +240,11 @@ impl Int4Gpt2Model {
         out.truncate(len as usize);
         Ok(out)
     }
+}
+
+fn stage_name(r: &sys::agpu_gpt2_stage_report) -> String {
+    let bytes: Vec<u8> = r.name.iter().take_while(|&&c| c != 0).map(|&c| c as u8).collect();
+    String::from_utf8_lossy(&bytes).into_owned()
 }
 
 impl Drop for Int4Gpt2Model {

@@ -15,6 +15,17 @@ pub struct agpu_ctx {
     _private: [u8; 0],
 }
 
+/// `agpu_gpt2_stage_report` of include/agpu_gpt2.h: one stage of forward_profiled / forward_diagnostic.
+#[repr(C)]
+#[derive(Clone, Copy, Debug, Default)]
+pub struct agpu_gpt2_stage_report {
+    pub name: [c_char; 24],
+    pub ms: f32,
+    pub pos0_first4: [f32; 4],
+    pub last_first4: [f32; 4],
+    pub non_finite: i32,
+}
+
 /// Opaque int4 GPT-2 model.
 #[repr(C)]
 pub struct agpu_gpt2 {
@@ -134,6 +145,8 @@ extern "C" {
     pub fn agpu_gpt2_generate_cached(m: *mut agpu_gpt2, prompt_host: *const u32, batch: i32, prompt_len: i32, max_new_tokens: i32, eos: i32, tokens_out_host: *mut u32, lengths_out_host: *mut i32, timing_ms_out_host: *mut f32) -> i32;
     pub fn agpu_gpt2_generate(m: *mut agpu_gpt2, prompt_host: *const u32, prompt_len: i32, max_new_tokens: i32, eos: i32, tokens_out_host: *mut u32, length_out_host: *mut i32) -> i32;
     pub fn agpu_gpt2_generate_cached_sampling(m: *mut agpu_gpt2, prompt_host: *const u32, prompt_len: i32, max_new_tokens: i32, top_k: i32, temperature: f32, rng_state: *mut u64, eos: i32, tokens_out_host: *mut u32, length_out_host: *mut i32) -> i32;
+    pub fn agpu_gpt2_forward_profiled(m: *mut agpu_gpt2, tokens: *const u32, seq_len: i32, logits_out: *mut f32, reports_out_host: *mut agpu_gpt2_stage_report, capacity: i32, n_reports_out_host: *mut i32) -> i32;
+    pub fn agpu_gpt2_forward_diagnostic(m: *mut agpu_gpt2, tokens: *const u32, seq_len: i32, logits_out: *mut f32, reports_out_host: *mut agpu_gpt2_stage_report, capacity: i32, n_reports_out_host: *mut i32, top5_tokens_out_host: *mut u32, top5_logits_out_host: *mut f32) -> i32;
     pub fn agpu_gpt2_forward_early_exit(m: *mut agpu_gpt2, tokens: *const u32, seq_len: i32, threshold: f32, logits_out: *mut f32, layers_used_out_host: *mut i32) -> i32;
     pub fn agpu_gpt2_generate_cached_early_exit(m: *mut agpu_gpt2, prompt_host: *const u32, prompt_len: i32, max_new_tokens: i32, threshold: f32, eos: i32, tokens_out_host: *mut u32, length_out_host: *mut i32, layers_out_host: *mut i32, steps_out_host: *mut i32) -> i32;
     pub fn agpu_gpt2_set_decode_mode(m: *mut agpu_gpt2, mode: i32) -> i32;

@@ -389,3 +389,63 @@ def test_long_prompts_in_a_batch(orc, agpu, dev, batch, prompt_len):
         (alone,), _ = one.generate_cached(prompts[b], 6, eos=-1)
         assert np.array_equal(outs[b], alone), b
 
+
+
+def test_gpt2_inference_example_program(orc, agpu, dev, tmp_path):
+    """The reference's example program (examples/std/gpt2-inference/src/main.rs:22-135) on this library: random fp32
+    weights in a safetensors file, a byte-level vocabulary trained here and written in tiktoken's format; the program
+    loads both, prints the diagnostic forward, and its uncached and KV-cached generations agree for all three prompts."""
+    import io
+    import importlib.util
+    import os
+    from async_gpu_amd import tokenizer, weights, workloads
+    from test_tokenizer import CORPUS, train
+    ranks, _ = train(CORPUS, 120)
+    tok = tokenizer.Gpt2Tokenizer(ranks)
+    vocab_path = str(tmp_path / "vocab.tiktoken")
+    tok.save_tiktoken_file(vocab_path)
+    cfg = dict(n_layer=2, n_embd=128, n_head=2, vocab=tok.vocab_size(), n_positions=96)
+    w = workloads.gpt2_fp32_weights(cfg, 8, std=0.08, nonzero_bias=True, random_ln=True)
+    model_path = str(tmp_path / "model.safetensors")
+    weights.save_gpt2_safetensors(model_path, w)
+    prog = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "async-gpu_amd", "examples", "gpt2_inference.py")
+    spec = importlib.util.spec_from_file_location("gpt2_inference_example", prog)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    out, err = io.StringIO(), io.StringIO()
+    assert mod.run(model_path, vocab_path, max_new_tokens=20, out=out, err=err)
+    text, diag = out.getvalue(), err.getvalue()
+    assert text.count("MATCH: cached and non-cached outputs agree") == 3 and "MISMATCH" not in text
+    assert "Model built on GPU" in text and text.count("ms/token)") == 6 and text.rstrip().endswith("Done.")
+    for line in ("[diag] Embedding pos0 first4:", "[diag] Layer 0 pos", "[diag] Layer 1 pos", "[diag] Final LN pos", "[diag] Top-5 tokens at pos"):
+        assert line in diag, diag
+    assert diag.count("  token ") == 5
+
+
+def test_forward_profiled_and_diagnostic(tiny, orc, agpu, dev):
+    """forward_profiled / forward_diagnostic (gpt2.rs:529-667): the stage list, positive timings, logits equal to the
+    forward's last row; the diagnostic's values against the oracle's intermediate results where it exposes them (the
+    logits) and against the model's own forward (embedding rows, top-5)."""
+    cfg, w, qz, om, gm = tiny
+    from async_gpu_amd import workloads
+    prompt = workloads.random_prompt(cfg, 4, 11)
+    gm.reset_cache()
+    ref = gm.forward_cached(prompt.reshape(1, -1), all_rows=False)[0]  # the last row through the same one-row head
+    logits, timings = gm.forward_profiled(prompt)
+    assert [n for n, _ in timings] == ["embedding"] + [f"block_{i}" for i in range(cfg["n_layer"])] + ["ln_f", "lm_head"]
+    assert all(ms > 0.0 for _, ms in timings)
+    assert np.array_equal(logits, ref)
+    assert gm.cache_len() == prompt.size
+    import io
+    buf = io.StringIO()
+    logits, reports, top_tok, top_val = gm.forward_diagnostic(prompt, out=buf)
+    assert np.array_equal(logits, ref)
+    emb0 = qz["wte"][prompt[0]] + qz["wpe"][0]
+    emb_last = qz["wte"][prompt[-1]] + qz["wpe"][prompt.size - 1]
+    assert np.array_equal(np.array(reports[0].pos0_first4[:]), emb0[:4]) and np.array_equal(np.array(reports[0].last_first4[:]), emb_last[:4])
+    assert all(r.non_finite == 0 for r in reports)
+    order = np.lexsort((np.arange(ref.size), -ref.astype(np.float64)))[:5]
+    assert list(top_tok) == list(order) and np.array_equal(top_val, ref[order])
+    om.reset_cache()
+    assert np.abs(om.forward(prompt, all_rows=False)[0] - logits).max() <= TOL_LOGITS
+    assert buf.getvalue().count("[diag]") >= 6
