@@ -23,39 +23,63 @@ pub enum Residency {
     HostDirty,
 }
 
-enum DeviceStorage {
-    Mapped { host: *mut c_void, dev: *mut c_void, reg: Arc<KernelRegistry> },
-    DeviceMem { dev: *mut c_void, reg: Arc<KernelRegistry> },
+/// Where the device side of an array lives: `dev` is what kernels are given; `alias` is the same bytes as the host sees
+/// them when the memory is pinned and mapped (small arrays), null when it is device memory that needs explicit copies.
+struct Backing {
+    dev: *mut c_void,
+    alias: *mut c_void,
+    bytes: usize,
+    reg: Arc<KernelRegistry>,
 }
 
-impl DeviceStorage {
-    fn dev_ptr(&self) -> u64 {
-        match self {
-            DeviceStorage::Mapped { dev, .. } | DeviceStorage::DeviceMem { dev, .. } => *dev as u64,
+impl Backing {
+    fn create(reg: &Arc<KernelRegistry>, bytes: usize, mapped: bool) -> Result<Backing> {
+        let (mut alias, mut dev): (*mut c_void, *mut c_void) = (std::ptr::null_mut(), std::ptr::null_mut());
+        if mapped {
+            reg.check(unsafe { sys::agpu_host_alloc_mapped(reg.raw(), bytes, &mut alias, &mut dev) })?;
+        } else {
+            reg.check(unsafe { sys::agpu_malloc(reg.raw(), bytes, &mut dev) })?;
         }
+        Ok(Backing { dev, alias, bytes, reg: Arc::clone(reg) })
+    }
+
+    /// Host bytes to the device side.  Mapped memory is written in place once nothing on the stream can still be reading it.
+    fn push(&self, src: *const c_void) -> Result<()> {
+        if self.alias.is_null() {
+            return self.reg.check(unsafe { sys::agpu_memcpy_h2d(self.reg.raw(), self.dev, src, self.bytes) });
+        }
+        self.reg.synchronize()?;
+        unsafe { std::ptr::copy_nonoverlapping(src as *const u8, self.alias as *mut u8, self.bytes) };
+        Ok(())
+    }
+
+    /// The device side back into host bytes, once the kernels that wrote it have finished.
+    fn pull(&self, dst: *mut c_void) -> Result<()> {
+        if self.alias.is_null() {
+            return self.reg.check(unsafe { sys::agpu_memcpy_d2h(self.reg.raw(), dst, self.dev, self.bytes) });
+        }
+        self.reg.synchronize()?;
+        unsafe { std::ptr::copy_nonoverlapping(self.alias as *const u8, dst as *mut u8, self.bytes) };
+        Ok(())
     }
 }
 
-impl Drop for DeviceStorage {
+impl Drop for Backing {
     fn drop(&mut self) {
         unsafe {
-            match self {
-                DeviceStorage::Mapped { host, reg, .. } => {
-                    sys::agpu_host_free_mapped(reg.raw(), *host);
-                }
-                DeviceStorage::DeviceMem { dev, reg } => {
-                    sys::agpu_free(reg.raw(), *dev);
-                }
+            if self.alias.is_null() {
+                sys::agpu_free(self.reg.raw(), self.dev);
+            } else {
+                sys::agpu_host_free_mapped(self.reg.raw(), self.alias);
             }
         }
     }
 }
 
 pub struct GpuArray<T: Copy + Send + 'static> {
-    host: UnsafeCell<Vec<T>>,
-    device: UnsafeCell<Option<DeviceStorage>>,
-    residency: Cell<Residency>,
-    len: usize,
+    elems: UnsafeCell<Vec<T>>,
+    backing: UnsafeCell<Option<Backing>>,
+    state: Cell<Residency>,
 }
 
 // Ownership may move between threads; shared access from two threads is not supported (Cell, UnsafeCell), as in the
@@ -64,113 +88,79 @@ unsafe impl<T: Copy + Send + 'static> Send for GpuArray<T> {}
 
 impl<T: Copy + Send + 'static> GpuArray<T> {
     pub fn from_vec(data: Vec<T>) -> Self {
-        let len = data.len();
-        GpuArray { host: UnsafeCell::new(data), device: UnsafeCell::new(None), residency: Cell::new(Residency::HostOnly), len }
+        GpuArray { elems: UnsafeCell::new(data), backing: UnsafeCell::new(None), state: Cell::new(Residency::HostOnly) }
     }
     pub fn from_slice(data: &[T]) -> Self {
         Self::from_vec(data.to_vec())
     }
     pub fn len(&self) -> usize {
-        self.len
+        self.host().len()
     }
     pub fn is_empty(&self) -> bool {
-        self.len == 0
+        self.len() == 0
     }
     pub fn residency(&self) -> Residency {
-        self.residency.get()
+        self.state.get()
     }
     pub fn should_use_mapped(&self) -> bool {
-        self.len * std::mem::size_of::<T>() < SIZE_THRESHOLD_BYTES
+        self.bytes() < SIZE_THRESHOLD_BYTES
     }
     fn bytes(&self) -> usize {
-        self.len * std::mem::size_of::<T>()
+        self.len() * std::mem::size_of::<T>()
+    }
+    fn host(&self) -> &Vec<T> {
+        unsafe { &*self.elems.get() }
+    }
+    fn backing(&self) -> Option<&Backing> {
+        unsafe { &*self.backing.get() }.as_ref()
     }
 
-    /// Device-to-host sync (gpu_array.rs:178-218); the caller holds the only reference to the host data.
-    fn sync_to_host_fallible(&self) -> Result<()> {
-        let storage = unsafe { &*self.device.get() };
-        let host = unsafe { &mut *self.host.get() };
-        if let Some(st) = storage {
-            match st {
-                DeviceStorage::Mapped { host: mapped, reg, .. } => {
-                    reg.synchronize()?; // the kernel that wrote the memory has finished
-                    unsafe { std::ptr::copy_nonoverlapping(*mapped as *const T, host.as_mut_ptr(), self.len) };
-                }
-                DeviceStorage::DeviceMem { dev, reg } => {
-                    reg.check(unsafe { sys::agpu_memcpy_d2h(reg.raw(), host.as_mut_ptr() as *mut c_void, *dev, self.bytes()) })?;
-                }
+    /// The one place where copies happen.  `newer_on_device` false: make the device side current (creating it on first
+    /// use) and return its address; true: make the host side current.  Either way the array ends up Synced.
+    fn reconcile(&self, reg: Option<&Arc<KernelRegistry>>, newer_on_device: bool) -> Result<u64> {
+        if newer_on_device {
+            if let Some(b) = self.backing() {
+                b.pull(unsafe { &mut *self.elems.get() }.as_mut_ptr() as *mut c_void)?;
             }
+            self.state.set(Residency::Synced);
+            return Ok(self.backing().map(|b| b.dev as u64).unwrap_or(0));
         }
-        self.residency.set(Residency::Synced);
-        Ok(())
+        if self.is_empty() {
+            self.state.set(Residency::Synced);
+            return Ok(0);
+        }
+        if self.backing().is_none() {
+            let reg = reg.expect("GpuArray: no registry to create the device side with");
+            let made = Backing::create(reg, self.bytes(), self.should_use_mapped())?;
+            unsafe { *self.backing.get() = Some(made) };
+        }
+        let b = self.backing().unwrap();
+        b.push(self.host().as_ptr() as *const c_void)?;
+        self.state.set(Residency::Synced);
+        Ok(b.dev as u64)
     }
 
     /// try_sync_to_host (gpu_array.rs:208-225): the host data, with a sync error returned instead of a panic.
     pub fn try_sync_to_host(&self) -> Result<&[T]> {
-        if self.residency.get() == Residency::DeviceOnly {
-            self.sync_to_host_fallible()?;
+        if self.state.get() == Residency::DeviceOnly {
+            self.reconcile(None, true)?;
         }
-        Ok(unsafe { &*self.host.get() })
+        Ok(self.host())
     }
 
     /// mark_device_dirty (gpu_array.rs:227-240): a kernel wrote the device copy.
     pub fn mark_device_dirty(&self) {
-        if self.residency.get() == Residency::Synced {
-            self.residency.set(Residency::DeviceOnly);
+        if self.state.get() == Residency::Synced {
+            self.state.set(Residency::DeviceOnly);
         }
     }
 
-    /// ensure_device (gpu_array.rs:241-340): the device address of the data, uploaded if the host copy is newer.
+    /// ensure_device (gpu_array.rs:241-340): the device address of the data, uploaded if the host copy is newer
+    /// (HostOnly: first upload; HostDirty: the host was written since the last one).
     pub fn ensure_device(&self, reg: &Arc<KernelRegistry>) -> Result<u64> {
-        match self.residency.get() {
-            Residency::HostOnly => {
-                if self.len == 0 {
-                    self.residency.set(Residency::Synced);
-                    return Ok(0);
-                }
-                let host = unsafe { &*self.host.get() };
-                let storage = if self.should_use_mapped() {
-                    let (mut h, mut d): (*mut c_void, *mut c_void) = (std::ptr::null_mut(), std::ptr::null_mut());
-                    reg.check(unsafe { sys::agpu_host_alloc_mapped(reg.raw(), self.bytes(), &mut h, &mut d) })?;
-                    unsafe { std::ptr::copy_nonoverlapping(host.as_ptr(), h as *mut T, self.len) };
-                    DeviceStorage::Mapped { host: h, dev: d, reg: Arc::clone(reg) }
-                } else {
-                    let mut d: *mut c_void = std::ptr::null_mut();
-                    reg.check(unsafe { sys::agpu_malloc(reg.raw(), self.bytes(), &mut d) })?;
-                    let st = DeviceStorage::DeviceMem { dev: d, reg: Arc::clone(reg) };
-                    reg.check(unsafe { sys::agpu_memcpy_h2d(reg.raw(), d, host.as_ptr() as *const c_void, self.bytes()) })?;
-                    st
-                };
-                let ptr = storage.dev_ptr();
-                unsafe { *self.device.get() = Some(storage) };
-                self.residency.set(Residency::Synced);
-                Ok(ptr)
-            }
-            Residency::HostDirty => {
-                let host = unsafe { &*self.host.get() };
-                let storage = unsafe { &*self.device.get() };
-                match storage {
-                    None => {
-                        // modified before the first upload: nothing on the device yet
-                        self.residency.set(Residency::HostOnly);
-                        self.ensure_device(reg)
-                    }
-                    Some(st) => {
-                        match st {
-                            DeviceStorage::Mapped { host: mapped, reg, .. } => {
-                                reg.synchronize()?; // no kernel may still be reading the old contents
-                                unsafe { std::ptr::copy_nonoverlapping(host.as_ptr(), *mapped as *mut T, self.len) };
-                            }
-                            DeviceStorage::DeviceMem { dev, reg } => {
-                                reg.check(unsafe { sys::agpu_memcpy_h2d(reg.raw(), *dev, host.as_ptr() as *const c_void, self.bytes()) })?;
-                            }
-                        }
-                        self.residency.set(Residency::Synced);
-                        Ok(st.dev_ptr())
-                    }
-                }
-            }
-            Residency::Synced | Residency::DeviceOnly => Ok(unsafe { &*self.device.get() }.as_ref().map(|s| s.dev_ptr()).unwrap_or(0)),
+        match self.state.get() {
+            Residency::HostOnly | Residency::HostDirty => self.reconcile(Some(reg), false),
+            Residency::Synced | Residency::DeviceOnly => Ok(self.backing().map(|b| b.dev as u64).unwrap_or(0)),
         }
     }
 }
@@ -185,20 +175,20 @@ impl<T: Copy + Send + Default + 'static> GpuArray<T> {
 impl<T: Copy + Send + 'static> Deref for GpuArray<T> {
     type Target = [T];
     fn deref(&self) -> &[T] {
-        if self.residency.get() == Residency::DeviceOnly {
-            self.sync_to_host_fallible().expect("GpuArray: device-to-host sync failed");
+        if self.state.get() == Residency::DeviceOnly {
+            self.reconcile(None, true).expect("GpuArray: device-to-host sync failed");
         }
-        unsafe { &*self.host.get() }
+        self.host()
     }
 }
 
 impl<T: Copy + Send + 'static> DerefMut for GpuArray<T> {
     fn deref_mut(&mut self) -> &mut [T] {
-        if self.residency.get() == Residency::DeviceOnly {
-            self.sync_to_host_fallible().expect("GpuArray: device-to-host sync failed");
+        if self.state.get() == Residency::DeviceOnly {
+            self.reconcile(None, true).expect("GpuArray: device-to-host sync failed");
         }
-        self.residency.set(Residency::HostDirty);
-        unsafe { &mut *self.host.get() }
+        self.state.set(Residency::HostDirty);
+        self.elems.get_mut().as_mut_slice()
     }
 }
 
@@ -226,7 +216,7 @@ impl<T: Copy + Send + 'static> AsDevicePtr for GpuArray<T> {
         GpuArray::ensure_device(self, reg)
     }
     fn device_len(&self) -> usize {
-        self.len
+        self.len()
     }
     fn mark_device_dirty(&self) {
         GpuArray::mark_device_dirty(self)
@@ -234,38 +224,36 @@ impl<T: Copy + Send + 'static> AsDevicePtr for GpuArray<T> {
 }
 
 #[cfg(test)]
-mod tests {
-    use super::*;
+mod host_side {
+    use super::{GpuArray, Residency};
 
-    // The host-only life cycle, as the reference tests it (gpu_array.rs:434-514).
+    // What can be checked without a device: the states a host-only array goes through (the reference checks the same
+    // properties in gpu_array.rs:434-514), and on which side of 64 KiB an array falls.
     #[test]
-    fn from_vec_creates_host_only() {
-        let arr = GpuArray::from_vec(vec![1.0f32, 2.0, 3.0]);
-        assert_eq!(arr.residency(), Residency::HostOnly);
-        assert_eq!(arr.len(), 3);
-        assert!(!arr.is_empty());
+    fn a_fresh_array_lives_on_the_host() {
+        let a = GpuArray::from_slice(&[4u32, 5, 6, 7]);
+        assert!(a.residency() == Residency::HostOnly && a.len() == 4 && !a.is_empty());
+        assert_eq!(&a[..], &[4, 5, 6, 7]);
     }
 
     #[test]
-    fn deref_mut_marks_host_dirty() {
-        let mut arr = GpuArray::from_vec(vec![1.0f32, 2.0, 3.0]);
-        arr[0] = 99.0;
-        assert_eq!(arr.residency(), Residency::HostDirty);
-        assert_eq!(arr[0], 99.0);
+    fn writing_through_the_array_makes_the_host_newer() {
+        let mut a: GpuArray<f64> = vec![0.5, 1.5].into();
+        a[1] = -2.0;
+        assert!(a.residency() == Residency::HostDirty);
+        assert_eq!(a.try_sync_to_host().unwrap(), &[0.5, -2.0]);
     }
 
     #[test]
-    fn size_thresholds() {
-        assert!(GpuArray::from_vec(vec![0.0f32; 100]).should_use_mapped());
-        assert!(!GpuArray::from_vec(vec![0.0f32; 16384]).should_use_mapped());
-        assert!(GpuArray::from_vec(vec![0.0f32; 16383]).should_use_mapped());
+    fn sixty_four_kib_is_the_first_size_in_device_memory() {
+        for (n, mapped) in [(1usize, true), (16383, true), (16384, false), (100_000, false)] {
+            assert_eq!(GpuArray::<f32>::zeroed(n).should_use_mapped(), mapped, "{n} floats");
+        }
     }
 
     #[test]
-    fn empty_and_zeroed() {
-        let arr = GpuArray::<f32>::from_vec(vec![]);
-        assert!(arr.is_empty());
-        let z = GpuArray::<f32>::zeroed(100);
-        assert!(z.iter().all(|&x| x == 0.0));
+    fn an_empty_array_is_empty() {
+        assert!(GpuArray::<u8>::from_vec(Vec::new()).is_empty());
+        assert!(GpuArray::<i32>::zeroed(9).iter().all(|&v| v == 0));
     }
 }
