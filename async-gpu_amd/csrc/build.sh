@@ -17,6 +17,15 @@ pids+=($!)
 for p in "${pids[@]}"; do wait "$p"; done
 "$HIPCC" --offload-arch=gfx950 -shared -fPIC -o ../libagpu_hip.so build/*.o -fopenmp
 echo "built $(cd .. && pwd)/libagpu_hip.so"
+# The same library with time stamps inside the one-launch decode step (bench_configs.py --stamps): the two sources that
+# know about them compiled again with -DAGPU_PK_TRACE, every other object shared.
+mkdir -p build/trace
+cp build/*.o build/trace/
+"$HIPCC" "${FLAGS[@]}" -DAGPU_PK_TRACE -c decode_xcd.hip -o build/trace/decode_xcd.o &
+"$HIPCC" "${FLAGS[@]}" -DAGPU_PK_TRACE -c gpt2_model.hip -o build/trace/gpt2_model.o &
+wait
+"$HIPCC" --offload-arch=gfx950 -shared -fPIC -o ../libagpu_hip_trace.so build/trace/*.o -fopenmp
+echo "built $(cd .. && pwd)/libagpu_hip_trace.so"
 # C++ host-layer test (include/agpu_nn.hpp); runs on the GPU box from tests/test_gpu_cpp.py
 g++ -O1 -std=c++17 -I../../include ../../tests/cpp/test_nn.cpp -o ../../tests/cpp/test_nn \
     -L.. -lagpu_hip -Wl,-rpath,'$ORIGIN/../../async-gpu_amd' -Wl,-rpath,/opt/rocm/lib -L/opt/rocm/lib -lamdhip64

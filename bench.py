@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, GB/s
 # of the LM-head GEMV (profiles/gemv_lm_head_pmc_traffic.md) and of the one-launch decode step
 # (profiles/decode_step_gpt2_small_pmc_traffic.md); None where not measured.
 TRAFFIC_BYTES_LM_HEAD = 24617000
-TRAFFIC_BYTES_DECODE_STEP = 96900000  # at contexts 64 .. 132; 85.1 MB algorithmic there
+TRAFFIC_BYTES_DECODE_STEP = 101696400  # at contexts 64 .. 132; 85.1 MB algorithmic there
 
 
 def step_bytes(cfg, group, context_len):
@@ -172,7 +172,8 @@ def main():
     lm = roofline_lm_head(model.ctx, cfg, group, workloads)
     if one_launch:
         achieved = sb / (us_launch * 1e-6) / 1e9
-        roof = {"bound": "hbm", "kernel": "decode_step_kernel<0> (one launch = one decode step: 48 Linears, 12 attentions, LM head, arg-max)",
+        roof = {"bound": "hbm", "kernel": "decode_xcd_kernel<0> (one launch = one decode step, the eight XCDs as tensor-parallel ranks: "
+                          "48 Linears, 12 attentions, 24 partial-sum exchanges, LM head, arg-max)",
                 "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5),
                 "traffic": TRAFFIC_BYTES_DECODE_STEP, "bytes_per_launch": int(sb), "us_per_launch": round(us_launch, 3),
                 "context_mid": ctx_mid,
@@ -205,8 +206,8 @@ def main():
                    "decode_path": "one launch per token" if one_launch else "one launch per stage (HIP graph)",
                    "context_at_start": ctx0, "steps_event_ms": round(ms_events, 4), "model_build_s": round(build_s, 2)},
         "latency_floor_ms": None if floor_ms is None else round(floor_ms, 5),
-        "latency_floor_note": "the one-launch step's stage chain with empty bodies: every wait, barrier and tagged store, no "
-                              "weights and no arithmetic",
+        "latency_floor_note": "the one-launch step's stage chain with empty bodies: every wait, barrier and store of an "
+                              "activation, no weights and no arithmetic",
         "roofline": roof,
         "roofline_lm_head": lm,
     }

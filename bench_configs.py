@@ -5,6 +5,7 @@ attention prefill / decode, and GPT-2 XL-shaped decode at batch 1 and 16.  Print
 case.  Kernel cases are timed as graph replays with HIP events on the context's stream.
 
     python3 bench_configs.py [--xl-layers 48] [--skip-xl] [--skip-kernels] [--prefill-only]
+    python3 bench_configs.py --stamps [small|xl]     time stamps inside the one-launch decode step (libagpu_hip_trace.so)
 """
 import argparse
 import ctypes as C
@@ -30,9 +31,17 @@ def main():
     ap.add_argument("--prefill-only", action="store_true", help="only the whole-model prefill of GPT-2 small (for kernel traces)")
     ap.add_argument("--eager", action="store_true", help="XL-shaped decode at batch 16 without HIP graphs (for kernel traces)")
     ap.add_argument("--cpu", action="store_true", help="also time the CPU oracle on configs 1-3 (single thread, as the reference CPU path)")
+    ap.add_argument("--xl-batch", type=int, nargs="+", default=[1, 16], help="batch sizes of the XL-shaped decode")
+    ap.add_argument("--with-copy", action="store_true",
+                    help="finish with ten 64 MiB device copies (calibration of FETCH_SIZE / WRITE_SIZE in rocprofv3 --pmc runs)")
+    ap.add_argument("--stamps", choices=("small", "xl"), help="per-stage time stamps of one one-launch decode step (needs libagpu_hip_trace.so)")
     args = ap.parse_args()
     entry.load_package()
     from async_gpu_amd import _lib, gpt2, workloads
+
+    if args.stamps:
+        stamp_table(args.stamps, args.xl_layers, _lib, gpt2, workloads)
+        return
 
     ctx = _lib.Context(0)
 
@@ -58,9 +67,90 @@ def main():
     if not args.skip_kernels:
         kernel_cases(ctx, emit, bench_linear, workloads, args)
         prefill_cases(ctx, emit, _lib, gpt2, workloads)
-    if args.skip_xl:
-        return
-    xl_cases(ctx, emit, args, _lib, gpt2, workloads)
+    if not args.skip_xl:
+        xl_cases(ctx, emit, args, _lib, gpt2, workloads)
+    if args.with_copy:
+        n = 64 << 20
+        a, b = ctx.malloc(n), ctx.malloc(n)
+        for _ in range(10):
+            ctx.call("agpu_memcpy_d2d", b, a, n)
+        ctx.sync()
+        emit(calibration_copy_bytes=n)
+
+
+def stamp_table(which, xl_layers, _lib, gpt2, workloads):
+    """Where the time of a one-launch decode step goes: thread 0 of every workgroup stamps the device clock (10 ns ticks)
+    at fixed points of every stage; printed per stage as median / slowest over the workgroups that took part, in ns from
+    the launch's first stamp.  Linear workgroups: input arrived, staged in LDS, dot products done, outputs stored.
+    Attention: q arrived, outputs stored.  Relays: partial sums of all XCDs in, sum stored into the mirror."""
+    from async_gpu_amd import ops
+    _lib._SO = os.path.join(os.path.dirname(_lib._SO), "libagpu_hip_trace.so")
+    cfg = workloads.GPT2_SMALL if which == "small" else dict(workloads.GPT2_XL, n_layer=xl_layers)
+    quant = lambda wt, g: ops.int4_quantize_host(wt, g, _lib.QUANT_SCRIPT)
+    qz = workloads.gpt2_quantized_layerwise(cfg, 3, 32, quant)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpt2.Gpt2Config(cfg["n_layer"], cfg["n_embd"], cfg["n_head"], vocab_size=cfg["vocab"]), qz)
+    prompt = workloads.random_prompt(cfg, 3, 64 if which == "small" else 256)
+    (_,), t = gm.generate_cached(prompt, 33, eos=-1)
+    assert gm.decode_is_one_launch()
+    lib = _lib.cdll()
+    fn = lib.agpu_gpt2_decode_trace
+    fn.restype = C.c_int32
+    fn.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]
+    n_stages = 4 * cfg["n_layer"] + 1
+    buf = np.zeros(256 * n_stages * 8, np.uint64)
+    g, ns = C.c_int32(0), C.c_int32(0)
+    for _ in range(3):  # the last of three steps is the one looked at
+        rc = fn(gm.handle, 0, buf.ctypes.data, C.addressof(g), C.addressof(ns))
+        assert rc == 0, rc
+    G, NS = g.value, ns.value
+    tr = buf[:G * NS * 8].reshape(G, NS, 8).astype(np.int64)
+    t0 = tr[tr > 0].min()
+    tr = np.where(tr > 0, (tr - t0) * 10, -1)
+    hx = (cfg["n_head"] + 7) // 8
+    n_relay, n_att = 4, hx * (2 if hx <= 2 else 1)  # roles per XCD as decode_xcd.hip plans them
+    in_xcd = np.arange(G) >> 3
+    relay, att = in_xcd < n_relay, (in_xcd >= n_relay) & (in_xcd < n_relay + n_att)
+    lin = ~relay & ~att
+
+    def ms(a):
+        a = a[a >= 0]
+        return f"{int(np.median(a)):7d} / {int(a.max()):7d}" if a.size else "      - /       -"
+
+    print(f"{which}: context {gm.cache_len() - 1}, step {t[1] / 32:.4f} ms with the stamps compiled in; median / slowest, ns since the first stamp")
+    print("| layer | stage | workgroups | input arrived | staged | dot products done | stored |")
+    print("|---|---|---|---|---|---|---|")
+    names = ("LN1 + QKV", "proj (partial sums)", "LN2 + fc + GELU", "fc-proj (partial sums)")
+    shown = [0, 1, 2, cfg["n_layer"] // 2, cfg["n_layer"] - 1]
+    for L in shown:
+        for k in range(4):
+            s = 4 * L + k
+            w = tr[lin][:, s, :]
+            w = w[w[:, 1] >= 0]
+            print(f"| {L} | {names[k]} | {len(w)} | {ms(w[:, 1])} | {ms(w[:, 2])} | {ms(w[:, 4])} | {ms(w[:, 3])} |")
+            if k == 0:
+                a = tr[att][:, s, :]
+                a = a[a[:, 1] >= 0]
+                print(f"| {L} | attention | {len(a)} | {ms(a[:, 1])} | - | {ms(a[:, 2])} | {ms(a[:, 3])} |")
+            if k in (1, 3):
+                r = tr[relay][:, s, :]
+                print(f"| {L} | exchange {k // 2 + 1} (relays) | {len(r)} | {ms(r[:, 6])} | - | - | {ms(r[:, 7])} |")
+    h = tr[~relay][:, NS - 1, :]
+    h = h[h[:, 1] >= 0]
+    print(f"| - | final LN + LM head | {len(h)} | {ms(h[:, 1])} | {ms(h[:, 2])} | {ms(h[:, 4])} (first chunk) | {ms(h[:, 3])} |")
+    # one layer's chain from the medians: stage to stage
+    L = shown[3]
+    q, p_, f, o = (tr[lin][:, 4 * L + k, :] for k in range(4))
+    nq = tr[lin][:, 4 * (L + 1), :]
+    a = tr[att][:, 4 * L, :]
+    r1, r2 = tr[relay][:, 4 * L + 1, :], tr[relay][:, 4 * L + 3, :]
+    med = lambda x, c: int(np.median(x[x[:, c] >= 0][:, c]))
+    chain = [("LN1 + QKV in the workgroup", med(q, 3) - med(q, 1)), ("-> attention (L2)", med(a, 1) - med(q, 3)),
+             ("attention in the workgroup", med(a, 3) - med(a, 1)), ("-> proj (L2)", med(p_, 1) - med(a, 3)),
+             ("proj in the workgroup", med(p_, 3) - med(p_, 1)), ("-> exchange 1 -> fc (memory, sum, L2)", med(f, 1) - med(p_, 3)),
+             ("LN2 + fc in the workgroup", med(f, 3) - med(f, 1)), ("-> fc-proj (L2)", med(o, 1) - med(f, 3)),
+             ("fc-proj in the workgroup", med(o, 3) - med(o, 1)), ("-> exchange 2 -> next QKV (memory, sum, L2)", med(nq, 1) - med(o, 3))]
+    print(f"\nlayer {L}, stage to stage (medians, ns): " + "; ".join(f"{n} {v}" for n, v in chain) + f"; sum {sum(v for _, v in chain)}")
+    print(f"relays of layer {L}: partial sums in {ms(r1[:, 6])} and {ms(r2[:, 6])}, sums stored {ms(r1[:, 7])} and {ms(r2[:, 7])}")
 
 
 def prefill_cases(ctx, emit, _lib, gpt2, workloads, lengths=(1024, 512, 128, 32)):
@@ -182,7 +272,7 @@ def xl_cases(ctx, emit, args, _lib, gpt2, workloads):
     build_s = time.time() - t0
     per_w = 0.5 + 4.0 / 32
     wbytes = cfg["n_layer"] * (12 * d * d * per_w + (3 * d + d + ff + d) * 4 + 4 * d * 4) + d * V * per_w
-    for B in (1, 16):
+    for B in args.xl_batch:
         model.set_decode_mode(model.DECODE_EAGER if args.eager and B > 1 else model.DECODE_AUTO)
         prompts = workloads.random_prompt(cfg, 4, 256, batch=B)
         model.reset_cache()
