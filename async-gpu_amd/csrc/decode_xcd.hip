@@ -628,7 +628,7 @@ __device__ __forceinline__ void ln_stats(const float4 *stat, float inv_k, float 
 // ---- one Linear of a layer, for a workgroup that has a unit of it ----
 // The finishing threads (one per column of the workgroup's units) request bias first; then the input; then every lane
 // its groups of its column; the waves of a unit meet in LDS and the finishing thread completes the column: bias, GELU,
-// the tagged store (into the XCD's mirror, or as a partial sum into memory), and for K and V columns the row of the cache.
+// the store (into the XCD's mirror, or as a partial sum into memory), and for K and V columns the row of the cache.
 template <int MODE>
 __device__ __forceinline__ void lay_stage(const Params &p, const Stage &st, Ctl &c, const Regs &r, float *xs, float *xsum, float4 *stat,
                                           float *red, float *mirror, int pos, uint32_t tok, int li, int tid) {
