@@ -63,6 +63,7 @@ SIGNATURES = {
     "agpu_ctx_set_strict_sync": (_i32, [_vp, _i32]),
     "agpu_ctx_test_hold": (_i32, [_vp, _i32]),
     "agpu_ln_int4_linear": (_i32, [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32]),
+    "agpu_int4_linear_pieces": (_i32, [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32, _vp, _vp, _vp]),
     "agpu_bench_int4_linear": (_i32, [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32,
                                       _i32, C.c_int64, C.c_int64, _i32, _vp]),
     "agpu_int4_dequantize": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32]),

@@ -24,6 +24,9 @@ struct AttnParams {
     float *kv_partial;
     unsigned int *counters;
     int strict;  // the context's strict_sync
+    // Decode kernel, q_len == 1 and batch <= 16 only: the outputs once more as the bf16 pieces of the next Linear's
+    // input (row = sequence, k = head * 64 + e; layout in linear_common.h), or null.
+    uint4 *px_pieces;
 };
 
 // max_kv_len bounds kv_len for launches that read it from pos_dev (sizes the key split).

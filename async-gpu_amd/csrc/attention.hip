@@ -8,6 +8,7 @@
 //     split the keys, 16 lanes share one key (float4 each), partial (m, l, o) merge in a fixed order.
 #include "agpu_internal.h"
 #include "attention.h"
+#include "linear_common.h"
 
 namespace {
 
@@ -516,11 +517,22 @@ __device__ __forceinline__ void merge_partial(float &m, float &l, float4 &o, flo
 constexpr int PASS = 8;
 constexpr int kMaxKeySplits = 8;
 
+// Wave 0 of a workgroup that has finished head h of sequence b: the 64 outputs, one per lane, also as bf16 pieces
+// (8 consecutive values per 16 bytes; `row` is LDS of the wave's own, and a wave's LDS operations complete in order).
+__device__ __forceinline__ void decode_pieces(const AttnParams &p, float *row, float val, int b, int h, int lane) {
+    row[lane] = val;
+    if (lane < 8) {
+        const float4 f0 = *reinterpret_cast<const float4 *>(row + 8 * lane), f1 = *reinterpret_cast<const float4 *>(row + 8 * lane + 4);
+        const float v[8] = {f0.x, f0.y, f0.z, f0.w, f1.x, f1.y, f1.z, f1.w};
+        px_store_pieces(p.px_pieces, h * DH + 8 * lane, b, v);
+    }
+}
+
 template <bool SPLIT>  // keys split over gridDim.z workgroups
 __global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
     __shared__ float sm[64], sl[64];
     __shared__ __align__(16) float so[64][DH];  // one row per lane group
-    __shared__ float so2[16][DH];               // one row per wave
+    __shared__ __align__(16) float so2[16][DH];  // one row per wave
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6;
     const int gq = lane >> 4, sub = lane & 15;
     const int qi = blockIdx.x, hb = blockIdx.y;
@@ -598,7 +610,9 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
         for (int w = 0; w < W; ++w) acc += so2[w][lane];
         float *orow = p.o + (size_t)b * p.o_batch_stride + (size_t)h * p.o_head_stride + (size_t)qi * p.o_row_stride;
         if constexpr (!SPLIT) {
-            orow[lane] = acc / l_all;
+            const float val = acc / l_all;
+            orow[lane] = val;
+            if (p.px_pieces) decode_pieces(p, so2[0], val, b, h, lane);
             return;
         }
         const int row = qi * gridDim.y + hb;
@@ -637,7 +651,9 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(const AttnParams p) {
             lsum += lz[zz] * f;
             osum += oz[zz] * f;
         }
-        orow[lane] = osum / lsum;
+        const float val = osum / lsum;
+        orow[lane] = val;
+        if (p.px_pieces) decode_pieces(p, so2[0], val, b, h, lane);
     }
 }
 

@@ -60,6 +60,12 @@ struct agpu_gpt2 {
     // activations (grown on demand, never inside a captured region)
     DevBuf hid, qkv, att, ffn, lnb, last, logits, tok_in;
     DevBuf kfrag, vfrag;  // K and V of one layer as bf16 operand fragments (prefill of one sequence from position 0)
+    // batched decode (5 .. 16 sequences): the inputs of the Linears as bf16 pieces left by their producers (hidden rows
+    // times the next LayerNorm's gains + their statistics, attention outputs, MLP activations), and per normalising
+    // Linear the two folded LayerNorm vectors: [layer][A qkv, B qkv, A fc, B fc], then the head's
+    DevBuf px_h, px_att, px_ffn, px_stats, px_fold;
+    bool px_fold_ready = false;
+    bool px_off = false;  // AGPU_NO_PX in the environment: keep to the kernels that split their inputs themselves
     uint32_t *cur_tok = nullptr, *next_tok = nullptr, *out_tok = nullptr;
     int out_capacity = 0;  // steps recorded in out_tok
     int *pos_dev = nullptr, *step_dev = nullptr;
@@ -209,7 +215,9 @@ unsigned long long step_addresses(const agpu_gpt2 *m, bool one_launch) {
         mix(p);
     if (one_launch)  // the step's plan; a graph of per-stage launches does not refer to it
         for (const void *p : {(const void *)m->pk.arena, (const void *)m->pk.stages_dev, (const void *)m->pk.state, (const void *)m->pk.ln_fold}) mix(p);
-    for (const DevBuf *b : {&m->hid, &m->qkv, &m->att, &m->ffn, &m->lnb, &m->last, &m->logits, &m->tok_in}) mix(b->p);
+    for (const DevBuf *b : {&m->hid, &m->qkv, &m->att, &m->ffn, &m->lnb, &m->last, &m->logits, &m->tok_in, &m->px_h, &m->px_att, &m->px_ffn,
+                            &m->px_stats, &m->px_fold})
+        mix(b->p);
     for (const Block &b : m->blocks) {
         for (const void *p : {(const void *)b.ln1_g, (const void *)b.ln1_b, (const void *)b.ln2_g, (const void *)b.ln2_b}) mix(p);
         for (const Int4Lin &l : b.lin) {
@@ -230,6 +238,12 @@ void drop_graphs(agpu_gpt2 *m) {
     // the plan of the one-launch step holds the same addresses
     agpu_step_plan_free(&m->pk);
     m->pk_tried = false;
+}
+
+// A weight setter has replaced a tensor: nothing captured or folded from the old ones may be used again.
+void weights_changed(agpu_gpt2 *m) {
+    drop_graphs(m);
+    m->px_fold_ready = false;
 }
 
 // Grow a buffer; existing graphs hold the old address, so they are dropped.
@@ -335,11 +349,66 @@ int32_t ln_linear(agpu_gpt2 *m, const float *x, const float *gamma, const float 
     return agpu_ln_int4_linear_kv(ctx, x, gamma, beta, eps, w.packed, w.scales, w.bias, residual, y, R, N, w.K, g, flags, kv, kv_done);
 }
 
+// Batched decode on pieces (int4_skinny.hip): one new position for 5 .. 16 sequences, every Linear's input left as bf16
+// pieces by the kernel that produced it.  Shapes: group a multiple of 32 up to 512, d and 4d multiples of 32, at most 64
+// tiles of 32 columns per hidden row.
+bool px_shape_ok(const agpu_gpt2 *m, int B, int new_len) {
+    const int g = m->cfg.group_size;
+    return !m->px_off && new_len == 1 && B > 4 && B <= 16 && g % 32 == 0 && g <= 512 && m->d % 32 == 0 && m->ff % 32 == 0 && m->d <= 2048;
+}
+bool px_active(const agpu_gpt2 *m, int B, int new_len) { return px_shape_ok(m, B, new_len) && m->px_fold_ready; }
+
+size_t px_fold_layer_floats(const agpu_gpt2 *m) { return 2 * ((size_t)3 * m->d + m->ff); }
+
+// Buffers and folded LayerNorm vectors of the pieces path; never inside a captured region.
+int32_t px_prepare(agpu_gpt2 *m) {
+    agpu_ctx *ctx = m->ctx;
+    const size_t d = m->d, ff = m->ff;
+    const bool int4_head = m->cfg.lm_head == AGPU_LM_HEAD_INT4;
+    int32_t rc;
+    auto grow = [&](DevBuf &b, size_t bytes) -> int32_t {
+        if (b.bytes >= bytes) return AGPU_OK;
+        int32_t r = ensure(m, b, bytes);
+        // rows beyond the batch are never written by anybody: zeros, not whatever the allocation held
+        if (r == AGPU_OK) r = agpu_hip(ctx, hipMemsetAsync(b.p, 0, bytes, ctx->stream), "hipMemsetAsync");
+        return r;
+    };
+    if ((rc = grow(m->px_h, d / 32 * 192 * 16)) != AGPU_OK) return rc;
+    if ((rc = grow(m->px_att, d / 32 * 192 * 16)) != AGPU_OK) return rc;
+    if ((rc = grow(m->px_ffn, ff / 32 * 192 * 16)) != AGPU_OK) return rc;
+    if ((rc = grow(m->px_stats, d / 32 * 16 * sizeof(float2))) != AGPU_OK) return rc;
+    if ((rc = grow(m->px_fold, (px_fold_layer_floats(m) * m->cfg.n_layer + (int4_head ? 2 * (size_t)m->Vpad : 0)) * sizeof(float))) != AGPU_OK)
+        return rc;
+    if (m->px_fold_ready) return AGPU_OK;
+    const int g = m->cfg.group_size;
+    float *fold = (float *)m->px_fold.p;
+    for (int L = 0; L < m->cfg.n_layer; ++L) {
+        const Block &b = m->blocks[L];
+        float *base = fold + px_fold_layer_floats(m) * L;
+        const Int4Lin &wq = b.lin[AGPU_LINEAR_QKV], &wf = b.lin[AGPU_LINEAR_FC];
+        if ((rc = agpu_px_fold_launch(ctx, wq.packed, wq.scales, (int)d, 3 * (int)d, g, b.ln1_g, b.ln1_b, base, base + 3 * d)) != AGPU_OK) return rc;
+        if ((rc = agpu_px_fold_launch(ctx, wf.packed, wf.scales, (int)d, (int)ff, g, b.ln2_g, b.ln2_b, base + 6 * d, base + 6 * d + ff)) != AGPU_OK)
+            return rc;
+    }
+    if (int4_head) {
+        float *hb = fold + px_fold_layer_floats(m) * m->cfg.n_layer;
+        if ((rc = agpu_px_fold_launch(ctx, m->lm_head.packed, m->lm_head.scales, (int)d, m->Vpad, g, m->lnf_g, m->lnf_b, hb, hb + m->Vpad)) != AGPU_OK)
+            return rc;
+    }
+    m->px_fold_ready = true;
+    return AGPU_OK;
+}
+
 int32_t launch_embed(agpu_gpt2 *m, const uint32_t *tokens, int B, int new_len) {
     const int R = B * new_len, d = m->d;
     hipLaunchKernelGGL(embed_rows_kernel, dim3((unsigned)(((size_t)R * d + 255) / 256)), dim3(256), 0, m->ctx->stream, tokens,
                        m->wte, m->wpe, (float *)m->hid.p, R, new_len, d, m->pos_dev, m->V, m->P);
-    return AGPU_LAUNCH_CHECK(m->ctx, "embed_rows_kernel");
+    int32_t rc = AGPU_LAUNCH_CHECK(m->ctx, "embed_rows_kernel");
+    if (rc == AGPU_OK && px_active(m, B, new_len)) {
+        const PxOut out{(uint4 *)m->px_h.p, m->blocks[0].ln1_g, (float2 *)m->px_stats.p};
+        rc = agpu_px_split_rows_launch(m->ctx, (const float *)m->hid.p, R, d, out);
+    }
+    return rc;
 }
 
 // Prompts long enough for eight key tiles (whole numbers of key tiles when there are several) into an empty cache: the QKV Linear also writes K and V as
@@ -370,6 +439,41 @@ int32_t launch_block(agpu_gpt2 *m, int L, int B, int new_len, int max_kv) {
     const Int4Lin &wq = b.lin[AGPU_LINEAR_QKV], &wp = b.lin[AGPU_LINEAR_PROJ], &wf = b.lin[AGPU_LINEAR_FC],
                   &wo = b.lin[AGPU_LINEAR_FC_PROJ];
     float *kc = m->kcache + L * layer_stride, *vc = m->vcache + L * layer_stride;
+    if (px_active(m, B, new_len)) {
+        // batched decode on pieces: QKV (LayerNorm folded, K/V rows to the cache) -> attention (outputs also as pieces) ->
+        // proj + residual (hidden rows, their pieces times LN2's gains, their statistics) -> fc + GELU (pieces) ->
+        // fc-proj + residual (hidden rows, pieces times the next LayerNorm's gains, statistics)
+        const float *fold = (const float *)m->px_fold.p + px_fold_layer_floats(m) * L;
+        uint4 *xh = (uint4 *)m->px_h.p, *xa = (uint4 *)m->px_att.p, *xf = (uint4 *)m->px_ffn.p;
+        float2 *st = (float2 *)m->px_stats.p;
+        GemvArgs ga{};
+        ga.packed = wq.packed; ga.scales = wq.scales; ga.bias = wq.bias; ga.y = qkv; ga.ln_eps = eps;
+        ga.M = R; ga.N = 3 * d; ga.K = d; ga.group = g;
+        ga.kcache = kc; ga.vcache = vc; ga.pos_dev = m->pos_dev; ga.n_heads = H; ga.n_positions = P;
+        if ((rc = agpu_int4_skinny_px_launch(ctx, ga, PxIn{xh, st, d / 32, fold, fold + 3 * d}, PxOut{})) != AGPU_OK) return rc;
+        AttnParams ap{};
+        ap.q = qkv; ap.k = kc; ap.v = vc; ap.o = att;
+        ap.n_heads = H; ap.batch = B; ap.q_len = 1; ap.kv_len = 0; ap.q_offset = 0; ap.kv_stride = P; ap.causal = 1;
+        ap.q_batch_stride = 3 * d; ap.q_head_stride = DH; ap.q_row_stride = 3 * d;
+        ap.o_batch_stride = d; ap.o_head_stride = DH; ap.o_row_stride = d;
+        ap.pos_dev = m->pos_dev;
+        ap.px_pieces = xa;
+        if ((rc = agpu_attention_launch(ctx, ap, max_kv)) != AGPU_OK) return rc;
+        GemvArgs gp{};
+        gp.packed = wp.packed; gp.scales = wp.scales; gp.bias = wp.bias; gp.residual = hid; gp.y = hid;
+        gp.M = R; gp.N = d; gp.K = d; gp.group = g;
+        if ((rc = agpu_int4_skinny_px_launch(ctx, gp, PxIn{xa, nullptr, 0, nullptr, nullptr}, PxOut{xh, b.ln2_g, st})) != AGPU_OK) return rc;
+        GemvArgs gf{};
+        gf.packed = wf.packed; gf.scales = wf.scales; gf.bias = wf.bias; gf.y = ffn; gf.ln_eps = eps;
+        gf.M = R; gf.N = ff; gf.K = d; gf.group = g; gf.flags = gelu_flag;
+        if ((rc = agpu_int4_skinny_px_launch(ctx, gf, PxIn{xh, st, d / 32, fold + 6 * d, fold + 6 * d + ff}, PxOut{xf, nullptr, nullptr})) != AGPU_OK)
+            return rc;
+        GemvArgs go{};
+        go.packed = wo.packed; go.scales = wo.scales; go.bias = wo.bias; go.residual = hid; go.y = hid;
+        go.M = R; go.N = d; go.K = ff; go.group = g;
+        const float *next_gamma = L + 1 < m->cfg.n_layer ? m->blocks[L + 1].ln1_g : m->lnf_g;
+        return agpu_int4_skinny_px_launch(ctx, go, PxIn{xf, nullptr, 0, nullptr, nullptr}, PxOut{xh, next_gamma, st});
+    }
     if (new_len == 1 && R <= 16 && g % 8 == 0 && agpu_int4_gemv_can_fuse_ln(R, d)) {
         // decode: LN1 + QKV + bias with the K/V rows written straight into the cache
         GemvArgs ga{};
@@ -432,12 +536,20 @@ int32_t launch_block(agpu_gpt2 *m, int L, int B, int new_len, int max_kv) {
 
 // Final LayerNorm + LM head on `rows` rows of head_in -> m->logits.  With `feed` (single row only) the same launch
 // also picks the arg-max and feeds it back as the next token; *fed tells whether it did.
-int32_t launch_head(agpu_gpt2 *m, const float *head_in, int rows, const ArgmaxAdvance *feed = nullptr, bool *fed = nullptr) {
+int32_t launch_head(agpu_gpt2 *m, const float *head_in, int rows, const ArgmaxAdvance *feed = nullptr, bool *fed = nullptr, bool px = false) {
     agpu_ctx *ctx = m->ctx;
     const int d = m->d, g = m->cfg.group_size;
     const float eps = m->cfg.layer_norm_epsilon;
     float *logits = (float *)m->logits.p;
     if (fed) *fed = false;
+    if (m->cfg.lm_head == AGPU_LM_HEAD_INT4 && px) {
+        // the last block has left the hidden rows as pieces times the final LayerNorm's gains
+        const float *hb = (const float *)m->px_fold.p + px_fold_layer_floats(m) * m->cfg.n_layer;
+        GemvArgs ga{};
+        ga.packed = m->lm_head.packed; ga.scales = m->lm_head.scales; ga.y = logits; ga.ln_eps = eps;
+        ga.M = rows; ga.N = m->Vpad; ga.K = d; ga.group = g;
+        return agpu_int4_skinny_px_launch(ctx, ga, PxIn{(const uint4 *)m->px_h.p, (const float2 *)m->px_stats.p, d / 32, hb, hb + m->Vpad}, PxOut{});
+    }
     if (m->cfg.lm_head == AGPU_LM_HEAD_INT4) {
         if (feed && rows == 1) {
             GemvArgs ga{};
@@ -474,7 +586,7 @@ int32_t launch_forward(agpu_gpt2 *m, const uint32_t *tokens, int B, int new_len,
     if (rc != AGPU_OK) return rc;
     // final LayerNorm + LM head on the rows whose logits are wanted
     if (all_rows_logits) return launch_head(m, (float *)m->hid.p, B * new_len);
-    if (new_len == 1) return launch_head(m, (float *)m->hid.p, B, B == 1 ? feed : nullptr, fed);
+    if (new_len == 1) return launch_head(m, (float *)m->hid.p, B, B == 1 ? feed : nullptr, fed, px_active(m, B, new_len));
     if ((rc = launch_gather_last(m, B, new_len)) != AGPU_OK) return rc;
     return launch_head(m, (float *)m->last.p, B);
 }
@@ -497,6 +609,8 @@ int32_t ensure_buffers(agpu_gpt2 *m, int B, int new_len, bool all_rows_logits) {
         if ((rc = ensure(m, m->kfrag, bytes)) != AGPU_OK) return rc;
         if ((rc = ensure(m, m->vfrag, bytes)) != AGPU_OK) return rc;
     }
+    // last: growing any buffer above drops nothing this needs, and nothing below may move a buffer
+    if (px_shape_ok(m, B, new_len) && (rc = px_prepare(m)) != AGPU_OK) return rc;
     return AGPU_OK;
 }
 
@@ -825,6 +939,7 @@ AGPU_EXPORT int32_t agpu_gpt2_create(agpu_ctx *ctx, const agpu_gpt2_config *cfg,
                          cfg->n_embd, cfg->n_head);
     if (cfg->n_embd % 8 != 0) return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "gpt2_create: n_embd must be divisible by 8");
     agpu_gpt2 *m = new (std::nothrow) agpu_gpt2();
+    if (m) m->px_off = getenv("AGPU_NO_PX") != nullptr;
     if (!m) return AGPU_ERR_NULL_POINTER;
     m->ctx = ctx;
     ctx->refs.fetch_add(1);
@@ -869,7 +984,8 @@ AGPU_EXPORT int32_t agpu_gpt2_destroy(agpu_gpt2 *m) {
     free_lin(m->lm_head);
     for (void *p : {(void *)m->wte, (void *)m->wpe, (void *)m->lnf_g, (void *)m->lnf_b, (void *)m->wte_t, (void *)m->kcache,
                     (void *)m->vcache, (void *)m->cur_tok, (void *)m->next_tok, (void *)m->out_tok, (void *)m->pos_dev,
-                    m->hid.p, m->qkv.p, m->att.p, m->ffn.p, m->lnb.p, m->last.p, m->logits.p, m->tok_in.p, m->kfrag.p, m->vfrag.p})
+                    m->hid.p, m->qkv.p, m->att.p, m->ffn.p, m->lnb.p, m->last.p, m->logits.p, m->tok_in.p, m->kfrag.p, m->vfrag.p,
+                    m->px_h.p, m->px_att.p, m->px_ffn.p, m->px_stats.p, m->px_fold.p})
         if (p) (void)hipFree(p);
     for (hipEvent_t e : {m->ev0, m->ev1, m->ev2})
         if (e) (void)hipEventDestroy(e);
@@ -889,7 +1005,7 @@ AGPU_EXPORT int32_t agpu_gpt2_set_embeddings(agpu_gpt2 *m, const float *wte, con
     AGPU_REQUIRE_CTX(ctx);
     // the plan of the one-launch step holds sums over the final LayerNorm's gains and offsets
     (void)hipStreamSynchronize(ctx->stream);
-    drop_graphs(m);
+    weights_changed(m);
     int32_t rc = set_vec(ctx, &m->wte, wte, (size_t)m->V * m->d, on_device);
     if (rc == AGPU_OK) rc = set_vec(ctx, &m->wpe, wpe, (size_t)m->P * m->d, on_device);
     if (rc == AGPU_OK) rc = set_vec(ctx, &m->lnf_g, lnf_g, m->d, on_device);
@@ -914,7 +1030,7 @@ AGPU_EXPORT int32_t agpu_gpt2_set_layer_norms(agpu_gpt2 *m, int32_t layer, const
     Block &b = m->blocks[layer];
     // the plan of the one-launch step holds sums over the gains and offsets
     (void)hipStreamSynchronize(m->ctx->stream);
-    drop_graphs(m);
+    weights_changed(m);
     int32_t rc = set_vec(m->ctx, &b.ln1_g, ln1_g, m->d, on_device);
     if (rc == AGPU_OK) rc = set_vec(m->ctx, &b.ln1_b, ln1_b, m->d, on_device);
     if (rc == AGPU_OK) rc = set_vec(m->ctx, &b.ln2_g, ln2_g, m->d, on_device);
@@ -929,7 +1045,7 @@ AGPU_EXPORT int32_t agpu_gpt2_set_int4_linear(agpu_gpt2 *m, int32_t layer, int32
     int32_t rc = check_layer(m, layer, which, K, N);
     if (rc != AGPU_OK) return rc;
     if (!packed || !scales) return agpu_fail(m->ctx, AGPU_ERR_NULL_POINTER, "gpt2_set_int4_linear: null pointer");
-    drop_graphs(m);
+    weights_changed(m);
     Int4Lin &l = *lin_slot(m, layer, which);
     rc = alloc_lin(m, l, K, N, layer < 0, bias != nullptr && layer >= 0);
     if (rc != AGPU_OK) return rc;

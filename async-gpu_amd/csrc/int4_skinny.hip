@@ -40,8 +40,19 @@ __device__ unsigned long long sk_trace[8][8];
         if (threadIdx.x == 0 && blockIdx.x + gridDim.x * blockIdx.y < 8)                                      \
             sk_trace[blockIdx.x + gridDim.x * blockIdx.y][slot] = wall_clock64();                             \
     } while (0)
+// the kernel on pieces: lane 0 of every wave of the first eight workgroups of the launches with the selected (N, K)
+__device__ unsigned long long px_trace[8][16][8];
+__device__ int px_trace_sel[2];
+#define PX_STAMP(slot)                                                                                               \
+    do {                                                                                                             \
+        if ((threadIdx.x & 63) == 0 && blockIdx.x + gridDim.x * blockIdx.y < 8 && p.a.N == px_trace_sel[0] && p.a.K == px_trace_sel[1]) \
+            px_trace[blockIdx.x + gridDim.x * blockIdx.y][threadIdx.x >> 6][slot] = wall_clock64();                  \
+    } while (0)
 #else
 #define SK_STAMP(slot) \
+    do {               \
+    } while (0)
+#define PX_STAMP(slot) \
     do {               \
     } while (0)
 #endif
@@ -54,12 +65,6 @@ struct SkinnyParams {
     unsigned int *counters;
     int strict;           // the context's strict_sync
 };
-
-// the leading 16 bits of two floats as one register: a in the low half
-__device__ __forceinline__ uint32_t sk_pack_top(float a, float b) {
-    return __builtin_amdgcn_perm(__float_as_uint(b), __float_as_uint(a), 0x07060302u);
-}
-__device__ __forceinline__ float sk_top_bits(float v) { return __uint_as_float(__float_as_uint(v) & 0xffff0000u); }
 
 // 8 nibbles of one column -> the bf16 numbers 16 + n, pairs (0,4) (1,5) (2,6) (3,7)
 __device__ __forceinline__ bf16x8 sk_nibbles_plus16(uint32_t w) {
@@ -418,7 +423,414 @@ int32_t agpu_int4_skinny_launch(agpu_ctx *ctx, const GemvArgs &a) {
     return narrow ? skinny_go<false, false, 16, 2>(ctx, p, grid, lds) : skinny_go<false, false, 16, 4>(ctx, p, grid, lds);
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// The batched decode Linear on pieces that its producer has already split.
+//
+// In the kernel above every workgroup of a launch turns all 16 x K inputs into bf16 pieces itself (13 vector instructions
+// per element on one CU: 2 us of a 10 us launch for K = 1600) and normalises the rows itself.  Inside a decode step
+// every input of a Linear is the output of a kernel of the same step, so the producer can leave the pieces instead:
+//   pieces  [K/32 trips][3 pieces lo, mid, hi][64 lanes] x 16 bytes, lane = 16 * (k % 32 / 8) + row, the 8 k of a lane in
+//           the order (0,4,1,5,2,6,3,7): exactly the A operand of v_mfma_f32_16x16x32_bf16, so a wave requests the
+//           three registers of a trip with three 1 KiB loads, next to the trip's weights, and no LDS or barrier comes
+//           before its MFMAs;
+//   stats   [K/32][16 rows] (mean, M2) of the raw values of a row over 32 columns (M2 = sum of squared distances from
+//           that mean), merged by the consumer in tile order (Chan et al.) into the row's mean and variance.
+// A LayerNorm in front of the Linear is folded into it: the producer multiplies by the gains before splitting,
+//   y_n = rstd (sum_k x_k g_k W_kn - mean A_n) + B_n + bias_n,   A_n = sum_k g_k W_kn,   B_n = sum_k b_k W_kn,
+// with A and B computed once per model (px_fold_kernel, double accumulation over the dequantized weights), so the
+// statistics are needed only when the sums are finished.  Same arithmetic otherwise: exact products, fp32 scales.
+
+struct PxParams {
+    GemvArgs a;             // x, ln_gamma, ln_beta unused
+    PxIn in;
+    PxOut out;
+    int trips_per_split;
+    float *partial;
+    unsigned int *counters;
+    int strict;
+};
+
+namespace {
+
+// What a producer leaves of 8 consecutive outputs of row `row` from column n0 (a multiple of 8): the row's statistics
+// over the 32 columns around them (the four lanes of a quad hold one row's 32 columns, in order; all four must call)
+// and the pieces of the values times the next LayerNorm's gains g (ones where there is none).  valid: the row exists.
+__device__ __forceinline__ void px_emit8(const PxOut &o, int n0, int row, bool valid, const float (&raw)[8], const float (&g)[8]) {
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = valid ? raw[e] : 0.0f;
+    if (o.stats) {
+        float s = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+        s += dpp_move<0xb1, 0xf>(0.0f, s);
+        s += dpp_move<0x4e, 0xf>(0.0f, s);
+        const float mean = s * (1.0f / 32.0f);
+        float q = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float d = v[e] - mean;
+            q = fmaf(d, d, q);
+        }
+        q += dpp_move<0xb1, 0xf>(0.0f, q);
+        q += dpp_move<0x4e, 0xf>(0.0f, q);
+        if ((n0 & 31) == 0) o.stats[(size_t)(n0 >> 5) * 16 + row] = make_float2(mean, q);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] *= g[e];
+    px_store_pieces(o.pieces, n0, row, v);
+}
+
+// the gains of 8 columns from n0, or ones
+__device__ __forceinline__ void px_gains(const PxOut &o, int n0, bool ok, float (&g)[8]) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) g[e] = 1.0f;
+    if (o.gamma && ok) {
+        const float4 g0 = *reinterpret_cast<const float4 *>(o.gamma + n0), g1 = *reinterpret_cast<const float4 *>(o.gamma + n0 + 4);
+        g[0] = g0.x; g[1] = g0.y; g[2] = g0.z; g[3] = g0.w; g[4] = g1.x; g[5] = g1.y; g[6] = g1.z; g[7] = g1.w;
+    }
+}
+
+// Rows of fp32 values -> pieces (+ statistics): for values no kernel of this file produces (the embedding rows).
+// One wave per trip of 32 columns.
+__global__ __launch_bounds__(64) void px_split_rows_kernel(const float *x, int M, int K, PxOut o) {
+    const int lane = threadIdx.x, row = lane >> 2, n0 = 32 * blockIdx.x + 8 * (lane & 3);
+    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, g[8];
+    px_gains(o, n0, true, g);
+    if (row < M) {
+        const float4 a = *reinterpret_cast<const float4 *>(x + (size_t)row * K + n0), b = *reinterpret_cast<const float4 *>(x + (size_t)row * K + n0 + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    }
+    px_emit8(o, n0, row, row < M, v, g);
+}
+
+// A_n = sum_k g_k W_kn, B_n = sum_k b_k W_kn of an int4 Linear behind a LayerNorm (W_kn = (nibble - 8) scale,
+// nn/ops/quantize.rs:158-162), in double.
+__global__ void px_fold_kernel(const uint32_t *packed, const float *scales, int K, int N, int group, const float *g, const float *b,
+                               float *A, float *B) {
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= N) return;
+    double a = 0.0, o = 0.0;
+    for (int kp = 0; kp < K / 8; ++kp) {
+        const uint32_t w = packed[(size_t)kp * N + n];
+        const double sc = (double)scales[(size_t)((8 * kp) / group) * N + n];
+        for (int i = 0; i < 8; ++i) {
+            const double q = (double)((int)((w >> (4 * i)) & 15u) - 8) * sc;
+            a += (double)g[8 * kp + i] * q;
+            o += (double)b[8 * kp + i] * q;
+        }
+    }
+    A[n] = (float)a;
+    B[n] = (float)o;
+}
+
+// One workgroup = one tile of 16 CPL columns x one K split of up to SK_MAX_TRIPS trips; waves take trips round robin.
+// LDS: red [W][16][16 CPL] per-wave sums, then fin [16][16 CPL] finished outputs for the pieces of the next Linear.
+template <bool LNF, int CPL>
+__global__ __launch_bounds__(1024) void int4_skinny_px_kernel(const PxParams p) {
+    constexpr int NW = 16, TPW = (SK_MAX_TRIPS + NW - 1) / NW, COLS = 16 * CPL, MT = 16, n_out = MT * COLS;
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ float s_mean[MT], s_rstd[MT];
+    __shared__ int s_last;
+    const GemvArgs &a = p.a;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6, T = blockDim.x;
+    const int rs = lane >> 4, cg = lane & 15;
+    const int tile = blockIdx.x, ksplit = gridDim.y, split = blockIdx.y;
+    const int trips_total = a.K / 32;
+    const int t0 = split * p.trips_per_split;
+    const int t1 = min(trips_total, t0 + p.trips_per_split);
+    float *red = reinterpret_cast<float *>(smem);
+    float *fin = red + (size_t)W * n_out;
+
+    PX_STAMP(0);
+    // requested first, used last: the row statistics (lane t: tile t) of the first two rows this wave finishes
+    constexpr int SE = 2;
+    float2 st_in[SE];
+    auto load_stats = [&](int row) {
+        float2 st = make_float2(0.f, 0.f);
+        if (row < a.M && lane < p.in.tiles) st = p.in.stats[(size_t)lane * 16 + row];
+        return st;
+    };
+    if (LNF) {
+#pragma unroll
+        for (int h = 0; h < SE; ++h) st_in[h] = load_stats(wave + h * W);
+    }
+    const int e_row = (tid >> 2) & 15, e_n0 = tile * COLS + 32 * (tid >> 6) + 8 * (tid & 3);
+    const int c0 = tile * COLS + cg * CPL;
+    const bool col_ok = c0 < a.N;
+    uint32_t w4[TPW][CPL];
+    float sc4[TPW][CPL];
+    uint4 af[TPW][3];
+#pragma unroll
+    for (int u = 0; u < TPW; ++u) {
+        const int trip = t0 + wave + u * W;
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) {
+            w4[u][c] = 0u;
+            sc4[u][c] = 0.0f;
+        }
+        af[u][0] = af[u][1] = af[u][2] = make_uint4(0u, 0u, 0u, 0u);
+        if (trip < t1) {
+            const uint4 *xp = p.in.pieces + (size_t)trip * 192 + lane;
+            af[u][0] = xp[0];
+            af[u][1] = xp[64];
+            af[u][2] = xp[128];
+            if (col_ok) {
+                const uint32_t *wp = a.packed + (size_t)(4 * trip + rs) * a.N + c0;
+                const float *sp = a.scales + (size_t)((trip * 32) / a.group) * a.N + c0;
+                if (CPL == 4) {
+                    const uint4 wv = *reinterpret_cast<const uint4 *>(wp);
+                    const float4 sv = *reinterpret_cast<const float4 *>(sp);
+                    w4[u][0] = wv.x; w4[u][1] = wv.y; w4[u][CPL - 2] = wv.z; w4[u][CPL - 1] = wv.w;
+                    sc4[u][0] = sv.x; sc4[u][1] = sv.y; sc4[u][CPL - 2] = sv.z; sc4[u][CPL - 1] = sv.w;
+                } else {
+                    const uint2 wv = *reinterpret_cast<const uint2 *>(wp);
+                    const float2 sv = *reinterpret_cast<const float2 *>(sp);
+                    w4[u][0] = wv.x; w4[u][1] = wv.y;
+                    sc4[u][0] = sv.x; sc4[u][1] = sv.y;
+                }
+            }
+        }
+    }
+    // operands of this thread's first output, requested early
+    float e_bias = 0.0f, e_res = 0.0f, e_fa = 0.0f, e_fb = 0.0f;
+    if (tid < n_out) {
+        const int m = tid / COLS, n = tile * COLS + (tid - m * COLS);
+        if (m < a.M && n < a.N) {
+            if (a.bias) e_bias = a.bias[n];
+            if (a.residual) e_res = a.residual[(size_t)m * a.N + n];
+            if (LNF) {
+                e_fa = p.in.fold_a[n];
+                e_fb = p.in.fold_b[n];
+            }
+        }
+    }
+    PX_STAMP(1);
+    floatx4 acc[CPL];
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) acc[c] = floatx4{0.f, 0.f, 0.f, 0.f};
+    const uint4 m24 = make_uint4(0xC1C0C1C0u, 0xC1C0C1C0u, 0xC1C0C1C0u, 0xC1C0C1C0u);  // -24 eight times
+    const bf16x8 b24 = __builtin_bit_cast(bf16x8, m24);
+#pragma unroll
+    for (int u = 0; u < TPW; ++u) {
+        if (t0 + wave + u * W >= t1) break;  // wave-uniform
+        const bf16x8 a_lo = __builtin_bit_cast(bf16x8, af[u][0]);
+        const bf16x8 a_mid = __builtin_bit_cast(bf16x8, af[u][1]);
+        const bf16x8 a_hi = __builtin_bit_cast(bf16x8, af[u][2]);
+        floatx4 z = {0.f, 0.f, 0.f, 0.f};
+        z = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, b24, z, 0, 0, 0);
+        z = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_mid, b24, z, 0, 0, 0);
+        z = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, b24, z, 0, 0, 0);
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) {
+            const bf16x8 b = sk_nibbles_plus16(w4[u][c]);
+            floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, b, z, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_mid, b, d, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, b, d, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[c][r] = fmaf(sc4[u][c], d[r], acc[c][r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        float *dst = red + (wave * MT + 4 * rs + r) * COLS + cg * CPL;
+        if (CPL == 4) *reinterpret_cast<float4 *>(dst) = make_float4(acc[0][r], acc[1][r], acc[CPL - 2][r], acc[CPL - 1][r]);
+        else *reinterpret_cast<float2 *>(dst) = make_float2(acc[0][r], acc[1][r]);
+    }
+    PX_STAMP(2);
+    // the gains of the 8 outputs this thread will turn into pieces: on their way during the reduction
+    float e_g[8];
+    px_gains(p.out, e_n0, p.out.pieces && tid < 2 * COLS && e_n0 < a.N, e_g);
+    if (LNF) {
+        // mean and 1 / sqrt(variance + eps) of every row from the producer's tiles of 32 columns (at most 64 of them),
+        // merged in tile order; a workgroup of fewer than 8 waves fetches the statistics of its later rows only now
+        for (int h = 0; wave + h * W < MT; ++h) {  // wave-uniform
+            const int row = wave + h * W;
+            const float2 st = h < SE ? st_in[h < SE ? h : 0] : load_stats(row);
+            const float mean = wave_sum(st.x) / (float)p.in.tiles;
+            const float dm = lane < p.in.tiles && row < a.M ? st.x - mean : 0.0f;
+            const float m2 = wave_sum(fmaf(32.0f * dm, dm, st.y));
+            if (lane == 0) {
+                s_mean[row] = mean;
+                s_rstd[row] = 1.0f / sqrtf(m2 / (float)a.K + a.ln_eps);
+            }
+        }
+    }
+    __syncthreads();
+    PX_STAMP(3);
+    // sum over K -> output element i of the tile (fold, bias, GELU, residual, store, K/V row), kept for the pieces
+    auto finish = [&](int i, float v) {
+        const int m = i / COLS, n = tile * COLS + (i - m * COLS);
+        const bool early = i == tid;
+        if (LNF) {
+            const float fa = early ? e_fa : p.in.fold_a[n], fb = early ? e_fb : p.in.fold_b[n];
+            v = fmaf(s_rstd[m], fmaf(-s_mean[m], fa, v), fb);
+        }
+        v = finish_output(a, v, early ? e_bias : (a.bias ? a.bias[n] : 0.0f),
+                          early ? e_res : (a.residual ? a.residual[(size_t)m * a.N + n] : 0.0f), m, n);
+        if (p.out.pieces) fin[i] = v;
+    };
+    for (int i = tid; i < n_out; i += T) {
+        const int m = i / COLS, n = tile * COLS + (i - m * COLS);
+        if (m < a.M && n < a.N) {
+            float v = 0.0f;
+            for (int w2 = 0; w2 < W; ++w2) v += red[w2 * n_out + i];
+            if (ksplit == 1) finish(i, v);
+            else __hip_atomic_store(&p.partial[((size_t)split * a.M + m) * a.N + n], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    PX_STAMP(4);
+    if (ksplit > 1) {
+        partials_published(p.strict);
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned int tk = take_ticket(&p.counters[tile], p.strict);
+            s_last = (tk == (unsigned int)(ksplit - 1));
+        }
+        __syncthreads();
+        PX_STAMP(5);
+        if (!s_last) return;  // uniform over the workgroup
+        for (int i = tid; i < n_out; i += T) {
+            const int m = i / COLS, n = tile * COLS + (i - m * COLS);
+            if (m < a.M && n < a.N) {
+                const float *src = p.partial + (size_t)m * a.N + n;
+                const size_t stride = (size_t)a.M * a.N;
+                float v = 0.0f;
+                for (int sp0 = 0; sp0 < ksplit; sp0 += 8) {  // 8 loads in flight, summed in split order
+                    float part[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+                        part[u] = sp0 + u < ksplit
+                                      ? __hip_atomic_load(src + (size_t)(sp0 + u) * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                      : 0.0f;
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+                        if (sp0 + u < ksplit) v += part[u];
+                }
+                finish(i, v);
+            }
+        }
+        if (tid == 0) __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    PX_STAMP(6);
+    if (!p.out.pieces) return;
+    __syncthreads();
+    // thread (8 columns = tid % 4 of a tile of 32, row = tid / 4 % 16, tile of 32 = tid / 64): whole waves, a quad per
+    // (row, tile of 32)
+    if (tid < 2 * COLS) {
+        const int cb = e_n0 - tile * COLS;
+        const bool valid = e_row < a.M && e_n0 < a.N;
+        float v[8];
+        const float4 f0 = *reinterpret_cast<const float4 *>(fin + e_row * COLS + cb), f1 = *reinterpret_cast<const float4 *>(fin + e_row * COLS + cb + 4);
+        v[0] = f0.x; v[1] = f0.y; v[2] = f0.z; v[3] = f0.w; v[4] = f1.x; v[5] = f1.y; v[6] = f1.z; v[7] = f1.w;
+        if (e_n0 < a.N) px_emit8(p.out, e_n0, e_row, valid, v, e_g);
+    }
+    PX_STAMP(7);
+}
+
+template <bool LNF, int CPL>
+int32_t px_go(agpu_ctx *ctx, const PxParams &p, dim3 grid, int W, size_t lds) {
+    static std::atomic<unsigned long long> lds_raised{0};
+    const unsigned long long dev_bit = 1ull << (ctx->device & 63);
+    if (lds > 48 * 1024 && !(lds_raised.load(std::memory_order_relaxed) & dev_bit)) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(int4_skinny_px_kernel<LNF, CPL>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 17 * 16 * 64 * 4);
+        if (e != hipSuccess) return agpu_hip(ctx, e, "hipFuncSetAttribute");
+        lds_raised.fetch_or(dev_bit, std::memory_order_relaxed);
+    }
+    hipLaunchKernelGGL((int4_skinny_px_kernel<LNF, CPL>), grid, dim3(64 * W), lds, ctx->stream, p);
+    return AGPU_LAUNCH_CHECK(ctx, "int4_skinny_px_kernel");
+}
+
+}  // namespace
+
+bool agpu_int4_skinny_px_supported(const GemvArgs &a, const PxIn &in, const PxOut &out) {
+    if (!(a.M > 4 && a.M <= 16 && a.group % 32 == 0 && a.group <= 512 && a.K % 32 == 0 && a.N % 4 == 0)) return false;
+    if (((uintptr_t)a.packed | (uintptr_t)a.scales | (uintptr_t)in.pieces | (uintptr_t)out.pieces | (uintptr_t)out.gamma) % 16 != 0) return false;
+    if (!in.pieces) return false;
+    if (in.stats && (in.tiles != a.K / 32 || in.tiles > 64 || !in.fold_a || !in.fold_b)) return false;
+    if (out.pieces && a.N % 32 != 0) return false;
+    return true;
+}
+
+int32_t agpu_int4_skinny_px_launch(agpu_ctx *ctx, const GemvArgs &a, const PxIn &in, const PxOut &out) {
+    if (!agpu_int4_skinny_px_supported(a, in, out))
+        return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "int4_skinny on pieces: M=%d N=%d K=%d group=%d not taken", a.M, a.N, a.K, a.group);
+    PxParams p{};
+    p.a = a;
+    p.in = in;
+    p.out = out;
+    p.strict = ctx->strict_sync;
+    const int trips_total = a.K / 32;
+    const int tpg = a.group / 32;  // trips per scale group; a split covers whole groups
+    const int tps_max = SK_MAX_TRIPS / tpg * tpg;
+    const int ksplit = ceil_div(trips_total, tps_max);
+    const int tps = ceil_div(ceil_div(trips_total, ksplit), tpg) * tpg;
+    if (ksplit > 1 && (size_t)ksplit * a.M * a.N * sizeof(float) > ctx->ws_bytes / 2)
+        return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_skinny: split-K partials exceed the workspace (M=%d N=%d K=%d)", a.M, a.N, a.K);
+    const bool narrow = ceil_div(a.N, 32) * ksplit <= ctx->num_cus;
+    const int cols = narrow ? 32 : 64;
+    const int col_blocks = ceil_div(a.N, cols);
+    if (col_blocks > ctx->n_counters) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_skinny: N=%d too large", a.N);
+    p.trips_per_split = tps;
+    const int W = tps < 16 ? (tps < 2 ? 2 : tps) : 16;  // two waves at least: the pieces are written by 2 cols threads
+    const size_t lds = sizeof(float) * (size_t)(W + 1) * 16 * cols;
+    p.partial = reinterpret_cast<float *>(ctx->workspace);
+    p.counters = ctx->counters;
+    const dim3 grid(col_blocks, ksplit);
+    if (in.stats) return narrow ? px_go<true, 2>(ctx, p, grid, W, lds) : px_go<true, 4>(ctx, p, grid, W, lds);
+    return narrow ? px_go<false, 2>(ctx, p, grid, W, lds) : px_go<false, 4>(ctx, p, grid, W, lds);
+}
+
+int32_t agpu_px_split_rows_launch(agpu_ctx *ctx, const float *x, int M, int K, const PxOut &out) {
+    if (K % 32 != 0 || M < 1 || M > 16 || !out.pieces) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "px_split_rows: M=%d K=%d", M, K);
+    hipLaunchKernelGGL(px_split_rows_kernel, dim3(K / 32), dim3(64), 0, ctx->stream, x, M, K, out);
+    return AGPU_LAUNCH_CHECK(ctx, "px_split_rows_kernel");
+}
+
+int32_t agpu_px_fold_launch(agpu_ctx *ctx, const uint32_t *packed, const float *scales, int K, int N, int group, const float *gamma,
+                            const float *beta, float *A, float *B) {
+    hipLaunchKernelGGL(px_fold_kernel, dim3(ceil_div(N, 256)), dim3(256), 0, ctx->stream, packed, scales, K, N, group, gamma, beta, A, B);
+    return AGPU_LAUNCH_CHECK(ctx, "px_fold_kernel");
+}
+
+AGPU_EXPORT int32_t agpu_int4_linear_pieces(agpu_ctx *ctx, const float *x, const float *gamma, const float *beta, float eps,
+                                            const uint32_t *packed, const float *scales, const float *bias, const float *residual,
+                                            float *y, int32_t M, int32_t N, int32_t K, int32_t group, uint32_t flags,
+                                            const float *out_gamma, void *out_pieces, float *out_stats) {
+    AGPU_REQUIRE_CTX(ctx);
+    AGPU_REQUIRE_PTR(ctx, x);
+    AGPU_REQUIRE_PTR(ctx, packed);
+    AGPU_REQUIRE_PTR(ctx, scales);
+    AGPU_REQUIRE_PTR(ctx, y);
+    if ((gamma == nullptr) != (beta == nullptr)) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "int4_linear_pieces: gamma and beta go together");
+    if (M < 5 || M > 16 || K < 32 || K % 32 != 0 || N < 4 || (gamma && K > 2048))
+        return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "int4_linear_pieces: M=%d N=%d K=%d not taken", M, N, K);
+    // scratch, second half of the context's: pieces of x | statistics | A | B
+    const size_t pieces_bytes = (size_t)(K / 32) * 192 * sizeof(uint4), stats_bytes = (size_t)(K / 32) * 16 * sizeof(float2);
+    const size_t need = pieces_bytes + stats_bytes + 2 * (size_t)N * sizeof(float);
+    if (need + 8192 > ctx->ws_bytes / 2) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_linear_pieces: %zu bytes of scratch needed", need);
+    char *base = ctx->workspace + ctx->ws_bytes / 2;
+    uint4 *pieces = reinterpret_cast<uint4 *>(base);
+    float2 *stats = reinterpret_cast<float2 *>(base + pieces_bytes);
+    float *fa = reinterpret_cast<float *>(base + pieces_bytes + stats_bytes), *fb = fa + N;
+    int32_t rc = agpu_px_split_rows_launch(ctx, x, M, K, PxOut{pieces, gamma, gamma ? stats : nullptr});
+    if (rc == AGPU_OK && gamma) rc = agpu_px_fold_launch(ctx, packed, scales, K, N, group, gamma, beta, fa, fb);
+    if (rc != AGPU_OK) return rc;
+    GemvArgs a{};
+    a.packed = packed; a.scales = scales; a.bias = bias; a.residual = residual; a.y = y; a.ln_eps = eps;
+    a.M = M; a.N = N; a.K = K; a.group = group; a.flags = flags;
+    const PxIn in{pieces, gamma ? stats : nullptr, gamma ? K / 32 : 0, gamma ? fa : nullptr, gamma ? fb : nullptr};
+    const PxOut out{reinterpret_cast<uint4 *>(out_pieces), out_pieces ? out_gamma : nullptr, out_pieces ? reinterpret_cast<float2 *>(out_stats) : nullptr};
+    return agpu_int4_skinny_px_launch(ctx, a, in, out);
+}
+
 #ifdef AGPU_SK_TRACE
+AGPU_EXPORT int32_t agpu_dev_px_trace_select(int32_t N, int32_t K) {
+    const int sel[2] = {N, K};
+    return (int32_t)hipMemcpyToSymbol(HIP_SYMBOL(px_trace_sel), sel, sizeof(sel));
+}
+AGPU_EXPORT int32_t agpu_dev_px_trace(unsigned long long *out_host) {
+    return (int32_t)hipMemcpyFromSymbol(out_host, HIP_SYMBOL(px_trace), sizeof(unsigned long long) * 8 * 16 * 8);
+}
 AGPU_EXPORT int32_t agpu_dev_skinny_trace(unsigned long long *out_host) {
     return (int32_t)hipMemcpyFromSymbol(out_host, HIP_SYMBOL(sk_trace), sizeof(unsigned long long) * 64);
 }

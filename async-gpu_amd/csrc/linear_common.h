@@ -109,6 +109,48 @@ int32_t agpu_ln_int4_linear_kv(agpu_ctx *ctx, const float *x, const float *gamma
 bool agpu_int4_skinny_supported(const GemvArgs &a);
 bool agpu_int4_skinny_can_fuse_ln(int M, int N, int K);
 int32_t agpu_int4_skinny_launch(agpu_ctx *ctx, const GemvArgs &a);
+// The same Linear inside a decode step, on inputs its producer has already split into bf16 pieces (layout and
+// arithmetic: csrc/int4_skinny.hip).  PxIn: the pieces of x [K/32][3][64] x 16 bytes; with stats (per row and 32
+// columns, `tiles` = K / 32 <= 64 of them) the LayerNorm in front of the Linear is applied through fold_a / fold_b.
+// PxOut (all optional): the pieces of this Linear's outputs for the next one, times `gamma` where given, and their
+// statistics.  Needs N % 32 == 0 to write pieces.
+struct PxIn {
+    const uint4 *pieces;
+    const float2 *stats;
+    int tiles;
+    const float *fold_a, *fold_b;
+};
+struct PxOut {
+    uint4 *pieces;
+    const float *gamma;
+    float2 *stats;
+};
+// the leading 16 bits of two floats as one register: a in the low half
+__device__ __forceinline__ uint32_t sk_pack_top(float a, float b) {
+    return __builtin_amdgcn_perm(__float_as_uint(b), __float_as_uint(a), 0x07060302u);
+}
+__device__ __forceinline__ float sk_top_bits(float v) { return __uint_as_float(__float_as_uint(v) & 0xffff0000u); }
+// 8 consecutive k (from k0, a multiple of 8) of row `row` -> the lane's 16 bytes of the three piece planes of its trip:
+// x = hi + mid + lo exactly, each piece the leading 8 bits of what the ones before it left; k order (0,4,1,5,2,6,3,7).
+__device__ __forceinline__ void px_store_pieces(uint4 *pieces, int k0, int row, const float (&v)[8]) {
+    float r1[8], r2[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        r1[e] = v[e] - sk_top_bits(v[e]);
+        r2[e] = r1[e] - sk_top_bits(r1[e]);
+    }
+    uint4 *dst = pieces + (size_t)(k0 >> 5) * 192 + 16 * ((k0 & 31) >> 3) + row;
+    dst[0] = make_uint4(sk_pack_top(r2[0], r2[4]), sk_pack_top(r2[1], r2[5]), sk_pack_top(r2[2], r2[6]), sk_pack_top(r2[3], r2[7]));
+    dst[64] = make_uint4(sk_pack_top(r1[0], r1[4]), sk_pack_top(r1[1], r1[5]), sk_pack_top(r1[2], r1[6]), sk_pack_top(r1[3], r1[7]));
+    dst[128] = make_uint4(sk_pack_top(v[0], v[4]), sk_pack_top(v[1], v[5]), sk_pack_top(v[2], v[6]), sk_pack_top(v[3], v[7]));
+}
+bool agpu_int4_skinny_px_supported(const GemvArgs &a, const PxIn &in, const PxOut &out);
+int32_t agpu_int4_skinny_px_launch(agpu_ctx *ctx, const GemvArgs &a, const PxIn &in, const PxOut &out);
+// fp32 rows [M <= 16, K] -> pieces (+ statistics), for values the Linear kernels do not produce themselves.
+int32_t agpu_px_split_rows_launch(agpu_ctx *ctx, const float *x, int M, int K, const PxOut &out);
+// A_n = sum_k gamma_k W_kn and B_n = sum_k beta_k W_kn of an int4 Linear [K, N] (dense, stride N).
+int32_t agpu_px_fold_launch(agpu_ctx *ctx, const uint32_t *packed, const float *scales, int K, int N, int group, const float *gamma,
+                            const float *beta, float *A, float *B);
 // Whether the GEMV can apply LayerNorm itself for this shape (otherwise normalise first).
 bool agpu_int4_gemv_can_fuse_ln(int M, int K);
 

@@ -51,6 +51,22 @@ def int4_linear(x, packed, scales, bias=None, residual=None, group=32, flags=0, 
     return y if x.dim() <= 2 else y.reshape(*x.shape[:-1], N)
 
 
+def int4_linear_pieces(x, packed, scales, bias=None, residual=None, group=32, flags=0, ln=None, out_gamma=None, want_pieces=False):
+    """The batched decode Linear of the model driver (5 .. 16 rows) on bf16 pieces of x, as agpu_int4_linear_pieces
+    describes it.  Returns y, or (y, pieces [N/32, 3, 64, 8] int16 bit patterns, stats [N/32, 16, 2]) with want_pieces."""
+    M, K = x.shape
+    N = packed.shape[1]
+    y = torch.empty((M, N), dtype=torch.float32, device=x.device)
+    pieces = stats = None
+    if want_pieces:
+        pieces = torch.zeros((N // 32, 3, 64, 8), dtype=torch.int16, device=x.device)
+        stats = torch.zeros((N // 32, 16, 2), dtype=torch.float32, device=x.device)
+    g, b, eps = ln if ln is not None else (None, None, 0.0)
+    context(x.device.index or 0).call("agpu_int4_linear_pieces", _f32(x), g, b, float(eps), packed, scales, bias, residual, y, M, N, K,
+                                      group, flags, out_gamma, pieces, stats)
+    return (y, pieces, stats) if want_pieces else y
+
+
 def int4_matmul(a, b, group=128):
     """ops::int4_matmul (nn/ops/gemm.rs:1186-1266): B [K, N] is quantized on the fly (per column, groups of 128 along
     K, the Rust quantizer's rounding; on the device here, on the host after a download in the reference), then

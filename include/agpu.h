@@ -190,6 +190,23 @@ int32_t agpu_ln_int4_linear(agpu_ctx *ctx, const float *x, const float *gamma, c
                             const float *residual, float *y, int32_t M, int32_t N, int32_t K,
                             int32_t group, uint32_t flags);
 
+/* The batched decode Linear as the model driver chains it inside a decode step of 5 .. 16 sequences (no counterpart in
+ * the reference, which runs one kernel for every M, compute_gemm.rs:2849-2910): there every Linear's input is left by
+ * the kernel that produced it as the exact sum of three bf16 pieces per element, in the matrix cores' operand order,
+ * together with row statistics per 32 columns, and a LayerNorm in front of a Linear is folded into it.  This call runs
+ * that chain for one Linear on fp32 rows, for tests and measurements: split x (times gamma) into pieces, fold
+ * (gamma, beta) into two vectors over the N columns, then y = epilogue(LayerNorm(x) W) as agpu_ln_int4_linear
+ * (gamma = beta = NULL: no LayerNorm).  5 <= M <= 16, K % 32 == 0, group a multiple of 32 up to 512, N % 4 == 0,
+ * K <= 2048 with LayerNorm.  Optionally it also leaves what the next Linear would read: out_pieces (device,
+ * N / 32 * 3072 bytes, needs N % 32 == 0): y times out_gamma (NULL: times one) as pieces
+ * [N/32][3: low, middle, high][64: 16 * (n % 32 / 8) + row] x 8 bf16 in the order n % 8 = 0,4,1,5,2,6,3,7; out_stats
+ * (device, N / 32 * 16 pairs of floats or NULL): per 32 columns and row the mean of y and the sum of squared
+ * distances from it.  Uses the second half of the context's scratch. */
+int32_t agpu_int4_linear_pieces(agpu_ctx *ctx, const float *x, const float *gamma, const float *beta, float eps,
+                                const uint32_t *packed, const float *scales, const float *bias, const float *residual,
+                                float *y, int32_t M, int32_t N, int32_t K, int32_t group, uint32_t flags,
+                                const float *out_gamma, void *out_pieces, float *out_stats);
+
 /* Measurement helper (no counterpart in the reference, whose benches time host-side loops,
  * nn/ops/norm.rs:578-633): records `reps` back-to-back launches of agpu_ln_int4_linear
  * (gamma/beta may be NULL) into a HIP graph, replays it and writes the mean microseconds per

@@ -105,6 +105,7 @@ extern "C" {
     pub fn agpu_int4_linear_static(device: i32, hip_stream: *mut c_void, x: *const f32, packed: *const u32, scales: *const f32, bias: *const f32, residual: *const f32, y: *mut f32, M: i32, N: i32, K: i32, group: i32, flags: u32, err_out: *mut c_char, err_cap: i32) -> i32;
     pub fn agpu_int4_gemv_tune(ctx: *mut agpu_ctx, max_wgs: i32, max_rows_per_wg: i32, max_waves_per_wg: i32) -> i32;
     pub fn agpu_ln_int4_linear(ctx: *mut agpu_ctx, x: *const f32, gamma: *const f32, beta: *const f32, eps: f32, packed: *const u32, scales: *const f32, bias: *const f32, residual: *const f32, y: *mut f32, M: i32, N: i32, K: i32, group: i32, flags: u32) -> i32;
+    pub fn agpu_int4_linear_pieces(ctx: *mut agpu_ctx, x: *const f32, gamma: *const f32, beta: *const f32, eps: f32, packed: *const u32, scales: *const f32, bias: *const f32, residual: *const f32, y: *mut f32, M: i32, N: i32, K: i32, group: i32, flags: u32, out_gamma: *const f32, out_pieces: *mut c_void, out_stats: *mut f32) -> i32;
     pub fn agpu_bench_int4_linear(ctx: *mut agpu_ctx, x: *const f32, gamma: *const f32, beta: *const f32, eps: f32, packed: *const u32, scales: *const f32, bias: *const f32, residual: *const f32, y: *mut f32, M: i32, N: i32, K: i32, group: i32, flags: u32, n_weight_sets: i32, packed_set_stride: i64, scales_set_stride: i64, reps: i32, us_per_launch_out_host: *mut f32) -> i32;
     pub fn agpu_int4_dequantize(ctx: *mut agpu_ctx, packed: *const u32, scales: *const f32, w_out: *mut f32, K: i32, N: i32, group: i32) -> i32;
     pub fn agpu_int4_quantize(ctx: *mut agpu_ctx, weight_t: *const f32, packed: *mut u32, scales: *mut f32, K: i32, N: i32, group: i32, mode: i32) -> i32;

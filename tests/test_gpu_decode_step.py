@@ -211,6 +211,44 @@ def test_one_launch_step_on_raw_nibbles_over_the_whole_range(orc, agpu, dev):
             assert float(np.abs(lp - lg).max()) <= TOL_LOGITS * scale
 
 
+@pytest.mark.parametrize("mode", ["one_launch", "per_stage"])
+def test_weights_replaced_under_cached_graphs_are_the_ones_the_next_call_uses(orc, agpu, dev, mode):
+    """Every setter that can replace a buffer or a folded vector drops the cached graphs and the step's plan: a model
+    that has decoded, then gets other LayerNorm vectors, one other Linear and other embeddings, decodes like a model built
+    with them from scratch (and like neither of the two it was before)."""
+    from async_gpu_amd import gpt2, workloads
+    cfg = workloads.GPT2_TINY
+    qa = _quantized(orc, cfg, 51, nonzero_bias=True, random_ln=True)
+    qb = _quantized(orc, cfg, 52, nonzero_bias=True, random_ln=True)
+    prompt = workloads.random_prompt(cfg, 9, 6)
+
+    def run(m):
+        m.set_decode_mode(m.DECODE_AUTO if mode == "one_launch" else m.DECODE_PER_STAGE)
+        (t,), _ = m.generate_cached(prompt, 24, eos=-1)
+        assert m.decode_is_one_launch() == (mode == "one_launch")
+        return t, m.last_logits().copy()
+
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg), qa)
+    ta, la = run(gm)
+    # a mix: embeddings and LayerNorms of b, Linears of a except layer 1's fc, the head of b
+    mix = dict(qa, wte=qb["wte"], wpe=qb["wpe"], lnf_g=qb["lnf_g"], lnf_b=qb["lnf_b"], lm_head=qb["lm_head"])
+    mix["layers"] = [dict(L) for L in qa["layers"]]
+    for li, L in enumerate(mix["layers"]):
+        for k in ("ln1_g", "ln1_b", "ln2_g", "ln2_b"):
+            L[k] = qb["layers"][li][k]
+    mix["layers"][1]["fc"] = qb["layers"][1]["fc"]
+    gm.set_embeddings(mix["wte"], mix["wpe"], mix["lnf_g"], mix["lnf_b"])
+    for li, L in enumerate(mix["layers"]):
+        gm.set_layer_norms(li, L["ln1_g"], L["ln1_b"], L["ln2_g"], L["ln2_b"])
+    gm.set_int4_linear(1, "fc", *mix["layers"][1]["fc"])
+    gm.set_int4_linear(-1, 0, mix["lm_head"][0], mix["lm_head"][1], None)
+    tm, lm = run(gm)
+    fresh = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg), mix)
+    tf, lf = run(fresh)
+    assert np.array_equal(tm, tf) and np.array_equal(lm, lf)
+    assert not np.array_equal(la, lm)
+
+
 def test_sampling_runs_on_the_one_launch_step(orc, agpu, dev):
     from async_gpu_amd import gpt2, ops, workloads
     cfg = workloads.GPT2_TINY

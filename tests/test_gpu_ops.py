@@ -152,6 +152,64 @@ def test_batched_decode_layer_norm(agpu, orc, dev, M, K, N, g):
     assert np.abs(y - ref).max() <= TOL_LINEAR
 
 
+def _pieces_to_rows(pieces, M):
+    """[N/32, 3, 64, 8] bf16 bit patterns, lane = 16 * (n % 32 / 8) + row, n % 8 in the order 0,4,1,5,2,6,3,7 -> the three
+    piece matrices [3, M, N] as float64."""
+    bits = pieces.astype(np.uint16).astype(np.uint32) << 16
+    vals = bits.view(np.float32).astype(np.float64)                  # [T, 3, 64, 8]
+    T = vals.shape[0]
+    vals = vals.reshape(T, 3, 4, 16, 8)                              # trip, piece, k block, row, slot
+    order = np.array([0, 4, 1, 5, 2, 6, 3, 7])
+    out = np.empty_like(vals)
+    out[..., order] = vals                                           # slot j holds k = order[j]
+    return out.transpose(1, 3, 0, 2, 4).reshape(3, 16, T * 32)[:, :M]
+
+
+@pytest.mark.parametrize("M", [5, 16])
+@pytest.mark.parametrize("K,N,g,ln", [(1600, 4800, 32, True), (1600, 1600, 32, False), (6400, 1600, 32, False), (1600, 6400, 32, True),
+                                      (768, 2304, 64, True), (3072, 768, 128, False), (2048, 96, 32, True), (64, 32, 32, False),
+                                      (1600, 50432, 32, True)])
+def test_batched_decode_on_pieces(agpu, orc, dev, M, K, N, g, ln):
+    """The batched decode Linear as the model chains it: x split once into three exact bf16 pieces, LayerNorm folded into
+    the Linear (statistics merged from tiles of 32 columns), and the outputs left as pieces times the next LayerNorm's
+    gains with their own statistics.  Against the f64 oracle; the pieces must add up to the stored outputs exactly."""
+    from async_gpu_amd import ops, workloads
+    rng = np.random.default_rng(M * 7 + K + N + g)
+    packed, scales, bias = workloads.random_int4_linear(rng, K, N, g, bias=True)
+    # rows of different size, each with a mean up to its own standard deviation: the folded LayerNorm subtracts
+    # mean * A_n from the sum at the end, so its rounding error grows like sqrt(1 + mean^2 / variance) of a row
+    x = ((rng.standard_normal((M, K)) + (rng.uniform(-1, 1, (M, 1)) if ln else 0)) * np.exp(rng.uniform(-2, 2, (M, 1)))).astype(np.float32)
+    gamma = (1 + 0.2 * rng.standard_normal(K)).astype(np.float32)
+    beta = (0.2 * rng.standard_normal(K)).astype(np.float32)
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    og = (1 + 0.3 * rng.standard_normal(N)).astype(np.float32)
+    lnp = (to_dev(gamma, dev), to_dev(beta, dev), 1e-5) if ln else None
+    y, pieces, stats = ops.int4_linear_pieces(to_dev(x, dev), to_dev(packed, dev), to_dev(scales, dev), bias=to_dev(bias, dev),
+                                              residual=to_dev(res, dev), group=g, ln=lnp, out_gamma=to_dev(og, dev), want_pieces=True)
+    y = y.cpu().numpy()
+    xin = orc.layer_norm(x, gamma, beta, 1e-5) if ln else x
+    ref = orc.int4_gemm_f64(xin, packed, scales, g, bias=bias) + res
+    if ln:
+        assert np.abs(y - ref).max() <= TOL_LINEAR
+    else:
+        bound = np.abs(x).astype(np.float64) @ np.abs(orc.int4_dequantize(packed, scales, g)).astype(np.float64)
+        assert np.all(np.abs(y - ref) <= 3e-6 * bound + 1e-6 * np.abs(ref) + 1e-6)
+    # what the next Linear would read
+    pc = _pieces_to_rows(pieces.cpu().numpy(), M)
+    want = (y * og[None, :]).astype(np.float32).astype(np.float64)
+    assert np.array_equal(pc[0] + pc[1] + pc[2], want)
+    assert np.all(np.abs(pc[0]) <= np.abs(want) * 2.0 ** -14 + 1e-300) and np.all(np.abs(pc[1]) <= np.abs(want) * 2.0 ** -7 + 1e-300)
+    st = stats.cpu().numpy()[:, :M]                                   # [N/32, M, 2]
+    tiles = y.astype(np.float64).reshape(M, N // 32, 32)
+    mean = tiles.mean(-1).T
+    m2 = ((tiles - tiles.mean(-1, keepdims=True)) ** 2).sum(-1).T
+    assert np.allclose(st[..., 0], mean, rtol=1e-5, atol=1e-6) and np.allclose(st[..., 1], m2, rtol=1e-4, atol=1e-6)
+    # without the pieces: same outputs, bit for bit
+    y2 = ops.int4_linear_pieces(to_dev(x, dev), to_dev(packed, dev), to_dev(scales, dev), bias=to_dev(bias, dev),
+                                residual=to_dev(res, dev), group=g, ln=lnp).cpu().numpy()
+    assert np.array_equal(y, y2)
+
+
 def test_batched_decode_special_rows(agpu, orc, dev):
     """A NaN or infinity poisons its own row only; an all-zero row gives the bias; two calls give the same bits."""
     from async_gpu_amd import ops, workloads
