@@ -6,6 +6,7 @@ HIPCC=${HIPCC:-/opt/rocm/bin/hipcc}
 FLAGS=(--offload-arch=gfx950 -O3 -std=c++17 -fPIC -fvisibility=hidden -ffp-contract=off
        -Xclang -target-feature -Xclang -packed-fp32-ops -Wall -Wno-unused-function)
 mkdir -p build
+rm -f build/*.o build/trace/*.o  # objects of sources that no longer exist must not be linked
 pids=()
 for src in *.hip; do
   obj="build/${src%.hip}.o"
