@@ -783,6 +783,11 @@ int32_t ensure_out_tokens(agpu_gpt2 *m, int steps, int B) {
 // Replays `steps` decode steps; the host only tracks the position to pick the graph.
 int32_t run_decode_steps(agpu_gpt2 *m, int B, int steps) {
     constexpr int kStepsPerGraph = 16;  // agpu_gpt2_decode_steps captures the same number ahead of its timed region
+    // the batched decode on pieces wants its buffers and folded LayerNorm vectors before a step is launched or captured
+    if (px_shape_ok(m, B, 1)) {
+        const int32_t rc = px_prepare(m);
+        if (rc != AGPU_OK) return rc;
+    }
     int s = 0;
     if (B == 1 && steps >= kStepsPerGraph && pk_ready(m)) {
         for (; s + kStepsPerGraph <= steps; s += kStepsPerGraph) {

@@ -183,6 +183,37 @@ def test_batch_of_independent_sequences(orc, agpu, dev):
     assert lg.shape == (5, cfg["vocab"])
 
 
+@pytest.mark.parametrize("batch,group,d,heads", [(5, 32, 192, 3), (11, 64, 256, 4), (16, 128, 768, 12), (8, 32, 1280, 20)])
+def test_batched_decode_on_pieces_in_the_model(orc, agpu, dev, batch, group, d, heads, monkeypatch):
+    """Decode steps of 5 .. 16 sequences run the Linears on bf16 pieces left by their producers, with LayerNorm folded
+    in: logits of a decode step against the f64 oracle for the first and the last sequence, tokens against the oracle,
+    and the same model with that path switched off (every Linear splitting and normalising its own input) within the
+    rounding of the two orders of summation."""
+    from async_gpu_amd import gpt2, workloads
+    cfg = dict(n_layer=3, n_embd=d, n_head=heads, vocab=1003, n_positions=96)
+    w, qz = _quantized(orc, cfg, 21 + batch, group=group, std=0.05, nonzero_bias=True, random_ln=True)
+    om = build_oracle_model(cfg, qz)
+    prompts = workloads.random_prompt(cfg, 5, 11, batch=batch)
+
+    def run():
+        gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg, max_batch=batch, group_size=group), qz)
+        outs, _ = gm.generate_cached(prompts, 9, eos=-1)
+        return outs, gm.last_logits(batch).copy()
+
+    outs, logits = run()
+    for b in (0, batch - 1):
+        ref, margins = om.generate(prompts[b], 9, cached=True, eos=-1)
+        _assert_tokens_match(outs[b], ref, margins, 11, f"row {b} of {batch}")
+        om.reset_cache()
+        om.forward(ref[:-2], all_rows=False)
+        lo = om.forward(ref[-2:-1], all_rows=False)  # the step that produced the last token
+        assert np.abs(logits[b] - lo[0]).max() <= TOL_LOGITS
+    monkeypatch.setenv("AGPU_NO_PX", "1")
+    outs2, logits2 = run()
+    assert all(np.array_equal(a, b) for a, b in zip(outs, outs2))
+    assert np.abs(logits - logits2).max() <= 1e-4 and not np.array_equal(logits, logits2)
+
+
 def test_xl_shaped_layers(orc, agpu, dev):
     """GPT-2 XL geometry (d=1600, 25 heads, ffn 6400) with 2 layers, batch 1 and 16."""
     from async_gpu_amd import gpt2, workloads
