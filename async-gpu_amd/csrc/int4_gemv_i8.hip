@@ -4,10 +4,11 @@
 // multiply-adds run on v_mfma_i32_16x16x64_i8 and the VALU only masks nibbles into bytes
 // (3 instructions per 8 nibbles), with results that are at least as accurate:
 //
-//   * x is turned into fixed point once per launch: with amax = max|x| of the row and s chosen so that
-//     |x * 2^s| < 2^30, X = rint(x * 2^s) is an int32 (exact for the large elements, off by at most
-//     amax * 2^-31 for the small ones; s is capped at 96, so elements below 2^-97 count as zero), split
-//     into four signed base-256 digits X = sum_d D_d * 256^d.
+//   * x is turned into fixed point once per launch, chunk by chunk (32 k = one MFMA slot): with amax = max|x| of the
+//     chunk and s chosen so that |x * 2^s| < 2^30, X = rint(x * 2^s) is an int32 (exact for the large elements, off
+//     by at most amax * 2^-31 for the small ones; s is capped at 96, so elements below 2^-97 count as zero), split
+//     into four signed base-256 digits X = sum_d D_d * 256^d.  The four threads that own a chunk agree on s by
+//     themselves (two DPP steps): no reduction over the workgroup stands between x and its digits.
 //   * B operand = the nibbles as bytes 0..15 straight from the packed words; A operand = the digits.
 //     The 16 rows of A are 4 slots x 4 digits; a slot is (row of x, 32-k chunk of the 64-k trip), and a
 //     slot's row is zero outside its chunk, so one MFMA yields, per slot, the four exact integer sums
@@ -94,13 +95,13 @@ __device__ __forceinline__ void block_reduce(float (&v)[N], float *scratch, int 
     }
 }
 
-// LDS: xd bytes [MT][tps][4 digits][4 q][16] | xsum float [MT][2 * tps rounded up to 4] | red float [tiles][32][MT][64]
+// LDS: xd bytes [MT][tps][4 digits][4 q][16] | xsum float4 [MT][2 * tps rounded up to 4]: per chunk 8 sum x, 2^-s, 2^(16-s) | red float [tiles][32][MT][64]
 // (rows >= 2 W of every region of red stay zero).  x never goes through LDS as floats: thread r owns packed row r (8 values) of
 // every x row in registers through LayerNorm, the fixed-point conversion and the chunk sums.
 template <int MT, bool LN, int SETS, bool AM = false>
 __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
     extern __shared__ __align__(16) float smem[];
-    __shared__ float s_scratch[3][MT * 16];
+    __shared__ float s_scratch[2][MT * 16];
     __shared__ int s_last[kMaxTilesPerPass];
     const GemvArgs &a = p.a;
     constexpr int COLS = 64;
@@ -111,9 +112,9 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
     const int trips_total = a.K / 64;
     const int t0 = split * tps, t1 = min(trips_total, t0 + tps);
     unsigned char *xd = reinterpret_cast<unsigned char *>(smem);
-    float *xsum = smem + MT * tps * 64;  // the digit planes take tps * 256 bytes per row
+    float4 *xsum = reinterpret_cast<float4 *>(smem + MT * tps * 64);  // the digit planes take tps * 256 bytes per row
     const int xsum_len = (2 * tps + 3) & ~3;
-    float *red = xsum + MT * xsum_len;
+    float *red = reinterpret_cast<float *>(xsum + MT * xsum_len);
     constexpr int n_out = MT * COLS;
     // Items of this workgroup: (tile j, trip t) for j < my_tiles, t < ntr, numbered j * ntr + t; wave w takes the
     // items w, w + W, ...  Two cursors walk that list: one for the loads, SETS items ahead of the one for the MFMAs.
@@ -181,7 +182,7 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
     for (int s = 0; s < SETS; ++s) if (s < p.sets_before) load_next(w0s[s], w1s[s], scs[s]);
     if (tid < 16) {  // neutral columns of the reduction scratch and the unused rows of red
         if (tid >= W)
-            for (int j = 0; j < 3 * MT; ++j) (&s_scratch[0][0])[j * 16 + tid] = 0.0f;
+            for (int j = 0; j < 2 * MT; ++j) (&s_scratch[0][0])[j * 16 + tid] = 0.0f;
     }
     {  // rows >= 2 W of every region of red
         const int per = (32 - 2 * W) * n_out;
@@ -214,8 +215,7 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
             for (int j = 0; j < 8; ++j) xv[m][j] = in_slice && m < a.M ? (xv[m][j] - mean[m]) * rstd * g8[j] + b8[j] : 0.0f;
         }
     }
-    // ---- fixed point: amax of the slice, digits, chunk sums ----
-    float amax[MT];
+    // ---- fixed point, chunk by chunk: amax of the chunk's 32 values (four threads), digits, chunk sums ----
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         float t = 0.0f;
@@ -224,20 +224,17 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
             const float v = fabsf(xv[m][j]);
             t = fmaxf(t, v == v ? v : __builtin_inff());  // a NaN counts as infinity
         }
-        amax[m] = in_slice ? t : 0.0f;
-    }
-    block_reduce<MT, true>(amax, s_scratch[2], lane, wave);
-    float c0m[MT], c1m[MT];
-#pragma unroll
-    for (int m = 0; m < MT; ++m) {
+        t = in_slice ? t : 0.0f;
+        t = fmaxf(t, dpp_move<0xb1, 0xf>(t, t));
+        const float amax = fmaxf(t, dpp_move<0x4e, 0xf>(t, t));  // 4 consecutive rows = one 32-k chunk
         // amax < 2^e with e from the exponent field (a denormal amax gives e = -126; s is capped anyway)
-        const int e = (int)((__float_as_uint(amax[m]) >> 23) & 0xffu) - 126;
+        const int e = (int)((__float_as_uint(amax) >> 23) & 0xffu) - 126;
         int s = 30 - e;
         s = s > 96 ? 96 : s;
-        const bool finite = amax[m] <= 3.0e38f;
+        const bool finite = amax <= 3.0e38f;
         const float up = finite ? __uint_as_float((uint32_t)(127 + s) << 23) : 0.0f;
-        c0m[m] = finite ? __uint_as_float((uint32_t)(127 - s) << 23) : __builtin_nanf("");
-        c1m[m] = finite ? __uint_as_float((uint32_t)(143 - s) << 23) : __builtin_nanf("");
+        const float c0 = finite ? __uint_as_float((uint32_t)(127 - s) << 23) : __builtin_nanf("");
+        const float c1 = finite ? __uint_as_float((uint32_t)(143 - s) << 23) : __builtin_nanf("");
         // Digits: with u = X + 0x00808080 the low three bytes of u ^ 0x00808080 are the signed digits
         // D_0..D_2 (each byte of u is D_i + 128) and the top byte is D_3.  A 4x4 byte transpose then gives,
         // per digit plane, the word of the even and of the odd nibbles of this thread's row.
@@ -265,7 +262,7 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
             unsigned char *dst = xd + ((size_t)(m * tps + tl) * 4) * 64 + 16 * (rr >> 1) + 8 * (rr & 1);
 #pragma unroll
             for (int d = 0; d < 4; ++d) *reinterpret_cast<uint2 *>(dst + d * 64) = make_uint2(dg[d][0], dg[d][1]);
-            if ((rl & 3) == 0) xsum[m * xsum_len + (rl >> 2)] = 8.0f * s8;
+            if ((rl & 3) == 0) xsum[m * xsum_len + (rl >> 2)] = make_float4(8.0f * s8, c0, c1, 0.0f);
         }
     }
     __syncthreads();
@@ -278,17 +275,14 @@ __global__ __launch_bounds__(1024) void int4_gemv_i8_kernel(const I8Params p) {
     const unsigned char *a_src = xd + ((size_t)(a_m < MT ? a_m : 0) * tps * 4 + (ai & 3)) * 64 + 16 * q;
     const int d_m = q >> 1;
     const bool d_ok = d_m < MT;
-    float c0f = 0.0f, c1f = 0.0f;
-#pragma unroll
-    for (int m = 0; m < MT; ++m)
-        if (d_m == m) { c0f = c0m[m]; c1f = c1m[m]; }
-    const float *d_xsum = xsum + (d_ok ? d_m : 0) * xsum_len + (q & 1);
+    const float4 *d_xsum = xsum + (d_ok ? d_m : 0) * xsum_len + (q & 1);
 
     float acc[4];
     auto consume = [&](const uint4 &w0v, const uint4 &w1v, const float4 &scv, int tl) {
         intx4 av = {0, 0, 0, 0};
         if (a_active) av = *reinterpret_cast<const intx4 *>(a_src + (size_t)tl * 256);
-        const float xs8 = d_ok ? d_xsum[2 * tl] : 0.0f;
+        const float4 ch = d_ok ? d_xsum[2 * tl] : make_float4(0.f, 0.f, 0.f, 0.f);  // the chunk's 8 sum x, 2^-s, 2^(16-s)
+        const float xs8 = ch.x, c0f = ch.y, c1f = ch.z;
         const uint32_t w0[4] = {w0v.x, w0v.y, w0v.z, w0v.w};
         const uint32_t w1[4] = {w1v.x, w1v.y, w1v.z, w1v.w};
         const float sc[4] = {scv.x, scv.y, scv.z, scv.w};
@@ -463,7 +457,7 @@ int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips
     if (col_blocks > ctx->n_counters - 1) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_gemv: N=%d too large", a.N);
     int tps_max = max_trips_per_split < 1 ? 1 : (max_trips_per_split > 128 ? 128 : max_trips_per_split);
     auto stage_bytes = [&](int tps) {
-        return (size_t)MT * tps * 256 + sizeof(float) * (size_t)MT * ((2 * tps + 3) & ~3);
+        return (size_t)MT * tps * 256 + sizeof(float4) * (size_t)MT * ((2 * tps + 3) & ~3);
     };
     while (tps_max > 1 && stage_bytes(tps_max) > 24 * 1024) --tps_max;
     int ksplit = ceil_div(trips_total, tps_max);

@@ -136,12 +136,12 @@ int32_t agpu_kernel_lookup(const agpu_ctx *ctx, const char *name, const char **e
  * (nn/ops/quantize.rs:109); otherwise AGPU_ERR_SHAPE_MISMATCH.
  *
  * Arithmetic for M <= 2 with group = 32 * 2^n, K % 64 == 0 and 16-byte aligned pointers (the decode shapes):
- * each x row is converted to 32-bit fixed point, X = rint(x * 2^s) with s chosen from the row's max |x| so
- * that |X| < 2^30, and the products with the nibbles are summed exactly in int32 per 32-k chunk; only the
- * per-group scale and the additions across groups round (fp32).  Consequences a caller can observe: an element
- * smaller than max|x| * 2^-31 of its row contributes as zero (the reference's fp32 fma chain would keep it, at a
- * weight below the chain's own rounding error); a row whose max |x| is below 2^-97 gives the bias / residual
- * alone; a row holding NaN or Inf gives NaN in every output of that row.  Results stay within
+ * each x row is converted to 32-bit fixed point chunk by chunk (32 consecutive k), X = rint(x * 2^s) with s chosen
+ * from the chunk's max |x| so that |X| < 2^30, and the products with the nibbles are summed exactly in int32 per
+ * chunk; only the per-group scale and the additions across groups round (fp32).  Consequences a caller can observe:
+ * an element smaller than 2^-31 of the largest |x| of its chunk contributes as zero (the reference's fp32 fma chain
+ * would keep it, at a weight below the chain's own rounding error); a chunk whose largest |x| is below 2^-97
+ * contributes nothing; a row holding NaN or Inf gives NaN in every output of that row.  Results stay within
  * 4e-7 * sum_k |x_k| |w_kn| of the exact dot product, tighter than the reference's fp32 chain.
  * AGPU_EPI_FORCE_FP32_GEMV selects the plain fp32 kernels instead.
  *
