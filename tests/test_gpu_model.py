@@ -214,6 +214,26 @@ def test_batched_decode_on_pieces_in_the_model(orc, agpu, dev, batch, group, d, 
     assert np.abs(logits - logits2).max() <= 1e-4 and not np.array_equal(logits, logits2)
 
 
+def test_batched_decode_on_pieces_with_the_f32_head_and_quick_gelu(orc, agpu, dev):
+    """The pieces path under the model's other options: the f32 LM head reads the hidden rows, not the pieces (rows of a
+    batch of 6 against the f64 oracle); the quick GELU goes through the same epilogue."""
+    from async_gpu_amd import gpt2, workloads
+    cfg = workloads.GPT2_TINY
+    w, qz = _quantized(orc, cfg, 14, nonzero_bias=True, random_ln=True)
+    prompts = workloads.random_prompt(cfg, 7, 8, batch=6)
+    om = build_oracle_model(cfg, qz, lm_head_int4=False)
+    gm = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg, max_batch=6, lm_head=gpt2.LM_HEAD_F32), qz)
+    outs, _ = gm.generate_cached(prompts, 12, eos=-1)
+    for b in (0, 5):
+        ref, margins = om.generate(prompts[b], 12, cached=True, eos=-1)
+        _assert_tokens_match(outs[b], ref, margins, 8, f"f32 head, row {b}")
+    # the quick GELU: a row of the batch equals the same sequence decoded alone (the one-launch step, checked elsewhere)
+    gq = gpt2.Int4Gpt2Model.from_quantized(gpu_config(cfg, max_batch=6, gelu=agpu._lib.GELU_QUICK), qz)
+    outs, _ = gq.generate_cached(prompts, 12, eos=-1)
+    (alone,), _ = gq.generate_cached(prompts[3], 12, eos=-1)
+    assert np.array_equal(outs[3], alone)
+
+
 def test_xl_shaped_layers(orc, agpu, dev):
     """GPT-2 XL geometry (d=1600, 25 heads, ffn 6400) with 2 layers, batch 1 and 16."""
     from async_gpu_amd import gpt2, workloads
