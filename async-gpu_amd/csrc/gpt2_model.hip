@@ -789,15 +789,19 @@ int32_t run_decode_steps(agpu_gpt2 *m, int B, int steps) {
         if (rc != AGPU_OK) return rc;
     }
     int s = 0;
-    if (B == 1 && steps >= kStepsPerGraph && pk_ready(m)) {
-        for (; s + kStepsPerGraph <= steps; s += kStepsPerGraph) {
+    if (B == 1 && steps >= 2 && pk_ready(m)) {
+        // graphs of sixteen launches, then one graph of what is left (a graph launch costs 5.5 us, a node inside one 1.5)
+        while (s < steps) {
+            const int n = std::min(kStepsPerGraph, steps - s);
+            if (n < 2) break;
             hipGraphExec_t exec;
-            const int32_t rc = decode_graph(m, 1, 0, &exec, kStepsPerGraph);
+            const int32_t rc = decode_graph(m, 1, 0, &exec, n);
             if (rc != AGPU_OK) return rc;
             const hipError_t e = hipGraphLaunch(exec, m->ctx->stream);
             if (e != hipSuccess) return agpu_hip(m->ctx, e, "hipGraphLaunch");
-            m->cache_len += kStepsPerGraph;
-            m->n_one_launch += kStepsPerGraph;
+            m->cache_len += n;
+            m->n_one_launch += n;
+            s += n;
         }
     }
     for (; s < steps; ++s) {
@@ -1317,7 +1321,10 @@ AGPU_EXPORT int32_t agpu_gpt2_decode_steps(agpu_gpt2 *m, int32_t batch, int32_t 
     if (rc != AGPU_OK) return rc;
     // capture outside the timed region
     hipGraphExec_t exec;
-    if (batch == 1 && steps >= 16 && pk_ready(m) && (rc = decode_graph(m, 1, 0, &exec, 16)) != AGPU_OK) return rc;
+    if (batch == 1 && steps >= 2 && pk_ready(m)) {
+        if (steps >= 16 && (rc = decode_graph(m, 1, 0, &exec, 16)) != AGPU_OK) return rc;
+        if (steps % 16 >= 2 && (rc = decode_graph(m, 1, 0, &exec, steps % 16)) != AGPU_OK) return rc;
+    }
     for (int s = 0; s < steps && m->decode_mode != AGPU_DECODE_EAGER; ++s)
         if ((rc = decode_graph(m, batch, kv_bucket(m, m->cache_len + 1 + s), &exec)) != AGPU_OK) return rc;
     if ((rc = agpu_hip(ctx, hipEventRecord(m->ev0, ctx->stream), "hipEventRecord")) != AGPU_OK) return rc;
