@@ -26,8 +26,9 @@
 //
 // Work decomposition: a workgroup owns up to four tiles of 64 columns x one K slice.  Its (tile, trip) pairs are
 // dealt to the waves round robin (item i goes to wave i % W), so any number of waves shares any number of trips
-// evenly, and a wave keeps up to SETS items in flight: their loads are issued before anything else, which for
-// the wide layers (the LM head) puts most of the matrix in flight while x is still being converted.  Waves reduce
+// evenly, and a wave keeps up to SETS items in flight.  A small layer's loads are all issued before anything else;
+// a wide layer (the LM head, three or more items per wave) is a stream that arrives the slower the more of it is
+// requested at once, so there a wave has one item on its way at a time, from the moment x is in LDS.  Waves reduce
 // through LDS in wave order; with ksplit > 1 partial sums are published write-through and the last workgroup to
 // take a ticket adds them in split order.  Rows with a NaN or infinity produce NaN outputs.
 #include "linear_common.h"
@@ -500,26 +501,30 @@ int32_t agpu_int4_gemv_i8_launch(agpu_ctx *ctx, const GemvArgs &a, int max_trips
     if (tiles_per_wg > 1) gx = ceil_div(col_blocks, tiles_per_wg);
     const size_t lds = stage_bytes(tps) + sizeof(float) * (size_t)tiles_per_wg * 32 * MT * 64;
     const int items_per_wave = ceil_div(tiles_per_wg * tps, W);
-    // With three or more items per wave a full request queue keeps the late waves from reaching the barriers of
-    // the x conversion before most of the matrix has arrived; one set up front and the rest after the digits was
-    // the fastest split on the LM head (8.1 us against 8.5 with two and 9.0 with all).
-    p.sets_before = items_per_wave > 2 ? 1 : 2;
+    // Up to two items per wave all of a workgroup's weights are requested before x is touched.  With three or more (the
+    // LM head) the matrix is a stream, and the stream arrives the slower the more of it is requested at once: one item
+    // in flight per wave, requested after the digits are in LDS, then item after item (LM head shapes K = 768 / 1600,
+    // weights from HBM: 7.65 / 12.1 us; with two sets 7.7 / 12.1, with four sets and one of them up front 8.05 / 13.4,
+    // with all four up front 8.8).
+    const bool stream = items_per_wave > 2;
+    p.sets_before = stream ? 0 : 2;
     const dim3 grid(gx, ksplit), block(64 * W);
     // fused arg-max: single row, unsplit K (else the separate kernel runs afterwards)
     const bool am = a.am_idx_out != nullptr && a.M == 1 && ksplit == 1 && (size_t)gx * sizeof(unsigned long long) <= ctx->ws_bytes / 2;
     if (am) {
         p.am_partial = reinterpret_cast<unsigned long long *>(ctx->workspace);
         p.am_counter = ctx->counters + (ctx->n_counters - 1);
-        if (a.ln_gamma) hipLaunchKernelGGL((int4_gemv_i8_kernel<1, true, 4, true>), grid, block, lds, ctx->stream, p);
-        else hipLaunchKernelGGL((int4_gemv_i8_kernel<1, false, 4, true>), grid, block, lds, ctx->stream, p);
+        // (the LM head: a stream; with one or two items per wave the single set costs the second item its overlap)
+        p.sets_before = stream ? 0 : 1;
+        if (a.ln_gamma) hipLaunchKernelGGL((int4_gemv_i8_kernel<1, true, 1, true>), grid, block, lds, ctx->stream, p);
+        else hipLaunchKernelGGL((int4_gemv_i8_kernel<1, false, 1, true>), grid, block, lds, ctx->stream, p);
         return AGPU_LAUNCH_CHECK(ctx, "int4_gemv_i8_kernel");
     }
 #define AGPU_I8_LAUNCH(MTv, LNv, Sv) hipLaunchKernelGGL((int4_gemv_i8_kernel<MTv, LNv, Sv>), grid, block, lds, ctx->stream, p)
 #define AGPU_I8_SETS(MTv, LNv)                         \
     do {                                               \
-        if (items_per_wave <= 1) AGPU_I8_LAUNCH(MTv, LNv, 1); \
-        else if (items_per_wave == 2) AGPU_I8_LAUNCH(MTv, LNv, 2); \
-        else AGPU_I8_LAUNCH(MTv, LNv, 4);              \
+        if (items_per_wave == 2) AGPU_I8_LAUNCH(MTv, LNv, 2); \
+        else AGPU_I8_LAUNCH(MTv, LNv, 1);              \
     } while (0)
     if (a.ln_gamma) {
         if (MT == 1) AGPU_I8_SETS(1, true);
