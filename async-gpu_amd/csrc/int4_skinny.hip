@@ -440,6 +440,12 @@ int32_t agpu_int4_skinny_launch(agpu_ctx *ctx, const GemvArgs &a) {
 // with A and B computed once per model (px_fold_kernel, double accumulation over the dequantized weights), so the
 // statistics are needed only when the sums are finished.  Same arithmetic otherwise: exact products, fp32 scales.
 
+#ifndef PX_AHEAD
+#define PX_AHEAD 2
+#endif
+#ifndef PX_WAVES
+#define PX_WAVES 16
+#endif
 struct PxParams {
     GemvArgs a;             // x, ln_gamma, ln_beta unused
     PxIn in;
@@ -524,9 +530,9 @@ __global__ void px_fold_kernel(const uint32_t *packed, const float *scales, int 
 
 // One workgroup = one tile of 16 CPL columns x one K split of up to SK_MAX_TRIPS trips; waves take trips round robin.
 // LDS: red [W][16][16 CPL] per-wave sums, then fin [16][16 CPL] finished outputs for the pieces of the next Linear.
-template <bool LNF, int CPL>
-__global__ __launch_bounds__(1024) void int4_skinny_px_kernel(const PxParams p) {
-    constexpr int NW = 16, TPW = (SK_MAX_TRIPS + NW - 1) / NW, COLS = 16 * CPL, MT = 16, n_out = MT * COLS;
+template <bool LNF, int CPL, int NW>
+__global__ __launch_bounds__(64 * NW) void int4_skinny_px_kernel(const PxParams p) {
+    constexpr int TPW = (SK_MAX_TRIPS + NW - 1) / NW, COLS = 16 * CPL, MT = 16, n_out = MT * COLS;
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float s_mean[MT], s_rstd[MT];
     __shared__ int s_last;
@@ -559,8 +565,10 @@ __global__ __launch_bounds__(1024) void int4_skinny_px_kernel(const PxParams p) 
     uint32_t w4[TPW][CPL];
     float sc4[TPW][CPL];
     uint4 af[TPW][3];
-#pragma unroll
-    for (int u = 0; u < TPW; ++u) {
+    // A wave's trips are requested two ahead of their use: with all of them on their way at once (320 KB per CU) the
+    // requests only queue.
+    constexpr int AHEAD = PX_AHEAD;
+    auto request = [&](int u) {
         const int trip = t0 + wave + u * W;
 #pragma unroll
         for (int c = 0; c < CPL; ++c) {
@@ -589,7 +597,10 @@ __global__ __launch_bounds__(1024) void int4_skinny_px_kernel(const PxParams p) 
                 }
             }
         }
-    }
+    };
+#pragma unroll
+    for (int u = 0; u < TPW; ++u)
+        if (u < AHEAD) request(u);
     // operands of this thread's first output, requested early
     float e_bias = 0.0f, e_res = 0.0f, e_fa = 0.0f, e_fb = 0.0f;
     if (tid < n_out) {
@@ -628,6 +639,7 @@ __global__ __launch_bounds__(1024) void int4_skinny_px_kernel(const PxParams p) 
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[c][r] = fmaf(sc4[u][c], d[r], acc[c][r]);
         }
+        if (u + AHEAD < TPW) request(u + AHEAD);
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -726,17 +738,17 @@ __global__ __launch_bounds__(1024) void int4_skinny_px_kernel(const PxParams p) 
     PX_STAMP(7);
 }
 
-template <bool LNF, int CPL>
+template <bool LNF, int CPL, int NW>
 int32_t px_go(agpu_ctx *ctx, const PxParams &p, dim3 grid, int W, size_t lds) {
     static std::atomic<unsigned long long> lds_raised{0};
     const unsigned long long dev_bit = 1ull << (ctx->device & 63);
     if (lds > 48 * 1024 && !(lds_raised.load(std::memory_order_relaxed) & dev_bit)) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(int4_skinny_px_kernel<LNF, CPL>),
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(int4_skinny_px_kernel<LNF, CPL, NW>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 17 * 16 * 64 * 4);
         if (e != hipSuccess) return agpu_hip(ctx, e, "hipFuncSetAttribute");
         lds_raised.fetch_or(dev_bit, std::memory_order_relaxed);
     }
-    hipLaunchKernelGGL((int4_skinny_px_kernel<LNF, CPL>), grid, dim3(64 * W), lds, ctx->stream, p);
+    hipLaunchKernelGGL((int4_skinny_px_kernel<LNF, CPL, NW>), grid, dim3(64 * W), lds, ctx->stream, p);
     return AGPU_LAUNCH_CHECK(ctx, "int4_skinny_px_kernel");
 }
 
@@ -771,13 +783,14 @@ int32_t agpu_int4_skinny_px_launch(agpu_ctx *ctx, const GemvArgs &a, const PxIn 
     const int col_blocks = ceil_div(a.N, cols);
     if (col_blocks > ctx->n_counters) return agpu_fail(ctx, AGPU_ERR_WORKSPACE, "int4_skinny: N=%d too large", a.N);
     p.trips_per_split = tps;
-    const int W = tps < 16 ? (tps < 2 ? 2 : tps) : 16;  // two waves at least: the pieces are written by 2 cols threads
+    constexpr int NW = PX_WAVES;
+    const int W = tps < NW ? (tps < 2 ? 2 : tps) : NW;  // two waves at least: the pieces are written by 2 cols threads
     const size_t lds = sizeof(float) * (size_t)(W + 1) * 16 * cols;
     p.partial = reinterpret_cast<float *>(ctx->workspace);
     p.counters = ctx->counters;
     const dim3 grid(col_blocks, ksplit);
-    if (in.stats) return narrow ? px_go<true, 2>(ctx, p, grid, W, lds) : px_go<true, 4>(ctx, p, grid, W, lds);
-    return narrow ? px_go<false, 2>(ctx, p, grid, W, lds) : px_go<false, 4>(ctx, p, grid, W, lds);
+    if (in.stats) return narrow ? px_go<true, 2, NW>(ctx, p, grid, W, lds) : px_go<true, 4, NW>(ctx, p, grid, W, lds);
+    return narrow ? px_go<false, 2, NW>(ctx, p, grid, W, lds) : px_go<false, 4, NW>(ctx, p, grid, W, lds);
 }
 
 int32_t agpu_px_split_rows_launch(agpu_ctx *ctx, const float *x, int M, int K, const PxOut &out) {
