@@ -16,7 +16,7 @@
 // staged through LDS, double buffered, in exactly the order the A operand wants them: thread t splits the 8 floats
 // k = 8 * (t % 8) .. + 7 of row t / 8 (and of row t / 8 + 32 when RB = 2) and writes one 16-byte fragment per
 // piece, so an MFMA's A operand is one conflict-free 1 KiB read.  B words and scales come straight from global
-// memory, one block ahead; a word (8 nibbles of one column) becomes the 8 bf16 of one B fragment in the order
+// memory, requested a whole block before their first use; a word (8 nibbles of one column) becomes the 8 bf16 of one B fragment in the order
 // (0, 2, 4, 6, 1, 3, 5, 7) of its nibbles, which is the order the x fragments are packed in as well.
 //   A fragment: lane (i, hh) = row i, the 8 k of half hh of a 16-k step
 //   B fragment: lane (j, hh) = column j, the same 8 k: packed row 4 * chunk + 2 * step + hh
@@ -49,6 +49,7 @@ struct GemmBfParams {
     int col_tiles;           // tiles per row of tiles; tile t = (t / col_tiles, t % col_tiles)
     int full_tiles;          // tiles 0 .. full_tiles - 1 have one workgroup each, the others tail_ks workgroups (slices of K)
     int tail_ks, n_tail;     // ... and how many tiles those others are
+    int xcd_rows;            // tiles numbered so that workgroups of one XCD share rows of tiles (see the kernel)
     float *partial;          // [tail_ks, n_tail tiles] partial results
     unsigned int *counters;  // one ticket per output tile, left at zero
     KvScatter kv;            // kcache == nullptr: none
@@ -95,6 +96,23 @@ constexpr float GB_NIBBLE_UNIT = 16.0f;  // what nibbles_to_bf16 divides by
 
 // RB row blocks of 32 per workgroup, CB column blocks of 32 per wave, NCH 32-k chunks per K block, GB_WAVES waves (4 or
 // 8; the first four stage x)
+#ifdef AGPU_GB_TRACE
+// Debug builds: shader-clock stamps of lane 0 of every wave of the first sixteen workgroups, per K block
+__device__ unsigned long long gb_trace[16][8][16][8];
+#define GB_STAMP(kbrel, slot)                                                                              \
+    do {                                                                                                   \
+        if (lane == 0 && blockIdx.x < 16 && (kbrel) < 16) gb_trace[blockIdx.x][wave][kbrel][slot] = clock64(); \
+    } while (0)
+__device__ unsigned long long gb_phase[2048][4];
+#define GB_PHASE(slot)                                                                     \
+    do {                                                                                   \
+        if (threadIdx.x == 0 && blockIdx.x < 2048) gb_phase[blockIdx.x][slot] = wall_clock64(); \
+    } while (0)
+#else
+#define GB_STAMP(kbrel, slot)
+#define GB_PHASE(slot)
+#endif
+
 template <int RB, int CB, int NCH, int GB_WAVES>
 __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const GemmBfParams p) {
     static_assert(NCH % 2 == 0, "staging works on 64-k halves");
@@ -105,6 +123,7 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
     __shared__ int s_last;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int j = lane & 31, hh = lane >> 5;
+    GB_PHASE(0);
     const int chunks = p.K / 32, kblocks = (chunks + NCH - 1) / NCH;
     // workgroup -> (tile, slice of K): whole tiles first, then the slices of the remaining tiles
     int tile_no, split, ksplit, bps;
@@ -116,7 +135,18 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
         const int t = blockIdx.x - p.full_tiles;
         split = t / p.n_tail; tile_no = p.full_tiles + (t - split * p.n_tail); ksplit = p.tail_ks; bps = p.blocks_per_split;
     }
-    const int tile_row = tile_no / p.col_tiles, tile_col = tile_no - tile_row * p.col_tiles;
+    // Workgroup b runs on XCD b % 8, each with an L2 of its own.  With the tiles numbered row by row every XCD would
+    // walk all of x and all of the weights (M = 1024, K = 768, N = 2304: 4.2 MB, more than its 4 MB); numbered so that
+    // an XCD owns whole rows of tiles, it reads an eighth of x and the weights.
+    int tile_row, tile_col;
+    if (p.xcd_rows) {
+        const int xcd = tile_no & 7, idx = tile_no >> 3, r = idx / p.col_tiles;
+        tile_row = r * 8 + xcd;
+        tile_col = idx - r * p.col_tiles;
+    } else {
+        tile_row = tile_no / p.col_tiles;
+        tile_col = tile_no - tile_row * p.col_tiles;
+    }
     const int m0 = tile_row * GB_BM, n0 = tile_col * GB_BN + wave * 32 * CB;
     const int kb0 = split * bps, kb1 = min(kblocks, kb0 + bps);
     const bool wave_active = n0 < p.N;
@@ -179,8 +209,8 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
                 const uint32_t *src = p.packed + (size_t)(4 * chunk + hh) * p.N + col[cb];
                 bw[set][c][cb][0] = src[0];
                 bw[set][c][cb][1] = src[2 * (size_t)p.N];
-                const float sc = p.scales[(size_t)(chunk >> p.chunk_shift) * p.N + col[cb]];
-                bs[set][c][cb] = valid ? sc * GB_NIBBLE_UNIT : 0.0f;
+                // as loaded: nothing may touch a value on the way in before its block, or the wave waits for it on the spot
+                bs[set][c][cb] = p.scales[(size_t)(chunk >> p.chunk_shift) * p.N + col[cb]];
             }
         }
     };
@@ -201,12 +231,13 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
 
     bf16x8 bf[2][CB][2];  // [chunk parity][column tile][step]: chunk c + 1 is converted while chunk c is in use
     float sc[2][CB];
-    auto convert = [&](int set, int c) {
+    auto convert = [&](int kb, int set, int c) {  // chunk c of block kb, whose words are in register set `set`
+        const bool valid = kb * NCH + c < chunks;
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
 #pragma unroll
             for (int st = 0; st < 2; ++st) bf[c & 1][cb][st] = nibbles_to_bf16(bw[set][c][cb][st]);
-            sc[c & 1][cb] = bs[set][c][cb];
+            sc[c & 1][cb] = valid ? bs[set][c][cb] * GB_NIBBLE_UNIT : 0.0f;
         }
     };
 
@@ -214,18 +245,22 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
     load_x(kb0, 0);
     load_b(kb0, 0);
     load_x(min(kb0 + 1, kblocks), 1);
+    load_b(min(kb0 + 1, kblocks), 1);
 #pragma unroll
     for (int ps = 0; ps < NP; ++ps) stage_half(kb0, 0, 0, ps);
-    convert(0, 0);
+    convert(kb0, 0, 0);
     __syncthreads();
+    GB_PHASE(1);
 
-    // One K block; P = its parity.  Reads what earlier iterations requested, then requests block + 1 (words) and
-    // block + 2 (x), then works on with the MFMAs of a group beside the vector work named at its end.
+    // One K block; P = its parity.  Reads what earlier iterations requested, requests x of block + 2 and, once this
+    // block's words are fragments, the words of block + 2 into their registers, and works on with the MFMAs of a group
+    // beside the vector work named at its end.
     auto block = [&](int kb, auto parity) {
         constexpr int P = decltype(parity)::value;
         floatx16 gs[2][CB];  // [group parity][column tile]: the sums of one chunk and row block
         const floatx16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         bf16x8 a[3][2];
+        GB_STAMP(kb - kb0, 0);
 #pragma unroll
         for (int piece = 0; piece < 3; ++piece)
 #pragma unroll
@@ -253,28 +288,41 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
                     for (int r = 0; r < 16; ++r) acc[prb][cb][r] = fmaf(sc[pc & 1][cb], gs[pg][cb][r], acc[prb][cb][r]);
             }
             // then the words of the next chunk become fragments (in place of those of the chunk before this one)
-            if (t % RB == 0 && c + 1 < NCH) convert(P, c + 1);
+            if (t % RB == 0 && c + 1 < NCH) convert(kb, P, c + 1);
             if (t == 0) {  // that was the first read of registers that a load of the previous iteration fills
                 __builtin_amdgcn_sched_barrier(0);
-                load_b(min(kb + 1, kblocks), P ^ 1);
                 load_x(min(kb + 2, kblocks), P);
+            }
+            // this block's words are all fragments now: their registers take the words of the block after the next, which
+            // then have a whole block's time to arrive
+            if (t == (NCH - 1) * RB) {
+                __builtin_amdgcn_sched_barrier(0);
+                load_b(min(kb + 2, kblocks), P);
             }
             if (t >= 1 && t - 1 < NP) stage_half(kb + 1, P ^ 1, P ^ 1, t - 1);
             __builtin_amdgcn_sched_barrier(0);  // a group's vector work stays beside its MFMAs
+            if (t < 4) GB_STAMP(kb - kb0, 1 + t);
         }
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
             for (int r = 0; r < 16; ++r)
                 acc[RB - 1][cb][r] = fmaf(sc[(NCH - 1) & 1][cb], gs[(NCH * RB - 1) & 1][cb][r], acc[RB - 1][cb][r]);
-        convert(P ^ 1, 0);  // chunk 0 of the next block
+        convert(kb + 1, P ^ 1, 0);  // chunk 0 of the next block
+        GB_STAMP(kb - kb0, 5);
         __syncthreads();
+        GB_STAMP(kb - kb0, 6);
     };
-    for (int kb = kb0; kb < kb1; kb += 2) {
+    // Pairs of blocks, then the odd one: with the second block of a pair behind a branch, the loop's head would also be
+    // reached from the end of a first block, and the compiler would make every pair wait for the loads just requested.
+    int kb = kb0;
+    for (; kb + 1 < kb1; kb += 2) {
         block(kb, std::integral_constant<int, 0>{});
-        if (kb + 1 < kb1) block(kb + 1, std::integral_constant<int, 1>{});
+        block(kb + 1, std::integral_constant<int, 1>{});
     }
+    if (kb < kb1) block(kb, std::integral_constant<int, 0>{});
 
+    GB_PHASE(2);
     // element (rb, cb, r) of this lane: row m0 + 32 rb + 8 (r / 4) + 4 hh + r % 4, column n0 + 32 cb + j
     auto row_of = [&](int rb, int r) { return m0 + 32 * rb + 8 * (r >> 2) + 4 * hh + (r & 3); };
     if (ksplit > 1) {
@@ -338,6 +386,7 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
         }
     }
     if (!wave_active) return;
+    const int kv_pos = p.kv.kcache ? *p.kv.pos_dev : 0;  // read once: inside the loops it was a load and a wait per element
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) {
         const int n = n0 + 32 * cb + j;
@@ -345,7 +394,12 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
         const float bias = p.bias ? p.bias[n] : 0.0f;
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
-            float vals[16];
+            float vals[16], res[16];
+            // all sixteen residuals requested before the first is used (rows past M repeat the last one): asked for one by
+            // one inside the loop below, each would be waited for before the next is requested
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                res[r] = p.residual ? p.residual[(size_t)min(row_of(rb, r), p.M - 1) * p.N + n] : 0.0f;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int m = row_of(rb, r);
@@ -354,13 +408,13 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
                 else if (p.flags & AGPU_EPI_GELU_QUICK) v = gelu_quick_dev(v);
                 vals[r] = v;
                 if (m < p.M) {
-                    if (p.residual) v += p.residual[(size_t)m * p.N + n];
+                    v += res[r];
                     p.y[(size_t)m * p.N + n] = v;
                     if (p.kv.kcache && n >= p.N / 3) {
                         const int dm = p.N / 3, jj = n - dm, in_v = jj >= dm ? 1 : 0, e = jj - in_v * dm;
                         const int b = m / p.kv.new_len, s = m - b * p.kv.new_len;
                         float *dst = in_v ? p.kv.vcache : p.kv.kcache;
-                        dst[((size_t)(b * p.kv.n_heads + (e >> 6)) * p.kv.n_positions + *p.kv.pos_dev + s) * 64 + (e & 63)] = v;
+                        dst[((size_t)(b * p.kv.n_heads + (e >> 6)) * p.kv.n_positions + kv_pos + s) * 64 + (e & 63)] = v;
                     }
                 }
             }
@@ -416,6 +470,10 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
             }
         }
     }
+#ifdef AGPU_GB_TRACE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores have left
+    GB_PHASE(3);
+#endif
 }
 
 enum class GemmVariant { Small, LongBlocks, Wide, Large };
@@ -448,6 +506,15 @@ bool agpu_int4_gemm_bf16_supported(const void *x, int M, int N, int K, int group
     (void)N;
     return M > 16 && group % 32 == 0 && ((group / 32) & (group / 32 - 1)) == 0 && K % 32 == 0 && ((uintptr_t)x % 16) == 0;
 }
+
+#ifdef AGPU_GB_TRACE
+AGPU_EXPORT int32_t agpu_dev_gb_phase(unsigned long long *out_host) {
+    return (int32_t)hipMemcpyFromSymbol(out_host, HIP_SYMBOL(gb_phase), sizeof(unsigned long long) * 2048 * 4);
+}
+AGPU_EXPORT int32_t agpu_dev_gb_trace(unsigned long long *out_host) {
+    return (int32_t)hipMemcpyFromSymbol(out_host, HIP_SYMBOL(gb_trace), sizeof(unsigned long long) * 16 * 8 * 16 * 8);
+}
+#endif
 
 int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t *packed, const float *scales, const float *bias,
                                    const float *residual, float *y, int M, int N, int K, int group, uint32_t flags,
@@ -514,6 +581,7 @@ int32_t agpu_int4_gemm_bf16_launch(agpu_ctx *ctx, const float *x, const uint32_t
         }
     }
     p.n_tail = tiles - p.full_tiles;
+    p.xcd_rows = ceil_div(M, BM) % 8 == 0 && p.full_tiles % 8 == 0 && p.n_tail % 8 == 0;
     p.partial = reinterpret_cast<float *>(ctx->workspace);
     p.counters = ctx->counters;
     const dim3 grid(p.full_tiles + p.n_tail * p.tail_ks);
