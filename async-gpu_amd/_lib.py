@@ -66,6 +66,7 @@ SIGNATURES = {
     "agpu_int4_linear_pieces": (_i32, [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32, _vp, _vp, _vp]),
     "agpu_bench_int4_linear": (_i32, [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _u32,
                                       _i32, C.c_int64, C.c_int64, _i32, _vp]),
+    "agpu_bench_read_stream": (_i32, [_vp, _vp, C.c_int64, _i32, C.c_int64, _i32, _vp]),
     "agpu_int4_dequantize": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32]),
     "agpu_int4_quantize": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32]),
     "agpu_int4_quantize_host": (_i32, [_vp, _vp, _vp, _i32, _i32, _i32, _i32]),

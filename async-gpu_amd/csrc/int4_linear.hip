@@ -8,6 +8,7 @@
 // (one word per lane) or 1 KiB (four words per lane) of contiguous memory.
 #include "elementwise.h"
 #include "linear_common.h"
+#include <algorithm>
 
 namespace {
 
@@ -299,6 +300,68 @@ AGPU_EXPORT int32_t agpu_bench_int4_linear(agpu_ctx *ctx, const float *x, const 
     if (rc != AGPU_OK || e != hipSuccess) {
         if (graph) (void)hipGraphDestroy(graph);
         return rc != AGPU_OK ? rc : agpu_hip(ctx, e, "hipStreamEndCapture");
+    }
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipGraphInstantiate");
+    float ms = 0.0f;
+    e = hipGraphLaunch(exec, ctx->stream);  // warm-up replay
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e == hipSuccess) rc = agpu_timer_start(ctx);
+    if (e == hipSuccess && rc == AGPU_OK) e = hipGraphLaunch(exec, ctx->stream);
+    if (e == hipSuccess && rc == AGPU_OK) rc = agpu_timer_stop(ctx, &ms);
+    (void)hipGraphExecDestroy(exec);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipGraphLaunch");
+    *us_per_launch_out_host = ms * 1000.0f / (float)reps;
+    return rc;
+}
+
+namespace {
+// Reads `vec16` 16-byte words and does nothing with them (the store never happens: it only keeps the loads alive).
+// Eight requests per thread on their way at a time, consecutive threads on consecutive words.
+__global__ __launch_bounds__(512) void read_stream_kernel(const uint4 *__restrict__ src, size_t vec16, unsigned int *sink) {
+    const size_t threads = (size_t)gridDim.x * blockDim.x;
+    uint4 acc = make_uint4(0, 0, 0, 0);
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < vec16; i += 8 * threads) {
+        uint4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = src[min(i + u * threads, vec16 - 1)];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            acc.x ^= v[u].x; acc.y |= v[u].y; acc.z ^= v[u].z; acc.w |= v[u].w;
+        }
+    }
+    if ((acc.x ^ acc.z) == 0x9e3779b9u && (acc.y & acc.w) == 0x7f4a7c15u) *sink = acc.x;
+}
+}  // namespace
+
+AGPU_EXPORT int32_t agpu_bench_read_stream(agpu_ctx *ctx, const void *buf, int64_t bytes, int32_t n_sets,
+                                           int64_t set_stride_bytes, int32_t reps, float *us_per_launch_out_host) {
+    AGPU_REQUIRE_CTX(ctx);
+    AGPU_REQUIRE_PTR(ctx, buf);
+    AGPU_REQUIRE_PTR(ctx, us_per_launch_out_host);
+    if (reps <= 0 || n_sets <= 0 || bytes < 16 || bytes % 16 || set_stride_bytes % 16 || ((uintptr_t)buf % 16))
+        return agpu_fail(ctx, AGPU_ERR_SHAPE_MISMATCH, "bench_read_stream: sizes must be positive multiples of 16 bytes");
+    if (!ctx->stream) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "bench_read_stream: needs a context with its own stream");
+    const size_t vec16 = (size_t)bytes / 16;
+    const unsigned wgs = (unsigned)std::min<size_t>((size_t)ctx->num_cus * 2, (vec16 + 511) / 512);
+    unsigned int *sink = reinterpret_cast<unsigned int *>(ctx->workspace);
+    auto launch = [&](int i) {
+        const char *src = static_cast<const char *>(buf) + (size_t)(i % n_sets) * (size_t)set_stride_bytes;
+        hipLaunchKernelGGL(read_stream_kernel, dim3(wgs), dim3(512), 0, ctx->stream, reinterpret_cast<const uint4 *>(src), vec16, sink);
+    };
+    launch(0);
+    int32_t rc = AGPU_LAUNCH_CHECK(ctx, "read_stream_kernel");
+    if (rc != AGPU_OK) return rc;
+    hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
+    if (e != hipSuccess) return agpu_hip(ctx, e, "hipStreamBeginCapture");
+    for (int i = 0; i < reps; ++i) launch(i);
+    hipGraph_t graph = nullptr;
+    e = hipStreamEndCapture(ctx->stream, &graph);
+    if (e != hipSuccess) {
+        if (graph) (void)hipGraphDestroy(graph);
+        return agpu_hip(ctx, e, "hipStreamEndCapture");
     }
     hipGraphExec_t exec = nullptr;
     e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);

@@ -58,7 +58,8 @@ def roofline_lm_head(ctx, cfg, group, workloads):
     recorded into a HIP graph and replayed; HIP events on the context's stream bracket the replay.
     Two figures: a rotation over 12 weight copies (290 MB, larger than the caches) is the HBM
     figure reported as `achieved`; the same weights every launch (cache resident, as in decode,
-    where the 78 MB model stays in the 256 MB Infinity Cache) is reported beside it."""
+    where the 78 MB model stays in the 256 MB Infinity Cache) is reported beside it, and so is
+    `read_only_launch_us`: a launch that only reads as many bytes from the same rotation and computes nothing."""
     import ctypes as C
     K, N = cfg["n_embd"], ((cfg["vocab"] + 255) // 256) * 256
     rng = np.random.default_rng(0)
@@ -78,6 +79,12 @@ def roofline_lm_head(ctx, cfg, group, workloads):
     us_hot = time_gemv(1)
     us = time_gemv(n_sets)
     gb = gemv_bytes(K, N, group)
+    # the same bytes read by a launch that computes nothing, over the same rotation: what "streaming" costs here at best
+    us_read = C.c_float(0)
+    set_bytes = packed.nbytes
+    read_bytes = (int(gb) + 15) // 16 * 16  # more than one copy of the packed words: the last copy is left out of the rotation
+    assert set_bytes < read_bytes <= 2 * set_bytes
+    ctx.call("agpu_bench_read_stream", dp, read_bytes, n_sets - 1, set_bytes, 240, C.addressof(us_read))
     for p in (dp, ds, dx, dy):
         ctx.free(p)
     achieved = gb / (us * 1e-6) / 1e9
@@ -85,7 +92,7 @@ def roofline_lm_head(ctx, cfg, group, workloads):
             "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5),
             "traffic": TRAFFIC_BYTES_LM_HEAD, "bytes_per_launch": int(gb), "us_per_launch": round(us, 3),
             "weight_sets_rotated": n_sets, "cache_resident_GBps": round(gb / (us_hot * 1e-6) / 1e9, 2),
-            "cache_resident_us_per_launch": round(us_hot, 3)}
+            "cache_resident_us_per_launch": round(us_hot, 3), "read_only_launch_us": round(float(us_read.value), 3)}
 
 
 def main():

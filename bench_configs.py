@@ -197,6 +197,17 @@ def kernel_cases(ctx, emit, bench_linear, workloads, args=None):
         us = bench_linear(1, K, N, reps=120, sets=sets)
         emit(case=f"int4 GEMV M=1 K={K} N={N} g=32 (LM head), {sets} rotating weight copies", us=round(us, 3),
              algorithmic_bytes=b, GBps=round(b / us / 1e3, 1), frac_hbm=round(b / us / 1e3 / HBM_GBS, 4))
+    # what a launch costs that only reads the bytes of these GEMVs (no arithmetic): the bound a streaming kernel of that
+    # size can be held against
+    for name, nbytes, sets in (("config 1 GEMV", 768 * 3072 // 2 + 24 * 3072 * 4, 256), ("LM head K=768", 768 * 50432 // 2 + 24 * 50432 * 4, 12),
+                               ("LM head K=1600", 1600 * 50432 // 2 + 50 * 50432 * 4, 6)):
+        nbytes = (nbytes + 15) // 16 * 16
+        buf = ctx.malloc(nbytes * sets)
+        us_c = C.c_float(0)
+        ctx.call("agpu_bench_read_stream", buf, nbytes, sets, nbytes, 240, C.addressof(us_c))
+        emit(case=f"read-only launch over the bytes of {name}, {sets} rotating copies", us=round(us_c.value, 3), bytes=nbytes,
+             GBps=round(nbytes / us_c.value / 1e3, 1), frac_hbm=round(nbytes / us_c.value / 1e3 / HBM_GBS, 4))
+        ctx.free(buf)
     # config 2: prefill QKV dequant-GEMM
     for M in (128, 512, 1024):
         us = bench_linear(M, 768, 2304, reps=50)

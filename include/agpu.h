@@ -220,6 +220,15 @@ int32_t agpu_bench_int4_linear(agpu_ctx *ctx, const float *x, const float *gamma
                                uint32_t flags, int32_t n_weight_sets, int64_t packed_set_stride,
                                int64_t scales_set_stride, int32_t reps, float *us_per_launch_out_host);
 
+/* Measurement helper (no counterpart in the reference): what a launch costs that only reads `bytes` bytes
+ * (a multiple of 16) and computes nothing: `reps` back-to-back launches in a HIP graph, launch i reading
+ * buf + (i % n_sets) * set_stride_bytes, mean microseconds per launch from HIP events.  The time of a
+ * kernel that streams the same bytes is to be read against this, not against bytes / peak bandwidth
+ * alone: a launch has a start, a ramp and an end however little it does.  Needs a context that owns
+ * its stream. */
+int32_t agpu_bench_read_stream(agpu_ctx *ctx, const void *buf, int64_t bytes, int32_t n_sets,
+                               int64_t set_stride_bytes, int32_t reps, float *us_per_launch_out_host);
+
 /* W[K,N] = (float)(nibble-8) * scale: the kernel's inline dequantisation
  * (compute_gemm.rs:2882-2886) / nn/ops/quantize.rs:158-162 as a standalone, bit-exact hook. */
 int32_t agpu_int4_dequantize(agpu_ctx *ctx, const uint32_t *packed, const float *scales, float *w_out,

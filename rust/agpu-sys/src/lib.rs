@@ -107,6 +107,7 @@ extern "C" {
     pub fn agpu_ln_int4_linear(ctx: *mut agpu_ctx, x: *const f32, gamma: *const f32, beta: *const f32, eps: f32, packed: *const u32, scales: *const f32, bias: *const f32, residual: *const f32, y: *mut f32, M: i32, N: i32, K: i32, group: i32, flags: u32) -> i32;
     pub fn agpu_int4_linear_pieces(ctx: *mut agpu_ctx, x: *const f32, gamma: *const f32, beta: *const f32, eps: f32, packed: *const u32, scales: *const f32, bias: *const f32, residual: *const f32, y: *mut f32, M: i32, N: i32, K: i32, group: i32, flags: u32, out_gamma: *const f32, out_pieces: *mut c_void, out_stats: *mut f32) -> i32;
     pub fn agpu_bench_int4_linear(ctx: *mut agpu_ctx, x: *const f32, gamma: *const f32, beta: *const f32, eps: f32, packed: *const u32, scales: *const f32, bias: *const f32, residual: *const f32, y: *mut f32, M: i32, N: i32, K: i32, group: i32, flags: u32, n_weight_sets: i32, packed_set_stride: i64, scales_set_stride: i64, reps: i32, us_per_launch_out_host: *mut f32) -> i32;
+    pub fn agpu_bench_read_stream(ctx: *mut agpu_ctx, buf: *const c_void, bytes: i64, n_sets: i32, set_stride_bytes: i64, reps: i32, us_per_launch_out_host: *mut f32) -> i32;
     pub fn agpu_int4_dequantize(ctx: *mut agpu_ctx, packed: *const u32, scales: *const f32, w_out: *mut f32, K: i32, N: i32, group: i32) -> i32;
     pub fn agpu_int4_quantize(ctx: *mut agpu_ctx, weight_t: *const f32, packed: *mut u32, scales: *mut f32, K: i32, N: i32, group: i32, mode: i32) -> i32;
     pub fn agpu_int4_quantize_host(weight_t_host: *const f32, packed_host: *mut u32, scales_host: *mut f32, K: i32, N: i32, group: i32, mode: i32) -> i32;
