@@ -88,7 +88,7 @@ def roofline_lm_head(ctx, cfg, group, workloads):
     for p in (dp, ds, dx, dy):
         ctx.free(p)
     achieved = gb / (us * 1e-6) / 1e9
-    return {"bound": "hbm", "kernel": "int4_gemv_i8_kernel<1,false,4> (LM head shape M=1 K=768 N=50432 g=32)",
+    return {"bound": "hbm", "kernel": "int4_gemv_i8_kernel<1,false,1> (LM head shape M=1 K=768 N=50432 g=32)",
             "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5),
             "traffic": TRAFFIC_BYTES_LM_HEAD, "bytes_per_launch": int(gb), "us_per_launch": round(us, 3),
             "weight_sets_rotated": n_sets, "cache_resident_GBps": round(gb / (us_hot * 1e-6) / 1e9, 2),
