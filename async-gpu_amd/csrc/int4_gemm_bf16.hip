@@ -479,19 +479,22 @@ __global__ __launch_bounds__(64 * GB_WAVES, 2) void int4_gemm_bf16_kernel(const 
 enum class GemmVariant { Small, LongBlocks, Wide, Large };
 
 GemmVariant pick_variant(const agpu_ctx *ctx, int M, int N, int K) {
-    // Workgroup tile: 32 rows x 128 columns (one 32 x 32 tile per wave), which puts the most waves on the chip for
-    // the layer sizes of GPT-2 small; 64 x 256 (every weight fragment serves two row blocks, every x fragment two
-    // column blocks) once that still leaves a workgroup per CU.  M = 1024, K = 768, N = 2304: 25.8 us with the
-    // small tile, 28.2 us with 32 x 256, 33.1 us with 64 x 256; K = 1600, N = 6400: 96.5 us with the large tile,
-    // 105.6 us with 32 x 256.
-    const bool large = ceil_div(N, 256) * ceil_div(M, 64) >= ctx->num_cus;
+    // Workgroup tile: 32 rows x 128 columns (one 32 x 32 tile per wave), which puts the most waves on the chip, unless
+    // a measurement says otherwise (us per launch, small tile against the other; swept over 64 .. 4096 rows):
+    //   64 x 256 (every weight fragment serves two row blocks, every x fragment two column blocks) from 1.5 such tiles
+    //   per CU and a long K: M = 1024, K = 1600, N = 6400 (1.56 per CU): 95 against 87; M = 4096, K = 1600, N = 4800: 228 against 196; M = 2048, N = 6400: 155 against 131;
+    //   M = 4096, K = 6400, N = 1600: 288 against 254; but M = 1024, K = 1600, N = 4800 (1.2 per CU): 64 against 75,
+    //   and with K = 768 the small tile wins at any size (M = 4096, N = 2304: 57 - 61 against 67).
+    const bool large = K >= 1536 && 2 * ceil_div(N, 256) * ceil_div(M, 64) >= 3 * ctx->num_cus;
     // K per block: 64; 128 for the small tile on small problems (fewer barriers and loop ends per k, but 159
     // registers against 126, three waves per SIMD against four: M = 512, K = 768, N = 2304: 17.5 us against 18.7 us;
     // M = 1024: 27.3 us against 25.8 us)
     const bool long_blocks = !large && (long long)ceil_div(N, 128) * ceil_div(M, 32) * ceil_div(K, 64) <= 5000;
-    // With a long K the split of x weighs more: eight waves share one 32-row x tile over 256 columns, the first four
-    // stage it (M = 1024, K = 1600, N = 1600: 32.8 us against 38.1 us; K = 768, N = 2304: 27.3 us against 25.2 us)
-    const bool wide = !large && !long_blocks && K >= 1536;
+    // 32 x 256 with eight waves, the first four staging x (a long K, where the split of x weighs more), only while the
+    // small tiles would not fill the chip and the matrix is wide enough for 256-column tiles: M = 512, K = 1600,
+    // N = 1600: 18.6 against 17.3; M = 1024, K = 2048, N = 1024: 23.1 against 21.4; but M = 1024, K = 3072, N = 768:
+    // 24.9 against 28.2; M = 512, K = 1600, N = 4800: 32.9 against 45.9; M = 1024, K = 6400, N = 1600: 81.6 against 89.3.
+    const bool wide = !large && !long_blocks && K >= 1536 && N >= 1024 && ceil_div(N, 128) * ceil_div(M, 32) <= ctx->num_cus;
     return large ? GemmVariant::Large : long_blocks ? GemmVariant::LongBlocks : wide ? GemmVariant::Wide : GemmVariant::Small;
 }
 

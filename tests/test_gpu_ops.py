@@ -315,13 +315,15 @@ def test_gemm_fp32_matrix_core_kernel(agpu, orc, dev, K, N, g, M):
 
 @pytest.mark.parametrize("K,N,g,M", [(32, 40, 32, 17), (96, 33, 32, 40), (160, 257, 32, 33), (768, 2304, 64, 100),
                                      (1024, 300, 256, 65), (6400, 1600, 32, 48), (64, 8200, 32, 2050),
-                                     (1600, 1608, 32, 1000), (768, 2304, 32, 1000), (768, 3072, 32, 520), (512, 1100, 32, 1024)])
+                                     (1600, 1608, 32, 1000), (768, 2304, 32, 1000), (768, 3072, 32, 520), (512, 1100, 32, 1024),
+                                     (768, 1000, 32, 256), (3072, 768, 32, 1024)])
 def test_gemm_bf16_matrix_core_shapes(agpu, orc, dev, K, N, g, M):
     """M > 16, group = 32 * 2^n, K % 32 == 0: one chunk, a K tail inside a 64-k block, ragged rows and columns,
     groups spanning several chunks, a long K (sliced over workgroups), enough tiles for the 64-row variant, a long K
     with many rows (the eight-wave variant), more tiles than CUs but not a multiple of them (the tiles left over are
-    sliced along K in the same launch: 64 of 576, 152 of 408, 32 of 288, with ragged last rows and columns); with a NaN
-    in one row and a wide dynamic range in another."""
+    sliced along K in the same launch: 64 of 576, 152 of 408, 32 of 288, with ragged last rows and columns); eight row
+    tiles, every tile sliced, ragged columns (tiles numbered XCD by XCD); the FFN-down shape with its residual; with a
+    NaN in one row and a wide dynamic range in another."""
     from async_gpu_amd import ops, workloads
     rng = np.random.default_rng(K + N + M + g)
     packed, scales, bias = workloads.random_int4_linear(rng, K, N, g, bias=True)
