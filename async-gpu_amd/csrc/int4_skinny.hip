@@ -817,6 +817,8 @@ AGPU_EXPORT int32_t agpu_int4_linear_pieces(agpu_ctx *ctx, const float *x, const
     if ((gamma == nullptr) != (beta == nullptr)) return agpu_fail(ctx, AGPU_ERR_NULL_POINTER, "int4_linear_pieces: gamma and beta go together");
     if (M < 5 || M > 16 || K < 32 || K % 32 != 0 || N < 4 || (gamma && K > 2048))
         return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "int4_linear_pieces: M=%d N=%d K=%d not taken", M, N, K);
+    if (((uintptr_t)x | (uintptr_t)gamma | (uintptr_t)out_gamma) % 16 != 0)  // read 16 bytes at a time
+        return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "int4_linear_pieces: x, gamma and out_gamma must be 16-byte aligned");
     // scratch, second half of the context's: pieces of x | statistics | A | B
     const size_t pieces_bytes = (size_t)(K / 32) * 192 * sizeof(uint4), stats_bytes = (size_t)(K / 32) * 16 * sizeof(float2);
     const size_t need = pieces_bytes + stats_bytes + 2 * (size_t)N * sizeof(float);

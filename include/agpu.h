@@ -197,7 +197,7 @@ int32_t agpu_ln_int4_linear(agpu_ctx *ctx, const float *x, const float *gamma, c
  * that chain for one Linear on fp32 rows, for tests and measurements: split x (times gamma) into pieces, fold
  * (gamma, beta) into two vectors over the N columns, then y = epilogue(LayerNorm(x) W) as agpu_ln_int4_linear
  * (gamma = beta = NULL: no LayerNorm).  5 <= M <= 16, K % 32 == 0, group a multiple of 32 up to 512, N % 4 == 0,
- * K <= 2048 with LayerNorm.  Optionally it also leaves what the next Linear would read: out_pieces (device,
+ * K <= 2048 with LayerNorm; x, gamma and out_gamma 16-byte aligned.  Optionally it also leaves what the next Linear would read: out_pieces (device,
  * N / 32 * 3072 bytes, needs N % 32 == 0): y times out_gamma (NULL: times one) as pieces
  * [N/32][3: low, middle, high][64: 16 * (n % 32 / 8) + row] x 8 bf16 in the order n % 8 = 0,4,1,5,2,6,3,7; out_stats
  * (device, N / 32 * 16 pairs of floats or NULL): per 32 columns and row the mean of y and the sum of squared
