@@ -34,3 +34,7 @@ echo "built tests/cpp/test_nn"
 g++ -O1 -std=c++17 -I../../include ../../tests/cpp/test_gpu_array_host.cpp -o ../../tests/cpp/test_gpu_array_host \
     -L.. -lagpu_hip -Wl,-rpath,'$ORIGIN/../../async-gpu_amd' -Wl,-rpath,/opt/rocm/lib -L/opt/rocm/lib -lamdhip64
 echo "built tests/cpp/test_gpu_array_host"
+# The GPT-2 example program over include/agpu_nn.hpp (tests/test_cpp_example.py, tests/test_gpu_model.py)
+g++ -O1 -std=c++17 -I../../include ../examples/gpt2_inference.cpp -o ../examples/gpt2_inference \
+    -L.. -lagpu_hip -Wl,-rpath,'$ORIGIN/..' -Wl,-rpath,/opt/rocm/lib -L/opt/rocm/lib -lamdhip64
+echo "built async-gpu_amd/examples/gpt2_inference"

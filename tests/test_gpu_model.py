@@ -473,6 +473,47 @@ def test_gpt2_inference_example_program(orc, agpu, dev, tmp_path):
     assert diag.count("  token ") == 5
 
 
+def test_gpt2_inference_cpp_example_program(orc, agpu, dev, tmp_path):
+    """The same program in C++ over include/agpu_nn.hpp (async-gpu_amd/examples/gpt2_inference.cpp), run as a process on
+    the same two files: its own safetensors reader and tokenizer, the same output lines, three MATCH lines, and the
+    tokens of every cached generation equal to those of the Python model built from the same file."""
+    import os
+    import subprocess
+    from async_gpu_amd import gpt2, tokenizer, weights, workloads
+    from test_tokenizer import CORPUS, train
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    prog = os.path.join(root, "async-gpu_amd", "examples", "gpt2_inference")
+    assert os.path.exists(prog), "async-gpu_amd/examples/gpt2_inference is not built: run async-gpu_amd/csrc/build.sh"
+    ranks, _ = train(CORPUS, 120)
+    tok = tokenizer.Gpt2Tokenizer(ranks)
+    vocab_path = str(tmp_path / "vocab.tiktoken")
+    tok.save_tiktoken_file(vocab_path)
+    cfg = dict(n_layer=2, n_embd=128, n_head=2, vocab=tok.vocab_size(), n_positions=96)
+    w = workloads.gpt2_fp32_weights(cfg, 8, std=0.08, nonzero_bias=True, random_ln=True)
+    model_path = str(tmp_path / "model.safetensors")
+    weights.save_gpt2_safetensors(model_path, w)
+    r = subprocess.run([prog, model_path, vocab_path, "--max-new-tokens", "20", "--print-tokens"], capture_output=True, text=True,
+                       timeout=110)
+    text, diag = r.stdout, r.stderr
+    assert r.returncode == 0, diag
+    assert text.startswith("HIP device initialized\nKernel registry loaded (12 ML kernels)\nLoaded ")
+    assert text.count("MATCH: cached and non-cached outputs agree") == 3 and "MISMATCH" not in text
+    assert "Model built on GPU" in text and text.count("ms/token)") == 6 and text.rstrip().endswith("Done.")
+    for line in ("[diag] Embedding pos0 first4:", "[diag] Layer 0 pos", "[diag] Layer 1 pos", "[diag] Final LN pos", "[diag] Top-5 tokens at pos"):
+        assert line in diag, diag
+    assert diag.count("  token ") == 5
+    got = [[int(x) for x in ln.split()[1:]] for ln in text.splitlines() if ln.startswith("Tokens:")]
+    from async_gpu_amd import _lib
+    model = gpt2.Int4Gpt2Model.from_file(model_path, group_size=32, mode=_lib.QUANT_RUST, lm_head=gpt2.LM_HEAD_F32)  # the program's defaults
+    try:
+        for prompt, ids in zip(("The capital of France is", "In a world where AI", "Once upon a time"), got):
+            (ref,), _ = model.generate_cached(np.asarray(tok.encode(prompt), np.uint32), 20)
+            assert ids == [int(t) for t in ref], prompt
+    finally:
+        model.close()
+    assert len(got) == 3
+
+
 def test_forward_profiled_and_diagnostic(tiny, orc, agpu, dev):
     """forward_profiled / forward_diagnostic (gpt2.rs:529-667): the stage list, positive timings, logits equal to the
     forward's last row; the diagnostic's values against the oracle's intermediate results where it exposes them (the
