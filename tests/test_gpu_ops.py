@@ -575,6 +575,29 @@ def test_config3_attention_decode(agpu, orc, dev, kv_len, stride):
         assert np.abs(o.cpu().numpy()[:, 0] - full[:, kv_len - 1]).max() <= 1e-5
 
 
+@pytest.mark.parametrize("H,q_len,kv_len,stride", [(12, 1, 600, 1024), (25, 1, 2048, 2048), (1, 1, 513, 513), (8, 8, 700, 1024),
+                                                   (3, 4, 1024, 1024), (64, 1, 777, 800), (2, 1, 5, 4096)])
+def test_attention_decode_keys_split(agpu, orc, dev, H, q_len, kv_len, stride):
+    """A few query rows over a long cache: the keys are split over up to eight workgroups per row, whose partial results
+    meet in the context's scratch behind a ticket that the kernel leaves at zero.  Shapes with empty key ranges, with 64
+    rows (the most that split), with one head; every shape three times in a row, then a shape that does not split, then
+    the first one again: the same bits every time and the oracle's values."""
+    from async_gpu_amd import ops, workloads
+    w = workloads.config3_attention(seed=H + kv_len, H=H, seq=stride)
+    q_offset = kv_len - q_len
+    q = w["q"][:, q_offset:kv_len].copy()
+    dq, dk, dv = to_dev(q, dev), to_dev(w["k"], dev), to_dev(w["v"], dev)
+    ref = orc.attention_kv(q, w["k"], w["v"], kv_len=kv_len, q_offset=q_offset)
+    outs = [ops.attention(dq, dk, dv, kv_len=kv_len, q_offset=q_offset).cpu().numpy() for _ in range(3)]
+    assert np.abs(outs[0] - ref).max() <= 1e-5
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+    short = ops.attention(dq[:, :1].contiguous(), dk[:, :256].contiguous(), dv[:, :256].contiguous(), kv_len=200, q_offset=199)
+    ref = orc.attention_kv(q[:, :1], w["k"][:, :256], w["v"][:, :256], kv_len=200, q_offset=199)
+    assert np.abs(short.cpu().numpy() - ref).max() <= 1e-5
+    again = ops.attention(dq, dk, dv, kv_len=kv_len, q_offset=q_offset).cpu().numpy()
+    assert np.array_equal(outs[0], again)
+
+
 @pytest.mark.parametrize("q_len,q_offset", [(4, 60), (8, 0), (40, 24), (33, 31)])
 def test_attention_chunked_prefill(agpu, orc, dev, q_len, q_offset):
     from async_gpu_amd import ops, workloads
