@@ -947,21 +947,33 @@ __device__ __forceinline__ void attn_role(const Params &p, CStage tab, Ctl &c, c
             PK_STAMP(1);
         }
         if (real) {
+            // Rounds go in pairs: a pair's two chains (four multiply-adds, four lane steps each) run side by side, and a
+            // pair beyond the range is skipped as a whole (wave-uniform).  A round without keys inside a pair has zeros
+            // in its registers and scores of -inf.
             float s[KVP];
             float bm = ninf;
 #pragma unroll
-            for (int t = 0; t < KVP; ++t) {
-                s[t] = ninf;
-                if (first + t >= n_rounds) continue;  // wave-uniform: no key of the range in this round
-                const float4 kk = as_f4(kv[2 * t]);
-                float dot = q.x * kk.x;
-                dot = fmaf(q.y, kk.y, dot);
-                dot = fmaf(q.z, kk.z, dot);
-                dot = fmaf(q.w, kk.w, dot);
-                dot = row16_sum(dot) * scale;
-                const int j = r0 + (first + t) * KR + wave * 4 + kq;
-                s[t] = j < r1 ? dot : ninf;
-                bm = fmaxf(bm, s[t]);
+            for (int t2 = 0; t2 < KVP; t2 += 2) {
+                s[t2] = s[t2 + 1] = ninf;
+                if (first + t2 >= n_rounds) continue;  // wave-uniform: no key of the range in this pair
+                float dot[2];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const float4 kk = as_f4(kv[2 * (t2 + u)]);
+                    float d = q.x * kk.x;
+                    d = fmaf(q.y, kk.y, d);
+                    d = fmaf(q.z, kk.z, d);
+                    d = fmaf(q.w, kk.w, d);
+                    dot[u] = d;
+                }
+                dot[0] = row16_sum(dot[0]) * scale;
+                dot[1] = row16_sum(dot[1]) * scale;
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int j = r0 + (first + t2 + u) * KR + wave * 4 + kq;
+                    s[t2 + u] = j < r1 ? dot[u] : ninf;
+                    bm = fmaxf(bm, s[t2 + u]);
+                }
             }
             float s_new = ninf;
             if (with_new && first == 0) {
@@ -979,15 +991,20 @@ __device__ __forceinline__ void attn_role(const Params &p, CStage tab, Ctl &c, c
                 l *= f;
                 o.x *= f; o.y *= f; o.z *= f; o.w *= f;
 #pragma unroll
-                for (int t = 0; t < KVP; ++t) {
-                    if (first + t >= n_rounds) continue;  // wave-uniform
-                    const float pr = s[t] > ninf ? __expf(s[t] - m2) : 0.0f;
-                    const float4 vv = as_f4(kv[2 * t + 1]);
-                    l += pr;
-                    o.x = fmaf(pr, vv.x, o.x);
-                    o.y = fmaf(pr, vv.y, o.y);
-                    o.z = fmaf(pr, vv.z, o.z);
-                    o.w = fmaf(pr, vv.w, o.w);
+                for (int t2 = 0; t2 < KVP; t2 += 2) {
+                    if (first + t2 >= n_rounds) continue;  // wave-uniform
+                    const float pr0 = s[t2] > ninf ? __expf(s[t2] - m2) : 0.0f;
+                    const float pr1 = s[t2 + 1] > ninf ? __expf(s[t2 + 1] - m2) : 0.0f;
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        const float pr = u == 0 ? pr0 : pr1;
+                        const float4 vv = as_f4(kv[2 * (t2 + u) + 1]);
+                        l += pr;
+                        o.x = fmaf(pr, vv.x, o.x);
+                        o.y = fmaf(pr, vv.y, o.y);
+                        o.z = fmaf(pr, vv.z, o.z);
+                        o.w = fmaf(pr, vv.w, o.w);
+                    }
                 }
                 if (s_new > ninf) {
                     const float pr = __expf(s_new - m2);
@@ -1007,8 +1024,8 @@ __device__ __forceinline__ void attn_role(const Params &p, CStage tab, Ctl &c, c
         if (!last_batch && real) prefetch_attn(st.kc, st.vc, p.P, kv, h, r0, r1, nfirst, wave, lane);
         if (last_batch) {
             if (real) {
-                // every lane of a 16-lane row holds the same l: the wave sum counts it 16 times (exactly)
-                const float lw = wave_sum(l) * 0.0625f;
+                // every lane of a 16-lane row holds the same l: the sum over the four rows is the wave's
+                const float lw = rows_sum(l);
                 o.x = rows_sum(o.x);
                 o.y = rows_sum(o.y);
                 o.z = rows_sum(o.z);
@@ -1023,15 +1040,19 @@ __device__ __forceinline__ void attn_role(const Params &p, CStage tab, Ctl &c, c
             PK_STAMP(5);
             float res = 0.0f;  // thread e < 64: o[e]; 64: m; 65: l of this workgroup
             if (real && wave <= 1) {  // whole waves: the weights travel between lanes
+                // every lane works out all W weights itself: W independent exponentials instead of one and W moves
+                // between lanes that each stand between two vector instructions
+                float wmv[W];
                 float mm = ninf;
 #pragma unroll
-                for (int w8 = 0; w8 < W; ++w8) mm = fmaxf(mm, wm[w8]);
-                const float mine = wm[lane & (W - 1)];
-                const float a_mine = mine > ninf ? __expf(mine - mm) : 0.0f;
+                for (int w8 = 0; w8 < W; ++w8) {
+                    wmv[w8] = wm[w8];
+                    mm = fmaxf(mm, wmv[w8]);
+                }
                 float den = 0.0f, num = 0.0f;
 #pragma unroll
                 for (int w8 = 0; w8 < W; ++w8) {
-                    const float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, a_mine), w8));
+                    const float a = wmv[w8] > ninf ? __expf(wmv[w8] - mm) : 0.0f;
                     den = fmaf(a, wl[w8], den);
                     num = fmaf(a, part[w8 * DH + lane], num);
                 }
