@@ -36,6 +36,11 @@ struct PkPlan {
     // Every activation vector of one step, in floats: two sets (steps use them in turn) of eight mirrors (one per XCD),
     // two sets of partial sums, then the arg-max candidates
     unsigned long long *arena = nullptr;
+    // The partial sums and the candidates, which cross XCDs through memory, live in device memory that no cache level
+    // keeps (a hop through it is about 0.2 us shorter); `arena` holds the mirrors only.  Such memory is never freed
+    // while the process runs: a plan returns it to a pool that later plans draw from.
+    float *xmem = nullptr;
+    size_t xmem_bytes = 0;
     size_t arena_elems = 0;  // floats of one mirror
     size_t parts_elems = 0;  // floats of one set of partial sums
     size_t cand_off = 0;     // where the arg-max candidates start (floats)

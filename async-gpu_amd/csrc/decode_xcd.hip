@@ -39,6 +39,7 @@
 #include "decode_step.h"
 
 #include <algorithm>
+#include <mutex>
 #include <vector>
 
 #include "linear_common.h"
@@ -90,7 +91,8 @@ static_assert(sizeof(Stage) % 16 == 0, "stage table is copied in 16-byte pieces"
 struct Params {
     const Stage *stages;  // [8][n_stages]
     int n_stages, n_layer;
-    float *arena;         // [2][8][mirror_elems] mirrors (two sets, one per XCD each), [2][parts_elems] partial sums, the arg-max candidates
+    float *arena;         // [2][8][mirror_elems] mirrors (two sets, one per XCD each)
+    float *xmem;          // [2][parts_elems] partial sums, the arg-max candidates: uncached memory; offsets count on from the mirrors'
     size_t mirror_elems, parts_elems;
     size_t cand_off;
     unsigned *state;      // [0] epoch, [1] error, [2] workgroups started so far
@@ -113,7 +115,7 @@ struct Params {
 
 struct Ctl {
     long oth;        // from a place in this step's set of mirrors to the same place in the other set (floats)
-    float *parts;    // arena + this step's set of partial sums (stage offsets count from the arena's start)
+    float *parts;    // this step's set of partial sums, less the mirrors' 16 mirror_elems (stage offsets count from the mirrors' start)
     long poth;       // the same distance for the partial sums
     uint32_t epoch;
     unsigned *err;
@@ -1251,7 +1253,7 @@ __global__ __launch_bounds__(T) void decode_xcd_kernel(const Params p) {
     const int par = (int)(c.epoch & 1u);
     float *mirror = p.arena + ((size_t)par * 8 + xcd) * p.mirror_elems;
     c.oth = (par ? -1L : 1L) * (long)(8 * p.mirror_elems);
-    c.parts = p.arena + (size_t)par * p.parts_elems;
+    c.parts = p.xmem + ((long)par * (long)p.parts_elems - (long)(16 * p.mirror_elems));
     c.poth = (par ? -1L : 1L) * (long)p.parts_elems;
     if (in_xcd < NR) {
         relay_role<MODE>(p, tab, c, mirror, pos, tok, tid, in_xcd);
@@ -1365,7 +1367,7 @@ __global__ __launch_bounds__(T) void decode_xcd_kernel(const Params p) {
     // ---- arg-max over the workgroups' candidates, token feed ----
     c.stage = p.n_stages;
     check_xcd(p, c, xcd, tid);
-    u64 *cand = reinterpret_cast<u64 *>(p.arena + p.cand_off);
+    u64 *cand = reinterpret_cast<u64 *>(p.xmem + (p.cand_off - 16 * p.mirror_elems));
     best = block_max48(best, L.scr, lane, wave);
     if (tid == 0) {
         // key (32) | index code (16) | low 16 bits of the epoch: the tag of a candidate
@@ -1618,6 +1620,48 @@ bool agpu_step_supported(const agpu_ctx *ctx, const PkModel &m) {
     return true;
 }
 
+// Uncached device memory for what crosses XCDs.  Memory of this kind that a kernel has read is never handed back to
+// the runtime while the process runs; a plan that ends gives its piece to this pool, the next plan of that device that
+// fits takes it from there.
+struct XmemPiece {
+    int device;
+    float *p;
+    size_t bytes;
+};
+static std::mutex g_xmem_mu;
+static std::vector<XmemPiece> g_xmem_pool;
+
+static hipError_t xmem_take(int device, size_t bytes, float **out, size_t *bytes_out) {
+    {
+        std::lock_guard<std::mutex> lock(g_xmem_mu);
+        size_t best = g_xmem_pool.size();
+        for (size_t i = 0; i < g_xmem_pool.size(); ++i)
+            if (g_xmem_pool[i].device == device && g_xmem_pool[i].bytes >= bytes &&
+                (best == g_xmem_pool.size() || g_xmem_pool[i].bytes < g_xmem_pool[best].bytes))
+                best = i;
+        if (best < g_xmem_pool.size()) {
+            *out = g_xmem_pool[best].p;
+            *bytes_out = g_xmem_pool[best].bytes;
+            g_xmem_pool.erase(g_xmem_pool.begin() + (long)best);
+            return hipSuccess;
+        }
+    }
+    void *p = nullptr;
+    const hipError_t e = hipExtMallocWithFlags(&p, bytes, hipDeviceMallocUncached);
+    if (e != hipSuccess) return e;
+    *out = static_cast<float *>(p);
+    *bytes_out = bytes;
+    return hipSuccess;
+}
+
+static void xmem_give(float *p, size_t bytes) {
+    int device = 0;
+    hipPointerAttribute_t attr{};
+    if (hipPointerGetAttributes(&attr, p) == hipSuccess) device = attr.device;
+    std::lock_guard<std::mutex> lock(g_xmem_mu);
+    g_xmem_pool.push_back(XmemPiece{device, p, bytes});
+}
+
 int32_t agpu_step_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
     agpu_step_plan_free(plan);
     if (!agpu_step_supported(ctx, m)) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "decode step: model shape not supported by the one-launch step");
@@ -1668,9 +1712,11 @@ int32_t agpu_step_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
     plan->cand_off = cand_off;
     plan->arena_elems = mirror_elems;
     plan->parts_elems = parts_elems;
-    const size_t arena_bytes = total * sizeof(float);
+    const size_t arena_bytes = part_base * sizeof(float);
+    plan->xmem_bytes = (total - part_base) * sizeof(float);
     if (e == hipSuccess) e = hipMalloc(&plan->stages_dev, st.size() * sizeof(Stage));
     if (e == hipSuccess) e = hipMalloc((void **)&plan->arena, arena_bytes);
+    if (e == hipSuccess) e = xmem_take(ctx->device, plan->xmem_bytes, &plan->xmem, &plan->xmem_bytes);
     if (e == hipSuccess) e = hipMalloc((void **)&plan->state, 64);
     if (e == hipSuccess) e = hipMemcpy(plan->stages_dev, st.data(), st.size() * sizeof(Stage), hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipMemsetAsync(plan->state, 0, 64, ctx->stream);
@@ -1736,6 +1782,7 @@ int32_t agpu_step_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
 void agpu_step_plan_free(PkPlan *plan) {
     if (plan->stages_dev) (void)hipFree(plan->stages_dev);
     if (plan->arena) (void)hipFree(plan->arena);
+    if (plan->xmem) xmem_give(plan->xmem, plan->xmem_bytes);
     if (plan->state) (void)hipFree(plan->state);
     if (plan->ln_fold) (void)hipFree(plan->ln_fold);
     *plan = PkPlan{};
@@ -1744,10 +1791,10 @@ void agpu_step_plan_free(PkPlan *plan) {
 // Every place "not written yet" (all-ones words), the candidates zero: on the stream the step runs on, and waited for
 // (a fill still under way when a step starts would leave words that are neither all-ones nor a value of the step).
 int32_t agpu_step_reset(agpu_ctx *ctx, const PkPlan &plan) {
-    const size_t total = plan.cand_off + 2 * (size_t)plan.grid + 2;
-    float *a = reinterpret_cast<float *>(plan.arena);
-    hipError_t e = hipMemsetAsync(a, 0xFF, plan.cand_off * sizeof(float), ctx->stream);
-    if (e == hipSuccess) e = hipMemsetAsync(a + plan.cand_off, 0, (total - plan.cand_off) * sizeof(float), ctx->stream);
+    const size_t total = plan.cand_off + 2 * (size_t)plan.grid + 2, part_base = 16 * plan.arena_elems;
+    hipError_t e = hipMemsetAsync(plan.arena, 0xFF, part_base * sizeof(float), ctx->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(plan.xmem, 0xFF, (plan.cand_off - part_base) * sizeof(float), ctx->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(plan.xmem + (plan.cand_off - part_base), 0, (total - plan.cand_off) * sizeof(float), ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     return agpu_hip(ctx, e, "decode step: arena");
 }
@@ -1772,6 +1819,7 @@ int32_t agpu_step_launch(agpu_ctx *ctx, const PkModel &m, const PkPlan &plan, in
     p.n_stages = plan.n_stages;
     p.n_layer = m.n_layer;
     p.arena = reinterpret_cast<float *>(plan.arena);
+    p.xmem = plan.xmem;
     p.mirror_elems = plan.arena_elems;
     p.parts_elems = plan.parts_elems;
     p.cand_off = plan.cand_off;

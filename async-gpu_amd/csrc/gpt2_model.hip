@@ -214,7 +214,7 @@ unsigned long long step_addresses(const agpu_gpt2 *m, bool one_launch) {
                           (const void *)m->lm_head.scales, (const void *)m->ctx->workspace, (const void *)m->ctx->counters})
         mix(p);
     if (one_launch)  // the step's plan; a graph of per-stage launches does not refer to it
-        for (const void *p : {(const void *)m->pk.arena, (const void *)m->pk.stages_dev, (const void *)m->pk.state, (const void *)m->pk.ln_fold}) mix(p);
+        for (const void *p : {(const void *)m->pk.arena, (const void *)m->pk.xmem, (const void *)m->pk.stages_dev, (const void *)m->pk.state, (const void *)m->pk.ln_fold}) mix(p);
     for (const DevBuf *b : {&m->hid, &m->qkv, &m->att, &m->ffn, &m->lnb, &m->last, &m->logits, &m->tok_in, &m->px_h, &m->px_att, &m->px_ffn,
                             &m->px_stats, &m->px_fold})
         mix(b->p);
@@ -1336,7 +1336,7 @@ AGPU_EXPORT int32_t agpu_gpt2_decode_steps(agpu_gpt2 *m, int32_t batch, int32_t 
 }
 
 #ifdef AGPU_PK_TRACE
-// Debug builds only: the one-launch step's arena (device pointer, bytes of one mirror, of one set of partial sums).
+// Debug builds only: the one-launch step's mirrors (device pointer, floats of one mirror) and the floats of one set of partial sums.
 AGPU_EXPORT int32_t agpu_gpt2_debug_arena(agpu_gpt2 *m, void **arena_out, unsigned long long *mirror_elems, unsigned long long *parts_elems) {
     if (!m || !m->pk.arena) return AGPU_ERR_UNSUPPORTED;
     *arena_out = m->pk.arena;
