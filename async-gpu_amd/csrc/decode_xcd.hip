@@ -64,7 +64,10 @@ constexpr int DH = 64;
 constexpr int NR = AGPU_XK_NR;  // relay workgroups per XCD
 constexpr int XI = 4;           // groups of four columns a relay thread owns at most
 constexpr uint32_t SENT = 0xFFFFFFFFu;  // "not written yet"
-constexpr int NPRE = 3;         // slots whose nibbles are converted ahead of the input
+#ifndef AGPU_XK_NPRE
+#define AGPU_XK_NPRE 4
+#endif
+constexpr int NPRE = AGPU_XK_NPRE;         // slots whose nibbles are converted ahead of the input
 
 enum : int { F_LN = 1, F_GELU_TANH = 2, F_GELU_QUICK = 4, F_HEAD = 8, F_SCATTER = 16, F_PARTIAL = 32 };
 
