@@ -46,6 +46,7 @@ struct PkPlan {
     size_t cand_off = 0;     // where the arg-max candidates start (floats)
     unsigned int *state = nullptr;  // [0] number of the last finished step, [1] error word (0 = none), [2] workgroups started, [8..15] XCD of each class
     int grid = 0;
+    int nr = 0;           // relay workgroups per XCD
     int att_per_xcd = 0;  // workgroups per XCD that only do attention
     int smax = 1;         // key ranges per head at most
     int lin_per_xcd = 0;  // Linear workgroups per XCD

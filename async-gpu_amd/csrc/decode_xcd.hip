@@ -61,7 +61,7 @@ constexpr int DH = 64;
 #ifndef AGPU_XK_NR
 #define AGPU_XK_NR 4
 #endif
-constexpr int NR = AGPU_XK_NR;  // relay workgroups per XCD
+constexpr int NR = AGPU_XK_NR;  // relay workgroups per XCD for models of up to 16 heads; one more beyond (Params.nr says)
 constexpr int XI = 4;           // groups of four columns a relay thread owns at most
 constexpr uint32_t SENT = 0xFFFFFFFFu;  // "not written yet"
 #ifndef AGPU_XK_NPRE
@@ -108,6 +108,7 @@ struct Params {
     float eps;
     int argmax_last;
     int att_per_xcd, smax, nlin;
+    int nr;               // relay workgroups per XCD
     int spin_limit;
     int xbuf;             // floats of one staging buffer
     int head_slots;       // how many of a workgroup's head slots (from its first) wait in LDS when the head stage begins
@@ -734,9 +735,9 @@ __device__ __forceinline__ void head_finish(const Params &p, const Stage &st, co
 // ---- relay ----
 constexpr int TK = 6;  // cache lines of one stage's weights a relay thread touches at most
 // One word of every 128 bytes of the XCD's share of a stage's weights, so that they wait in the XCD's L2 when the Linear
-// workgroups request them: thread tid of relay r takes the lines tid + r T + s NR T.  The loaded words are handed back;
+// workgroups request them: thread tid of relay r of nr takes the lines tid + r T + s nr T.  The loaded words are handed back;
 // the caller keeps them until after its next poll, so nothing but that poll waits for them.
-__device__ __forceinline__ void touch_stage(CStage e, int tid, int r, uint32_t (&tk)[TK]) {
+__device__ __forceinline__ void touch_stage(CStage e, int tid, int r, int nr, uint32_t (&tk)[TK]) {
     const int n_units = e->n_units;
     if (n_units <= 0) return;  // workgroup-uniform
     const int n_cparts = e->n_cparts, stride = e->stride, K = e->K;
@@ -749,7 +750,7 @@ __device__ __forceinline__ void touch_stage(CStage e, int tid, int r, uint32_t (
     const size_t row_b = (size_t)stride * 4;
 #pragma unroll
     for (int s = 0; s < TK; ++s) {
-        const int i = tid + r * T + s * NR * T;
+        const int i = tid + r * T + s * nr * T;
         if (i < n_all) {
             const int part = i / per_part, q = i - part * per_part;
             const int row = q / lpr, line = q - row * lpr;
@@ -763,12 +764,12 @@ __device__ __forceinline__ void touch_stage(CStage e, int tid, int r, uint32_t (
 // The exchanges of the step, for relay r of the XCD: thread (cq_local, part) = (tid >> 3, tid & 7) polls the partial
 // sum of XCD `part` for the groups of four columns r cqs + cq_local + 64 k; the eight lanes of such a group add up what
 // they got, and lane 0 of them adds bias and residual, keeps the result as the next residual and stores it into the mirror.
-template <int MODE>
+template <int MODE, int NRT>
 __device__ __forceinline__ void relay_role(const Params &p, CStage tab, Ctl &c, float *mirror, int pos, uint32_t tok, int tid, int r) {
     const bool real = MODE == 0;
     const int part = tid & 7, cql = tid >> 3;
     const int quads = p.d >> 2;
-    const int cqs = (quads + NR - 1) / NR;
+    const int cqs = (quads + NRT - 1) / NRT;
     const int n_it = (cqs + 63) >> 6;  // <= XI
     float4 res[XI];
     bool valid[XI];
@@ -792,8 +793,8 @@ __device__ __forceinline__ void relay_role(const Params &p, CStage tab, Ctl &c, 
     // the weights of the first half layers, as far ahead as the later ones will be touched
     if (real && p.touch_dist > 0)
         for (int hh = 0; hh < min(p.touch_dist + 1, n_half); ++hh) {
-            touch_stage(tab + 2 * hh, tid, r, tk0);
-            touch_stage(tab + 2 * hh + 1, tid, r, tk1);
+            touch_stage(tab + 2 * hh, tid, r, NRT, tk0);
+            touch_stage(tab + 2 * hh + 1, tid, r, NRT, tk1);
         }
     for (int x = 0; x < n_half; ++x) {
         CStage e = tab + 2 * x + 1;  // the partial-sum stage in front of this exchange
@@ -856,8 +857,8 @@ __device__ __forceinline__ void relay_role(const Params &p, CStage tab, Ctl &c, 
         PK_STAMP(7);
         // half layer x + 1 begins now: the weights of the one touch_dist further on
         if (real && p.touch_dist > 0 && x + 1 + p.touch_dist < n_half) {
-            touch_stage(tab + 2 * (x + 1 + p.touch_dist), tid, r, tk0);
-            touch_stage(tab + 2 * (x + 1 + p.touch_dist) + 1, tid, r, tk1);
+            touch_stage(tab + 2 * (x + 1 + p.touch_dist), tid, r, NRT, tk0);
+            touch_stage(tab + 2 * (x + 1 + p.touch_dist) + 1, tid, r, NRT, tk1);
         }
     }
 #pragma unroll
@@ -1211,7 +1212,7 @@ __device__ __forceinline__ void check_xcd(const Params &p, Ctl &c, int xcd, int 
     if ((w & 15u) != xcc_id()) atomicCAS(c.err, 0u, 0x2000u + (unsigned)xcd);
 }
 
-template <int MODE>
+template <int MODE, int NRT>  // NRT: relay workgroups per XCD (a constant of the instantiation: 1 % of a step against a kernel argument)
 __global__ __launch_bounds__(T) void decode_xcd_kernel(const Params p) {
     extern __shared__ __align__(16) float smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -1258,20 +1259,20 @@ __global__ __launch_bounds__(T) void decode_xcd_kernel(const Params p) {
     c.oth = (par ? -1L : 1L) * (long)(8 * p.mirror_elems);
     c.parts = p.xmem + ((long)par * (long)p.parts_elems - (long)(16 * p.mirror_elems));
     c.poth = (par ? -1L : 1L) * (long)p.parts_elems;
-    if (in_xcd < NR) {
-        relay_role<MODE>(p, tab, c, mirror, pos, tok, tid, in_xcd);
+    if (in_xcd < NRT) {
+        relay_role<MODE, NRT>(p, tab, c, mirror, pos, tok, tid, in_xcd);
         check_xcd(p, c, xcd, tid);
         PK_DUMP();
         return;
     }
-    const bool is_att = in_xcd < NR + p.att_per_xcd;
+    const bool is_att = in_xcd < NRT + p.att_per_xcd;
     const int nlin = p.nlin;
-    const int li = in_xcd - NR - p.att_per_xcd;  // Linear workgroup of its XCD
+    const int li = in_xcd - NRT - p.att_per_xcd;  // Linear workgroup of its XCD
     // in the head, Linear workgroups are numbered XCD by XCD (neighbouring tiles, which read neighbouring pieces of the
     // same weight rows, meet in one L2); attention workgroups follow them
-    const int att_a = in_xcd - NR;
+    const int att_a = in_xcd - NRT;
     const int rank = is_att ? 8 * nlin + att_a * 8 + xcd : xcd * nlin + li;
-    const int n_head_wgs = G - 8 * NR;
+    const int n_head_wgs = G - 8 * NRT;
     (void)per_xcd;
 
     if (is_att) {
@@ -1427,16 +1428,21 @@ bool linear_ok(const PkLinear &l) {
 }
 
 struct Roles {
-    int G, att_per_xcd, smax, nlin;
+    int G, att_per_xcd, smax, nlin, nr;
 };
 
 Roles plan_roles(const agpu_ctx *ctx, int H) {
     Roles r{};
     r.G = (ctx->num_cus / 8) * 8;
     const int hx = ceil_div(H, 8);  // heads of an XCD at most
-    r.smax = NR <= 2 ? (hx <= 2 ? 3 : (hx <= 4 ? 2 : 1)) : (NR <= 4 && hx <= 2 ? 2 : 1);
+    // Relays per XCD: with up to two heads per XCD four, which leaves room for two key ranges per head (more relays and
+    // one range are 1 % faster up to 256 keys of context and 9 % slower at 700); beyond, where a head has one range
+    // anyway, five (XL shape 0.950 -> 0.937 ms per step, large shape 0.528 -> 0.511; six: 0.935 and 0.536).
+    r.nr = hx <= 2 ? NR : NR + 1;
+    if (const char *env = getenv("AGPU_XK_RELAYS")) r.nr = atoi(env) == NR + 1 ? NR + 1 : NR;  // the two instantiations of the kernel
+    r.smax = r.nr <= 2 ? (hx <= 2 ? 3 : (hx <= 4 ? 2 : 1)) : (r.nr <= 4 && hx <= 2 ? 2 : 1);
     r.att_per_xcd = hx * r.smax;
-    r.nlin = r.G / 8 - NR - r.att_per_xcd;
+    r.nlin = r.G / 8 - r.nr - r.att_per_xcd;
     return r;
 }
 
@@ -1589,7 +1595,7 @@ bool build_tables(const PkModel &m, const Roles &r, int lin_groups, size_t part_
             prev_h2 = o_h2;
         }
         Stage hs;
-        if (!plan_head(hs, m.head, r.G - 8 * NR)) return false;
+        if (!plan_head(hs, m.head, r.G - 8 * r.nr)) return false;
         hs.in_off = prev_h2; hs.flags = F_LN | F_HEAD; hs.ln_g = m.lnf_g; hs.ln_b = m.lnf_b;
         hs.xbias = fold + fold_layer * m.n_layer; hs.bias = hs.xbias + m.head.N;  // A and B
         out[(size_t)x * n_st + 4 * m.n_layer] = hs;
@@ -1603,8 +1609,8 @@ bool build_tables(const PkModel &m, const Roles &r, int lin_groups, size_t part_
 bool agpu_step_supported(const agpu_ctx *ctx, const PkModel &m) {
     const Roles r = plan_roles(ctx, m.H);
     // eight XCDs of 32 CUs: the roles and the hand-offs through an L2 are laid out for this part
-    if (ctx->num_cus != 256 || r.nlin < 8 || m.H < 1 || r.G - 8 * NR > T) return false;
-    if (m.d != m.H * DH || m.d % 32 != 0 || m.d > XMAX || m.d / 4 > NR * 64 * XI) return false;
+    if (ctx->num_cus != 256 || r.nlin < 8 || m.H < 1 || r.G - 8 * r.nr > T) return false;
+    if (m.d != m.H * DH || m.d % 32 != 0 || m.d > XMAX || m.d / 4 > r.nr * 64 * XI) return false;
     if (m.ff % 32 != 0 || m.ff < 32 || m.V > 65535 || m.V < 1 || m.n_layer < 1 || m.group != 32) return false;
     if (!linear_ok(m.head) || m.head.K != m.d) return false;
     for (int L = 0; L < m.n_layer; ++L) {
@@ -1710,6 +1716,7 @@ int32_t agpu_step_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
     plan->n_stages = 4 * m.n_layer + 1;
     plan->grid = r.G;
     plan->att_per_xcd = r.att_per_xcd;
+    plan->nr = r.nr;
     plan->smax = r.smax;
     plan->lin_per_xcd = r.nlin;
     plan->cand_off = cand_off;
@@ -1748,9 +1755,9 @@ int32_t agpu_step_plan_build(agpu_ctx *ctx, const PkModel &m, PkPlan *plan) {
     // the largest request any plan can make, once per device: the attribute belongs to the kernel, not to a plan
     static bool attr_set[64] = {false};
     if (e == hipSuccess && !attr_set[ctx->device & 63]) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(decode_xcd_kernel<0>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(decode_xcd_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        for (const void *k : {reinterpret_cast<const void *>(decode_xcd_kernel<0, NR>), reinterpret_cast<const void *>(decode_xcd_kernel<1, NR>),
+                              reinterpret_cast<const void *>(decode_xcd_kernel<0, NR + 1>), reinterpret_cast<const void *>(decode_xcd_kernel<1, NR + 1>)})
+            if (e == hipSuccess) e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e == hipSuccess) attr_set[ctx->device & 63] = true;
     }
     // Where the workgroups land: b, b + 8, ... must share an XCD.  A launch shaped like the step's is looked at here;
@@ -1832,6 +1839,7 @@ int32_t agpu_step_launch(agpu_ctx *ctx, const PkModel &m, const PkPlan &plan, in
     p.pos_dev = m.pos_dev; p.step_dev = m.step_dev; p.out_capacity = m.out_capacity;
     p.d = m.d; p.H = m.H; p.P = m.P; p.V = m.V; p.eps = m.eps; p.argmax_last = m.argmax_last;
     p.att_per_xcd = plan.att_per_xcd;
+    p.nr = plan.nr;
     p.smax = plan.smax;
     p.nlin = plan.lin_per_xcd;
     p.spin_limit = plan.spin_limit > 0 ? plan.spin_limit : kSpinLimit;
@@ -1840,7 +1848,13 @@ int32_t agpu_step_launch(agpu_ctx *ctx, const PkModel &m, const PkPlan &plan, in
     p.red_floats = red_floats_for(plan.head_tpc);
     p.touch_dist = plan.touch_dist;
     p.trace = trace;
-    if (mode == 0) hipLaunchKernelGGL(decode_xcd_kernel<0>, dim3(plan.grid), dim3(T), plan.lds_bytes, ctx->stream, p);
-    else hipLaunchKernelGGL(decode_xcd_kernel<1>, dim3(plan.grid), dim3(T), plan.lds_bytes, ctx->stream, p);
+    if (plan.nr != NR && plan.nr != NR + 1) return agpu_fail(ctx, AGPU_ERR_UNSUPPORTED, "decode step: no kernel for %d relays per XCD", plan.nr);
+    if (plan.nr == NR) {
+        if (mode == 0) hipLaunchKernelGGL((decode_xcd_kernel<0, NR>), dim3(plan.grid), dim3(T), plan.lds_bytes, ctx->stream, p);
+        else hipLaunchKernelGGL((decode_xcd_kernel<1, NR>), dim3(plan.grid), dim3(T), plan.lds_bytes, ctx->stream, p);
+    } else {
+        if (mode == 0) hipLaunchKernelGGL((decode_xcd_kernel<0, NR + 1>), dim3(plan.grid), dim3(T), plan.lds_bytes, ctx->stream, p);
+        else hipLaunchKernelGGL((decode_xcd_kernel<1, NR + 1>), dim3(plan.grid), dim3(T), plan.lds_bytes, ctx->stream, p);
+    }
     return AGPU_LAUNCH_CHECK(ctx, "decode_xcd_kernel");
 }

@@ -107,7 +107,7 @@ def stamp_table(which, xl_layers, _lib, gpt2, workloads):
     t0 = tr[tr > 0].min()
     tr = np.where(tr > 0, (tr - t0) * 10, -1)
     hx = (cfg["n_head"] + 7) // 8
-    n_relay, n_att = 4, hx * (2 if hx <= 2 else 1)  # roles per XCD as decode_xcd.hip plans them
+    n_relay, n_att = (4 if hx <= 2 else 5), hx * (2 if hx <= 2 else 1)  # roles per XCD as decode_xcd.hip plans them
     in_xcd = np.arange(G) >> 3
     relay, att = in_xcd < n_relay, (in_xcd >= n_relay) & (in_xcd < n_relay + n_att)
     lin = ~relay & ~att
