@@ -512,6 +512,18 @@ def test_gpt2_inference_cpp_example_program(orc, agpu, dev, tmp_path):
     finally:
         model.close()
     assert len(got) == 3
+    # the tied int4 head (--int4-head) against the Python model with the same head
+    r = subprocess.run([prog, model_path, vocab_path, "--max-new-tokens", "12", "--print-tokens", "--int4-head", "--prompt", "Once upon a time"],
+                       capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stderr
+    assert r.stdout.count("MATCH: cached and non-cached outputs agree") == 1
+    ids = [[int(x) for x in ln.split()[1:]] for ln in r.stdout.splitlines() if ln.startswith("Tokens:")][0]
+    model = gpt2.Int4Gpt2Model.from_file(model_path, group_size=32, mode=_lib.QUANT_RUST, lm_head=gpt2.LM_HEAD_INT4)
+    try:
+        (ref,), _ = model.generate_cached(np.asarray(tok.encode("Once upon a time"), np.uint32), 12)
+        assert ids == [int(t) for t in ref]
+    finally:
+        model.close()
 
 
 def test_forward_profiled_and_diagnostic(tiny, orc, agpu, dev):
