@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, GB/s
 # of the LM-head GEMV (profiles/gemv_lm_head_pmc_traffic.md) and of the one-launch decode step
 # (profiles/decode_step_gpt2_small_pmc_traffic.md); None where not measured.
 TRAFFIC_BYTES_LM_HEAD = 24617000
-TRAFFIC_BYTES_DECODE_STEP = 101696400  # at contexts 64 .. 132; 85.1 MB algorithmic there
+TRAFFIC_BYTES_DECODE_STEP = 101621500  # at contexts 64 .. 132; 85.1 MB algorithmic there
 
 
 def step_bytes(cfg, group, context_len):
